@@ -1,0 +1,178 @@
+"""Benchmark of the CherryQ hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all]
+
+A step is one fused CherryLinear matvec (batch 1) over one packed layer resident in HBM.  The
+default workload is the headline configuration: LLaMA-7B gate/up shape 4096 -> 11008, 4-bit,
+group 128, 1/256 cherry channels.  Every step uses a different copy of the packed layer, cycling
+through enough copies (> 512 MB) that nothing is served from the 256 MB Infinity Cache.
+
+Prints one JSON line:  metric = microseconds per matvec (whole-job, HIP events around the K
+timed launches on the launch stream);  roofline = algorithmic bytes per launch / that time,
+against the 8 TB/s HBM peak;  cpu_baseline = the reference's CPU path (unpack + linear) as
+restated by the C oracle, timed on this host.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for p in (str(ROOT), str(ROOT / "mixed-precision-cuda-kernel_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (w_bits, in_features, out_features)
+    "llama7b_gate_up_w4": (4, 4096, 11008),
+    "llama7b_gate_up_w3": (3, 4096, 11008),
+    "llama7b_down_w4": (4, 11008, 4096),
+    "llama7b_down_w3": (3, 11008, 4096),
+    "llama7b_attn_w4": (4, 4096, 4096),
+    "llama7b_attn_w3": (3, 4096, 4096),
+    "llama13b_attn_w3": (3, 5120, 5120),
+    "llama13b_gate_up_w3": (3, 5120, 13824),
+    "llama13b_down_w3": (3, 13824, 5120),
+    "llama70b_attn_w4": (4, 8192, 8192),
+    "llama70b_kv_w4": (4, 8192, 1024),
+    "llama70b_gate_up_w4": (4, 8192, 28672),
+    "llama70b_down_w4": (4, 28672, 8192),
+}
+
+
+def algorithmic_bytes(bits, k, n, batch=1, group=128):
+    """Bytes one call must move: packed codes + scales + cherry rows + indices + x + y."""
+    c = -(-k // 256) // 8 * 8
+    kn = k - c
+    return kn // 8 * bits * n + -(-kn // group) * n * 2 + c * n * 2 + c * 2 + batch * k * 2 + batch * n * 2
+
+
+def make_copies(bits, k, n, group, min_bytes, seed=0):
+    """Distinct packed layers (random codes, plausible scales) totalling > min_bytes on the GPU."""
+    import numpy as np
+    import torch
+    from oracle import cherryq_oracle as orc
+    base = orc.synthetic_packed_fast(k, n, bits, group, seed=seed)
+    per = sum(v.nbytes for v in base.values())
+    ncopies = max(2, -(-min_bytes // per))
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    copies = []
+    for i in range(ncopies):
+        t = {name: torch.from_numpy(v).cuda() for name, v in base.items()}
+        if i:
+            t["qweight"] = torch.randint(0, 256, base["qweight"].shape, dtype=torch.uint8, device="cuda", generator=g)
+        copies.append(t)
+    return base, copies
+
+
+def time_gpu(bits, k, n, group, steps, warmup, batch=1):
+    import numpy as np
+    import torch
+    import quant_cuda
+    base, copies = make_copies(bits, k, n, group, 640 << 20)
+    x = torch.from_numpy(np.random.default_rng(1).standard_normal((batch, k)).astype(np.float16)).cuda()
+    out = torch.zeros(batch, n, dtype=torch.float16, device="cuda")
+
+    def step(i):
+        t = copies[i % len(copies)]
+        quant_cuda.matmul_cherryq(bits, x, t["qweight"], t["cherry_weight"], t["cherry_indices"], t["scales"], out,
+                                  group, accumulate=False)
+
+    stream = torch.cuda.current_stream()
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for i in range(steps):
+        step(warmup + i)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dev_us = e0.elapsed_time(e1) * 1e3 / steps
+    return dev_us, wall * 1e6 / steps, base, x, out, copies
+
+
+def cpu_baseline(bits, k, n, group, base, x_np):
+    """The reference CPU path -- QuantLinear.unpack() then linear -- restated in C (oracle),
+    timed on this host: cold = unpack + matvec, cached = matvec on the dense fp16 weight."""
+    import numpy as np
+    from oracle import c_oracle
+    threads = c_oracle.threads()
+    dense = np.zeros((n, k), dtype=np.float16)
+    c_oracle.dequant_matmul(x_np, base, bits, group, dense)  # warm-up
+    reps, cold = 0, []
+    t_end = time.perf_counter() + 8.0
+    while reps < 20 and (reps < 3 or time.perf_counter() < t_end):
+        t0 = time.perf_counter()
+        c_oracle.dequant_matmul(x_np, base, bits, group, dense)
+        cold.append(time.perf_counter() - t0)
+        reps += 1
+    cached = []
+    for _ in range(max(3, reps)):
+        t0 = time.perf_counter()
+        c_oracle.linear(x_np, dense)
+        cached.append(time.perf_counter() - t0)
+    cold_us = float(np.median(cold)) * 1e6
+    return {"value": round(cold_us, 1), "unit": "us/matvec", "cores": threads, "kind": "port",
+            "sample": f"{reps} calls of unpack()+linear on the same {k}x{n} {bits}-bit layer, median; "
+                      f"cached dense fp16 linear alone: {float(np.median(cached)) * 1e6:.1f} us"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--workload", default="llama7b_gate_up_w4", choices=sorted(WORKLOADS))
+    ap.add_argument("--group", type=int, default=128)
+    ap.add_argument("--all", action="store_true", help="also print a table of every workload to stderr")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures the hot path on ONE GPU; --gpus N > 1 is not supported "
+              "(the path shards by output columns without any exchange, see DESIGN.md).", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    torch.cuda.set_device(0)
+
+    if args.all:
+        for name, (bits, k, n) in WORKLOADS.items():
+            us, wall_us, *_ = time_gpu(bits, k, n, args.group, max(200, args.steps // 4), args.warmup)
+            ab = algorithmic_bytes(bits, k, n, 1, args.group)
+            print(f"{name:24s} {bits}-bit {k:5d}->{n:5d}: {us:7.2f} us/matvec  {ab / us / 1e3:7.1f} GB/s  "
+                  f"{ab / us / 1e3 / HBM_PEAK_GBS * 100:5.1f}% of 8 TB/s  (host wall {wall_us:.2f} us)",
+                  file=sys.stderr, flush=True)
+            torch.cuda.empty_cache()
+
+    bits, k, n = WORKLOADS[args.workload]
+    us, wall_us, base, x, out, copies = time_gpu(bits, k, n, args.group, args.steps, args.warmup)
+    ab = algorithmic_bytes(bits, k, n, 1, args.group)
+    gbs = ab / us / 1e3
+    result = {
+        "metric": "us_per_matvec", "value": round(us, 3), "unit": "us", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us / 1e3, 6),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16xu%d->f32" % bits,
+        "data": "synthetic",
+        "config": {"workload": args.workload, "w_bits": bits, "in_features": k, "out_features": n,
+                   "group_size": args.group, "batch": 1, "cherries": -(-k // 256) // 8 * 8,
+                   "weight_copies_rotated": len(copies), "host_wall_us_per_call": round(wall_us, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": ab, "kernel": f"cq::matvec_kernel<{bits}>"},
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(bits, k, n, args.group, base, x.cpu().numpy())
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

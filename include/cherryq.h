@@ -1,0 +1,125 @@
+/*
+ * libcherryq -- C ABI of the MI355X (gfx950) implementation of CherryQ's mixed-precision
+ * quantized linear: packed 3/4-bit group-wise weights + fp16 "cherry" input channels.
+ *
+ * This header is the drop-in boundary.  It replaces the pybind11 module `quant_cuda` of
+ * the reference (csrc/quant_cuda.cpp:72-77) and the four host launchers behind it
+ * (csrc/quant_cuda_kernel.cu:117-188, 675-716, 838-866, 925-953).  All pointers are
+ * device pointers owned by the caller; nothing here allocates, frees or synchronises.
+ * Every call enqueues work on `stream` (a hipStream_t passed as void*; NULL = the null
+ * stream) of the device that is current in the calling thread, and returns at once.
+ *
+ * Tensor layouts (row-major, contiguous), with K = in_features, N = out_features,
+ * C = num_cherries, Kn = K - C, b = w_bits, G = group_size:
+ *   vec            (B, K)            fp16 (or fp32 for the *_f32 entry point)
+ *   qweight        (Kn/8*b, N)       uint8   llama/qlinear.py:51-54, packing :86-116
+ *   cherry_weight  (C, N)            fp16    llama/qlinear.py:47-50
+ *   cherry_indices (C,)              int16, ascending (int32 for *_f32)  llama/qlinear.py:43-46
+ *   scales         (ceil(Kn/G), N)   fp16    llama/qlinear.py:55-58
+ *   mul            (B, N)            fp16, accumulated into (mul += x W^T) when
+ *                                    `accumulate` != 0, overwritten otherwise
+ *
+ * Return value: 0 on success; negative = rejected argument (CHERRYQ_E_*); positive = a
+ * hipError_t reported by the launch.  cherryq_status_string() names either.
+ */
+#ifndef CHERRYQ_H
+#define CHERRYQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CHERRYQ_VERSION 1
+
+enum {
+    CHERRYQ_OK = 0,
+    CHERRYQ_E_NULL = -1,        /* a required pointer is NULL */
+    CHERRYQ_E_SHAPE = -2,       /* dimensions inconsistent with the buffer schema */
+    CHERRYQ_E_GROUP = -3,       /* unsupported group size for this entry point */
+    CHERRYQ_E_WORKSPACE = -4,   /* workspace missing, misaligned or too small */
+    CHERRYQ_E_BITS = -5,        /* w_bits is not 3 or 4 */
+    CHERRYQ_E_ALIGN = -6,       /* a pointer is not aligned as the kernels require */
+    CHERRYQ_E_UNSUPPORTED = -7  /* valid request that this build does not implement */
+};
+
+int cherryq_version(void);
+const char *cherryq_status_string(int status);
+
+/*
+ * Split-K workspace.  The fused entry points split the reduction over K across
+ * workgroups; partial sums and per-tile arrival counters live in a caller-provided
+ * device buffer of at least cherryq_workspace_bytes() bytes, 256-byte aligned.  Its first
+ * cherryq_workspace_counter_bytes() bytes must be zero before the first call; every call
+ * leaves them zero again.  Calls that may overlap in time (different streams) must use
+ * different workspaces.  Has no counterpart in the reference, whose kernels add fp16
+ * partials into `mul` with atomics (csrc/quant_cuda_kernel.cu:833).
+ */
+size_t cherryq_workspace_bytes(int batch, int in_features, int out_features, int num_cherries);
+size_t cherryq_workspace_counter_bytes(int out_features);
+
+/*
+ * Replaces quant_cuda.vecquant4matmul_cherryq (csrc/quant_cuda.cpp:56-69,
+ * csrc/quant_cuda_kernel.cu:675-835).  group_size must be a multiple of 32 that is
+ * >= 128 (the reference rejects < 128, :684, and silently assumes a multiple of 128).
+ */
+int cherryq_vecquant4matmul_f16(const void *vec, const uint8_t *qweight, const void *cherry_weight,
+                                const int16_t *cherry_indices, const void *scales, void *mul,
+                                int batch, int in_features, int out_features, int num_cherries,
+                                int group_size, int accumulate, void *workspace,
+                                size_t workspace_bytes, void *stream);
+
+/*
+ * Replaces quant_cuda.vecquant3matmul_cherryq with fp16=True (csrc/quant_cuda.cpp:41-54,
+ * csrc/quant_cuda_kernel.cu:117-188, kernels :316-438 for group 64 and :558-672 for
+ * multiples of 128).  group_size must be a multiple of 32; the reference silently does
+ * nothing for group sizes other than 64 or a multiple of 128.
+ */
+int cherryq_vecquant3matmul_f16(const void *vec, const uint8_t *qweight, const void *cherry_weight,
+                                const int16_t *cherry_indices, const void *scales, void *mul,
+                                int batch, int in_features, int out_features, int num_cherries,
+                                int group_size, int accumulate, void *workspace,
+                                size_t workspace_bytes, void *stream);
+
+/*
+ * Replaces quant_cuda.vecquant3matmul_cherryq with fp16=False: fp32 vec / cherry_weight /
+ * scales / mul and int32 cherry_indices (csrc/quant_cuda_kernel.cu:191-314, 441-556;
+ * caller: benchmark_speed.py:20-32).
+ */
+int cherryq_vecquant3matmul_f32(const float *vec, const uint8_t *qweight, const float *cherry_weight,
+                                const int32_t *cherry_indices, const float *scales, float *mul,
+                                int batch, int in_features, int out_features, int num_cherries,
+                                int group_size, int accumulate, void *workspace,
+                                size_t workspace_bytes, void *stream);
+
+/*
+ * Replace quant_cuda.Dequantize3Normal / Dequantize4Normal (csrc/quant_cuda.cpp:26-38,
+ * csrc/quant_cuda_kernel.cu:838-1010): out[k, n] = (code(k, n) - c_b) * scales[k / G, n]
+ * for the Kn compacted normal positions, fp32 scales and fp32 out of shape (>= Kn, N).
+ * `height` is in_features.  The reference's 4-bit launcher indexes rows with the 3-bit
+ * block height (:934, :964) and so covers only part of the matrix; this one covers all
+ * of it.
+ */
+int cherryq_dequantize3_normal_f32(const uint8_t *qweight, const float *scales, float *out,
+                                   int height, int out_features, int cherry_size, int group_size,
+                                   void *stream);
+int cherryq_dequantize4_normal_f32(const uint8_t *qweight, const float *scales, float *out,
+                                   int height, int out_features, int cherry_size, int group_size,
+                                   void *stream);
+
+/*
+ * Device-side QuantLinear.unpack() (llama/qlinear.py:120-162): the dense (N, K) fp16
+ * weight, normal column normal[k] = RN16((code - c_b) * scale) bit for bit as the
+ * reference's torch code computes it, cherry column idx[c] = cherry_weight[c, :].
+ */
+int cherryq_unpack_f16(int w_bits, const uint8_t *qweight, const void *cherry_weight,
+                       const int16_t *cherry_indices, const void *scales, void *dense,
+                       int in_features, int out_features, int num_cherries, int group_size,
+                       void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CHERRYQ_H */

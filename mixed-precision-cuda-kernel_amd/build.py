@@ -1,0 +1,70 @@
+"""Builds libcherryq.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
+
+    python build.py            # rebuild if any source is newer than the library
+    python build.py --force
+
+No CUDAExtension / hipify: the sources are HIP written for CDNA4 and are compiled directly.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+HERE = Path(__file__).resolve().parent
+CSRC = HERE / "csrc"
+OBJ = HERE / "build"
+LIB = HERE / "libcherryq.so"
+SOURCES = ["cq_api.hip", "cq_generic.hip", "cq_matvec.hip"]
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
+]
+
+
+def _deps():
+    return list(CSRC.glob("*")) + [HERE.parent / "include" / "cherryq.h", Path(__file__)]
+
+
+def needs_build() -> bool:
+    if not LIB.exists():
+        return True
+    t = LIB.stat().st_mtime
+    return any(p.stat().st_mtime > t for p in _deps())
+
+
+def build(force: bool = False, verbose: bool = False) -> Path:
+    if not force and not needs_build():
+        return LIB
+    OBJ.mkdir(exist_ok=True)
+
+    def compile_one(src):
+        out = OBJ / (src + ".o")
+        cmd = [HIPCC, *FLAGS, "-c", str(CSRC / src), "-o", str(out)]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        msgs = "\n".join(l for l in (r.stdout + r.stderr).splitlines()
+                         if "packed-fp32-ops" not in l and l.strip())
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {src}:\n{msgs}")
+        if verbose and msgs:
+            print(msgs)
+        return out
+
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
+        objs = list(ex.map(compile_one, SOURCES))
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", str(LIB), *map(str, objs)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + r.stdout + r.stderr)
+    return LIB
+
+
+if __name__ == "__main__":
+    p = build(force="--force" in sys.argv, verbose=True)
+    print(f"built {p} ({p.stat().st_size} bytes)")

@@ -1,0 +1,173 @@
+// extern "C" entry points of libcherryq: argument validation and kernel selection.
+// Declarations and the reference interfaces they replace: include/cherryq.h.
+#include "../../include/cherryq.h"
+
+#include "cq_common.cuh"
+#include "cq_kernels.h"
+
+namespace cq {
+
+// The smallest units_per_wg any kernel uses is 1, which bounds the split count by the unit count.
+size_t workspace_counter_bytes(int N) {
+    size_t tiles = (size_t)ceil_div(N > 0 ? N : 1, kTileCols);
+    return (tiles * sizeof(unsigned) + 255) / 256 * 256;
+}
+
+size_t workspace_bytes(int B, int K, int N, int C) {
+    if (B < 1) B = 1;
+    if (K < 8) K = 8;
+    if (C < 0) C = 0;
+    if (C > K) C = K;
+    // one slot of partial sums per unit (128 normal positions or 32 cherry rows) bounds every
+    // split factor the kernels use; batch rows are processed at most 16 at a time
+    size_t units = (size_t)ceil_div(K - C, kUnitK) + (size_t)ceil_div(C, kCherryUnit) + 1;
+    size_t rows = (size_t)(B < 16 ? B : 16);
+    return workspace_counter_bytes(N) + units * rows * (size_t)(N > 0 ? N : 1) * sizeof(float);
+}
+
+static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+static int check_common(const void *vec, const void *qweight, const void *cherry_weight,
+                        const void *cherry_indices, const void *scales, const void *mul, int B, int K, int N,
+                        int C, int G, void *workspace, size_t workspace_bytes_given) {
+    if (B < 0 || K <= 0 || N <= 0 || C < 0 || C > K) return CHERRYQ_E_SHAPE;
+    if (K % 8 || N % 8 || C % 8) return CHERRYQ_E_SHAPE;
+    if (K - C <= 0 && C == 0) return CHERRYQ_E_SHAPE;
+    if (G <= 0 || G % 32) return CHERRYQ_E_GROUP;
+    if (!vec || !mul) return CHERRYQ_E_NULL;
+    if (K - C > 0 && (!qweight || !scales)) return CHERRYQ_E_NULL;
+    if (C > 0 && (!cherry_weight || !cherry_indices)) return CHERRYQ_E_NULL;
+    if (!aligned(qweight, 16) || !aligned(scales, 16) || !aligned(cherry_weight, 16) || !aligned(vec, 4) ||
+        !aligned(mul, 16) || !aligned(cherry_indices, 4))
+        return CHERRYQ_E_ALIGN;
+    if (!workspace || !aligned(workspace, 256) || workspace_bytes_given < workspace_bytes(B, K, N, C))
+        return CHERRYQ_E_WORKSPACE;
+    return CHERRYQ_OK;
+}
+
+template <int BITS>
+static int matmul_f16(const void *vec, const uint8_t *qweight, const void *cherry_weight,
+                      const int16_t *cherry_indices, const void *scales, void *mul, int B, int K, int N,
+                      int C, int G, int accumulate, void *workspace, size_t wsb, void *stream) {
+    int rc = check_common(vec, qweight, cherry_weight, cherry_indices, scales, mul, B, K, N, C, G, workspace,
+                          wsb);
+    if (rc) return rc;
+    if (B == 0) return CHERRYQ_OK;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const __half *x = reinterpret_cast<const __half *>(vec);
+    const __half *cw = reinterpret_cast<const __half *>(cherry_weight);
+    const __half *sc = reinterpret_cast<const __half *>(scales);
+    __half *y = reinterpret_cast<__half *>(mul);
+    hipError_t e;
+    if (matvec_supported(BITS, B, K, N, C, G)) {
+        e = hipSuccess;
+        for (int b = 0; b < B && e == hipSuccess; b++)
+            e = launch_matvec(BITS, x + (size_t)b * K, qweight, cw, cherry_indices, sc, y + (size_t)b * N, K,
+                              N, C, G, accumulate, workspace, s);
+    } else {
+        e = launch_generic<BITS, __half, int16_t>(x, qweight, cw, cherry_indices, sc, y, B, K, N, C, G,
+                                                  accumulate, workspace, s);
+    }
+    return (int)e;
+}
+
+}  // namespace cq
+
+extern "C" {
+
+int cherryq_version(void) { return CHERRYQ_VERSION; }
+
+const char *cherryq_status_string(int status) {
+    switch (status) {
+        case CHERRYQ_OK: return "ok";
+        case CHERRYQ_E_NULL: return "a required pointer is NULL";
+        case CHERRYQ_E_SHAPE: return "dimensions inconsistent with the packed buffer schema";
+        case CHERRYQ_E_GROUP: return "unsupported group_size for this entry point";
+        case CHERRYQ_E_WORKSPACE: return "workspace missing, misaligned or too small";
+        case CHERRYQ_E_BITS: return "w_bits must be 3 or 4";
+        case CHERRYQ_E_ALIGN: return "a pointer is not aligned as the kernels require";
+        case CHERRYQ_E_UNSUPPORTED: return "request not implemented by this build";
+        default: break;
+    }
+    if (status > 0) return hipGetErrorString((hipError_t)status);
+    return "unknown status";
+}
+
+size_t cherryq_workspace_bytes(int batch, int in_features, int out_features, int num_cherries) {
+    return cq::workspace_bytes(batch, in_features, out_features, num_cherries);
+}
+
+size_t cherryq_workspace_counter_bytes(int out_features) { return cq::workspace_counter_bytes(out_features); }
+
+int cherryq_vecquant4matmul_f16(const void *vec, const uint8_t *qweight, const void *cherry_weight,
+                                const int16_t *cherry_indices, const void *scales, void *mul, int batch,
+                                int in_features, int out_features, int num_cherries, int group_size,
+                                int accumulate, void *workspace, size_t workspace_bytes, void *stream) {
+    if (group_size < 128) return CHERRYQ_E_GROUP;  // csrc/quant_cuda_kernel.cu:684
+    return cq::matmul_f16<4>(vec, qweight, cherry_weight, cherry_indices, scales, mul, batch, in_features,
+                             out_features, num_cherries, group_size, accumulate, workspace, workspace_bytes,
+                             stream);
+}
+
+int cherryq_vecquant3matmul_f16(const void *vec, const uint8_t *qweight, const void *cherry_weight,
+                                const int16_t *cherry_indices, const void *scales, void *mul, int batch,
+                                int in_features, int out_features, int num_cherries, int group_size,
+                                int accumulate, void *workspace, size_t workspace_bytes, void *stream) {
+    return cq::matmul_f16<3>(vec, qweight, cherry_weight, cherry_indices, scales, mul, batch, in_features,
+                             out_features, num_cherries, group_size, accumulate, workspace, workspace_bytes,
+                             stream);
+}
+
+int cherryq_vecquant3matmul_f32(const float *vec, const uint8_t *qweight, const float *cherry_weight,
+                                const int32_t *cherry_indices, const float *scales, float *mul, int batch,
+                                int in_features, int out_features, int num_cherries, int group_size,
+                                int accumulate, void *workspace, size_t workspace_bytes, void *stream) {
+    int rc = cq::check_common(vec, qweight, cherry_weight, cherry_indices, scales, mul, batch, in_features,
+                              out_features, num_cherries, group_size, workspace, workspace_bytes);
+    if (rc) return rc;
+    if (batch == 0) return CHERRYQ_OK;
+    return (int)cq::launch_generic<3, float, int32_t>(vec, qweight, cherry_weight, cherry_indices, scales, mul,
+                                                      batch, in_features, out_features, num_cherries,
+                                                      group_size, accumulate, workspace,
+                                                      reinterpret_cast<hipStream_t>(stream));
+}
+
+static int dequantize_normal(int bits, const uint8_t *qweight, const float *scales, float *out, int height,
+                             int N, int C, int G, void *stream) {
+    if (height <= 0 || N <= 0 || C < 0 || C > height || height % 8 || N % 8 || C % 8) return CHERRYQ_E_SHAPE;
+    if (G <= 0 || G % 8) return CHERRYQ_E_GROUP;
+    if (height - C == 0) return CHERRYQ_OK;
+    if (!qweight || !scales || !out) return CHERRYQ_E_NULL;
+    if (!cq::aligned(qweight, 4) || !cq::aligned(scales, 16) || !cq::aligned(out, 16)) return CHERRYQ_E_ALIGN;
+    return (int)cq::launch_dequant_normal(bits, qweight, scales, out, height - C, N, G,
+                                          reinterpret_cast<hipStream_t>(stream));
+}
+
+int cherryq_dequantize3_normal_f32(const uint8_t *qweight, const float *scales, float *out, int height,
+                                   int out_features, int cherry_size, int group_size, void *stream) {
+    return dequantize_normal(3, qweight, scales, out, height, out_features, cherry_size, group_size, stream);
+}
+
+int cherryq_dequantize4_normal_f32(const uint8_t *qweight, const float *scales, float *out, int height,
+                                   int out_features, int cherry_size, int group_size, void *stream) {
+    return dequantize_normal(4, qweight, scales, out, height, out_features, cherry_size, group_size, stream);
+}
+
+int cherryq_unpack_f16(int w_bits, const uint8_t *qweight, const void *cherry_weight,
+                       const int16_t *cherry_indices, const void *scales, void *dense, int in_features,
+                       int out_features, int num_cherries, int group_size, void *stream) {
+    if (w_bits != 3 && w_bits != 4) return CHERRYQ_E_BITS;
+    int K = in_features, N = out_features, C = num_cherries;
+    if (K <= 0 || N <= 0 || C < 0 || C > K || K % 8 || N % 8 || C % 8) return CHERRYQ_E_SHAPE;
+    if (group_size <= 0 || group_size % 8) return CHERRYQ_E_GROUP;
+    if (!dense) return CHERRYQ_E_NULL;
+    if (K - C > 0 && (!qweight || !scales)) return CHERRYQ_E_NULL;
+    if (C > 0 && (!cherry_weight || !cherry_indices)) return CHERRYQ_E_NULL;
+    if (!cq::aligned(qweight, 4) || !cq::aligned(scales, 2) || !cq::aligned(dense, 2)) return CHERRYQ_E_ALIGN;
+    return (int)cq::launch_unpack(w_bits, qweight, reinterpret_cast<const __half *>(cherry_weight),
+                                  cherry_indices, reinterpret_cast<const __half *>(scales),
+                                  reinterpret_cast<__half *>(dense), K, N, C, group_size,
+                                  reinterpret_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

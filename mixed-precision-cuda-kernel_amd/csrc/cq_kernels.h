@@ -1,0 +1,31 @@
+// Internal launch interface between the C ABI (cq_api.hip) and the kernel files.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace cq {
+
+size_t workspace_counter_bytes(int N);
+size_t workspace_bytes(int B, int K, int N, int C);
+
+// cq_generic.hip
+template <int BITS, typename IO, typename IDX>
+hipError_t launch_generic(const IO *vec, const uint8_t *qweight, const IO *cherry_weight,
+                          const IDX *cherry_indices, const IO *scales, IO *mul, int B, int K, int N,
+                          int C, int G, int accumulate, void *workspace, hipStream_t stream);
+hipError_t launch_dequant_normal(int bits, const uint8_t *qweight, const float *scales, float *out, int Kn,
+                                 int N, int G, hipStream_t stream);
+hipError_t launch_unpack(int bits, const uint8_t *qweight, const __half *cherry_weight,
+                         const int16_t *cherry_indices, const __half *scales, __half *dense, int K, int N,
+                         int C, int G, hipStream_t stream);
+
+// cq_matvec.hip: batch-1 HBM-streaming matvec.  Returns false when the shape is not one it takes.
+bool matvec_supported(int bits, int B, int K, int N, int C, int G);
+hipError_t launch_matvec(int bits, const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
+                         const int16_t *cherry_indices, const __half *scales, __half *mul, int K, int N,
+                         int C, int G, int accumulate, void *workspace, hipStream_t stream);
+
+}  // namespace cq

@@ -1,0 +1,332 @@
+// Batch-1 fused dequant + matvec for gfx950, built as an HBM stream.
+//
+// Work unit: 128 compacted normal positions x 256 output columns (16 KB of 4-bit, 12 KB of
+// 3-bit weights), or 32 cherry rows x 256 columns.  One wavefront owns one unit: the 64 lanes
+// form 4 lane groups (16-lane DPP rows) that split the 128 positions four ways, and the 16
+// lanes of a row each own 16 adjacent columns, so every load is a dwordx4 and a row of lanes
+// reads 256 contiguous bytes of one byte row.  A wavefront issues all 16 (12) weight loads
+// up front and consumes them in order as they land.  Four wavefronts (four consecutive units
+// of one column tile) form a workgroup; the K reduction runs lane -> DPP row -> permlane
+// swaps across rows -> LDS across wavefronts -> split-K partials across workgroups.
+//
+// Codes never pass through an int->float conversion.  A code field masked in place inside a
+// 16-bit half is the fp16 subnormal  code * 2^(p-24)  (p = bit position of the field), which
+// v_dot2_f32_f16 multiplies exactly against fp16 activations and accumulates in fp32:
+//   4-bit: two byte rows are interleaved per column with one v_perm_b32; the low-nibble pair
+//          and the high-nibble pair are two masks and two dot2 (5 VALU ops per 4 weights).
+//   3-bit: three byte rows of a column give the 24-bit unit in two v_perm_b32; four masks pick
+//          the code pairs (0,3) (1,4) (5,6) (2,7), whose different bit positions are folded
+//          into the activations as exact powers of two (11 VALU ops per 8 weights).
+// The grid offset c_b = 7.5 / 3.5 is applied once per lane group as  -c_b * sum(x).
+//
+// Arithmetic contract: csrc/quant_cuda_kernel.cu:718-835 (4-bit) and 558-672 / 316-438
+// (3-bit); fp32 accumulation throughout, one rounding to fp16 at the end.
+#include "cq_common.cuh"
+#include "cq_kernels.h"
+
+namespace cq {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kMaxFastCherries = 128;  // two 64-lane chunks of cherry indices
+constexpr uint32_t kRsrcFlags = 0x00020000u;
+constexpr uint32_t kOob = 0x80000000u;  // byte offset beyond any buffer this kernel accepts
+
+__device__ inline float fdot2(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a), __builtin_bit_cast(half2_t, b), c, false);
+}
+
+// all-reduce over the 16 lanes of a DPP row by rotations 8, 4, 2, 1
+__device__ inline float row_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x122, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xf, 0xf, false));
+    return v;
+}
+
+__device__ inline int row_max(int v) {
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x128, 0xf, 0xf, false));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x124, 0xf, 0xf, false));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x122, 0xf, 0xf, false));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x121, 0xf, 0xf, false));
+    return v;
+}
+
+__device__ inline float half_bits_to_float(uint32_t h) {
+    return __half2float(__ushort_as_half((unsigned short)h));
+}
+
+// Sum `a` over lanes l, l^32 for the lower half of the wave and `b` for the upper half:
+// lanes < 32 return a[l] + a[l+32], lanes >= 32 return b[l-32] + b[l].
+__device__ inline float swap32_add(float a, float b) {
+    auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, a), __builtin_bit_cast(unsigned, b),
+                                              false, false);
+    return __builtin_bit_cast(float, r[0]) + __builtin_bit_cast(float, r[1]);
+}
+
+// Same across the two rows of each half: even rows return a[row] + a[row+1], odd rows b + b.
+__device__ inline float swap16_add(float a, float b) {
+    auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, a), __builtin_bit_cast(unsigned, b),
+                                              false, false);
+    return __builtin_bit_cast(float, r[0]) + __builtin_bit_cast(float, r[1]);
+}
+
+template <int BITS>
+struct Geo {
+    static constexpr int kRowsPerLaneGroup = BITS == 4 ? 16 : 12;  // byte rows holding 32 positions
+    static constexpr int kRowsPerUnit = 4 * kRowsPerLaneGroup;
+};
+
+template <int BITS>
+__global__ __launch_bounds__(256) void matvec_kernel(
+    const __half *__restrict__ x, const uint8_t *__restrict__ qweight, const __half *__restrict__ cherry_weight,
+    const int16_t *__restrict__ cherry_indices, const __half *__restrict__ scales, __half *__restrict__ mul,
+    float *__restrict__ partial, unsigned *__restrict__ tickets, int K, int N, int C, int G, int accumulate,
+    Plan plan) {
+    constexpr int R = Geo<BITS>::kRowsPerLaneGroup;
+    __shared__ uint32_t s_win[4][128];  // per wave: 256 fp16 activations starting at the unit's first position
+    __shared__ uint32_t s_pair[4][64];  // per wave: activation pairs laid out for the dot2 operands
+    __shared__ float s_red[4][kTileCols];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int kq = lane >> 4, nl = lane & 15;
+    const int lid = xcd_remap(blockIdx.x, gridDim.x);
+    const int tile = lid / plan.splits;
+    const int split = lid % plan.splits;
+    const int u = split * 4 + wave;
+    const int n0 = tile * kTileCols + nl * 16;
+    const bool col_ok = n0 < N;
+    const int Kn = K - C;
+
+    float tot[16];
+#pragma unroll
+    for (int c = 0; c < 16; c++) tot[c] = 0.f;
+
+    if (u < plan.units_normal) {
+        const int ubase = u * kUnitK;
+        // ---- small operands first: vmcnt retires in order, so these can be waited on while
+        // the weight loads issued after them are still in flight
+        const __amdgpu_buffer_rsrc_t ri =
+            __builtin_amdgcn_make_buffer_rsrc((void *)cherry_indices, 0, C * 2, kRsrcFlags);
+        const int i0 = (short)__builtin_amdgcn_raw_buffer_load_b16(ri, lane * 2, 0, 0);
+        const int i1 = (short)__builtin_amdgcn_raw_buffer_load_b16(ri, (lane + 64) * 2, 0, 0);
+        const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, K * 2, kRsrcFlags);
+        const uint32_t win0 = __builtin_amdgcn_raw_buffer_load_b32(rx, (ubase + 2 * lane) * 2, 0, 0);
+        const uint32_t win1 = __builtin_amdgcn_raw_buffer_load_b32(rx, (ubase + 128 + 2 * lane) * 2, 0, 0);
+        const int ng = ceil_div(Kn, G);
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)scales, 0, ng * N * 2, kRsrcFlags);
+        const int g = (ubase + 32 * kq) / G;
+        const uint32_t soff = col_ok ? (uint32_t)(g * N + n0) * 2u : kOob;
+        const u32x4 sc0 = __builtin_amdgcn_raw_buffer_load_b128(rs, soff, 0, 0);
+        const u32x4 sc1 = __builtin_amdgcn_raw_buffer_load_b128(rs, soff + 16, 0, 0);
+
+        // ---- the weight stream: R byte rows x 16 columns per lane, rows past the end read 0
+        const int qrows = Kn / 8 * BITS;
+        const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void *)qweight, 0, qrows * N, kRsrcFlags);
+        const uint32_t woff = col_ok ? (uint32_t)((u * Geo<BITS>::kRowsPerUnit + kq * R) * N + n0) : kOob;
+        u32x4 w[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) w[r] = __builtin_amdgcn_raw_buffer_load_b128(rw, woff + (uint32_t)(r * N), 0, 0);
+
+        // ---- gather the unit's 128 activations around the cherry channels
+        // t[m] = idx[m] - m is non-decreasing; position k sits after every m with t[m] <= k
+        const int t0 = lane < C ? i0 - lane : 0x7fffffff;
+        const int t1 = lane + 64 < C ? i1 - (lane + 64) : 0x7fffffff;
+        s_win[wave][lane] = win0;
+        s_win[wave][64 + lane] = win1;
+        // positions this lane prepares, relative to the lane group's first position
+        int j0, j1, p0 = 0, p1 = 0;
+        if (BITS == 4) {
+            j0 = 4 * (nl >> 1) + (nl & 1);  // even lanes: (4p, 4p+2), odd lanes: (4p+1, 4p+3)
+            j1 = j0 + 2;
+        } else {
+            const int q = nl & 3, t8 = 8 * (nl >> 2);  // code pairs (0,3) (1,4) (5,6) (2,7) of a unit
+            j0 = t8 + ((0x2510 >> (4 * q)) & 15);
+            j1 = t8 + ((0x7643 >> (4 * q)) & 15);
+            p0 = (0x6730 >> (4 * q)) & 15;  // bit position of the first code's field in its half
+            p1 = (0x5241 >> (4 * q)) & 15;
+        }
+        const int k0 = ubase + 32 * kq + j0, k1 = ubase + 32 * kq + j1;
+        int low0 = __popcll(__ballot(t0 < ubase)) + __popcll(__ballot(t1 < ubase));
+        int low1 = low0;
+        {
+            unsigned long long m = __ballot(t0 >= ubase && t0 < ubase + kUnitK);
+            while (m) {
+                int j = __builtin_ctzll(m);
+                int tj = __builtin_amdgcn_readlane(t0, j);
+                low0 += tj <= k0;
+                low1 += tj <= k1;
+                m &= m - 1;
+            }
+            m = __ballot(t1 >= ubase && t1 < ubase + kUnitK);
+            while (m) {
+                int j = __builtin_ctzll(m);
+                int tj = __builtin_amdgcn_readlane(t1, j);
+                low0 += tj <= k0;
+                low1 += tj <= k1;
+                m &= m - 1;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const unsigned short *winh = reinterpret_cast<const unsigned short *>(&s_win[wave][0]);
+        uint32_t h0 = (k0 < Kn) ? winh[(k0 - ubase) + low0] : 0u;
+        uint32_t h1 = (k1 < Kn) ? winh[(k1 - ubase) + low1] : 0u;
+        const float xsum = row_sum(half_bits_to_float(h0) + half_bits_to_float(h1));
+        int sh = 0;
+        if (BITS == 3) {
+            // scale the lane group's activations so that the largest has biased exponent 29;
+            // the per-field factors 2^-p (p <= 7) then stay far inside the fp16 normal range
+            const int e = row_max((int)max(h0 & 0x7fffu, h1 & 0x7fffu)) >> 10;
+            sh = 29 - e;
+            h0 = __half_as_ushort(__float2half_rn(ldexpf(half_bits_to_float(h0), sh - p0)));
+            h1 = __half_as_ushort(__float2half_rn(ldexpf(half_bits_to_float(h1), sh - p1)));
+        }
+        s_pair[wave][lane] = h0 | (h1 << 16);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        u32x4 xq[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) xq[i] = *reinterpret_cast<const u32x4 *>(&s_pair[wave][16 * kq + 4 * i]);
+
+        if (BITS == 4) {
+            float lo[16], hi[16];
+#pragma unroll
+            for (int c = 0; c < 16; c++) lo[c] = hi[c] = 0.f;
+#pragma unroll
+            for (int p = 0; p < 8; p++) {
+                const uint32_t xe = xq[p >> 1][(p & 1) * 2], xo = xq[p >> 1][(p & 1) * 2 + 1];
+#pragma unroll
+                for (int d = 0; d < 4; d++) {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        // bytes (row 2p col j, 0, row 2p+1 col j, 0)
+                        const uint32_t pr = __builtin_amdgcn_perm(w[2 * p][d], w[2 * p + 1][d],
+                                                                  0x0c000c00u | (uint32_t)(j << 16) | (uint32_t)(4 + j));
+                        lo[4 * d + j] = fdot2(pr & 0x000f000fu, xe, lo[4 * d + j]);
+                        hi[4 * d + j] = fdot2(pr & 0x00f000f0u, xo, hi[4 * d + j]);
+                    }
+                }
+            }
+            const float corr = -7.5f * xsum;
+#pragma unroll
+            for (int c = 0; c < 16; c++) {
+                const uint32_t sw = c < 8 ? sc0[c >> 1] : sc1[(c - 8) >> 1];
+                const float s = half_bits_to_float((c & 1) ? (sw >> 16) : (sw & 0xffffu));
+                tot[c] = (lo[c] * 16777216.0f + hi[c] * 1048576.0f + corr) * s;
+            }
+        } else {
+            float acc[16];
+#pragma unroll
+            for (int c = 0; c < 16; c++) acc[c] = 0.f;
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const uint32_t xa = xq[t][0], xb = xq[t][1], xc = xq[t][2], xd = xq[t][3];
+#pragma unroll
+                for (int d = 0; d < 4; d++) {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const uint32_t sel = 0x0c000000u | (uint32_t)(j << 16) | (uint32_t)(j << 8) | (uint32_t)(4 + j);
+                        // p1 = bits 0..15 of the 24-bit unit | its bits 8..15 again in the high half
+                        // p2 = bits 8..23 of the unit        | its bits 16..23 in the high half
+                        const uint32_t p1 = __builtin_amdgcn_perm(w[3 * t][d], w[3 * t + 1][d], sel);
+                        const uint32_t p2 = __builtin_amdgcn_perm(w[3 * t + 1][d], w[3 * t + 2][d], sel);
+                        float a = acc[4 * d + j];
+                        a = fdot2(p1 & 0x000e0007u, xa, a);                            // codes 0 | 3
+                        a = fdot2(p1 & 0x00700038u, xb, a);                            // codes 1 | 4
+                        a = fdot2(p2 & 0x001c0380u, xc, a);                            // codes 5 | 6
+                        a = fdot2((p1 & 0x000001c0u) | (p2 & 0x00e00000u), xd, a);     // codes 2 | 7
+                        acc[4 * d + j] = a;
+                    }
+                }
+            }
+            const float corr = -3.5f * xsum;
+#pragma unroll
+            for (int c = 0; c < 16; c++) {
+                const uint32_t sw = c < 8 ? sc0[c >> 1] : sc1[(c - 8) >> 1];
+                const float s = half_bits_to_float((c & 1) ? (sw >> 16) : (sw & 0xffffu));
+                tot[c] = (ldexpf(acc[c], 24 - sh) + corr) * s;
+            }
+        }
+    } else if (u < plan.units_total) {
+        // ---- cherry unit: 32 rows of fp16 weights, 8 per lane group, times x[idx[c]]
+        const int c0 = (u - plan.units_normal) * kCherryUnit + 8 * kq;
+        const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc((void *)cherry_weight, 0, C * N * 2, kRsrcFlags);
+        const uint32_t coff = col_ok ? (uint32_t)(c0 * N + n0) * 2u : kOob;
+        const __amdgpu_buffer_rsrc_t ri =
+            __builtin_amdgcn_make_buffer_rsrc((void *)cherry_indices, 0, C * 2, kRsrcFlags);
+        const int ci = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(ri, (c0 + (nl & 7)) * 2, 0, 0);
+        u32x4 cw[8][2];
+#pragma unroll
+        for (int r = 0; r < 8; r++) {
+            cw[r][0] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff + (uint32_t)(r * N * 2), 0, 0);
+            cw[r][1] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff + (uint32_t)(r * N * 2) + 16, 0, 0);
+        }
+        const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, K * 2, kRsrcFlags);
+        const uint32_t xoff = (nl < 8 && c0 + nl < C) ? (uint32_t)ci * 2u : kOob;
+        const float xv = half_bits_to_float(__builtin_amdgcn_raw_buffer_load_b16(rx, xoff, 0, 0));
+        s_pair[wave][lane] = __builtin_bit_cast(uint32_t, xv);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        float xc[8];
+#pragma unroll
+        for (int r = 0; r < 8; r++) xc[r] = __builtin_bit_cast(float, s_pair[wave][16 * kq + r]);
+#pragma unroll
+        for (int r = 0; r < 8; r++) {
+#pragma unroll
+            for (int c = 0; c < 16; c++) {
+                const uint32_t ww = cw[r][c >> 3][(c & 7) >> 1];
+                tot[c] += half_bits_to_float((c & 1) ? (ww >> 16) : (ww & 0xffffu)) * xc[r];
+            }
+        }
+    }
+
+    // ---- reduce over the four lane groups; lane group kq ends up with columns 4kq .. 4kq+3
+    float h8[8], q4[4];
+#pragma unroll
+    for (int i = 0; i < 8; i++) h8[i] = swap32_add(tot[i], tot[8 + i]);
+#pragma unroll
+    for (int i = 0; i < 4; i++) q4[i] = swap16_add(h8[i], h8[4 + i]);
+    *reinterpret_cast<float4 *>(&s_red[wave][16 * nl + 4 * kq]) = make_float4(q4[0], q4[1], q4[2], q4[3]);
+    __syncthreads();
+    float vals[1][1];
+    vals[0][0] = (s_red[0][tid] + s_red[1][tid]) + (s_red[2][tid] + s_red[3][tid]);
+    const int n = tile * kTileCols + tid;
+    splitk_finish<__half, 1, 1>(vals, 1, N, n, n < N, tile, split, plan.splits, partial, tickets, mul, accumulate);
+}
+
+bool matvec_supported(int bits, int B, int K, int N, int C, int G) {
+    (void)bits;
+    if (B < 1 || B > 4) return false;
+    if (C > kMaxFastCherries) return false;
+    if (G % 32) return false;
+    // byte offsets are 32-bit and kOob must lie beyond every buffer
+    const long long wbytes = (long long)(K - C) / 8 * 4 * N;
+    const long long cbytes = (long long)C * N * 2;
+    const long long sbytes = (long long)ceil_div(K - C, G) * N * 2;
+    if (wbytes >= 0x7fff0000ll || cbytes >= 0x7fff0000ll || sbytes >= 0x7fff0000ll) return false;
+    return K - C > 0;
+}
+
+hipError_t launch_matvec(int bits, const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
+                         const int16_t *cherry_indices, const __half *scales, __half *mul, int K, int N, int C,
+                         int G, int accumulate, void *workspace, hipStream_t stream) {
+    Plan plan = make_plan(K, N, C, 4);
+    unsigned *tickets = reinterpret_cast<unsigned *>(workspace);
+    float *partial =
+        reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + workspace_counter_bytes(N));
+    dim3 grid(plan.tiles * plan.splits), block(256);
+    if (bits == 4)
+        hipLaunchKernelGGL(matvec_kernel<4>, grid, block, 0, stream, vec, qweight, cherry_weight, cherry_indices,
+                           scales, mul, partial, tickets, K, N, C, G, accumulate, plan);
+    else
+        hipLaunchKernelGGL(matvec_kernel<3>, grid, block, 0, stream, vec, qweight, cherry_weight, cherry_indices,
+                           scales, mul, partial, tickets, K, N, C, G, accumulate, plan);
+    return hipGetLastError();
+}
+
+}  // namespace cq

@@ -1,0 +1,234 @@
+"""`quant_cuda` for MI355X: the reference extension's four entry points over libcherryq.
+
+Drop-in for the pybind11 module built from csrc/quant_cuda.cpp:72-77 of the reference:
+
+    vecquant3matmul_cherryq(vec, qweight, cherry_weight, cherry_indices, scaling_factors, mul, group_size, fp16)
+    vecquant4matmul_cherryq(vec, qweight, cherry_weight, cherry_indices, scaling_factors, mul, group_size)
+    Dequantize3Normal(qweight, scaling_factors, out, height, cherry_size, group_size)
+    Dequantize4Normal(qweight, scaling_factors, out, height, cherry_size, group_size)
+
+Same positional arguments, same in-place accumulate into `mul`, nothing returned.  The work is
+done by hand-written HIP kernels in libcherryq.so (C ABI: include/cherryq.h), reached through
+ctypes with raw device pointers; torch only supplies memory and the current stream.  There is no
+CPU or eager fallback: importing this module without the built library raises, and so does any
+call with tensors that are not on a GPU.
+
+Differences from the reference, all on the side of failing loudly (the reference launches on
+the legacy default stream without checking anything, csrc/quant_cuda_kernel.cu:140,699):
+kernels run on torch's current stream; dtype / device / shape / contiguity mismatches raise
+RuntimeError; group sizes the kernels cannot honour raise instead of silently doing nothing
+(csrc/quant_cuda_kernel.cu:139-179).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from pathlib import Path
+
+import torch
+
+_HERE = Path(__file__).resolve().parent
+_LIB_PATH = Path(os.environ.get("CHERRYQ_LIB", _HERE / "libcherryq.so"))
+
+if not _LIB_PATH.exists():
+    raise ImportError(
+        f"quant_cuda: {_LIB_PATH} is not built. Run `python {_HERE / 'build.py'}` "
+        "(hipcc, --offload-arch=gfx950); there is no fallback implementation.")
+
+_lib = ctypes.CDLL(str(_LIB_PATH))
+
+_vp, _int, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+_MATMUL_ARGS = [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _vp, _sz, _vp]
+for _name in ("cherryq_vecquant4matmul_f16", "cherryq_vecquant3matmul_f16", "cherryq_vecquant3matmul_f32"):
+    getattr(_lib, _name).argtypes = _MATMUL_ARGS
+    getattr(_lib, _name).restype = _int
+for _name in ("cherryq_dequantize3_normal_f32", "cherryq_dequantize4_normal_f32"):
+    getattr(_lib, _name).argtypes = [_vp, _vp, _vp, _int, _int, _int, _int, _vp]
+    getattr(_lib, _name).restype = _int
+_lib.cherryq_unpack_f16.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp]
+_lib.cherryq_unpack_f16.restype = _int
+_lib.cherryq_workspace_bytes.argtypes = [_int, _int, _int, _int]
+_lib.cherryq_workspace_bytes.restype = _sz
+_lib.cherryq_workspace_counter_bytes.argtypes = [_int]
+_lib.cherryq_workspace_counter_bytes.restype = _sz
+_lib.cherryq_status_string.argtypes = [_int]
+_lib.cherryq_status_string.restype = ctypes.c_char_p
+_lib.cherryq_version.restype = _int
+
+LIBRARY_PATH = str(_LIB_PATH)
+
+
+def _fail(status: int, what: str):
+    raise RuntimeError(f"{what}: {_lib.cherryq_status_string(status).decode()} (status {status})")
+
+
+def _check(t: torch.Tensor, name: str, dtype, ndim: int, device=None):
+    if not isinstance(t, torch.Tensor):
+        raise RuntimeError(f"{name} must be a torch.Tensor")
+    if t.dtype != dtype:
+        raise RuntimeError(f"{name}: expected dtype {dtype}, got {t.dtype}")
+    if t.dim() != ndim:
+        raise RuntimeError(f"{name}: expected {ndim} dimensions, got {tuple(t.shape)}")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on a GPU (got {t.device}); there is no CPU path")
+    if device is not None and t.device != device:
+        raise RuntimeError(f"{name} is on {t.device}, expected {device}")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+# Split-K scratch: one zero-initialised buffer per (device, stream), grown on demand.  The
+# kernels leave the counter region zero after every call, so the buffer is reusable as is.
+_workspaces: dict = {}
+
+
+def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
+    key = (device.index, stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def _ptr(t: torch.Tensor):
+    return t.data_ptr() if t.numel() else None
+
+
+def _matmul(fn, what, vec, qweight, cherry_weight, cherry_indices, scales, mul, group_size, w_bits,
+            io_dtype, idx_dtype, accumulate=True):
+    _check(vec, "vec", io_dtype, 2)
+    dev = vec.device
+    _check(qweight, "qweight", torch.uint8, 2, dev)
+    _check(cherry_weight, "cherry_weight", io_dtype, 2, dev)
+    _check(cherry_indices, "cherry_indices", idx_dtype, 1, dev)
+    _check(scales, "scaling_factors", io_dtype, 2, dev)
+    _check(mul, "mul", io_dtype, 2, dev)
+    batch, k = vec.shape
+    n = qweight.shape[1]
+    c = cherry_indices.shape[0]
+    group_size = int(group_size)
+    kn = k - c
+    if qweight.shape[0] * 8 != kn * w_bits:
+        raise RuntimeError(f"qweight has {qweight.shape[0]} rows, expected {(kn // 8) * w_bits} "
+                           f"for in_features={k}, num_cherries={c}, w_bits={w_bits}")
+    if tuple(cherry_weight.shape) != (c, n):
+        raise RuntimeError(f"cherry_weight shape {tuple(cherry_weight.shape)} != {(c, n)}")
+    if group_size <= 0:
+        raise RuntimeError(f"{what}: group_size must be positive, got {group_size}")
+    ng = -(-kn // group_size)
+    if tuple(scales.shape) != (ng, n):
+        raise RuntimeError(f"scaling_factors shape {tuple(scales.shape)} != {(ng, n)}")
+    if tuple(mul.shape) != (batch, n):
+        raise RuntimeError(f"mul shape {tuple(mul.shape)} != {(batch, n)}")
+    if batch == 0:
+        return
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        need = _lib.cherryq_workspace_bytes(batch, k, n, c)
+        ws = _workspace(dev, stream, need)
+        rc = fn(_ptr(vec), _ptr(qweight), _ptr(cherry_weight), _ptr(cherry_indices), _ptr(scales), _ptr(mul),
+                batch, k, n, c, group_size, 1 if accumulate else 0, ws.data_ptr(), ws.numel(), stream)
+    if rc != 0:
+        _fail(rc, what)
+
+
+def vecquant4matmul_cherryq(vec, qweight, cherry_weight, cherry_indices, scaling_factors, mul, group_size):
+    """mul += vec @ W^T for 4-bit packed W (reference: csrc/quant_cuda.cpp:56-69)."""
+    if int(group_size) < 128:
+        raise RuntimeError("`group_size` must be multiple of 128")  # csrc/quant_cuda_kernel.cu:684
+    _matmul(_lib.cherryq_vecquant4matmul_f16, "vecquant4matmul_cherryq", vec, qweight, cherry_weight,
+            cherry_indices, scaling_factors, mul, group_size, 4, torch.float16, torch.int16)
+
+
+def vecquant3matmul_cherryq(vec, qweight, cherry_weight, cherry_indices, scaling_factors, mul, group_size,
+                            fp16):
+    """mul += vec @ W^T for 3-bit packed W (reference: csrc/quant_cuda.cpp:41-54).
+
+    fp16=True: fp16 tensors, int16 indices.  fp16=False: fp32 tensors, int32 indices
+    (the call shape of benchmark_speed.py:20-32)."""
+    if fp16:
+        _matmul(_lib.cherryq_vecquant3matmul_f16, "vecquant3matmul_cherryq", vec, qweight, cherry_weight,
+                cherry_indices, scaling_factors, mul, group_size, 3, torch.float16, torch.int16)
+    else:
+        _matmul(_lib.cherryq_vecquant3matmul_f32, "vecquant3matmul_cherryq", vec, qweight, cherry_weight,
+                cherry_indices, scaling_factors, mul, group_size, 3, torch.float32, torch.int32)
+
+
+def matmul_cherryq(w_bits, vec, qweight, cherry_weight, cherry_indices, scaling_factors, out, group_size,
+                   accumulate=False):
+    """fp16 fused matmul that can overwrite `out` instead of accumulating into it, which spares
+    the caller the zero-fill the reference needs before every call (llama/qlinear.py:177).
+    No counterpart in the reference extension."""
+    if w_bits == 4:
+        if int(group_size) < 128:
+            raise RuntimeError("`group_size` must be multiple of 128")
+        fn = _lib.cherryq_vecquant4matmul_f16
+    elif w_bits == 3:
+        fn = _lib.cherryq_vecquant3matmul_f16
+    else:
+        raise NotImplementedError(f"{w_bits} bit kernel is not implemented yet.")
+    _matmul(fn, f"matmul_cherryq[{w_bits}bit]", vec, qweight, cherry_weight, cherry_indices, scaling_factors,
+            out, group_size, w_bits, torch.float16, torch.int16, accumulate=accumulate)
+
+
+def _dequantize_normal(fn, what, w_bits, qweight, scaling_factors, out, height, cherry_size, group_size):
+    _check(qweight, "qweight", torch.uint8, 2)
+    dev = qweight.device
+    _check(scaling_factors, "scaling_factors", torch.float32, 2, dev)
+    _check(out, "out", torch.float32, 2, dev)
+    height, cherry_size, group_size = int(height), int(cherry_size), int(group_size)
+    n = qweight.shape[1]
+    kn = height - cherry_size
+    if qweight.shape[0] * 8 != kn * w_bits:
+        raise RuntimeError(f"qweight has {qweight.shape[0]} rows, expected {(kn // 8) * w_bits}")
+    if group_size <= 0 or tuple(scaling_factors.shape) != (-(-kn // group_size), n):
+        raise RuntimeError(f"scaling_factors shape {tuple(scaling_factors.shape)} does not match "
+                           f"group_size={group_size}")
+    if out.shape[1] != n or out.shape[0] < kn:
+        raise RuntimeError(f"out shape {tuple(out.shape)} cannot hold ({kn}, {n})")
+    with torch.cuda.device(dev):
+        rc = fn(_ptr(qweight), _ptr(scaling_factors), _ptr(out), height, n, cherry_size, group_size,
+                torch.cuda.current_stream(dev).cuda_stream)
+    if rc != 0:
+        _fail(rc, what)
+
+
+def Dequantize3Normal(qweight, scaling_factors, out, height, cherry_size, group_size):
+    """out[k, n] = (code - 3.5) * scale for the compacted normal part (reference:
+    csrc/quant_cuda_kernel.cu:838-922)."""
+    _dequantize_normal(_lib.cherryq_dequantize3_normal_f32, "Dequantize3Normal", 3, qweight, scaling_factors,
+                       out, height, cherry_size, group_size)
+
+
+def Dequantize4Normal(qweight, scaling_factors, out, height, cherry_size, group_size):
+    """out[k, n] = (code - 7.5) * scale for the compacted normal part.  The reference's
+    launcher (csrc/quant_cuda_kernel.cu:925-1010) walks the rows with the 3-bit block height
+    and leaves part of `out` unwritten; this one writes all Kn rows."""
+    _dequantize_normal(_lib.cherryq_dequantize4_normal_f32, "Dequantize4Normal", 4, qweight, scaling_factors,
+                       out, height, cherry_size, group_size)
+
+
+def unpack_cherryq(w_bits, qweight, cherry_weight, cherry_indices, scaling_factors, in_features, group_size):
+    """Dense (out_features, in_features) fp16 weight, bit for bit what QuantLinear.unpack()
+    computes (llama/qlinear.py:120-162), produced on the GPU."""
+    _check(qweight, "qweight", torch.uint8, 2)
+    dev = qweight.device
+    _check(cherry_weight, "cherry_weight", torch.float16, 2, dev)
+    _check(cherry_indices, "cherry_indices", torch.int16, 1, dev)
+    _check(scaling_factors, "scaling_factors", torch.float16, 2, dev)
+    n = qweight.shape[1]
+    c = cherry_indices.shape[0]
+    kn = int(in_features) - c
+    if qweight.shape[0] * 8 != kn * w_bits:
+        raise RuntimeError(f"qweight has {qweight.shape[0]} rows, expected {(kn // 8) * w_bits}")
+    if tuple(scaling_factors.shape) != (-(-kn // int(group_size)), n):
+        raise RuntimeError(f"scaling_factors shape {tuple(scaling_factors.shape)} does not match")
+    dense = torch.empty((n, int(in_features)), dtype=torch.float16, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.cherryq_unpack_f16(w_bits, _ptr(qweight), _ptr(cherry_weight), _ptr(cherry_indices),
+                                     _ptr(scaling_factors), dense.data_ptr(), int(in_features), n, c,
+                                     int(group_size), torch.cuda.current_stream(dev).cuda_stream)
+    if rc != 0:
+        _fail(rc, "unpack_cherryq")
+    return dense

@@ -1,0 +1,396 @@
+"""Parity of the HIP path with the CPU oracle on identical packed inputs (MI355X only).
+
+Bars: dequantised weights bit-exact; fused outputs within rel-L2 <= 1e-3 of the oracle's
+dequantise-and-matmul (fp16 weights, wide accumulation, one rounding); one-hot activations read
+dequantised weights back through the fused kernels bit for bit.
+"""
+import ctypes
+import glob
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cherryq_oracle as orc
+from oracle import c_oracle
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3  # rel-L2 bar on fused outputs
+GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "golden_*.npz")))
+NAMES = ("cherry_indices", "cherry_weight", "qweight", "scales")
+
+
+@pytest.fixture(scope="module")
+def qc():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    import quant_cuda
+    return quant_cuda
+
+
+def dev(packed):
+    return {k: torch.from_numpy(np.ascontiguousarray(v)).cuda() for k, v in packed.items() if k in NAMES}
+
+
+def announce(*a):
+    print("[case]", *a, flush=True)
+    sys.stdout.flush()
+
+
+def run_fused(qc, bits, x, p, gs, mul=None):
+    d = dev(p)
+    xt = torch.from_numpy(x).cuda()
+    out = torch.zeros(x.shape[0], p["qweight"].shape[1], dtype=torch.float16, device="cuda") if mul is None \
+        else torch.from_numpy(mul).cuda()
+    if bits == 4:
+        qc.vecquant4matmul_cherryq(xt, d["qweight"], d["cherry_weight"], d["cherry_indices"], d["scales"], out, gs)
+    else:
+        qc.vecquant3matmul_cherryq(xt, d["qweight"], d["cherry_weight"], d["cherry_indices"], d["scales"], out,
+                                   gs, True)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def oracle_outputs(bits, x, p, gs):
+    k = x.shape[1]
+    dense = c_oracle.unpack(p, bits, gs, k)
+    y_deq = c_oracle.linear(x, dense, want_f64=True)[1]   # fp16 weights, wide accumulation
+    y_fused = c_oracle.fused(x, p, bits, gs)               # un-rounded weights, wide accumulation
+    return dense, y_deq, y_fused
+
+
+# ------------------------------------------------------------------------- golden fixtures
+
+@pytest.mark.parametrize("path", [p for p in GOLDEN if "_f32" not in p and "gall" not in p],
+                         ids=lambda p: os.path.basename(p)[7:-4])
+def test_fused_on_golden_fixtures(qc, path):
+    d = np.load(path)
+    bits, gs, k, n, c = (int(v) for v in d["meta"])
+    announce("golden", os.path.basename(path), bits, gs, k, n, c)
+    if bits == 4 and gs < 128:
+        pytest.skip("4-bit needs group_size >= 128, as in the reference")
+    p = {name: d[name] for name in NAMES}
+    y = run_fused(qc, bits, d["x"], p, gs)
+    assert orc.rel_l2(y, d["forward_dequantized"]) <= 2 * TOL  # reference's own fp16 CPU linear
+    _, y_deq, y_fused = oracle_outputs(bits, d["x"], p, gs)
+    assert orc.rel_l2(y, y_deq) <= TOL
+    assert orc.rel_l2(y, y_fused) <= TOL
+
+
+@pytest.mark.parametrize("path", [p for p in GOLDEN if "_f32" not in p], ids=lambda p: os.path.basename(p)[7:-4])
+def test_unpack_kernel_bit_exact_on_golden(qc, path):
+    d = np.load(path)
+    bits, gs, k, n, c = (int(v) for v in d["meta"])
+    announce("unpack golden", os.path.basename(path))
+    t = dev({name: d[name] for name in NAMES})
+    g = gs if gs != -1 else k
+    dense = qc.unpack_cherryq(bits, t["qweight"], t["cherry_weight"], t["cherry_indices"], t["scales"], k, g)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(dense.cpu().numpy(), d["unpack"])
+
+
+# ------------------------------------------------------------------------- BASELINE shapes
+
+SHAPES_B1 = [
+    (4, 4096, 4096), (3, 4096, 4096),            # config 0 (+ its 3-bit twin)
+    (4, 4096, 11008), (3, 4096, 11008),          # config 1: gate / up
+    (4, 11008, 4096), (3, 11008, 4096),          # config 1: down
+    (3, 5120, 5120), (3, 5120, 13824), (3, 13824, 5120),   # config 3 (13B)
+    (4, 8192, 1024), (4, 8192, 8192),            # config 4 (70B), smaller two
+]
+
+
+@pytest.mark.parametrize("bits,k,n", SHAPES_B1)
+def test_matvec_baseline_shapes(qc, bits, k, n):
+    announce("matvec", bits, k, n)
+    w, p = orc.synthetic_layer(k, n, bits, 128, seed=k + n + bits)
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((1, k)).astype(np.float16)
+    y = run_fused(qc, bits, x, p, 128)
+    _, y_deq, y_fused = oracle_outputs(bits, x, p, 128)
+    e_deq, e_fused = orc.rel_l2(y, y_deq), orc.rel_l2(y, y_fused)
+    print(f"  rel-L2 vs dequant-matmul {e_deq:.2e}, vs un-rounded contract {e_fused:.2e}")
+    assert e_deq <= TOL and e_fused <= TOL
+    # the result is the fp16 rounding of the fp32 sum: compare against the rounded contract
+    ulp_ok = np.abs(y.astype(np.float64) - y_fused) <= np.abs(y_fused) * 2 ** -10 + 1e-3
+    assert ulp_ok.mean() > 0.999
+
+
+@pytest.mark.parametrize("bits,k,n", [(4, 8192, 28672), (4, 28672, 8192)])
+def test_matvec_70b_large_shapes_properties(qc, bits, k, n):
+    """Full-size 70B shapes: random packed bytes (no quantisation pass), checked against the C
+    oracle on a column sample and through linearity."""
+    announce("matvec-large", bits, k, n)
+    p = orc.synthetic_packed_fast(k, n, bits, 128, seed=3)
+    rng = np.random.default_rng(11)
+    x1 = rng.standard_normal((1, k)).astype(np.float16)
+    y1 = run_fused(qc, bits, x1, p, 128)
+    cols = np.sort(rng.choice(n, size=512, replace=False))
+    sub = {"cherry_indices": p["cherry_indices"], "cherry_weight": np.ascontiguousarray(p["cherry_weight"][:, cols]),
+           "qweight": np.ascontiguousarray(p["qweight"][:, cols]), "scales": np.ascontiguousarray(p["scales"][:, cols])}
+    want = c_oracle.fused(x1, sub, bits, 128)
+    assert orc.rel_l2(y1[:, cols], want) <= TOL
+    # linearity: f(2 x) == 2 f(x) exactly (powers of two commute with every rounding involved)
+    y2 = run_fused(qc, bits, (x1 * np.float16(2)).astype(np.float16), p, 128)
+    np.testing.assert_array_equal(y2, (y1.astype(np.float32) * 2).astype(np.float16))
+
+
+@pytest.mark.parametrize("bits,k,n", [(4, 4096, 4096), (3, 4096, 4096), (4, 11008, 512), (3, 11008, 512)])
+def test_one_hot_reads_back_dequantised_weights(qc, bits, k, n):
+    """x = e_j returns column j of the dense weight: the fused decode is bit-exact."""
+    announce("one-hot", bits, k, n)
+    w, p = orc.synthetic_layer(k, n, bits, 128, seed=5)
+    dense = c_oracle.unpack(p, bits, 128, k)
+    idx = p["cherry_indices"].astype(np.int64)
+    nidx = orc.normal_indices(k, idx)
+    probes = [int(nidx[0]), int(nidx[1]), int(nidx[127]), int(nidx[128]), int(nidx[-1]), int(nidx[-113]),
+              int(idx[0]), int(idx[-1]), int(idx[0]) + 1 if idx[0] + 1 not in idx else int(nidx[5]),
+              int(nidx[len(nidx) // 2 + 3])]
+    for j in probes:
+        x = np.zeros((1, k), dtype=np.float16)
+        x[0, j] = 1
+        y = run_fused(qc, bits, x, p, 128)
+        np.testing.assert_array_equal(y[0], dense[:, j], err_msg=f"column {j}")
+    # a power-of-two activation scales the column exactly
+    x = np.zeros((1, k), dtype=np.float16)
+    x[0, probes[2]] = np.float16(2 ** -9)
+    y = run_fused(qc, bits, x, p, 128)
+    np.testing.assert_array_equal(y[0], (dense[:, probes[2]].astype(np.float32) * 2 ** -9).astype(np.float16))
+
+
+def test_accumulate_semantics_and_repeat_calls(qc):
+    """mul += result, like the reference entry point; repeated calls keep accumulating and the
+    split-K counters come back to zero every time."""
+    announce("accumulate")
+    bits, k, n = 4, 4096, 4096
+    w, p = orc.synthetic_layer(k, n, bits, 128, seed=2)
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((1, k)).astype(np.float16)
+    init = rng.standard_normal((1, n)).astype(np.float16)
+    d = dev(p)
+    xt = torch.from_numpy(x).cuda()
+    mul = torch.from_numpy(init).cuda()
+    y_fused = c_oracle.fused(x, p, bits, 128)
+    expect = init.astype(np.float64)
+    for rep in range(3):
+        qc.vecquant4matmul_cherryq(xt, d["qweight"], d["cherry_weight"], d["cherry_indices"], d["scales"], mul, 128)
+        torch.cuda.synchronize()
+        expect = (expect + y_fused).astype(np.float16).astype(np.float64)
+        assert orc.rel_l2(mul.cpu().numpy(), expect) <= TOL, rep
+    # determinism: same inputs, same bits
+    a = run_fused(qc, bits, x, p, 128)
+    b = run_fused(qc, bits, x, p, 128)
+    np.testing.assert_array_equal(a, b)
+
+
+def test_scale_invariance_small_and_large_activations(qc):
+    announce("scale-invariance")
+    for bits in (3, 4):
+        k, n = 4096, 1024
+        w, p = orc.synthetic_layer(k, n, bits, 128, seed=9)
+        rng = np.random.default_rng(4)
+        base = rng.standard_normal((1, k)).astype(np.float32)
+        for scale in (2.0 ** -12, 2.0 ** -6, 1.0, 2.0 ** 6):
+            x = (base * scale).astype(np.float16)
+            y = run_fused(qc, bits, x, p, 128)
+            assert orc.rel_l2(y, c_oracle.fused(x, p, bits, 128)) <= TOL, (bits, scale)
+
+
+# ------------------------------------------------------------------------- batches / variants
+
+@pytest.mark.parametrize("bits,k,n,b", [(3, 5120, 5120, 4), (3, 5120, 5120, 8), (3, 5120, 13824, 8),
+                                        (4, 8192, 1024, 16), (4, 4096, 4096, 2), (4, 4096, 4096, 5),
+                                        (3, 4096, 4096, 16), (4, 4096, 4096, 19)])
+def test_small_batches(qc, bits, k, n, b):
+    announce("batch", bits, k, n, b)
+    w, p = orc.synthetic_layer(k, n, bits, 128, seed=b)
+    rng = np.random.default_rng(b)
+    x = rng.standard_normal((b, k)).astype(np.float16)
+    y = run_fused(qc, bits, x, p, 128)
+    _, y_deq, y_fused = oracle_outputs(bits, x, p, 128)
+    assert orc.rel_l2(y, y_deq) <= TOL and orc.rel_l2(y, y_fused) <= TOL
+    for r in range(b):
+        assert orc.rel_l2(y[r], y_fused[r]) <= TOL, r
+
+
+@pytest.mark.parametrize("bits,gs,k,n,frac,b", [
+    (3, 64, 1024, 512, 1 / 64, 1), (3, 64, 1024, 512, 1 / 64, 3),     # group 64 (reference G64 kernels)
+    (4, 256, 2048, 512, 1 / 256, 1), (3, 256, 2048, 264, 1 / 256, 2),  # group 256, N not a multiple of 256
+    (4, 128, 1024, 8, 1 / 256, 1),                                    # no cherries (K < 2048), tiny N
+    (4, 128, 4096, 72, 1 / 16, 1), (3, 128, 4096, 72, 1 / 16, 4),     # 256 cherries: beyond the fast path
+    (3, 32, 512, 256, 1 / 32, 1), (4, 4096, 4096, 256, 1 / 256, 1),   # group 32; one group for all of K
+    (4, 128, 2048 + 8, 256, 1 / 256, 1), (3, 128, 2048 + 8, 256, 1 / 256, 1),  # ragged last unit (8 positions)
+])
+def test_layout_variants(qc, bits, gs, k, n, frac, b):
+    announce("variant", bits, gs, k, n, frac, b)
+    w, p = orc.synthetic_layer(k, n, bits, gs, seed=13, cherry_fraction=frac)
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((b, k)).astype(np.float16)
+    y = run_fused(qc, bits, x, p, gs)
+    _, y_deq, y_fused = oracle_outputs(bits, x, p, gs)
+    assert orc.rel_l2(y, y_deq) <= TOL and orc.rel_l2(y, y_fused) <= TOL
+
+
+def test_cherry_positions_edge_cases(qc):
+    """Cherries at the very start / end, adjacent runs, and clustered inside one unit."""
+    announce("cherry-edges")
+    k, n, gs = 4096, 256, 128
+    rng = np.random.default_rng(3)
+    for bits in (3, 4):
+        for idx in ([0, 1, 2, 3, 4, 5, 6, 7, 4088, 4089, 4090, 4091, 4092, 4093, 4094, 4095],
+                    list(range(300, 316)),
+                    [5, 127, 128, 129, 255, 256, 1000, 1001, 2047, 2048, 2049, 3000, 3071, 3072, 4000, 4095]):
+            w = (rng.standard_normal((n, k)) * 0.02).astype(np.float16)
+            p = orc.pack(w, np.array(idx), bits, gs)
+            x = rng.standard_normal((1, k)).astype(np.float16)
+            y = run_fused(qc, bits, x, p, gs)
+            assert orc.rel_l2(y, c_oracle.fused(x, p, bits, gs)) <= TOL, (bits, idx[:3])
+            # every cherry column and its neighbours, one-hot
+            dense = c_oracle.unpack(p, bits, gs, k)
+            for j in sorted(set(idx[:3] + idx[-3:] + [min(idx[-1] + 1, k - 1), max(idx[0] - 1, 0)])):
+                e = np.zeros((1, k), dtype=np.float16)
+                e[0, j] = 1
+                np.testing.assert_array_equal(run_fused(qc, bits, e, p, gs)[0], dense[:, j])
+
+
+def test_fp32_entry_point_benchmark_speed_shape(qc):
+    """vecquant3matmul_cherryq(..., fp16=False): fp32 tensors, int32 indices, batch 16, repeated
+    accumulation into the same `mul` -- the call pattern of the reference's benchmark_speed.py."""
+    announce("fp32")
+    b, k, n, c = 16, 4096, 13824 // 8, 16
+    rng = np.random.default_rng(0)
+    vec = rng.standard_normal((b, k)).astype(np.float32)
+    qweight = rng.integers(1, 5, size=(1530, n), dtype=np.uint8)
+    cw = rng.standard_normal((c, n)).astype(np.float32)
+    idx = np.arange(16, dtype=np.int32)
+    scales = np.ones((32, n), dtype=np.float32)
+    mul = torch.zeros(b, n, device="cuda")
+    args = [torch.from_numpy(a).cuda() for a in (vec, qweight, cw, idx, scales)]
+    for _ in range(2):
+        qc.vecquant3matmul_cherryq(*args, mul, 128, False)
+    torch.cuda.synchronize()
+    u = orc.unpack_codes(qweight, 3).astype(np.float64) - 3.5
+    nidx = orc.normal_indices(k, idx)
+    want = 2 * (vec[:, nidx].astype(np.float64) @ u + vec[:, idx].astype(np.float64) @ cw.astype(np.float64))
+    np.testing.assert_allclose(mul.cpu().numpy(), want, rtol=2e-5, atol=2e-3)
+
+
+def test_unsupported_requests_raise(qc):
+    announce("errors")
+    k, n = 1024, 256
+    w, p = orc.synthetic_layer(k, n, 4, 128, seed=1)
+    d = dev(p)
+    x = torch.zeros(1, k, dtype=torch.float16, device="cuda")
+    out = torch.zeros(1, n, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError, match="multiple of 128"):
+        qc.vecquant4matmul_cherryq(x, d["qweight"], d["cherry_weight"], d["cherry_indices"], d["scales"], out, 64)
+    with pytest.raises(RuntimeError):
+        qc.vecquant4matmul_cherryq(x, d["qweight"], d["cherry_weight"], d["cherry_indices"], d["scales"], out, 256)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        qc.vecquant4matmul_cherryq(x, d["qweight"].t().contiguous().t(), d["cherry_weight"], d["cherry_indices"],
+                                   d["scales"], out, 128)
+    with pytest.raises(RuntimeError, match="dtype"):
+        qc.vecquant4matmul_cherryq(x.float(), d["qweight"], d["cherry_weight"], d["cherry_indices"], d["scales"],
+                                   out, 128)
+    with pytest.raises(RuntimeError):
+        qc.vecquant4matmul_cherryq(x[:, :512].contiguous(), d["qweight"], d["cherry_weight"], d["cherry_indices"],
+                                   d["scales"], out, 128)
+
+
+# ------------------------------------------------------------------------- dense dequant
+
+@pytest.mark.parametrize("bits,k,n,gs", [(4, 4096, 4096, 128), (3, 4096, 4096, 128), (3, 11008, 520, 128),
+                                         (4, 2048, 264, 256), (3, 1024, 512, 64)])
+def test_unpack_kernel_bit_exact(qc, bits, k, n, gs):
+    announce("unpack", bits, k, n, gs)
+    w, p = orc.synthetic_layer(k, n, bits, gs, seed=k)
+    t = dev(p)
+    dense = qc.unpack_cherryq(bits, t["qweight"], t["cherry_weight"], t["cherry_indices"], t["scales"], k, gs)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(dense.cpu().numpy(), c_oracle.unpack(p, bits, gs, k))
+
+
+@pytest.mark.parametrize("bits,k,n,gs", [(3, 4096, 1024, 128), (4, 4096, 1024, 128), (4, 11008, 264, 128)])
+def test_dequantize_normal_entry_points(qc, bits, k, n, gs):
+    announce("DequantizeNormal", bits, k, n)
+    w, p = orc.synthetic_layer(k, n, bits, gs, seed=k + 1)
+    c = p["cherry_indices"].shape[0]
+    s32 = p["scales"].astype(np.float32)
+    out = torch.full((k, n), -1.0, device="cuda")
+    fn = qc.Dequantize3Normal if bits == 3 else qc.Dequantize4Normal
+    fn(torch.from_numpy(p["qweight"]).cuda(), torch.from_numpy(s32).cuda(), out, k, c, gs)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    np.testing.assert_array_equal(got[:k - c], c_oracle.dequantize_normal(p["qweight"], s32, bits, k, c, gs))
+    assert np.all(got[k - c:] == -1.0)  # rows past Kn stay untouched
+
+
+# ------------------------------------------------------------------------- module level
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_quantlinear_module_end_to_end(qc, bits):
+    """pack() on the host, move to the GPU, fused forward vs dequantised forward vs oracle."""
+    announce("module", bits)
+    from llama.cherry_linear import QuantLinear as TrainLinear
+    from llama.qlinear import QuantLinear as PackedLinear
+    k, n = 4096, 512
+    torch.manual_seed(bits)
+    lin = TrainLinear(k, n, bias=True, w_bits=bits, group_size=128, cherryq=True).half()
+    lin.weight.data.normal_(0, 0.02)
+    lin.bias.data.normal_(0, 0.1)
+    lin.eval()
+    score = lin.weight.float().abs().amax(0)
+    lin.register_cherry_indices(torch.argsort(score, descending=True)[:lin.num_cherries])
+    q = PackedLinear(bits, 128, lin.quantizer, 1 / 256, k, n, bias=True)
+    q.pack(lin)
+    p = {name: getattr(q, name).numpy().copy() for name in NAMES}
+    want_p = orc.pack(lin.weight.numpy(), lin.cherry_indices.numpy(), bits, 128)
+    for name in NAMES:
+        np.testing.assert_array_equal(p[name], want_p[name], err_msg=name)
+    q = q.cuda()
+    x = torch.randn(2, 3, k, dtype=torch.float16, device="cuda")
+    y = q(x)
+    assert y.shape == (2, 3, n) and y.dtype == torch.float16
+    xn = x.reshape(-1, k).cpu().numpy()
+    want = c_oracle.fused(xn, p, bits, 128).astype(np.float16).astype(np.float64) + q.bias.cpu().numpy().astype(np.float64)
+    assert orc.rel_l2(y.reshape(-1, n).cpu().numpy(), want) <= TOL
+    dense_dev = q.unpack()
+    np.testing.assert_array_equal(dense_dev.cpu().numpy(), c_oracle.unpack(p, bits, 128, k))
+    with PackedLinear.dmode(layerwise_dequantize=False):
+        y2 = q(x)
+    assert q.dequantized
+    assert orc.rel_l2(y2.reshape(-1, n).cpu().numpy(), want) <= 2 * TOL
+    with pytest.raises(RuntimeError):
+        q(x)  # fused mode after the packed buffers were dropped
+
+
+def test_direct_c_abi_call_with_raw_pointers(qc):
+    """The entry point as a non-Python host would call it: raw device pointers, explicit
+    workspace, explicit stream."""
+    announce("raw C ABI")
+    bits, k, n = 4, 4096, 2048
+    w, p = orc.synthetic_layer(k, n, bits, 128, seed=17)
+    d = dev(p)
+    c = p["cherry_indices"].shape[0]
+    x = torch.randn(1, k, dtype=torch.float16, device="cuda")
+    out = torch.full((1, n), 7.0, dtype=torch.float16, device="cuda")
+    lib = ctypes.CDLL(qc.LIBRARY_PATH)
+    lib.cherryq_workspace_bytes.restype = ctypes.c_size_t
+    need = lib.cherryq_workspace_bytes(1, k, n, c)
+    ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.Stream()
+    fn = lib.cherryq_vecquant4matmul_f16
+    fn.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 6 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    fn.restype = ctypes.c_int
+    torch.cuda.synchronize()
+    rc = fn(x.data_ptr(), d["qweight"].data_ptr(), d["cherry_weight"].data_ptr(), d["cherry_indices"].data_ptr(),
+            d["scales"].data_ptr(), out.data_ptr(), 1, k, n, c, 128, 0, ws.data_ptr(), need, stream.cuda_stream)
+    assert rc == 0
+    stream.synchronize()
+    want = c_oracle.fused(x.cpu().numpy(), p, bits, 128)
+    assert orc.rel_l2(out.cpu().numpy(), want) <= TOL  # accumulate=0 overwrote the 7.0 fill
+    counters = lib.cherryq_workspace_counter_bytes
+    counters.restype = ctypes.c_size_t
+    assert int(ws[:counters(n)].cpu().sum()) == 0
