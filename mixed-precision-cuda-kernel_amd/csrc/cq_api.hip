@@ -2,10 +2,19 @@
 // Declarations and the reference interfaces they replace: include/cherryq.h.
 #include "../../include/cherryq.h"
 
+#include <stdlib.h>
+
 #include "cq_common.cuh"
 #include "cq_kernels.h"
 
 namespace cq {
+
+// CHERRYQ_FORCE_GENERIC=1 routes every fused call through the generic kernel (a second,
+// independently written HIP path; used by the tests to cross-check the specialised kernels).
+static bool force_generic() {
+    const char *e = getenv("CHERRYQ_FORCE_GENERIC");
+    return e && e[0] == '1';
+}
 
 // The smallest units_per_wg any kernel uses is 1, which bounds the split count by the unit count.
 size_t workspace_counter_bytes(int N) {
@@ -59,7 +68,7 @@ static int matmul_f16(const void *vec, const uint8_t *qweight, const void *cherr
     const __half *sc = reinterpret_cast<const __half *>(scales);
     __half *y = reinterpret_cast<__half *>(mul);
     hipError_t e;
-    if (matvec_supported(BITS, B, K, N, C, G)) {
+    if (!force_generic() && matvec_supported(BITS, B, K, N, C, G)) {
         e = hipSuccess;
         for (int b = 0; b < B && e == hipSuccess; b++)
             e = launch_matvec(BITS, x + (size_t)b * K, qweight, cw, cherry_indices, sc, y + (size_t)b * N, K,

@@ -59,19 +59,22 @@ __device__ inline float half_bits_to_float(uint32_t h) {
     return __half2float(__ushort_as_half((unsigned short)h));
 }
 
-// Sum `a` over lanes l, l^32 for the lower half of the wave and `b` for the upper half:
-// lanes < 32 return a[l] + a[l+32], lanes >= 32 return b[l-32] + b[l].
+// v_permlane32_swap_b32 exchanges lanes 32..63 of its first operand with lanes 0..31 of its
+// second; v_permlane16_swap_b32 exchanges the odd 16-lane rows of the first with the even rows
+// of the second.  Written as inline assembly because the compiler builtin of this toolchain
+// returns the first result twice; the s_nop pad the VALU->permlane-swap data hazards that the
+// compiler cannot see through an asm statement.
+//
+// swap32_add: lanes < 32 return a[l] + a[l+32], lanes >= 32 return b[l-32] + b[l].
 __device__ inline float swap32_add(float a, float b) {
-    auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, a), __builtin_bit_cast(unsigned, b),
-                                              false, false);
-    return __builtin_bit_cast(float, r[0]) + __builtin_bit_cast(float, r[1]);
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return a + b;
 }
 
-// Same across the two rows of each half: even rows return a[row] + a[row+1], odd rows b + b.
+// swap16_add: even rows return a[row] + a[row+1], odd rows return b[row-1] + b[row].
 __device__ inline float swap16_add(float a, float b) {
-    auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, a), __builtin_bit_cast(unsigned, b),
-                                              false, false);
-    return __builtin_bit_cast(float, r[0]) + __builtin_bit_cast(float, r[1]);
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return a + b;
 }
 
 template <int BITS>

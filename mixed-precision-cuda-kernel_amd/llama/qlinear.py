@@ -121,7 +121,7 @@ class QuantLinear(nn.Module):
         """Fill the packed buffers from a fake-quant training module.  llama/qlinear.py:67-118.
         The buffers end up on the CPU, as in the reference."""
         if linear.bias is not None:
-            self.bias = linear.bias.half().cpu()
+            self.bias = linear.bias.detach().to(torch.float16).cpu().clone()
         weight = linear.weight
         cherry = linear.cherry_indices.sort().values.long()
         self.cherry_indices = cherry.to(dtype=torch.int16).cpu()
