@@ -49,16 +49,16 @@ int cherryq_version(void);
 const char *cherryq_status_string(int status);
 
 /*
- * Split-K workspace.  The fused entry points split the reduction over K across
- * workgroups; partial sums and per-tile arrival counters live in a caller-provided
- * device buffer of at least cherryq_workspace_bytes() bytes, 256-byte aligned.  Its first
- * cherryq_workspace_counter_bytes() bytes must be zero before the first call; every call
- * leaves them zero again.  Calls that may overlap in time (different streams) must use
- * different workspaces.  Has no counterpart in the reference, whose kernels add fp16
- * partials into `mul` with atomics (csrc/quant_cuda_kernel.cu:833).
+ * Split-K workspace.  The fused entry points split the reduction over K across workgroups,
+ * which meet in one 64-bit accumulator word per output element (fixed-point running sum plus
+ * an arrival count, added with a single atomic; see csrc/cq_common.cuh).  The words live in a
+ * caller-provided device buffer of at least cherryq_workspace_bytes() bytes, 256-byte aligned.
+ * The buffer must be all zero before the first call; every call leaves it all zero again.
+ * Calls that may overlap in time (different streams) must use different workspaces.  Has no
+ * counterpart in the reference, whose kernels add fp16 partials into `mul` with atomics
+ * (csrc/quant_cuda_kernel.cu:833).
  */
 size_t cherryq_workspace_bytes(int batch, int in_features, int out_features, int num_cherries);
-size_t cherryq_workspace_counter_bytes(int out_features);
 
 /*
  * Replaces quant_cuda.vecquant4matmul_cherryq (csrc/quant_cuda.cpp:56-69,

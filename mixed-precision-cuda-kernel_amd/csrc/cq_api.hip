@@ -16,22 +16,14 @@ static bool force_generic() {
     return e && e[0] == '1';
 }
 
-// The smallest units_per_wg any kernel uses is 1, which bounds the split count by the unit count.
-size_t workspace_counter_bytes(int N) {
-    size_t tiles = (size_t)ceil_div(N > 0 ? N : 1, kTileCols);
-    return (tiles * sizeof(unsigned) + 255) / 256 * 256;
-}
-
+// One 64-bit accumulator word per output element of the largest batch chunk a kernel handles.
 size_t workspace_bytes(int B, int K, int N, int C) {
+    (void)K;
+    (void)C;
     if (B < 1) B = 1;
-    if (K < 8) K = 8;
-    if (C < 0) C = 0;
-    if (C > K) C = K;
-    // one slot of partial sums per unit (128 normal positions or 32 cherry rows) bounds every
-    // split factor the kernels use; batch rows are processed at most 16 at a time
-    size_t units = (size_t)ceil_div(K - C, kUnitK) + (size_t)ceil_div(C, kCherryUnit) + 1;
     size_t rows = (size_t)(B < 16 ? B : 16);
-    return workspace_counter_bytes(N) + units * rows * (size_t)(N > 0 ? N : 1) * sizeof(float);
+    size_t bytes = rows * (size_t)(N > 0 ? N : 1) * sizeof(unsigned long long);
+    return (bytes + 255) / 256 * 256;
 }
 
 static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
@@ -105,8 +97,6 @@ const char *cherryq_status_string(int status) {
 size_t cherryq_workspace_bytes(int batch, int in_features, int out_features, int num_cherries) {
     return cq::workspace_bytes(batch, in_features, out_features, num_cherries);
 }
-
-size_t cherryq_workspace_counter_bytes(int out_features) { return cq::workspace_counter_bytes(out_features); }
 
 int cherryq_vecquant4matmul_f16(const void *vec, const uint8_t *qweight, const void *cherry_weight,
                                 const int16_t *cherry_indices, const void *scales, void *mul, int batch,

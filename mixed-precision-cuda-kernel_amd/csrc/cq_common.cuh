@@ -8,7 +8,7 @@
 namespace cq {
 
 constexpr int kTileCols = 256;  // output columns per workgroup tile (256 B of one byte row)
-constexpr int kUnitK = 128;     // compacted normal positions per work unit
+constexpr int kUnitK = 128;     // compacted normal positions per work unit (generic kernel)
 constexpr int kCherryUnit = 32; // cherry rows per work unit
 constexpr int kXcds = 8;        // MI355X: 8 accelerator complex dies, workgroups dealt round-robin
 
@@ -23,15 +23,24 @@ struct Plan {
     int splits;         // workgroups per column tile (split-K factor)
 };
 
-__host__ __device__ inline Plan make_plan(int K, int N, int C, int units_per_wg) {
+__host__ __device__ inline Plan make_plan(int K, int N, int C, int units_per_wg, int unit_k = kUnitK) {
     Plan p;
     p.tiles = ceil_div(N, kTileCols);
-    p.units_normal = ceil_div(K - C, kUnitK);
+    p.units_normal = ceil_div(K - C, unit_k);
     p.units_total = p.units_normal + ceil_div(C, kCherryUnit);
     p.units_per_wg = units_per_wg;
     p.splits = ceil_div(p.units_total, units_per_wg);
     if (p.splits < 1) p.splits = 1;
     return p;
+}
+
+// Units per workgroup for the streaming kernels: as many as possible (fewer split-K atomics on
+// the same word, which serialise at roughly 80 ns each) while the grid still has at least
+// `min_wgs` workgroups to cover the 256 CUs.
+inline int choose_units_per_wg(int K, int N, int C, int max_units, int min_wgs, int unit_k = kUnitK) {
+    int u = max_units;
+    while (u > 1 && make_plan(K, N, C, u, unit_k).tiles * make_plan(K, N, C, u, unit_k).splits < min_wgs) u >>= 1;
+    return u;
 }
 
 // Workgroups are dealt to the 8 XCDs round-robin by their linear id.  Renumber so that
@@ -64,66 +73,78 @@ __device__ inline int gather_offset(const IDX *__restrict__ idx, int C, int k) {
     return lo;
 }
 
-// Split-K epilogue.  Every workgroup of a column tile stores its partial sums, then takes a
-// ticket; the workgroup that draws the last ticket adds the partials in split order (a fixed
-// order, so results do not depend on scheduling) and writes `mul` with a single rounding.
+// Split-K epilogue: one 64-bit atomic per output element.
+//
+// Each output element owns a 64-bit accumulator word in the workspace:
+//     bits 63..8  running sum of the partial sums, two's-complement fixed point, 2^-34 units
+//     bits  7..0  number of workgroups that have contributed so far
+// A workgroup adds  (fixed(partial) << 8) + 1  with a single agent-scope atomic that returns
+// the previous word.  Integer addition is associative, so the total does not depend on the order
+// in which workgroups arrive, and the thread that sees the count reach `splits` holds the
+// complete sum: it converts it back, writes `mul` with one rounding and stores 0 to the word,
+// which is thereby ready for the next call.  One memory round trip, no barrier, no second pass.
+//
+// Fixed point loses nothing that fp16 output can show: the resolution 2^-34 is 2^10 times finer
+// than the smallest fp16 subnormal step, and the range +-2^21 is 32 times fp16's largest value
+// (partials are clamped to it; a NaN partial is clamped too and so reads as a huge value).
+// Agent-scope release/acquire fences are deliberately not used: on this multi-XCD part they
+// write back and invalidate a whole L2 and serialise the workgroups.
+constexpr float kFixScale = 17179869184.0f;        // 2^34
+constexpr double kFixInvScale = 1.0 / 17179869184.0;
+constexpr float kFixClamp = 2097151.0f;             // 2^21 - 1
+constexpr int kMaxSplits = 255;
+
+__device__ inline unsigned long long splitk_encode(float partial) {
+    float p = fminf(fmaxf(partial, -kFixClamp), kFixClamp);
+    long long q = __double2ll_rn((double)p * (double)kFixScale);
+    return ((unsigned long long)q << 8) + 1ull;
+}
+
 // `vals[b][c]` are this thread's partial sums for columns n0 + c, batch rows b < B.
 template <typename IO, int MAXB, int COLS>
-__device__ inline void splitk_finish(float (&vals)[MAXB][COLS], int B, int N, int n0, bool active,
-                                     int tile, int split, int splits, float *__restrict__ partial,
-                                     unsigned *__restrict__ tickets, IO *__restrict__ mul,
+__device__ inline void splitk_finish(float (&vals)[MAXB][COLS], int B, int N, int n0, bool active, int splits,
+                                     unsigned long long *__restrict__ acc, IO *__restrict__ mul,
                                      int accumulate) {
+    if (!active) return;
     if (splits > 1) {
-        if (active) {
-#pragma unroll
-            for (int b = 0; b < MAXB; b++)
-                if (b < B) {
-                    float *p = partial + ((size_t)split * B + b) * N + n0;
-#pragma unroll
-                    for (int c = 0; c < COLS; c++) p[c] = vals[b][c];
-                }
-        }
-        __shared__ int s_last;
-        __threadfence();
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            unsigned old = __hip_atomic_fetch_add(&tickets[tile], 1u, __ATOMIC_ACQ_REL,
-                                                  __HIP_MEMORY_SCOPE_AGENT);
-            s_last = (old == (unsigned)(splits - 1));
-        }
-        __syncthreads();
-        if (!s_last) return;
-        __threadfence();
-        if (active) {
-#pragma unroll
-            for (int b = 0; b < MAXB; b++)
-                if (b < B) {
-#pragma unroll
-                    for (int c = 0; c < COLS; c++) vals[b][c] = 0.f;
-                    for (int s = 0; s < splits; s++) {
-                        const float *p = partial + ((size_t)s * B + b) * N + n0;
-#pragma unroll
-                        for (int c = 0; c < COLS; c++)
-                            vals[b][c] += __builtin_nontemporal_load(p + c);
-                    }
-                }
-        }
-        if (threadIdx.x == 0)
-            __hip_atomic_store(&tickets[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    if (active) {
+        unsigned long long now[MAXB][COLS];
 #pragma unroll
         for (int b = 0; b < MAXB; b++)
             if (b < B) {
-                IO *o = mul + (size_t)b * N + n0;
 #pragma unroll
                 for (int c = 0; c < COLS; c++) {
-                    float v = vals[b][c];
-                    if (accumulate) v += to_float(o[c]);
-                    o[c] = from_float<IO>(v);
+                    const unsigned long long add = splitk_encode(vals[b][c]);
+                    now[b][c] = __hip_atomic_fetch_add(acc + (size_t)b * N + n0 + c, add, __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT) + add;
                 }
             }
+#pragma unroll
+        for (int b = 0; b < MAXB; b++)
+            if (b < B) {
+#pragma unroll
+                for (int c = 0; c < COLS; c++) {
+                    if ((int)(now[b][c] & 0xffull) != splits) continue;  // someone else finishes this one
+                    __hip_atomic_store(acc + (size_t)b * N + n0 + c, 0ull, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                    float v = (float)((double)((long long)now[b][c] >> 8) * kFixInvScale);
+                    IO *o = mul + (size_t)b * N + n0 + c;
+                    if (accumulate) v += to_float(*o);
+                    *o = from_float<IO>(v);
+                }
+            }
+        return;
     }
+#pragma unroll
+    for (int b = 0; b < MAXB; b++)
+        if (b < B) {
+            IO *o = mul + (size_t)b * N + n0;
+#pragma unroll
+            for (int c = 0; c < COLS; c++) {
+                float v = vals[b][c];
+                if (accumulate) v += to_float(o[c]);
+                o[c] = from_float<IO>(v);
+            }
+        }
 }
 
 }  // namespace cq

@@ -41,8 +41,8 @@ template <int BITS, typename IO, typename IDX>
 __global__ __launch_bounds__(64) void generic_kernel(
     const IO *__restrict__ vec, const uint8_t *__restrict__ qweight,
     const IO *__restrict__ cherry_weight, const IDX *__restrict__ cherry_indices,
-    const IO *__restrict__ scales, IO *__restrict__ mul, float *__restrict__ partial,
-    unsigned *__restrict__ tickets, int B, int K, int N, int C, int G, int accumulate, Plan plan) {
+    const IO *__restrict__ scales, IO *__restrict__ mul, unsigned long long *__restrict__ acc_words, int B,
+    int K, int N, int C, int G, int accumulate, Plan plan) {
     const int lane = threadIdx.x;
     const int lid = xcd_remap(blockIdx.x, gridDim.x);
     const int tile = lid / plan.splits;
@@ -144,23 +144,22 @@ __global__ __launch_bounds__(64) void generic_kernel(
             }
         }
     }
-    splitk_finish<IO, kMaxB, 4>(acc, B, N, n0, active, tile, split, plan.splits, partial, tickets, mul,
-                                accumulate);
+    splitk_finish<IO, kMaxB, 4>(acc, B, N, n0, active, plan.splits, acc_words, mul, accumulate);
 }
 
 template <int BITS, typename IO, typename IDX>
 hipError_t launch_generic(const IO *vec, const uint8_t *qweight, const IO *cherry_weight,
                           const IDX *cherry_indices, const IO *scales, IO *mul, int B, int K, int N,
                           int C, int G, int accumulate, void *workspace, hipStream_t stream) {
-    Plan plan = make_plan(K, N, C, 4);
-    unsigned *tickets = reinterpret_cast<unsigned *>(workspace);
-    float *partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) +
-                                               workspace_counter_bytes(N));
+    int upw = 4;
+    while (make_plan(K, N, C, upw).splits > kMaxSplits) upw <<= 1;
+    Plan plan = make_plan(K, N, C, upw);
+    unsigned long long *acc_words = reinterpret_cast<unsigned long long *>(workspace);
     for (int b0 = 0; b0 < B; b0 += kMaxB) {
         int nb = min(kMaxB, B - b0);
         hipLaunchKernelGGL((generic_kernel<BITS, IO, IDX>), dim3(plan.tiles * plan.splits), dim3(64), 0,
                            stream, vec + (size_t)b0 * K, qweight, cherry_weight, cherry_indices, scales,
-                           mul + (size_t)b0 * N, partial, tickets, nb, K, N, C, G, accumulate, plan);
+                           mul + (size_t)b0 * N, acc_words, nb, K, N, C, G, accumulate, plan);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }

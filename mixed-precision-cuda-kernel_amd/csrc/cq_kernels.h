@@ -8,7 +8,6 @@
 
 namespace cq {
 
-size_t workspace_counter_bytes(int N);
 size_t workspace_bytes(int B, int K, int N, int C);
 
 // cq_generic.hip

@@ -24,15 +24,34 @@
 #include "cq_common.cuh"
 #include "cq_kernels.h"
 
+#ifdef CQ_TRACE
+extern __device__ unsigned long long *g_cq_trace;  // defined by the profiling harness
+#endif
+
 namespace cq {
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
+// Optional per-wave phase timestamps for a profiling harness; compiled out in the library.
+#ifdef CQ_TRACE
+#define CQ_STAMP(slot)                                                                                       \
+    do {                                                                                                     \
+        if (g_cq_trace && lane == 0)                                                                         \
+            g_cq_trace[((size_t)blockIdx.x * NW + wave) * 8 + (slot)] = wall_clock64();                      \
+    } while (0)
+#else
+#define CQ_STAMP(slot) do { } while (0)
+#endif
+
 constexpr int kMaxFastCherries = 128;  // two 64-lane chunks of cherry indices
 constexpr uint32_t kRsrcFlags = 0x00020000u;
 constexpr uint32_t kOob = 0x80000000u;  // byte offset beyond any buffer this kernel accepts
+#ifndef CQ_STREAM_POLICY
+#define CQ_STREAM_POLICY 2
+#endif
+constexpr int kStreamPolicy = CQ_STREAM_POLICY;  // cache policy of the weight stream: 2 = nt (read once)
 
 __device__ inline float fdot2(uint32_t a, uint32_t b, float c) {
     return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a), __builtin_bit_cast(half2_t, b), c, false);
@@ -77,30 +96,37 @@ __device__ inline float swap16_add(float a, float b) {
     return a + b;
 }
 
-template <int BITS>
+// KPL = compacted positions per lane group (16 or 32); a unit is 4 * KPL positions.
+template <int BITS, int KPL>
 struct Geo {
-    static constexpr int kRowsPerLaneGroup = BITS == 4 ? 16 : 12;  // byte rows holding 32 positions
+    static constexpr int kUnit = 4 * KPL;
+    static constexpr int kRowsPerLaneGroup = KPL * BITS / 8;  // byte rows holding KPL positions
     static constexpr int kRowsPerUnit = 4 * kRowsPerLaneGroup;
+    static constexpr int kPairs = KPL / 2;  // activation pair dwords per lane group
 };
 
-template <int BITS>
-__global__ __launch_bounds__(256) void matvec_kernel(
+// NW = wavefronts (= units) per workgroup: 4 for large layers, 2 or 1 when the layer is so small
+// that larger workgroups would leave CUs without work.
+template <int BITS, int NW, int KPL>
+__global__ __launch_bounds__(64 * NW) void matvec_kernel(
     const __half *__restrict__ x, const uint8_t *__restrict__ qweight, const __half *__restrict__ cherry_weight,
     const int16_t *__restrict__ cherry_indices, const __half *__restrict__ scales, __half *__restrict__ mul,
-    float *__restrict__ partial, unsigned *__restrict__ tickets, int K, int N, int C, int G, int accumulate,
-    Plan plan) {
-    constexpr int R = Geo<BITS>::kRowsPerLaneGroup;
-    __shared__ uint32_t s_win[4][128];  // per wave: 256 fp16 activations starting at the unit's first position
-    __shared__ uint32_t s_pair[4][64];  // per wave: activation pairs laid out for the dot2 operands
-    __shared__ float s_red[4][kTileCols];
+    unsigned long long *__restrict__ acc_words, int K, int N, int C, int G, int accumulate, Plan plan) {
+    using G_ = Geo<BITS, KPL>;
+    constexpr int R = G_::kRowsPerLaneGroup;
+    constexpr int UK = G_::kUnit;
+    __shared__ uint32_t s_win[NW][128];  // per wave: 256 fp16 activations starting at the unit's first position
+    __shared__ uint32_t s_pair[NW][64];  // per wave: activation pairs laid out for the dot2 operands
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int kq = lane >> 4, nl = lane & 15;
-    const int lid = xcd_remap(blockIdx.x, gridDim.x);
-    const int tile = lid / plan.splits;
-    const int split = lid % plan.splits;
-    const int u = split * 4 + wave;
+    // Consecutive workgroups take neighbouring column tiles of the same rows, so that the
+    // workgroups in flight at any moment read whole byte rows (DRAM page locality); walking one
+    // 256-byte strip down the rows instead costs ~40 % of the bandwidth on square layers.
+    const int tile = blockIdx.x % plan.tiles;
+    const int split = blockIdx.x / plan.tiles;
+    const int u = split * NW + wave;
     const int n0 = tile * kTileCols + nl * 16;
     const bool col_ok = n0 < N;
     const int Kn = K - C;
@@ -108,32 +134,49 @@ __global__ __launch_bounds__(256) void matvec_kernel(
     float tot[16];
 #pragma unroll
     for (int c = 0; c < 16; c++) tot[c] = 0.f;
+    CQ_STAMP(0);
 
     if (u < plan.units_normal) {
-        const int ubase = u * kUnitK;
+        const int ubase = u * UK;
         // ---- small operands first: vmcnt retires in order, so these can be waited on while
         // the weight loads issued after them are still in flight
         const __amdgpu_buffer_rsrc_t ri =
             __builtin_amdgcn_make_buffer_rsrc((void *)cherry_indices, 0, C * 2, kRsrcFlags);
+#ifdef CQ_EXP_NOIDX
+        const int i0 = 16000 + lane, i1 = 17000 + lane;
+#else
         const int i0 = (short)__builtin_amdgcn_raw_buffer_load_b16(ri, lane * 2, 0, 0);
         const int i1 = (short)__builtin_amdgcn_raw_buffer_load_b16(ri, (lane + 64) * 2, 0, 0);
+#endif
         const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, K * 2, kRsrcFlags);
+#ifdef CQ_EXP_NOWIN
+        const uint32_t win0 = 0x3c003c00u + lane, win1 = 0x3c003c00u;
+#else
         const uint32_t win0 = __builtin_amdgcn_raw_buffer_load_b32(rx, (ubase + 2 * lane) * 2, 0, 0);
         const uint32_t win1 = __builtin_amdgcn_raw_buffer_load_b32(rx, (ubase + 128 + 2 * lane) * 2, 0, 0);
+#endif
         const int ng = ceil_div(Kn, G);
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)scales, 0, ng * N * 2, kRsrcFlags);
-        const int g = (ubase + 32 * kq) / G;
+        const int g = (ubase + KPL * kq) / G;
         const uint32_t soff = col_ok ? (uint32_t)(g * N + n0) * 2u : kOob;
+#ifdef CQ_EXP_NOSCALE
+        const u32x4 sc0 = {0x20002000u + soff, 0x20002000u, 0x20002000u, 0x20002000u}, sc1 = sc0;
+#else
         const u32x4 sc0 = __builtin_amdgcn_raw_buffer_load_b128(rs, soff, 0, 0);
         const u32x4 sc1 = __builtin_amdgcn_raw_buffer_load_b128(rs, soff + 16, 0, 0);
+#endif
 
+#ifdef CQ_EXP_WAIT_SMALL
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
         // ---- the weight stream: R byte rows x 16 columns per lane, rows past the end read 0
         const int qrows = Kn / 8 * BITS;
         const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void *)qweight, 0, qrows * N, kRsrcFlags);
-        const uint32_t woff = col_ok ? (uint32_t)((u * Geo<BITS>::kRowsPerUnit + kq * R) * N + n0) : kOob;
+        const uint32_t woff = col_ok ? (uint32_t)((u * G_::kRowsPerUnit + kq * R) * N + n0) : kOob;
         u32x4 w[R];
 #pragma unroll
-        for (int r = 0; r < R; r++) w[r] = __builtin_amdgcn_raw_buffer_load_b128(rw, woff + (uint32_t)(r * N), 0, 0);
+        for (int r = 0; r < R; r++)
+            w[r] = __builtin_amdgcn_raw_buffer_load_b128(rw, woff + (uint32_t)(r * N), 0, kStreamPolicy);
 
         // ---- gather the unit's 128 activations around the cherry channels
         // t[m] = idx[m] - m is non-decreasing; position k sits after every m with t[m] <= k
@@ -153,11 +196,11 @@ __global__ __launch_bounds__(256) void matvec_kernel(
             p0 = (0x6730 >> (4 * q)) & 15;  // bit position of the first code's field in its half
             p1 = (0x5241 >> (4 * q)) & 15;
         }
-        const int k0 = ubase + 32 * kq + j0, k1 = ubase + 32 * kq + j1;
+        const int k0 = ubase + KPL * kq + j0, k1 = ubase + KPL * kq + j1;
         int low0 = __popcll(__ballot(t0 < ubase)) + __popcll(__ballot(t1 < ubase));
         int low1 = low0;
         {
-            unsigned long long m = __ballot(t0 >= ubase && t0 < ubase + kUnitK);
+            unsigned long long m = __ballot(t0 >= ubase && t0 < ubase + UK);
             while (m) {
                 int j = __builtin_ctzll(m);
                 int tj = __builtin_amdgcn_readlane(t0, j);
@@ -165,7 +208,7 @@ __global__ __launch_bounds__(256) void matvec_kernel(
                 low1 += tj <= k1;
                 m &= m - 1;
             }
-            m = __ballot(t1 >= ubase && t1 < ubase + kUnitK);
+            m = __ballot(t1 >= ubase && t1 < ubase + UK);
             while (m) {
                 int j = __builtin_ctzll(m);
                 int tj = __builtin_amdgcn_readlane(t1, j);
@@ -177,8 +220,9 @@ __global__ __launch_bounds__(256) void matvec_kernel(
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         const unsigned short *winh = reinterpret_cast<const unsigned short *>(&s_win[wave][0]);
-        uint32_t h0 = (k0 < Kn) ? winh[(k0 - ubase) + low0] : 0u;
-        uint32_t h1 = (k1 < Kn) ? winh[(k1 - ubase) + low1] : 0u;
+        const bool prep = nl < G_::kPairs;  // lanes that prepare an activation pair
+        uint32_t h0 = (prep && k0 < Kn) ? winh[(k0 - ubase) + low0] : 0u;
+        uint32_t h1 = (prep && k1 < Kn) ? winh[(k1 - ubase) + low1] : 0u;
         const float xsum = row_sum(half_bits_to_float(h0) + half_bits_to_float(h1));
         int sh = 0;
         if (BITS == 3) {
@@ -192,16 +236,28 @@ __global__ __launch_bounds__(256) void matvec_kernel(
         s_pair[wave][lane] = h0 | (h1 << 16);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        u32x4 xq[4];
+        u32x4 xq[G_::kPairs / 4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) xq[i] = *reinterpret_cast<const u32x4 *>(&s_pair[wave][16 * kq + 4 * i]);
+        for (int i = 0; i < G_::kPairs / 4; i++)
+            xq[i] = *reinterpret_cast<const u32x4 *>(&s_pair[wave][16 * kq + 4 * i]);
+        CQ_STAMP(1);
 
+#ifdef CQ_EXP_NOCOMPUTE
+        {
+            uint32_t acc_x = 0;
+#pragma unroll
+            for (int r = 0; r < R; r++) acc_x ^= w[r][0] ^ w[r][1] ^ w[r][2] ^ w[r][3];
+            tot[0] = __builtin_bit_cast(float, (acc_x & 0xffu) | xq[0][0]) * xsum;
+        }
+        if (false) {
+#else
         if (BITS == 4) {
+#endif
             float lo[16], hi[16];
 #pragma unroll
             for (int c = 0; c < 16; c++) lo[c] = hi[c] = 0.f;
 #pragma unroll
-            for (int p = 0; p < 8; p++) {
+            for (int p = 0; p < R / 2; p++) {
                 const uint32_t xe = xq[p >> 1][(p & 1) * 2], xo = xq[p >> 1][(p & 1) * 2 + 1];
 #pragma unroll
                 for (int d = 0; d < 4; d++) {
@@ -227,7 +283,7 @@ __global__ __launch_bounds__(256) void matvec_kernel(
 #pragma unroll
             for (int c = 0; c < 16; c++) acc[c] = 0.f;
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
+            for (int t = 0; t < R / 3; t++) {
                 const uint32_t xa = xq[t][0], xb = xq[t][1], xc = xq[t][2], xd = xq[t][3];
 #pragma unroll
                 for (int d = 0; d < 4; d++) {
@@ -260,19 +316,22 @@ __global__ __launch_bounds__(256) void matvec_kernel(
         const int c0 = (u - plan.units_normal) * kCherryUnit + 8 * kq;
         const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc((void *)cherry_weight, 0, C * N * 2, kRsrcFlags);
         const uint32_t coff = col_ok ? (uint32_t)(c0 * N + n0) * 2u : kOob;
+        // the activation gather x[idx[c]] is a dependent chain; run it before the weight loads are
+        // queued, while this wave has nothing else outstanding
         const __amdgpu_buffer_rsrc_t ri =
             __builtin_amdgcn_make_buffer_rsrc((void *)cherry_indices, 0, C * 2, kRsrcFlags);
         const int ci = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(ri, (c0 + (nl & 7)) * 2, 0, 0);
+        const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, K * 2, kRsrcFlags);
+        const uint32_t xoff = (nl < 8 && c0 + nl < C) ? (uint32_t)ci * 2u : kOob;
+        const uint32_t xraw = __builtin_amdgcn_raw_buffer_load_b16(rx, xoff, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);  // keep the weight loads behind the gather in the queue
         u32x4 cw[8][2];
 #pragma unroll
         for (int r = 0; r < 8; r++) {
-            cw[r][0] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff + (uint32_t)(r * N * 2), 0, 0);
-            cw[r][1] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff + (uint32_t)(r * N * 2) + 16, 0, 0);
+            cw[r][0] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff + (uint32_t)(r * N * 2), 0, kStreamPolicy);
+            cw[r][1] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff + (uint32_t)(r * N * 2) + 16, 0, kStreamPolicy);
         }
-        const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, K * 2, kRsrcFlags);
-        const uint32_t xoff = (nl < 8 && c0 + nl < C) ? (uint32_t)ci * 2u : kOob;
-        const float xv = half_bits_to_float(__builtin_amdgcn_raw_buffer_load_b16(rx, xoff, 0, 0));
-        s_pair[wave][lane] = __builtin_bit_cast(uint32_t, xv);
+        s_pair[wave][lane] = __builtin_bit_cast(uint32_t, half_bits_to_float(xraw));
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         float xc[8];
@@ -288,18 +347,46 @@ __global__ __launch_bounds__(256) void matvec_kernel(
         }
     }
 
+    CQ_STAMP(2);
     // ---- reduce over the four lane groups; lane group kq ends up with columns 4kq .. 4kq+3
-    float h8[8], q4[4];
+    float h8[8], q4[1][4];
 #pragma unroll
     for (int i = 0; i < 8; i++) h8[i] = swap32_add(tot[i], tot[8 + i]);
 #pragma unroll
-    for (int i = 0; i < 4; i++) q4[i] = swap16_add(h8[i], h8[4 + i]);
-    *reinterpret_cast<float4 *>(&s_red[wave][16 * nl + 4 * kq]) = make_float4(q4[0], q4[1], q4[2], q4[3]);
-    __syncthreads();
-    float vals[1][1];
-    vals[0][0] = (s_red[0][tid] + s_red[1][tid]) + (s_red[2][tid] + s_red[3][tid]);
-    const int n = tile * kTileCols + tid;
-    splitk_finish<__half, 1, 1>(vals, 1, N, n, n < N, tile, split, plan.splits, partial, tickets, mul, accumulate);
+    for (int i = 0; i < 4; i++) q4[0][i] = swap16_add(h8[i], h8[4 + i]);
+    if (NW == 1) {
+        const int n = n0 + 4 * kq;
+        CQ_STAMP(3);
+#ifdef CQ_EXP_NOEPILOGUE
+        if (n < N && q4[0][0] == 123.f) mul[n] = __float2half(q4[0][1]);
+#else
+        splitk_finish<__half, 1, 4>(q4, 1, N, n, n < N, plan.splits, acc_words, mul, accumulate);
+#endif
+        CQ_STAMP(4);
+    } else {
+        // ---- across the workgroup's wavefronts through LDS, then 4 / NW columns per thread
+        __shared__ float s_red[NW][kTileCols];
+        *reinterpret_cast<float4 *>(&s_red[wave][16 * nl + 4 * kq]) = make_float4(q4[0][0], q4[0][1], q4[0][2], q4[0][3]);
+        __syncthreads();
+        constexpr int CPT = NW <= 4 ? 4 / NW : 1;  // columns per thread; 8 waves: first 256 threads
+        float vals[1][CPT];
+#pragma unroll
+        for (int c = 0; c < CPT; c++) {
+            float v = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < NW; wv++) v += s_red[wv][(tid * CPT + c) & (kTileCols - 1)];
+            vals[0][c] = v;
+        }
+        const int n = tile * kTileCols + tid * CPT;
+        CQ_STAMP(3);
+#ifdef CQ_EXP_NOEPILOGUE
+        if (n < N && vals[0][0] == 123.f) mul[n] = __float2half(vals[0][0]);
+#else
+        splitk_finish<__half, 1, CPT>(vals, 1, N, n, n < N && tid * CPT < kTileCols, plan.splits, acc_words, mul,
+                                      accumulate);
+#endif
+        CQ_STAMP(4);
+    }
 }
 
 bool matvec_supported(int bits, int B, int K, int N, int C, int G) {
@@ -312,24 +399,69 @@ bool matvec_supported(int bits, int B, int K, int N, int C, int G) {
     const long long cbytes = (long long)C * N * 2;
     const long long sbytes = (long long)ceil_div(K - C, G) * N * 2;
     if (wbytes >= 0x7fff0000ll || cbytes >= 0x7fff0000ll || sbytes >= 0x7fff0000ll) return false;
+    if (make_plan(K, N, C, 8, 64).splits > kMaxSplits) return false;
     return K - C > 0;
+}
+
+#ifndef CQ_MIN_WGS
+#define CQ_MIN_WGS 256
+#endif
+
+template <int BITS, int NW, int KPL>
+static hipError_t launch_matvec_nw(const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
+                                   const int16_t *cherry_indices, const __half *scales, __half *mul, int K, int N,
+                                   int C, int G, int accumulate, void *workspace, hipStream_t stream) {
+    const Plan plan = make_plan(K, N, C, NW, 4 * KPL);
+    hipLaunchKernelGGL((matvec_kernel<BITS, NW, KPL>), dim3(plan.tiles * plan.splits), dim3(64 * NW), 0, stream,
+                       vec, qweight, cherry_weight, cherry_indices, scales, mul,
+                       reinterpret_cast<unsigned long long *>(workspace), K, N, C, G, accumulate, plan);
+    return hipGetLastError();
+}
+
+// Positions per lane group.  Small layers are latency bound: 64-position units (8 KB per wave)
+// put twice the wavefronts in flight and halve the compute each one still has to do when its
+// data lands.  Large layers are throughput bound and prefer 128-position units (fewer waves,
+// less fixed work per byte).  Measured crossover on MI355X: about 64 MB of packed weights.
+int matvec_kpl(int bits, int K, int N, int C) {
+#ifdef CQ_KPL
+    (void)bits; (void)K; (void)N; (void)C;
+    return CQ_KPL;
+#else
+    const long long bytes = (long long)(K - C) / 8 * bits * N;
+    return bytes < (64ll << 20) ? 16 : 32;
+#endif
+}
+
+int matvec_waves_per_wg(int K, int N, int C, int kpl) {
+    const int max_waves = kpl == 16 ? 8 : 4;
+    int nw = choose_units_per_wg(K, N, C, max_waves, CQ_MIN_WGS, 4 * kpl);
+    while (nw < max_waves && make_plan(K, N, C, nw, 4 * kpl).splits > kMaxSplits) nw <<= 1;
+    return nw;
 }
 
 hipError_t launch_matvec(int bits, const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
                          const int16_t *cherry_indices, const __half *scales, __half *mul, int K, int N, int C,
                          int G, int accumulate, void *workspace, hipStream_t stream) {
-    Plan plan = make_plan(K, N, C, 4);
-    unsigned *tickets = reinterpret_cast<unsigned *>(workspace);
-    float *partial =
-        reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + workspace_counter_bytes(N));
-    dim3 grid(plan.tiles * plan.splits), block(256);
-    if (bits == 4)
-        hipLaunchKernelGGL(matvec_kernel<4>, grid, block, 0, stream, vec, qweight, cherry_weight, cherry_indices,
-                           scales, mul, partial, tickets, K, N, C, G, accumulate, plan);
-    else
-        hipLaunchKernelGGL(matvec_kernel<3>, grid, block, 0, stream, vec, qweight, cherry_weight, cherry_indices,
-                           scales, mul, partial, tickets, K, N, C, G, accumulate, plan);
-    return hipGetLastError();
+    const int kpl = matvec_kpl(bits, K, N, C);
+    const int nw = matvec_waves_per_wg(K, N, C, kpl);
+#define CQ_LAUNCH(B, W, P)                                                                                   \
+    return launch_matvec_nw<B, W, P>(vec, qweight, cherry_weight, cherry_indices, scales, mul, K, N, C, G,   \
+                                     accumulate, workspace, stream)
+#define CQ_PICK_NW(B, P)                                                                                     \
+    do {                                                                                                     \
+        if (nw >= 8 && P == 16) CQ_LAUNCH(B, 8, 16);                                                         \
+        if (nw >= 4) CQ_LAUNCH(B, 4, P);                                                                     \
+        if (nw == 2) CQ_LAUNCH(B, 2, P);                                                                     \
+        CQ_LAUNCH(B, 1, P);                                                                                  \
+    } while (0)
+    if (bits == 4) {
+        if (kpl == 16) CQ_PICK_NW(4, 16);
+        CQ_PICK_NW(4, 32);
+    }
+    if (kpl == 16) CQ_PICK_NW(3, 16);
+    CQ_PICK_NW(3, 32);
+#undef CQ_PICK_NW
+#undef CQ_LAUNCH
 }
 
 }  // namespace cq

@@ -49,8 +49,6 @@ _lib.cherryq_unpack_f16.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _int, _int, _
 _lib.cherryq_unpack_f16.restype = _int
 _lib.cherryq_workspace_bytes.argtypes = [_int, _int, _int, _int]
 _lib.cherryq_workspace_bytes.restype = _sz
-_lib.cherryq_workspace_counter_bytes.argtypes = [_int]
-_lib.cherryq_workspace_counter_bytes.restype = _sz
 _lib.cherryq_status_string.argtypes = [_int]
 _lib.cherryq_status_string.restype = ctypes.c_char_p
 _lib.cherryq_version.restype = _int
@@ -78,7 +76,7 @@ def _check(t: torch.Tensor, name: str, dtype, ndim: int, device=None):
 
 
 # Split-K scratch: one zero-initialised buffer per (device, stream), grown on demand.  The
-# kernels leave the counter region zero after every call, so the buffer is reusable as is.
+# kernels leave it all zero after every call, so the buffer is reusable as is.
 _workspaces: dict = {}
 
 
@@ -86,7 +84,7 @@ def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
     key = (device.index, stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        ws = torch.zeros(max(nbytes, 1 << 18), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
 
@@ -123,12 +121,14 @@ def _matmul(fn, what, vec, qweight, cherry_weight, cherry_indices, scales, mul, 
         raise RuntimeError(f"mul shape {tuple(mul.shape)} != {(batch, n)}")
     if batch == 0:
         return
-    with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
-        need = _lib.cherryq_workspace_bytes(batch, k, n, c)
-        ws = _workspace(dev, stream, need)
-        rc = fn(_ptr(vec), _ptr(qweight), _ptr(cherry_weight), _ptr(cherry_indices), _ptr(scales), _ptr(mul),
-                batch, k, n, c, group_size, 1 if accumulate else 0, ws.data_ptr(), ws.numel(), stream)
+    if torch.cuda.current_device() != dev.index:
+        with torch.cuda.device(dev):
+            return _matmul(fn, what, vec, qweight, cherry_weight, cherry_indices, scales, mul, group_size,
+                           w_bits, io_dtype, idx_dtype, accumulate)
+    stream = torch.cuda.current_stream().cuda_stream
+    ws = _workspace(dev, stream, _lib.cherryq_workspace_bytes(batch, k, n, c))
+    rc = fn(_ptr(vec), _ptr(qweight), _ptr(cherry_weight), _ptr(cherry_indices), _ptr(scales), _ptr(mul),
+            batch, k, n, c, group_size, 1 if accumulate else 0, ws.data_ptr(), ws.numel(), stream)
     if rc != 0:
         _fail(rc, what)
 

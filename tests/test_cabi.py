@@ -31,7 +31,7 @@ def test_header_declares_the_expected_entry_points():
     names = declared_functions()
     for n in ("cherryq_vecquant4matmul_f16", "cherryq_vecquant3matmul_f16", "cherryq_vecquant3matmul_f32",
               "cherryq_dequantize3_normal_f32", "cherryq_dequantize4_normal_f32", "cherryq_unpack_f16",
-              "cherryq_workspace_bytes", "cherryq_workspace_counter_bytes", "cherryq_version",
+              "cherryq_workspace_bytes", "cherryq_version",
               "cherryq_status_string"):
         assert n in names
 
@@ -51,13 +51,10 @@ def test_version_and_status_strings(lib):
 
 def test_workspace_sizes(lib):
     lib.cherryq_workspace_bytes.restype = ctypes.c_size_t
-    lib.cherryq_workspace_counter_bytes.restype = ctypes.c_size_t
-    c = lib.cherryq_workspace_counter_bytes(11008)
-    assert c % 256 == 0 and c >= 43 * 4
     a = lib.cherryq_workspace_bytes(1, 4096, 11008, 16)
     b = lib.cherryq_workspace_bytes(16, 4096, 11008, 16)
-    assert a >= c + 33 * 11008 * 4 and b >= c + 16 * 33 * 11008 * 4
-    assert lib.cherryq_workspace_bytes(64, 4096, 11008, 16) == b
+    assert a % 256 == 0 and a >= 11008 * 8 and b >= 16 * 11008 * 8
+    assert lib.cherryq_workspace_bytes(64, 4096, 11008, 16) == b  # batches run 16 rows at a time
 
 
 def _call(fn, *, vec=0x1000, qw=0x1000, cw=0x1000, idx=0x1000, sc=0x1000, mul=0x1000, b=1, k=4096, n=4096,
@@ -82,6 +79,7 @@ def test_argument_validation_rejects_before_launch(lib):
     assert _call(f3f, idx=None) == -1
     assert _call(f4, ws=None) == -4
     assert _call(f4, wsb=1024) == -4
+    assert _call(f4, n=11008, wsb=11008 * 8 - 1) == -4
     assert _call(f4, ws=0x1010) == -4
     assert _call(f4, qw=0x1001) == -6
     assert _call(f4, b=-1) == -2
