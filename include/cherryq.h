@@ -49,16 +49,21 @@ int cherryq_version(void);
 const char *cherryq_status_string(int status);
 
 /*
- * Split-K workspace.  The fused entry points split the reduction over K across workgroups,
- * which meet in one 64-bit accumulator word per output element (fixed-point running sum plus
- * an arrival count, added with a single atomic; see csrc/cq_common.cuh).  The words live in a
- * caller-provided device buffer of at least cherryq_workspace_bytes() bytes, 256-byte aligned.
- * The buffer must be all zero before the first call; every call leaves it all zero again.
- * Calls that may overlap in time (different streams) must use different workspaces.  Has no
- * counterpart in the reference, whose kernels add fp16 partials into `mul` with atomics
- * (csrc/quant_cuda_kernel.cu:833).
+ * Device memory the fused entry points need beside their operands (the reference's kernels need
+ * none: they add fp16 partials into `mul` with atomics, csrc/quant_cuda_kernel.cu:833).
+ *
+ * workspace: where the K splits of different workgroups meet -- one 64-bit accumulator word per
+ *   output element (fixed-point running sum plus an arrival count, added with a single atomic)
+ *   and one arrival ticket per 256-column tile.  At least cherryq_workspace_bytes() bytes,
+ *   256-byte aligned.  It must be all zero before the first call; every call leaves it all zero
+ *   again, whatever the shapes of earlier calls were.
+ * scratch: uninitialised memory for the batched path (batch >= 2): per-split partial tiles and
+ *   the activations laid out in matrix-core operand order.  At least cherryq_scratch_bytes()
+ *   bytes (0 for batch 1, then it may be NULL), 256-byte aligned.
+ * Calls that may overlap in time (different streams) must use different workspace and scratch.
  */
 size_t cherryq_workspace_bytes(int batch, int in_features, int out_features, int num_cherries);
+size_t cherryq_scratch_bytes(int batch, int in_features, int out_features, int num_cherries);
 
 /*
  * Replaces quant_cuda.vecquant4matmul_cherryq (csrc/quant_cuda.cpp:56-69,
@@ -69,7 +74,8 @@ int cherryq_vecquant4matmul_f16(const void *vec, const uint8_t *qweight, const v
                                 const int16_t *cherry_indices, const void *scales, void *mul,
                                 int batch, int in_features, int out_features, int num_cherries,
                                 int group_size, int accumulate, void *workspace,
-                                size_t workspace_bytes, void *stream);
+                                size_t workspace_bytes, void *scratch, size_t scratch_bytes,
+                                void *stream);
 
 /*
  * Replaces quant_cuda.vecquant3matmul_cherryq with fp16=True (csrc/quant_cuda.cpp:41-54,
@@ -81,7 +87,8 @@ int cherryq_vecquant3matmul_f16(const void *vec, const uint8_t *qweight, const v
                                 const int16_t *cherry_indices, const void *scales, void *mul,
                                 int batch, int in_features, int out_features, int num_cherries,
                                 int group_size, int accumulate, void *workspace,
-                                size_t workspace_bytes, void *stream);
+                                size_t workspace_bytes, void *scratch, size_t scratch_bytes,
+                                void *stream);
 
 /*
  * Replaces quant_cuda.vecquant3matmul_cherryq with fp16=False: fp32 vec / cherry_weight /
@@ -92,7 +99,8 @@ int cherryq_vecquant3matmul_f32(const float *vec, const uint8_t *qweight, const 
                                 const int32_t *cherry_indices, const float *scales, float *mul,
                                 int batch, int in_features, int out_features, int num_cherries,
                                 int group_size, int accumulate, void *workspace,
-                                size_t workspace_bytes, void *stream);
+                                size_t workspace_bytes, void *scratch, size_t scratch_bytes,
+                                void *stream);
 
 /*
  * Replace quant_cuda.Dequantize3Normal / Dequantize4Normal (csrc/quant_cuda.cpp:26-38,

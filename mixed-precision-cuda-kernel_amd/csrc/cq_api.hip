@@ -17,20 +17,38 @@ static bool force_generic() {
 }
 
 // One 64-bit accumulator word per output element of the largest batch chunk a kernel handles.
-size_t workspace_bytes(int B, int K, int N, int C) {
-    (void)K;
-    (void)C;
+static void clamp_dims(int &B, int &K, int &N, int &C) {
     if (B < 1) B = 1;
+    if (K < 8) K = 8;
+    if (N < 8) N = 8;
+    if (C < 0) C = 0;
+    if (C > K) C = K;
+}
+
+// zero-kept: accumulator words (batch 1 and the generic kernel) and, for batches, the tickets
+size_t workspace_bytes(int B, int K, int N, int C) {
+    clamp_dims(B, K, N, C);
     size_t rows = (size_t)(B < 16 ? B : 16);
-    size_t bytes = rows * (size_t)(N > 0 ? N : 1) * sizeof(unsigned long long);
-    return (bytes + 255) / 256 * 256;
+    size_t bytes = (rows * (size_t)N * sizeof(unsigned long long) + 255) / 256 * 256;
+    if (B >= 2) {
+        size_t b2 = batch_workspace(K, N, C).workspace_total;
+        if (b2 > bytes) bytes = b2;
+    }
+    return bytes;
+}
+
+// uninitialised: partial tiles and prepared activations of the matrix-core path
+size_t scratch_bytes(int B, int K, int N, int C) {
+    clamp_dims(B, K, N, C);
+    return B >= 2 ? batch_workspace(K, N, C).scratch_total : 0;
 }
 
 static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 static int check_common(const void *vec, const void *qweight, const void *cherry_weight,
                         const void *cherry_indices, const void *scales, const void *mul, int B, int K, int N,
-                        int C, int G, void *workspace, size_t workspace_bytes_given) {
+                        int C, int G, void *workspace, size_t workspace_bytes_given, void *scratch,
+                        size_t scratch_bytes_given) {
     if (B < 0 || K <= 0 || N <= 0 || C < 0 || C > K) return CHERRYQ_E_SHAPE;
     if (K % 8 || N % 8 || C % 8) return CHERRYQ_E_SHAPE;
     if (K - C <= 0 && C == 0) return CHERRYQ_E_SHAPE;
@@ -43,15 +61,18 @@ static int check_common(const void *vec, const void *qweight, const void *cherry
         return CHERRYQ_E_ALIGN;
     if (!workspace || !aligned(workspace, 256) || workspace_bytes_given < workspace_bytes(B, K, N, C))
         return CHERRYQ_E_WORKSPACE;
+    const size_t need = scratch_bytes(B, K, N, C);
+    if (need && (!scratch || !aligned(scratch, 256) || scratch_bytes_given < need)) return CHERRYQ_E_WORKSPACE;
     return CHERRYQ_OK;
 }
 
 template <int BITS>
 static int matmul_f16(const void *vec, const uint8_t *qweight, const void *cherry_weight,
                       const int16_t *cherry_indices, const void *scales, void *mul, int B, int K, int N,
-                      int C, int G, int accumulate, void *workspace, size_t wsb, void *stream) {
+                      int C, int G, int accumulate, void *workspace, size_t wsb, void *scratch, size_t scb,
+                      void *stream) {
     int rc = check_common(vec, qweight, cherry_weight, cherry_indices, scales, mul, B, K, N, C, G, workspace,
-                          wsb);
+                          wsb, scratch, scb);
     if (rc) return rc;
     if (B == 0) return CHERRYQ_OK;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
@@ -60,11 +81,10 @@ static int matmul_f16(const void *vec, const uint8_t *qweight, const void *cherr
     const __half *sc = reinterpret_cast<const __half *>(scales);
     __half *y = reinterpret_cast<__half *>(mul);
     hipError_t e;
-    if (!force_generic() && matvec_supported(BITS, B, K, N, C, G)) {
-        e = hipSuccess;
-        for (int b = 0; b < B && e == hipSuccess; b++)
-            e = launch_matvec(BITS, x + (size_t)b * K, qweight, cw, cherry_indices, sc, y + (size_t)b * N, K,
-                              N, C, G, accumulate, workspace, s);
+    if (!force_generic() && B == 1 && matvec_supported(BITS, B, K, N, C, G)) {
+        e = launch_matvec(BITS, x, qweight, cw, cherry_indices, sc, y, K, N, C, G, accumulate, workspace, s);
+    } else if (!force_generic() && batch_supported(BITS, B, K, N, C, G)) {
+        e = launch_batch(BITS, x, qweight, cw, cherry_indices, sc, y, B, K, N, C, G, accumulate, workspace, scratch, s);
     } else {
         e = launch_generic<BITS, __half, int16_t>(x, qweight, cw, cherry_indices, sc, y, B, K, N, C, G,
                                                   accumulate, workspace, s);
@@ -98,31 +118,39 @@ size_t cherryq_workspace_bytes(int batch, int in_features, int out_features, int
     return cq::workspace_bytes(batch, in_features, out_features, num_cherries);
 }
 
+size_t cherryq_scratch_bytes(int batch, int in_features, int out_features, int num_cherries) {
+    return cq::scratch_bytes(batch, in_features, out_features, num_cherries);
+}
+
 int cherryq_vecquant4matmul_f16(const void *vec, const uint8_t *qweight, const void *cherry_weight,
                                 const int16_t *cherry_indices, const void *scales, void *mul, int batch,
                                 int in_features, int out_features, int num_cherries, int group_size,
-                                int accumulate, void *workspace, size_t workspace_bytes, void *stream) {
+                                int accumulate, void *workspace, size_t workspace_bytes, void *scratch,
+                                size_t scratch_bytes, void *stream) {
     if (group_size < 128) return CHERRYQ_E_GROUP;  // csrc/quant_cuda_kernel.cu:684
     return cq::matmul_f16<4>(vec, qweight, cherry_weight, cherry_indices, scales, mul, batch, in_features,
                              out_features, num_cherries, group_size, accumulate, workspace, workspace_bytes,
-                             stream);
+                             scratch, scratch_bytes, stream);
 }
 
 int cherryq_vecquant3matmul_f16(const void *vec, const uint8_t *qweight, const void *cherry_weight,
                                 const int16_t *cherry_indices, const void *scales, void *mul, int batch,
                                 int in_features, int out_features, int num_cherries, int group_size,
-                                int accumulate, void *workspace, size_t workspace_bytes, void *stream) {
+                                int accumulate, void *workspace, size_t workspace_bytes, void *scratch,
+                                size_t scratch_bytes, void *stream) {
     return cq::matmul_f16<3>(vec, qweight, cherry_weight, cherry_indices, scales, mul, batch, in_features,
                              out_features, num_cherries, group_size, accumulate, workspace, workspace_bytes,
-                             stream);
+                             scratch, scratch_bytes, stream);
 }
 
 int cherryq_vecquant3matmul_f32(const float *vec, const uint8_t *qweight, const float *cherry_weight,
                                 const int32_t *cherry_indices, const float *scales, float *mul, int batch,
                                 int in_features, int out_features, int num_cherries, int group_size,
-                                int accumulate, void *workspace, size_t workspace_bytes, void *stream) {
+                                int accumulate, void *workspace, size_t workspace_bytes, void *scratch,
+                                size_t scratch_bytes, void *stream) {
     int rc = cq::check_common(vec, qweight, cherry_weight, cherry_indices, scales, mul, batch, in_features,
-                              out_features, num_cherries, group_size, workspace, workspace_bytes);
+                              out_features, num_cherries, group_size, workspace, workspace_bytes, scratch,
+                              scratch_bytes);
     if (rc) return rc;
     if (batch == 0) return CHERRYQ_OK;
     return (int)cq::launch_generic<3, float, int32_t>(vec, qweight, cherry_weight, cherry_indices, scales, mul,

@@ -27,4 +27,16 @@ hipError_t launch_matvec(int bits, const __half *vec, const uint8_t *qweight, co
                          const int16_t *cherry_indices, const __half *scales, __half *mul, int K, int N,
                          int C, int G, int accumulate, void *workspace, hipStream_t stream);
 
+// cq_batch.hip: 2..16 batch rows per pass on the matrix cores.
+struct BatchWorkspace {
+    size_t tickets, workspace_total;                       // zero-kept workspace: offset, size
+    size_t partial, xa, rowsum, rowshift, scratch_total;  // uninitialised scratch: offsets, size
+};
+BatchWorkspace batch_workspace(int K, int N, int C);
+bool batch_supported(int bits, int B, int K, int N, int C, int G);
+hipError_t launch_batch(int bits, const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
+                        const int16_t *cherry_indices, const __half *scales, __half *mul, int B, int K, int N,
+                        int C, int G, int accumulate, void *workspace, void *scratch, hipStream_t stream);
+size_t scratch_bytes(int B, int K, int N, int C);
+
 }  // namespace cq

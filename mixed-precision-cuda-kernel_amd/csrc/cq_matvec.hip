@@ -391,7 +391,7 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
 
 bool matvec_supported(int bits, int B, int K, int N, int C, int G) {
     (void)bits;
-    if (B < 1 || B > 4) return false;
+    if (B != 1) return false;
     if (C > kMaxFastCherries) return false;
     if (G % 32) return false;
     // byte offsets are 32-bit and kOob must lie beyond every buffer

@@ -38,7 +38,7 @@ if not _LIB_PATH.exists():
 _lib = ctypes.CDLL(str(_LIB_PATH))
 
 _vp, _int, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
-_MATMUL_ARGS = [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _vp, _sz, _vp]
+_MATMUL_ARGS = [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _vp, _sz, _vp, _sz, _vp]
 for _name in ("cherryq_vecquant4matmul_f16", "cherryq_vecquant3matmul_f16", "cherryq_vecquant3matmul_f32"):
     getattr(_lib, _name).argtypes = _MATMUL_ARGS
     getattr(_lib, _name).restype = _int
@@ -49,6 +49,8 @@ _lib.cherryq_unpack_f16.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _int, _int, _
 _lib.cherryq_unpack_f16.restype = _int
 _lib.cherryq_workspace_bytes.argtypes = [_int, _int, _int, _int]
 _lib.cherryq_workspace_bytes.restype = _sz
+_lib.cherryq_scratch_bytes.argtypes = [_int, _int, _int, _int]
+_lib.cherryq_scratch_bytes.restype = _sz
 _lib.cherryq_status_string.argtypes = [_int]
 _lib.cherryq_status_string.restype = ctypes.c_char_p
 _lib.cherryq_version.restype = _int
@@ -75,9 +77,11 @@ def _check(t: torch.Tensor, name: str, dtype, ndim: int, device=None):
         raise RuntimeError(f"{name} must be contiguous")
 
 
-# Split-K scratch: one zero-initialised buffer per (device, stream), grown on demand.  The
-# kernels leave it all zero after every call, so the buffer is reusable as is.
+# Per (device, stream): a zero-initialised workspace (the kernels leave it all zero after every
+# call, so it is reusable as is) and an uninitialised scratch buffer for the batched path.  Both
+# grow on demand.
 _workspaces: dict = {}
+_scratches: dict = {}
 
 
 def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
@@ -87,6 +91,17 @@ def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
         ws = torch.zeros(max(nbytes, 1 << 18), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
+
+
+def _scratch(device: torch.device, stream: int, nbytes: int):
+    if nbytes == 0:
+        return None
+    key = (device.index, stream)
+    sc = _scratches.get(key)
+    if sc is None or sc.numel() < nbytes:
+        sc = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _scratches[key] = sc
+    return sc
 
 
 def _ptr(t: torch.Tensor):
@@ -127,8 +142,10 @@ def _matmul(fn, what, vec, qweight, cherry_weight, cherry_indices, scales, mul, 
                            w_bits, io_dtype, idx_dtype, accumulate)
     stream = torch.cuda.current_stream().cuda_stream
     ws = _workspace(dev, stream, _lib.cherryq_workspace_bytes(batch, k, n, c))
+    sc = _scratch(dev, stream, _lib.cherryq_scratch_bytes(batch, k, n, c)) if batch > 1 else None
     rc = fn(_ptr(vec), _ptr(qweight), _ptr(cherry_weight), _ptr(cherry_indices), _ptr(scales), _ptr(mul),
-            batch, k, n, c, group_size, 1 if accumulate else 0, ws.data_ptr(), ws.numel(), stream)
+            batch, k, n, c, group_size, 1 if accumulate else 0, ws.data_ptr(), ws.numel(),
+            sc.data_ptr() if sc is not None else None, sc.numel() if sc is not None else 0, stream)
     if rc != 0:
         _fail(rc, what)
 

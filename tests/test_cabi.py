@@ -31,7 +31,7 @@ def test_header_declares_the_expected_entry_points():
     names = declared_functions()
     for n in ("cherryq_vecquant4matmul_f16", "cherryq_vecquant3matmul_f16", "cherryq_vecquant3matmul_f32",
               "cherryq_dequantize3_normal_f32", "cherryq_dequantize4_normal_f32", "cherryq_unpack_f16",
-              "cherryq_workspace_bytes", "cherryq_version",
+              "cherryq_workspace_bytes", "cherryq_scratch_bytes", "cherryq_version",
               "cherryq_status_string"):
         assert n in names
 
@@ -52,16 +52,21 @@ def test_version_and_status_strings(lib):
 def test_workspace_sizes(lib):
     lib.cherryq_workspace_bytes.restype = ctypes.c_size_t
     a = lib.cherryq_workspace_bytes(1, 4096, 11008, 16)
-    b = lib.cherryq_workspace_bytes(16, 4096, 11008, 16)
-    assert a % 256 == 0 and a >= 11008 * 8 and b >= 16 * 11008 * 8
-    assert lib.cherryq_workspace_bytes(64, 4096, 11008, 16) == b  # batches run 16 rows at a time
+    b = 16 * 11008 * 8
+    assert a % 256 == 0 and a >= 11008 * 8 and lib.cherryq_workspace_bytes(16, 4096, 11008, 16) >= b
+    assert lib.cherryq_workspace_bytes(64, 4096, 11008, 16) == lib.cherryq_workspace_bytes(16, 4096, 11008, 16)
+    assert lib.cherryq_workspace_bytes(2, 4096, 11008, 16) == b + 256  # batches: + one ticket per tile
+    lib.cherryq_scratch_bytes.restype = ctypes.c_size_t
+    assert lib.cherryq_scratch_bytes(1, 4096, 11008, 16) == 0
+    assert lib.cherryq_scratch_bytes(2, 4096, 11008, 16) >= 8 * 16 * 11008 * 4 + 33 * 4096
 
 
 def _call(fn, *, vec=0x1000, qw=0x1000, cw=0x1000, idx=0x1000, sc=0x1000, mul=0x1000, b=1, k=4096, n=4096,
-          c=16, g=128, acc=1, ws=0x1000, wsb=1 << 30, stream=None):
-    fn.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 6 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+          c=16, g=128, acc=1, ws=0x1000, wsb=1 << 30, scr=None, scrb=0, stream=None):
+    fn.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 6 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
+                                                               ctypes.c_size_t, ctypes.c_void_p]
     fn.restype = ctypes.c_int
-    return fn(vec, qw, cw, idx, sc, mul, b, k, n, c, g, acc, ws, wsb, stream)
+    return fn(vec, qw, cw, idx, sc, mul, b, k, n, c, g, acc, ws, wsb, scr, scrb, stream)
 
 
 def test_argument_validation_rejects_before_launch(lib):
@@ -82,6 +87,8 @@ def test_argument_validation_rejects_before_launch(lib):
     assert _call(f4, n=11008, wsb=11008 * 8 - 1) == -4
     assert _call(f4, ws=0x1010) == -4
     assert _call(f4, qw=0x1001) == -6
+    assert _call(f4, b=4) == -4           # batches need scratch
+    assert _call(f4, b=4, scr=0x2000, scrb=1024) == -4
     assert _call(f4, b=-1) == -2
     assert _call(f4, b=0) == 0            # empty batch: nothing to do, nothing launched
 

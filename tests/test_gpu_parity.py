@@ -216,6 +216,77 @@ def test_small_batches(qc, bits, k, n, b):
         assert orc.rel_l2(y[r], y_fused[r]) <= TOL, r
 
 
+@pytest.mark.parametrize("bits,k,n", [(4, 4096, 4096), (3, 4096, 4096), (4, 11008, 512), (3, 5120, 768)])
+def test_batch_one_hot_rows_are_bit_exact(qc, bits, k, n):
+    """16 one-hot activation rows through the matrix-core path: row i returns dequantised column
+    j_i bit for bit (subnormal code fields, per-row normalisation and the A/B operand order)."""
+    announce("batch one-hot", bits, k, n)
+    w, p = orc.synthetic_layer(k, n, bits, 128, seed=8)
+    dense = c_oracle.unpack(p, bits, 128, k)
+    idx = p["cherry_indices"].astype(np.int64)
+    nidx = orc.normal_indices(k, idx)
+    cols = [int(nidx[0]), int(nidx[1]), int(nidx[2]), int(nidx[3]), int(nidx[7]), int(nidx[8]), int(nidx[31]),
+            int(nidx[32]), int(nidx[127]), int(nidx[128]), int(nidx[-1]), int(nidx[-9]), int(idx[0]), int(idx[7]),
+            int(idx[8]), int(idx[-1])]
+    x = np.zeros((16, k), dtype=np.float16)
+    for i, j in enumerate(cols):
+        x[i, j] = 1
+    y = run_fused(qc, bits, x, p, 128)
+    for i, j in enumerate(cols):
+        np.testing.assert_array_equal(y[i], dense[:, j], err_msg=f"row {i} column {j}")
+    # rows of very different magnitude in one batch; powers of two keep the products exact
+    scale = np.array([2.0 ** e for e in (-14, -10, -6, -3, 0, 1, 3, 5, 7, 9, 11, 12, 13, 14, 15, 15)])
+    xs = (x.astype(np.float64) * scale[:, None]).astype(np.float16)
+    ys = run_fused(qc, bits, xs, p, 128)
+    want = c_oracle.fused(xs, p, bits, 128)
+    with np.errstate(over="ignore"):
+        np.testing.assert_array_equal(ys, want.astype(np.float16))
+
+
+@pytest.mark.parametrize("bits,k,n,b", [(4, 8192, 8192, 16), (4, 8192, 28672, 16), (4, 28672, 8192, 16),
+                                        (3, 13824, 5120, 8), (3, 5120, 13824, 4)])
+def test_batch_large_shapes(qc, bits, k, n, b):
+    """Configs 3 and 4 at their batch sizes: random packed bytes, C oracle on a column sample."""
+    announce("batch-large", bits, k, n, b)
+    p = orc.synthetic_packed_fast(k, n, bits, 128, seed=4)
+    rng = np.random.default_rng(b)
+    x = rng.standard_normal((b, k)).astype(np.float16)
+    y = run_fused(qc, bits, x, p, 128)
+    cols = np.sort(rng.choice(n, size=256, replace=False))
+    sub = {"cherry_indices": p["cherry_indices"], "cherry_weight": np.ascontiguousarray(p["cherry_weight"][:, cols]),
+           "qweight": np.ascontiguousarray(p["qweight"][:, cols]), "scales": np.ascontiguousarray(p["scales"][:, cols])}
+    assert orc.rel_l2(y[:, cols], c_oracle.fused(x, sub, bits, 128)) <= TOL
+    # the batch path agrees with the batch-1 path row by row (different kernels, same contract)
+    y0 = run_fused(qc, bits, x[:1], p, 128)
+    assert orc.rel_l2(y[0], y0[0]) <= TOL
+
+
+def test_batch_accumulate_scale_invariance_and_determinism(qc):
+    announce("batch-misc")
+    for bits in (3, 4):
+        k, n, b = 4096, 1024, 8
+        w, p = orc.synthetic_layer(k, n, bits, 128, seed=bits + 20)
+        rng = np.random.default_rng(5)
+        base = rng.standard_normal((b, k)).astype(np.float32)
+        for scale in (2.0 ** -12, 2.0 ** -5, 1.0, 2.0 ** 5):
+            x = (base * scale).astype(np.float16)
+            y = run_fused(qc, bits, x, p, 128)
+            assert orc.rel_l2(y, c_oracle.fused(x, p, bits, 128)) <= TOL, (bits, scale)
+        x = base.astype(np.float16)
+        init = rng.standard_normal((b, n)).astype(np.float16)
+        y1 = run_fused(qc, bits, x, p, 128, mul=init.copy())
+        want = (init.astype(np.float64) + c_oracle.fused(x, p, bits, 128))
+        assert orc.rel_l2(y1, want) <= TOL
+        np.testing.assert_array_equal(run_fused(qc, bits, x, p, 128), run_fused(qc, bits, x, p, 128))
+        # the generic kernel (independent code) agrees
+        os.environ["CHERRYQ_FORCE_GENERIC"] = "1"
+        try:
+            yg = run_fused(qc, bits, x, p, 128)
+        finally:
+            os.environ["CHERRYQ_FORCE_GENERIC"] = "0"
+        assert orc.rel_l2(run_fused(qc, bits, x, p, 128), yg) <= TOL
+
+
 @pytest.mark.parametrize("bits,gs,k,n,frac,b", [
     (3, 64, 1024, 512, 1 / 64, 1), (3, 64, 1024, 512, 1 / 64, 3),     # group 64 (reference G64 kernels)
     (4, 256, 2048, 512, 1 / 256, 1), (3, 256, 2048, 264, 1 / 256, 2),  # group 256, N not a multiple of 256
@@ -383,11 +454,13 @@ def test_direct_c_abi_call_with_raw_pointers(qc):
     ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
     stream = torch.cuda.Stream()
     fn = lib.cherryq_vecquant4matmul_f16
-    fn.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 6 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    fn.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 6 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
+                                                               ctypes.c_size_t, ctypes.c_void_p]
     fn.restype = ctypes.c_int
     torch.cuda.synchronize()
     rc = fn(x.data_ptr(), d["qweight"].data_ptr(), d["cherry_weight"].data_ptr(), d["cherry_indices"].data_ptr(),
-            d["scales"].data_ptr(), out.data_ptr(), 1, k, n, c, 128, 0, ws.data_ptr(), need, stream.cuda_stream)
+            d["scales"].data_ptr(), out.data_ptr(), 1, k, n, c, 128, 0, ws.data_ptr(), need, None, 0,
+            stream.cuda_stream)
     assert rc == 0
     stream.synchronize()
     want = c_oracle.fused(x.cpu().numpy(), p, bits, 128)
