@@ -166,6 +166,20 @@ def main():
     torch.cuda.set_device(0)
 
     if args.all:
+        # the small-batch path (matrix cores) on the shapes BASELINE names for it
+        for name, b in (("llama13b_attn_w3", 4), ("llama13b_attn_w3", 8), ("llama13b_gate_up_w3", 8),
+                        ("llama13b_down_w3", 8), ("llama70b_attn_w4", 16), ("llama70b_kv_w4", 16),
+                        ("llama70b_gate_up_w4", 16), ("llama70b_down_w4", 16), ("llama7b_gate_up_w4", 16)):
+            bits, k, n = WORKLOADS[name]
+            us, wall_us, *_ = time_gpu(bits, k, n, args.group, max(200, args.steps // 4), args.warmup, batch=b,
+                                      use_graph=not args.no_graph)
+            ab = algorithmic_bytes(bits, k, n, b, args.group)
+            fl = 2.0 * b * k * n
+            print(f"{name:24s} {bits}-bit {k:5d}->{n:5d} batch {b:2d}: {us:7.2f} us  {ab / us / 1e3:7.1f} GB/s "
+                  f"{ab / us / 1e3 / HBM_PEAK_GBS * 100:5.1f}% of 8 TB/s  {fl / us / 1e6:6.1f} TFLOP/s "
+                  f"({fl / us / 1e6 / 2500 * 100:4.1f}% of fp16 MFMA peak; prep + main kernel)",
+                  file=sys.stderr, flush=True)
+            torch.cuda.empty_cache()
         for name, (bits, k, n) in WORKLOADS.items():
             us, wall_us, *_ = time_gpu(bits, k, n, args.group, max(200, args.steps // 4), args.warmup,
                                       use_graph=not args.no_graph)

@@ -30,6 +30,18 @@
 #include "cq_common.cuh"
 #include "cq_kernels.h"
 
+// Optional per-wave phase timestamps for a profiling harness; compiled out in the library.
+#ifdef CQ_TRACE
+extern __device__ unsigned long long *g_cq_trace;
+#define CQB_STAMP(slot)                                                                                      \
+    do {                                                                                                     \
+        if (g_cq_trace && (threadIdx.x & 63) == 0)                                                           \
+            g_cq_trace[((size_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 8 + (slot)] = wall_clock64();         \
+    } while (0)
+#else
+#define CQB_STAMP(slot) do { } while (0)
+#endif
+
 namespace cq {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -38,16 +50,24 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kBatchRows = 16;        // MFMA M dimension; smaller batches are zero padded
 constexpr int kBatchWaves = 4;        // wavefronts per workgroup
-constexpr int kBatchMaxSplits = 8;    // bounds the partial-tile workspace
+constexpr int kBatchMaxSplits = 8;    // bounds the partial-tile scratch and the last workgroup's reads
 constexpr uint32_t kRsrcFlagsB = 0x00020000u;
 constexpr uint32_t kOobB = 0x80000000u;
 
 // position order inside one 8-position MFMA slice of a lane group, and the bit position p of
 // each code's field inside its 16-bit half (value seen by the matrix core = code * 2^(p-24))
-__device__ __constant__ int kOrd4[8] = {0, 2, 1, 3, 4, 6, 5, 7};
-__device__ __constant__ int kPos4[8] = {0, 0, 4, 4, 0, 0, 4, 4};
-__device__ __constant__ int kOrd3[8] = {0, 3, 1, 4, 5, 6, 2, 7};
-__device__ __constant__ int kPos3[8] = {0, 1, 3, 4, 7, 2, 6, 5};
+//   4-bit: ord = {0, 2, 1, 3, 4, 6, 5, 7}   p = {0, 0, 4, 4, 0, 0, 4, 4}
+//   3-bit: ord = {0, 3, 1, 4, 5, 6, 2, 7}   p = {0, 1, 3, 4, 7, 2, 6, 5}
+template <int BITS>
+__host__ __device__ constexpr int slice_ord(int kk) {
+    return BITS == 4 ? ((kk & 4) | ((kk & 1) << 1) | ((kk >> 1) & 1)) : (int)((0x72654130u >> (4 * kk)) & 7u);
+}
+template <int BITS>
+__host__ __device__ constexpr int slice_pos(int kk) {
+    return BITS == 4 ? ((kk & 2) ? 4 : 0) : (int)((0x56274310u >> (4 * kk)) & 7u);
+}
+static_assert(slice_ord<4>(1) == 2 && slice_ord<4>(2) == 1 && slice_ord<4>(6) == 5 && slice_pos<4>(3) == 4, "");
+static_assert(slice_ord<3>(1) == 3 && slice_ord<3>(6) == 2 && slice_pos<3>(4) == 7 && slice_pos<3>(7) == 5, "");
 
 BatchWorkspace batch_workspace(int K, int N, int C) {
     BatchWorkspace w;
@@ -99,16 +119,44 @@ __global__ __launch_bounds__(256) void batch_prep_kernel(const __half *__restric
         }
         return;
     }
+    // t[m] = idx[m] - m is non-decreasing; position k sits after every cherry m with t[m] <= k.
+    // Stage t in LDS (one pass over the indices) and walk this thread's 8 consecutive positions.
+    constexpr int kCap = 2048;
+    __shared__ int s_t[kCap];
     if (t < kBatchRows) s_max[t] = 0;
+    const bool staged = C <= kCap;
+    if (staged)
+        for (int mm = t; mm < C; mm += 256) s_t[mm] = (int)cherry_indices[mm] - mm;
     __syncthreads();
+    const int kb = u * kUnitK + 32 * q + 8 * s;
+    int lows[8];
+    if (staged) {
+        int lo = 0, hi = C;
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            const bool le = s_t[mid] <= kb;
+            lo = le ? mid + 1 : lo;
+            hi = le ? hi : mid;
+        }
+        lows[0] = lo;
+#pragma unroll
+        for (int j = 1; j < 8; j++) {
+            while (lo < C && s_t[lo] <= kb + j) lo++;
+            lows[j] = lo;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; j++) lows[j] = gather_offset(cherry_indices, C, kb + j);
+    }
     float v[8];
     unsigned m = 0;
     float sum = 0.f;
 #pragma unroll
     for (int kk = 0; kk < 8; kk++) {
-        const int k = u * kUnitK + 32 * q + 8 * s + (BITS == 4 ? kOrd4[kk] : kOrd3[kk]);
+        const int j = slice_ord<BITS>(kk);
+        const int k = kb + j;
         unsigned short hb = 0;
-        if (k < Kn && i < B) hb = __half_as_ushort(x[(size_t)i * K + k + gather_offset(cherry_indices, C, k)]);
+        if (k < Kn && i < B) hb = __half_as_ushort(x[(size_t)i * K + k + lows[j]]);
         v[kk] = __half2float(__ushort_as_half(hb));
         m = max(m, (unsigned)(hb & 0x7fffu));
         sum += v[kk];
@@ -120,7 +168,7 @@ __global__ __launch_bounds__(256) void batch_prep_kernel(const __half *__restric
     unsigned short h[8];
 #pragma unroll
     for (int kk = 0; kk < 8; kk++)
-        h[kk] = __half_as_ushort(__float2half_rn(ldexpf(v[kk], sh - (BITS == 4 ? kPos4[kk] : kPos3[kk]))));
+        h[kk] = __half_as_ushort(__float2half_rn(ldexpf(v[kk], sh - slice_pos<BITS>(kk))));
     xa[(size_t)u * 256 + t] = make_uint4(h[0] | h[1] << 16, h[2] | h[3] << 16, h[4] | h[5] << 16, h[6] | h[7] << 16);
     if (t < kBatchRows) {
         float tot = 0.f;
@@ -132,133 +180,185 @@ __global__ __launch_bounds__(256) void batch_prep_kernel(const __half *__restric
 }
 
 // ---- main kernel -------------------------------------------------------------------------------
+// Everything one unit needs from memory; two of these alternate so that the loads of the next
+// unit are in flight while the matrix cores work on the current one.
+struct UnitRegs {
+    u32x4 w[16];    // 16 (12) byte rows x 16 columns
+    u32x4 sc0, sc1; // 16 group scales (fp16)
+    uint4 a[4];     // prepared activations, one MFMA A operand per step
+    float4 rsum;    // row sums of the activations for the lane's 4 batch rows
+    int4 rsh;       // their normalisation shifts
+};
+
+struct BatchCtx {
+    __amdgpu_buffer_rsrc_t rw, rs, rc;
+    const uint4 *xa;
+    const float *rowsum;
+    const int *rowshift;
+    int N, G, units_normal, lane, kq, n0;
+    bool col_ok;
+};
+
 template <int BITS>
-__global__ __launch_bounds__(64 * kBatchWaves) void batch_kernel(
+__device__ __forceinline__ void issue_unit(UnitRegs &r, const BatchCtx &cx, int u) {
+    constexpr int R = BITS == 4 ? 16 : 12;
+    const uint4 *xau = cx.xa + (size_t)u * 256 + cx.lane;
+    const uint32_t woff = cx.col_ok ? (uint32_t)((u * 4 * R + cx.kq * R) * cx.N + cx.n0) : kOobB;
+#pragma unroll
+    for (int i = 0; i < R; i++)
+        r.w[i] = __builtin_amdgcn_raw_buffer_load_b128(cx.rw, woff + (uint32_t)(i * cx.N), 0, 2);
+    const int g = (u * kUnitK) / cx.G;
+    const uint32_t soff = cx.col_ok ? (uint32_t)(g * cx.N + cx.n0) * 2u : kOobB;
+    r.sc0 = __builtin_amdgcn_raw_buffer_load_b128(cx.rs, soff, 0, 0);
+    r.sc1 = __builtin_amdgcn_raw_buffer_load_b128(cx.rs, soff + 16, 0, 0);
+#pragma unroll
+    for (int s = 0; s < 4; s++) r.a[s] = xau[s * 64];
+    r.rsum = *reinterpret_cast<const float4 *>(cx.rowsum + u * kBatchRows + 4 * cx.kq);
+    r.rsh = *reinterpret_cast<const int4 *>(cx.rowshift + u * kBatchRows + 4 * cx.kq);
+}
+
+// tot[c][r]: column n0 + c, batch row 4 * kq + r
+template <int BITS>
+__device__ __forceinline__ void compute_unit(const UnitRegs &r, float4_t (&tot)[16]) {
+    constexpr float kGrid = BITS == 4 ? 7.5f : 3.5f;
+    float4_t d[16];
+#pragma unroll
+    for (int c = 0; c < 16; c++) d[c] = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        const half8_t av = __builtin_bit_cast(half8_t, r.a[s]);
+#pragma unroll
+        for (int dw = 0; dw < 4; dw++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                u32x4 b;
+                if (BITS == 4) {
+                    const uint32_t sel = 0x0c000c00u | (uint32_t)(j << 16) | (uint32_t)(4 + j);
+                    const uint32_t p0 = __builtin_amdgcn_perm(r.w[4 * s][dw], r.w[4 * s + 1][dw], sel);
+                    const uint32_t p1 = __builtin_amdgcn_perm(r.w[4 * s + 2][dw], r.w[4 * s + 3][dw], sel);
+                    b = (u32x4){p0 & 0x000f000fu, p0 & 0x00f000f0u, p1 & 0x000f000fu, p1 & 0x00f000f0u};
+                } else {
+                    const uint32_t sel = 0x0c000000u | (uint32_t)(j << 16) | (uint32_t)(j << 8) | (uint32_t)(4 + j);
+                    const uint32_t p1 = __builtin_amdgcn_perm(r.w[3 * s][dw], r.w[3 * s + 1][dw], sel);
+                    const uint32_t p2 = __builtin_amdgcn_perm(r.w[3 * s + 1][dw], r.w[3 * s + 2][dw], sel);
+                    b = (u32x4){p1 & 0x000e0007u, p1 & 0x00700038u, p2 & 0x001c0380u,
+                                (p1 & 0x000001c0u) | (p2 & 0x00e00000u)};
+                }
+                d[4 * dw + j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, __builtin_bit_cast(half8_t, b),
+                                                                      d[4 * dw + j], 0, 0, 0);
+            }
+        }
+    }
+    // tile -> totals: undo the normalisation, apply the grid offset and the group scale
+    const float f[4] = {ldexpf(1.f, 24 - r.rsh.x), ldexpf(1.f, 24 - r.rsh.y), ldexpf(1.f, 24 - r.rsh.z),
+                        ldexpf(1.f, 24 - r.rsh.w)};
+    const float o[4] = {-kGrid * r.rsum.x, -kGrid * r.rsum.y, -kGrid * r.rsum.z, -kGrid * r.rsum.w};
+#pragma unroll
+    for (int c = 0; c < 16; c++) {
+        const uint32_t sw = c < 8 ? r.sc0[c >> 1] : r.sc1[(c - 8) >> 1];
+        const float sc = __half2float(__ushort_as_half((unsigned short)((c & 1) ? (sw >> 16) : (sw & 0xffffu))));
+#pragma unroll
+        for (int q = 0; q < 4; q++) tot[c][q] += sc * (d[c][q] * f[q] + o[q]);
+    }
+}
+
+// cherry unit: 32 dense fp16 rows, 8 per lane group; B operands packed by v_perm_b32
+__device__ __forceinline__ void cherry_unit(const BatchCtx &cx, int u, float4_t (&tot)[16]) {
+    const int c0 = (u - cx.units_normal) * kCherryUnit + 8 * cx.kq;
+    const uint32_t coff = cx.col_ok ? (uint32_t)(c0 * cx.N + cx.n0) * 2u : kOobB;
+    u32x4 cw[8][2];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        cw[i][0] = __builtin_amdgcn_raw_buffer_load_b128(cx.rc, coff + (uint32_t)(i * cx.N * 2), 0, 2);
+        cw[i][1] = __builtin_amdgcn_raw_buffer_load_b128(cx.rc, coff + (uint32_t)(i * cx.N * 2) + 16, 0, 2);
+    }
+    const half8_t av = __builtin_bit_cast(half8_t, cx.xa[(size_t)u * 256 + cx.lane]);
+#pragma unroll
+    for (int c = 0; c < 16; c++) {
+        const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;  // (row r half, row r+1 half)
+        u32x4 b;
+#pragma unroll
+        for (int rp = 0; rp < 4; rp++)
+            b[rp] = __builtin_amdgcn_perm(cw[2 * rp + 1][c >> 3][(c & 7) >> 1], cw[2 * rp][c >> 3][(c & 7) >> 1], sel);
+        tot[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, __builtin_bit_cast(half8_t, b), tot[c], 0, 0, 0);
+    }
+}
+
+template <int BITS>
+__global__ __launch_bounds__(64 * kBatchWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void batch_kernel(
     const uint8_t *__restrict__ qweight, const __half *__restrict__ cherry_weight,
     const __half *__restrict__ scales, __half *__restrict__ mul, const uint4 *__restrict__ xa,
     const float *__restrict__ rowsum, const int *__restrict__ rowshift, float *__restrict__ partial,
     unsigned *__restrict__ tickets, int B, int K, int N, int C, int G, int accumulate, Plan plan,
     int units_per_wave) {
-    constexpr int R = BITS == 4 ? 16 : 12;  // byte rows per lane group per unit
-    constexpr float kGrid = BITS == 4 ? 7.5f : 3.5f;
     __shared__ float s_red[kBatchWaves][kBatchRows][kTileCols];  // 64 KB
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kq = lane >> 4, nl = lane & 15;
     const int tile = blockIdx.x % plan.tiles;
     const int split = blockIdx.x / plan.tiles;
-    const int n0 = tile * kTileCols + nl * 16;
-    const bool col_ok = n0 < N;
     const int Kn = K - C;
-    const int qrows = Kn / 8 * BITS;
-    const int ng = ceil_div(Kn, G);
-    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void *)qweight, 0, qrows * N, kRsrcFlagsB);
-    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)scales, 0, ng * N * 2, kRsrcFlagsB);
-    const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc((void *)cherry_weight, 0, C * N * 2, kRsrcFlagsB);
+    BatchCtx cx;
+    cx.rw = __builtin_amdgcn_make_buffer_rsrc((void *)qweight, 0, Kn / 8 * BITS * N, kRsrcFlagsB);
+    cx.rs = __builtin_amdgcn_make_buffer_rsrc((void *)scales, 0, ceil_div(Kn, G) * N * 2, kRsrcFlagsB);
+    cx.rc = __builtin_amdgcn_make_buffer_rsrc((void *)cherry_weight, 0, C * N * 2, kRsrcFlagsB);
+    cx.xa = xa;
+    cx.rowsum = rowsum;
+    cx.rowshift = rowshift;
+    cx.N = N;
+    cx.G = G;
+    cx.units_normal = plan.units_normal;
+    cx.lane = lane;
+    cx.kq = kq;
+    cx.n0 = tile * kTileCols + nl * 16;
+    cx.col_ok = cx.n0 < N;
 
-    // tot[c][r]: column n0 + c, batch row 4 * kq + r
     float4_t tot[16];
 #pragma unroll
     for (int c = 0; c < 16; c++) tot[c] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-    const int u_first = split * plan.units_per_wg + wave;
+    // this wave's units: u0, u0 + 4, u0 + 8, ...  (the 4 waves interleave).  Two units per round:
+    // both sets of loads are issued before the first unit is consumed, so the second unit's
+    // 16 KB arrive while the matrix cores work on the first.
+    // this wave's units: u0, u0 + 4, u0 + 8, ...  (the 4 waves interleave).  One register set per
+    // wave keeps the kernel at two waves per SIMD, which overlap each other's loads and MFMAs.
+    CQB_STAMP(0);
+    const int u0 = split * plan.units_per_wg + wave;
     for (int it = 0; it < units_per_wave; it++) {
-        const int u = u_first + it * kBatchWaves;
-        if (u >= plan.units_total) break;
-        const uint4 *xau = xa + (size_t)u * 256 + lane;
-        if (u < plan.units_normal) {
-            const uint32_t woff = col_ok ? (uint32_t)((u * 4 * R + kq * R) * N + n0) : kOobB;
-            u32x4 w[R];
-#pragma unroll
-            for (int r = 0; r < R; r++) w[r] = __builtin_amdgcn_raw_buffer_load_b128(rw, woff + (uint32_t)(r * N), 0, 2);
-            const int g = (u * kUnitK) / G;
-            const uint32_t soff = col_ok ? (uint32_t)(g * N + n0) * 2u : kOobB;
-            const u32x4 sc0 = __builtin_amdgcn_raw_buffer_load_b128(rs, soff, 0, 0);
-            const u32x4 sc1 = __builtin_amdgcn_raw_buffer_load_b128(rs, soff + 16, 0, 0);
-            uint4 a[4];
-#pragma unroll
-            for (int s = 0; s < 4; s++) a[s] = xau[s * 64];
-            const float4 rsum = *reinterpret_cast<const float4 *>(rowsum + u * kBatchRows + 4 * kq);
-            const int4 rsh = *reinterpret_cast<const int4 *>(rowshift + u * kBatchRows + 4 * kq);
-
-            float4_t d[16];
-#pragma unroll
-            for (int c = 0; c < 16; c++) d[c] = (float4_t){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int s = 0; s < 4; s++) {
-                const half8_t av = __builtin_bit_cast(half8_t, a[s]);
-#pragma unroll
-                for (int dw = 0; dw < 4; dw++) {
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        u32x4 b;
-                        if (BITS == 4) {
-                            const uint32_t sel = 0x0c000c00u | (uint32_t)(j << 16) | (uint32_t)(4 + j);
-                            const uint32_t p0 = __builtin_amdgcn_perm(w[4 * s][dw], w[4 * s + 1][dw], sel);
-                            const uint32_t p1 = __builtin_amdgcn_perm(w[4 * s + 2][dw], w[4 * s + 3][dw], sel);
-                            b = (u32x4){p0 & 0x000f000fu, p0 & 0x00f000f0u, p1 & 0x000f000fu, p1 & 0x00f000f0u};
-                        } else {
-                            const uint32_t sel = 0x0c000000u | (uint32_t)(j << 16) | (uint32_t)(j << 8) | (uint32_t)(4 + j);
-                            const uint32_t p1 = __builtin_amdgcn_perm(w[3 * s][dw], w[3 * s + 1][dw], sel);
-                            const uint32_t p2 = __builtin_amdgcn_perm(w[3 * s + 1][dw], w[3 * s + 2][dw], sel);
-                            b = (u32x4){p1 & 0x000e0007u, p1 & 0x00700038u, p2 & 0x001c0380u,
-                                        (p1 & 0x000001c0u) | (p2 & 0x00e00000u)};
-                        }
-                        d[4 * dw + j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, __builtin_bit_cast(half8_t, b),
-                                                                              d[4 * dw + j], 0, 0, 0);
-                    }
-                }
-            }
-            // tile -> totals: undo the normalisation, apply the grid offset and the group scale
-            const float f[4] = {ldexpf(1.f, 24 - rsh.x), ldexpf(1.f, 24 - rsh.y), ldexpf(1.f, 24 - rsh.z),
-                                ldexpf(1.f, 24 - rsh.w)};
-            const float o[4] = {-kGrid * rsum.x, -kGrid * rsum.y, -kGrid * rsum.z, -kGrid * rsum.w};
-#pragma unroll
-            for (int c = 0; c < 16; c++) {
-                const uint32_t sw = c < 8 ? sc0[c >> 1] : sc1[(c - 8) >> 1];
-                const float sc = __half2float(__ushort_as_half((unsigned short)((c & 1) ? (sw >> 16) : (sw & 0xffffu))));
-#pragma unroll
-                for (int r = 0; r < 4; r++) tot[c][r] += sc * (d[c][r] * f[r] + o[r]);
-            }
-        } else {
-            // cherry unit: 32 dense fp16 rows, 8 per lane group
-            const int c0 = (u - plan.units_normal) * kCherryUnit + 8 * kq;
-            const uint32_t coff = col_ok ? (uint32_t)(c0 * N + n0) * 2u : kOobB;
-            u32x4 cw[8][2];
-#pragma unroll
-            for (int r = 0; r < 8; r++) {
-                cw[r][0] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff + (uint32_t)(r * N * 2), 0, 2);
-                cw[r][1] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff + (uint32_t)(r * N * 2) + 16, 0, 2);
-            }
-            const half8_t av = __builtin_bit_cast(half8_t, xau[0]);
-#pragma unroll
-            for (int c = 0; c < 16; c++) {
-                const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;  // (row r half, row r+1 half)
-                u32x4 b;
-#pragma unroll
-                for (int rp = 0; rp < 4; rp++)
-                    b[rp] = __builtin_amdgcn_perm(cw[2 * rp + 1][c >> 3][(c & 7) >> 1], cw[2 * rp][c >> 3][(c & 7) >> 1], sel);
-                tot[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, __builtin_bit_cast(half8_t, b), tot[c], 0, 0, 0);
-            }
+        const int ua = u0 + it * kBatchWaves;
+        if (ua < plan.units_normal) {
+            UnitRegs ra;
+            issue_unit<BITS>(ra, cx, ua);
+            compute_unit<BITS>(ra, tot);
         }
     }
+    for (int it = 0; it < units_per_wave; it++) {
+        const int u = u0 + it * kBatchWaves;
+        if (u >= plan.units_normal && u < plan.units_total) cherry_unit(cx, u, tot);
+    }
 
-    // ---- across the workgroup's wavefronts through LDS (float4 stores: 4 adjacent columns)
+    CQB_STAMP(1);
+    // ---- across the workgroup's wavefronts through LDS.  Column 16 nl + c is stored at
+    // 16 nl + ((c + nl) & 15): for a fixed c the 16 lanes of a row then hit 16 different banks.
 #pragma unroll
-    for (int c4 = 0; c4 < 16; c4 += 4)
+    for (int c = 0; c < 16; c++)
 #pragma unroll
-        for (int r = 0; r < 4; r++)
-            *reinterpret_cast<float4 *>(&s_red[wave][4 * kq + r][16 * nl + c4]) =
-                make_float4(tot[c4][r], tot[c4 + 1][r], tot[c4 + 2][r], tot[c4 + 3][r]);
+        for (int r = 0; r < 4; r++) s_red[wave][4 * kq + r][16 * nl + ((c + nl) & 15)] = tot[c][r];
     __syncthreads();
     float vals[kBatchRows];
+    {
+        const int sw = (tid & ~15) | (((tid & 15) + (tid >> 4)) & 15);  // where column `tid` was stored
 #pragma unroll
-    for (int b = 0; b < kBatchRows; b++)
-        vals[b] = (s_red[0][b][tid] + s_red[1][b][tid]) + (s_red[2][b][tid] + s_red[3][b][tid]);
+        for (int b = 0; b < kBatchRows; b++)
+            vals[b] = (s_red[0][b][sw] + s_red[1][b][sw]) + (s_red[2][b][sw] + s_red[3][b][sw]);
+    }
     const int n = tile * kTileCols + tid;
     const bool active = n < N;
 
-    // ---- across workgroups: partial tiles + ticket (see splitk_finish in cq_common.cuh for why no fences)
+    // ---- across workgroups: per-split partial tiles + one ticket per column tile.  (One atomic
+    // per output element, as in the batch-1 kernel, is slower here: 16 rows make 16x the atomics.)
+    // Partials travel as agent-scope sc1 stores / loads, no cache-wide fences; see cq_common.cuh.
+    CQB_STAMP(2);
     if (plan.splits > 1) {
         if (active)
 #pragma unroll
@@ -275,23 +375,31 @@ __global__ __launch_bounds__(64 * kBatchWaves) void batch_kernel(
             *s_last = (old == (unsigned)(plan.splits - 1));
         }
         __syncthreads();
+        CQB_STAMP(3);
         if (!*s_last) return;
         if (tid == 0) __hip_atomic_store(&tickets[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (active) {
 #pragma unroll
             for (int b = 0; b < kBatchRows; b++) vals[b] = 0.f;
-            for (int s = 0; s < plan.splits; s++) {
-                float p[kBatchRows];
+            // up to 3 splits (48 loads) in flight at a time, added in split order
+            for (int s0 = 0; s0 < plan.splits; s0 += 3) {
+                float p[3][kBatchRows];
 #pragma unroll
-                for (int b = 0; b < kBatchRows; b++)
-                    p[b] = (b < B) ? __hip_atomic_load(partial + ((size_t)s * kBatchRows + b) * N + n, __ATOMIC_RELAXED,
-                                                       __HIP_MEMORY_SCOPE_AGENT)
-                                   : 0.f;
+                for (int ds = 0; ds < 3; ds++)
 #pragma unroll
-                for (int b = 0; b < kBatchRows; b++) vals[b] += p[b];
+                    for (int b = 0; b < kBatchRows; b++)
+                        p[ds][b] = (b < B && s0 + ds < plan.splits)
+                                       ? __hip_atomic_load(partial + ((size_t)(s0 + ds) * kBatchRows + b) * N + n,
+                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                       : 0.f;
+#pragma unroll
+                for (int ds = 0; ds < 3; ds++)
+#pragma unroll
+                    for (int b = 0; b < kBatchRows; b++) vals[b] += p[ds][b];
             }
         }
     }
+    CQB_STAMP(4);
     if (active) {
 #pragma unroll
         for (int b = 0; b < kBatchRows; b++)
@@ -329,11 +437,12 @@ static hipError_t launch_batch_bits(const __half *vec, const uint8_t *qweight, c
     float *partial = reinterpret_cast<float *>(base + ws.partial);
     unsigned *tickets = reinterpret_cast<unsigned *>(reinterpret_cast<char *>(workspace) + ws.tickets);
     const Plan unit_plan = make_plan(K, N, C, 1, kUnitK);
-    // units per wave: the fewest that keep the split count within the partial workspace, more
-    // when the grid would still hold >= 512 workgroups (less split-K traffic)
+    // units per wave: one if the split count then fits the partial workspace (every wave's loads
+    // go out at once and the kernel is one memory latency deep); more only for very long K, or
+    // when the grid would otherwise exceed ~4 workgroups per CU (less split-K traffic)
     int upv = 1;
     while (ceil_div(unit_plan.units_total, kBatchWaves * upv) > kBatchMaxSplits) upv++;
-    while (upv < 8 && unit_plan.tiles * ceil_div(unit_plan.units_total, kBatchWaves * (upv + 1)) >= 512) upv++;
+    while (upv < 8 && unit_plan.tiles * ceil_div(unit_plan.units_total, kBatchWaves * (upv + 1)) >= 1024) upv++;
     const Plan plan = make_plan(K, N, C, kBatchWaves * upv, kUnitK);
     for (int b0 = 0; b0 < B; b0 += kBatchRows) {
         const int nb = min(kBatchRows, B - b0);
