@@ -144,6 +144,36 @@ def cpu_baseline(bits, k, n, group, base, x_np):
                       f"cached dense fp16 linear alone: {float(np.median(cached)) * 1e6:.1f} us"}
 
 
+def decode_benchmark(prompt_len=128, new_tokens=128, w_bits=4, seed=0):
+    """BASELINE config 2: random-init LLaMA-7B-shape decoder (32 layers, hidden 4096, 32 heads,
+    MLP 11008, vocab 32000, all seven linears per layer 4-bit CherryLinear, group 128, 1/256
+    cherries), greedy decoding at batch 1: 128 random prompt ids, then 128 generated tokens.
+    The token step is one captured HIP graph; decode tokens/s excludes the prompt."""
+    import numpy as np
+    import torch
+    import cherryq_decoder as cd
+    cfg = cd.DecoderConfig(w_bits=w_bits, max_position_embeddings=prompt_len + new_tokens)
+    model = cd.CherryLlamaDecoder(cfg, seed=seed)
+    prompt = torch.randint(0, cfg.vocab_size, (prompt_len,), generator=torch.Generator().manual_seed(seed))
+    model.capture(fork=True)
+    model.generate(prompt, 8)                                   # warm-up
+    out, _, total = model.generate(prompt, new_tokens)          # throughput: one sync at the end
+    _, times, _ = model.generate(prompt, new_tokens, sync_each_token=True)  # latency per token
+    bytes_per_token = model.step_bytes()
+    tok_s = new_tokens / total
+    res = {"model": "llama7b-shape random init", "w_bits": w_bits, "prompt_tokens": prompt_len,
+           "generated_tokens": new_tokens, "tokens_per_s": round(tok_s, 1),
+           "ms_per_token_median_synced": round(float(np.median(times)) * 1e3, 4),
+           "packed_bytes_per_token": bytes_per_token,
+           "hbm_gbs": round(bytes_per_token * tok_s / 1e9, 1),
+           "frac_of_hbm_peak": round(bytes_per_token * tok_s / 1e9 / HBM_PEAK_GBS, 4),
+           "launch": "one HIP graph per token, q/k/v and gate/up on forked streams",
+           "first_tokens": out[:8].tolist()}
+    del model
+    torch.cuda.empty_cache()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -153,6 +183,7 @@ def main():
     ap.add_argument("--group", type=int, default=128)
     ap.add_argument("--all", action="store_true", help="also print a table of every workload to stderr")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-decode", action="store_true", help="skip the 7B-shape decode measurement")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a graph replay")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -194,6 +225,8 @@ def main():
                                                 use_graph=not args.no_graph)
     ab = algorithmic_bytes(bits, k, n, 1, args.group)
     gbs = ab / us / 1e3
+    x_host = x.cpu().numpy()
+    n_copies = len(copies)
     result = {
         "metric": "us_per_matvec", "value": round(us, 3), "unit": "us", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us / 1e3, 6),
@@ -201,15 +234,19 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "w_bits": bits, "in_features": k, "out_features": n,
                    "group_size": args.group, "batch": 1, "cherries": -(-k // 256) // 8 * 8,
-                   "weight_copies_rotated": len(copies),
+                   "weight_copies_rotated": n_copies,
                    "launch": "eager" if args.no_graph else "hip_graph_replay",
                    "eager_host_wall_us_per_call": round(wall_us, 2)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
                      "algorithmic_bytes_per_launch": ab, "kernel": f"cq::matvec_kernel<{bits}>"},
     }
+    if not args.no_decode:
+        del copies, x, out
+        torch.cuda.empty_cache()
+        result["decode"] = decode_benchmark()
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(bits, k, n, args.group, base, x.cpu().numpy())
+        result["cpu_baseline"] = cpu_baseline(bits, k, n, args.group, base, x_host)
     print(json.dumps(result), flush=True)
 
 

@@ -127,6 +127,25 @@ int cherryq_unpack_f16(int w_bits, const uint8_t *qweight, const void *cherry_we
                        int in_features, int out_features, int num_cherries, int group_size,
                        void *stream);
 
+/*
+ * Decode-step glue for a LLaMA-shaped decoder, batch 1, fp16: what sits between two fused
+ * matvecs in the caller's token step (llama/modeling_llama_quant.py of the reference: RMSNorm
+ * :75-89, rotary embedding :179-210, attention over the KV cache :391-402 and :671-696, gated
+ * MLP :251), one launch each, so that the step can be captured as a short HIP graph.  They have
+ * no counterpart in the reference's extension, which leaves these operations to PyTorch.
+ * `position` is a device pointer to the current token position (so a captured graph can be
+ * replayed while the caller increments it); caches are [kv_head][max_len][head_dim].
+ */
+int cherryq_decode_add_rmsnorm_f16(void *hidden, const void *delta /* may be NULL */, const void *weight,
+                                   void *normed, int hidden_size, float eps, void *stream);
+int cherryq_decode_rope_cache_f16(void *q, const void *k, const void *v, void *k_cache, void *v_cache,
+                                  const int *position, int n_heads, int n_kv_heads, int head_dim, int max_len,
+                                  float theta, void *stream);
+int cherryq_decode_attention_f16(const void *q, const void *k_cache, const void *v_cache, void *out,
+                                 const int *position, int n_heads, int n_kv_heads, int head_dim, int max_len,
+                                 void *stream);
+int cherryq_decode_silu_mul_f16(const void *gate, const void *up, void *out, int n, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,317 @@
+"""A minimal LLaMA-shaped decoder whose seven per-layer projections are packed CherryQ linears,
+for batch-1 greedy decoding on one MI355X.
+
+It reproduces the mathematics of the reference's model (llama/modeling_llama_quant.py: embedding
+:949, RMSNorm :75-89, rotary embedding :95-210, attention with KV cache :630-710, gated MLP
+:221-251, decoder layer :754-775, final norm + unquantised fp16 lm_head :1064,1132,1222) without
+its HF-transformers scaffolding, and the per-token timing loop of benchmark_perplexity.py:92-113.
+
+Every projection is a `llama.qlinear.QuantLinear` (the reference's buffer schema); a token step
+calls the fused kernels through `quant_cuda`, and the operations between them (residual +
+RMSNorm, rotary + cache write, single-query attention, SiLU * up) through the decode entry points
+of libcherryq.  The whole step is captured once in a HIP graph and replayed per token; q/k/v and
+gate/up, which do not depend on each other, are captured on forked streams.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from dataclasses import dataclass
+
+import torch
+import torch.nn as nn
+
+import quant_cuda
+from llama.qlinear import QuantLinear
+from llama.quantizer import FullSymQuantizer
+
+_lib = quant_cuda._lib
+_vp, _int, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+_lib.cherryq_decode_add_rmsnorm_f16.argtypes = [_vp, _vp, _vp, _vp, _int, _f, _vp]
+_lib.cherryq_decode_rope_cache_f16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _f, _vp]
+_lib.cherryq_decode_attention_f16.argtypes = [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp]
+_lib.cherryq_decode_silu_mul_f16.argtypes = [_vp, _vp, _vp, _int, _vp]
+for _n in ("cherryq_decode_add_rmsnorm_f16", "cherryq_decode_rope_cache_f16", "cherryq_decode_attention_f16",
+           "cherryq_decode_silu_mul_f16"):
+    getattr(_lib, _n).restype = _int
+
+
+def _ok(rc, what):
+    if rc != 0:
+        quant_cuda._fail(rc, what)
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+@dataclass
+class DecoderConfig:
+    hidden_size: int = 4096
+    intermediate_size: int = 11008
+    num_hidden_layers: int = 32
+    num_attention_heads: int = 32
+    num_key_value_heads: int = 32
+    vocab_size: int = 32000
+    rms_norm_eps: float = 1e-6
+    rope_theta: float = 10000.0
+    max_position_embeddings: int = 256
+    w_bits: int = 4
+    group_size: int = 128
+    cherry_fraction: float = 1 / 256
+
+    @property
+    def head_dim(self):
+        return self.hidden_size // self.num_attention_heads
+
+
+def random_packed_linear(cfg: DecoderConfig, in_features, out_features, gen: torch.Generator, device) -> QuantLinear:
+    """A QuantLinear with random but well-formed packed buffers, generated on the device:
+    uniform codes, scales such that the dequantised weights have a standard deviation of about
+    0.02 (LLaMA's init), sorted random cherry columns with N(0, 0.02) fp16 weights."""
+    q = QuantLinear(cfg.w_bits, cfg.group_size, FullSymQuantizer, cfg.cherry_fraction, in_features, out_features,
+                    bias=False)
+    c = q.num_cherries
+    code_std = math.sqrt((4 ** cfg.w_bits - 1) / 12.0)
+    q.qweight = torch.randint(0, 256, q.qweight.shape, dtype=torch.uint8, device=device, generator=gen)
+    q.scales = ((torch.rand(q.scales.shape, device=device, generator=gen) * 0.5 + 0.75) * (0.02 / code_std)).half()
+    q.cherry_weight = (torch.randn(q.cherry_weight.shape, device=device, generator=gen) * 0.02).half()
+    q.cherry_indices = torch.randperm(in_features, device=device, generator=gen)[:c].sort().values.to(torch.int16)
+    return q
+
+
+class DecoderLayer(nn.Module):
+    def __init__(self, cfg: DecoderConfig, gen, device):
+        super().__init__()
+        h, kv = cfg.hidden_size, cfg.num_key_value_heads * cfg.head_dim
+        self.q_proj = random_packed_linear(cfg, h, h, gen, device)
+        self.k_proj = random_packed_linear(cfg, h, kv, gen, device)
+        self.v_proj = random_packed_linear(cfg, h, kv, gen, device)
+        self.o_proj = random_packed_linear(cfg, h, h, gen, device)
+        self.gate_proj = random_packed_linear(cfg, h, cfg.intermediate_size, gen, device)
+        self.up_proj = random_packed_linear(cfg, h, cfg.intermediate_size, gen, device)
+        self.down_proj = random_packed_linear(cfg, cfg.intermediate_size, h, gen, device)
+        self.input_layernorm = nn.Parameter(torch.ones(h, dtype=torch.float16, device=device), requires_grad=False)
+        self.post_attention_layernorm = nn.Parameter(torch.ones(h, dtype=torch.float16, device=device),
+                                                     requires_grad=False)
+
+
+class CherryLlamaDecoder(nn.Module):
+    """Random-init decoder; `generate()` does greedy decoding with a captured token step."""
+
+    def __init__(self, cfg: DecoderConfig, seed: int = 0, device="cuda"):
+        super().__init__()
+        self.cfg = cfg
+        self.device_ = torch.device(device)
+        gen = torch.Generator(device=self.device_).manual_seed(seed)
+        h = cfg.hidden_size
+        self.embed_tokens = (torch.randn(cfg.vocab_size, h, device=self.device_, generator=gen) * 0.02).half()
+        self.layers = nn.ModuleList([DecoderLayer(cfg, gen, self.device_) for _ in range(cfg.num_hidden_layers)])
+        self.norm = torch.ones(h, dtype=torch.float16, device=self.device_)
+        self.lm_head = (torch.randn(cfg.vocab_size, h, device=self.device_, generator=gen) * 0.02).half()
+        L, kvh, ml, hd = cfg.num_hidden_layers, cfg.num_key_value_heads, cfg.max_position_embeddings, cfg.head_dim
+        self.k_cache = torch.zeros(L, kvh, ml, hd, dtype=torch.float16, device=self.device_)
+        self.v_cache = torch.zeros_like(self.k_cache)
+        # static step buffers (a captured graph replays on fixed addresses)
+        f16 = dict(dtype=torch.float16, device=self.device_)
+        self.pos = torch.zeros(1, dtype=torch.int32, device=self.device_)
+        self.token = torch.zeros(1, dtype=torch.int64, device=self.device_)
+        self.next_token = torch.zeros(1, dtype=torch.int64, device=self.device_)
+        self.hid = torch.zeros(1, h, **f16)
+        self.normed = torch.zeros(1, h, **f16)
+        self.q = torch.zeros(1, h, **f16)
+        self.k = torch.zeros(1, kvh * hd, **f16)
+        self.v = torch.zeros(1, kvh * hd, **f16)
+        self.attn = torch.zeros(1, h, **f16)
+        self.proj = torch.zeros(1, h, **f16)
+        self.gate = torch.zeros(1, cfg.intermediate_size, **f16)
+        self.up = torch.zeros(1, cfg.intermediate_size, **f16)
+        self.act = torch.zeros(1, cfg.intermediate_size, **f16)
+        self.logits16 = torch.zeros(1, cfg.vocab_size, **f16)
+        self.logits = torch.zeros(1, cfg.vocab_size, dtype=torch.float32, device=self.device_)
+        self.lm_head_t = self.lm_head.t()
+        self._graph = None
+        self._side = [torch.cuda.Stream(device=self.device_) for _ in range(2)]
+
+    # ---- packed bytes a token step must read (for the roofline of tokens/s)
+    def step_bytes(self) -> int:
+        n = self.lm_head.numel() * 2
+        for layer in self.layers:
+            for m in layer.children():
+                n += sum(b.numel() * b.element_size() for b in (m.qweight, m.scales, m.cherry_weight, m.cherry_indices))
+        return n
+
+    def _linear(self, m: QuantLinear, x, out):
+        quant_cuda.matmul_cherryq(m.w_bits, x, m.qweight, m.cherry_weight, m.cherry_indices, m.scales, out,
+                                  m.group_size, accumulate=False)
+
+    def _fork(self, fns):
+        """Run independent launches on forked streams (inside a capture this becomes a fork/join)."""
+        main = torch.cuda.current_stream()
+        fns[0]()
+        for fn, st in zip(fns[1:], self._side):
+            st.wait_stream(main)
+            with torch.cuda.stream(st):
+                fn()
+        for st in self._side[:len(fns) - 1]:
+            main.wait_stream(st)
+
+    def _step(self, fork=True):
+        """One token: self.token at position self.pos -> self.logits, self.next_token; pos += 1."""
+        cfg = self.cfg
+        nh, nkv, hd, ml = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.max_position_embeddings
+        torch.index_select(self.embed_tokens, 0, self.token, out=self.hid)
+        delta = None
+        for li, layer in enumerate(self.layers):
+            _ok(_lib.cherryq_decode_add_rmsnorm_f16(self.hid.data_ptr(), delta, layer.input_layernorm.data_ptr(),
+                                                    self.normed.data_ptr(), cfg.hidden_size, cfg.rms_norm_eps,
+                                                    _stream()), "add_rmsnorm")
+            qkv = [lambda l=layer: self._linear(l.q_proj, self.normed, self.q),
+                   lambda l=layer: self._linear(l.k_proj, self.normed, self.k),
+                   lambda l=layer: self._linear(l.v_proj, self.normed, self.v)]
+            if fork:
+                self._fork(qkv)
+            else:
+                for fn in qkv:
+                    fn()
+            _ok(_lib.cherryq_decode_rope_cache_f16(self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(),
+                                                   self.k_cache[li].data_ptr(), self.v_cache[li].data_ptr(),
+                                                   self.pos.data_ptr(), nh, nkv, hd, ml, cfg.rope_theta, _stream()),
+                "rope_cache")
+            _ok(_lib.cherryq_decode_attention_f16(self.q.data_ptr(), self.k_cache[li].data_ptr(),
+                                                  self.v_cache[li].data_ptr(), self.attn.data_ptr(),
+                                                  self.pos.data_ptr(), nh, nkv, hd, ml, _stream()), "attention")
+            self._linear(layer.o_proj, self.attn, self.proj)
+            _ok(_lib.cherryq_decode_add_rmsnorm_f16(self.hid.data_ptr(), self.proj.data_ptr(),
+                                                    layer.post_attention_layernorm.data_ptr(), self.normed.data_ptr(),
+                                                    cfg.hidden_size, cfg.rms_norm_eps, _stream()), "add_rmsnorm")
+            gu = [lambda l=layer: self._linear(l.gate_proj, self.normed, self.gate),
+                  lambda l=layer: self._linear(l.up_proj, self.normed, self.up)]
+            if fork:
+                self._fork(gu)
+            else:
+                for fn in gu:
+                    fn()
+            _ok(_lib.cherryq_decode_silu_mul_f16(self.gate.data_ptr(), self.up.data_ptr(), self.act.data_ptr(),
+                                                 cfg.intermediate_size, _stream()), "silu_mul")
+            self._linear(layer.down_proj, self.act, self.proj)
+            delta = self.proj.data_ptr()
+        _ok(_lib.cherryq_decode_add_rmsnorm_f16(self.hid.data_ptr(), delta, self.norm.data_ptr(),
+                                                self.normed.data_ptr(), cfg.hidden_size, cfg.rms_norm_eps, _stream()),
+            "final norm")
+        torch.matmul(self.normed, self.lm_head_t, out=self.logits16)  # unquantised fp16 head
+        self.logits.copy_(self.logits16)
+        torch.argmax(self.logits, dim=-1, out=self.next_token)
+        self.pos.add_(1)
+
+    def reset(self):
+        self.pos.zero_()
+        self.k_cache.zero_()
+        self.v_cache.zero_()
+
+    def capture(self, fork=True):
+        """Warm up (allocates the per-stream workspaces) and capture one token step."""
+        self.reset()
+        s = torch.cuda.Stream(device=self.device_)
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            for _ in range(2):
+                self._step(fork)
+            s.synchronize()
+            self._graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self._graph, stream=s):
+                self._step(fork)
+        torch.cuda.current_stream().wait_stream(s)
+        self.reset()
+
+    @torch.inference_mode()
+    def generate(self, prompt_ids: torch.Tensor, max_new_tokens: int, use_graph=True, sync_each_token=False):
+        """Greedy decoding.  The prompt is fed token by token through the same step (prefill is
+        not timed separately here).  Returns (generated ids, per-token seconds of the decode part
+        when sync_each_token, total decode seconds)."""
+        import time
+        assert prompt_ids.dim() == 1 and prompt_ids.numel() + max_new_tokens <= self.cfg.max_position_embeddings
+        if use_graph and self._graph is None:
+            self.capture()
+        self.reset()
+        run = self._graph.replay if use_graph else self._step
+        prompt_ids = prompt_ids.to(self.device_)
+        for i in range(prompt_ids.numel()):
+            self.token.copy_(prompt_ids[i:i + 1])
+            run()
+        out = torch.zeros(max_new_tokens, dtype=torch.int64, device=self.device_)
+        torch.cuda.synchronize()
+        times = []
+        t0 = time.perf_counter()
+        for i in range(max_new_tokens):
+            tick = time.perf_counter()
+            self.token.copy_(self.next_token)
+            out[i:i + 1].copy_(self.next_token)
+            run()
+            if sync_each_token:
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - tick)
+        torch.cuda.synchronize()
+        return out, times, time.perf_counter() - t0
+
+    @torch.inference_mode()
+    def step_logits(self, ids: torch.Tensor, use_graph=False, fork=False) -> torch.Tensor:
+        """Logits after each token of `ids`, produced by the token step (teacher forcing)."""
+        if use_graph and self._graph is None:
+            self.capture(fork)
+        self.reset()
+        ids = ids.to(self.device_)
+        rows = []
+        for i in range(ids.numel()):
+            self.token.copy_(ids[i:i + 1])
+            if use_graph:
+                self._graph.replay()
+            else:
+                self._step(fork)
+            rows.append(self.logits.clone())
+        torch.cuda.synchronize()
+        return torch.cat(rows, dim=0)
+
+    # ---- reference: same model with dense fp16 weights and plain torch ops -------------------
+    @torch.inference_mode()
+    def reference_logits(self, ids: torch.Tensor) -> torch.Tensor:
+        """Logits for every position of `ids` (teacher forcing) from dequantised weights and torch
+        operations only (fp32 softmax/norm as in the reference's eager path)."""
+        cfg = self.cfg
+        ids = ids.to(self.device_)
+        T, nh, nkv, hd = ids.numel(), cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+
+        def norm(x, w):
+            xf = x.float()
+            return w * (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + cfg.rms_norm_eps)).half()
+
+        pos = torch.arange(T, device=self.device_, dtype=torch.float32)
+        inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, hd, 2, device=self.device_, dtype=torch.float32) / hd))
+        fr = torch.outer(pos, inv)
+        emb = torch.cat([fr, fr], dim=-1)
+        cos, sin = emb.cos().half()[None], emb.sin().half()[None]  # (1, T, hd)
+
+        def rot(x):
+            x1, x2 = x[..., :hd // 2], x[..., hd // 2:]
+            return torch.cat([-x2, x1], dim=-1)
+
+        h = self.embed_tokens[ids]
+        mask = torch.full((T, T), float("-inf"), device=self.device_).triu(1)
+        for layer in self.layers:
+            dense = {n: m.unpack() for n, m in layer.named_children()}
+            x = norm(h, layer.input_layernorm)
+            q = (x @ dense["q_proj"].t()).view(T, nh, hd).transpose(0, 1)
+            k = (x @ dense["k_proj"].t()).view(T, nkv, hd).transpose(0, 1)
+            v = (x @ dense["v_proj"].t()).view(T, nkv, hd).transpose(0, 1)
+            q = q * cos + rot(q) * sin
+            k = k * cos + rot(k) * sin
+            rep = nh // nkv
+            k, v = k.repeat_interleave(rep, 0), v.repeat_interleave(rep, 0)
+            att = (q @ k.transpose(1, 2)) / math.sqrt(hd)
+            att = torch.softmax(att.float() + mask, dim=-1).half()
+            a = (att @ v).transpose(0, 1).reshape(T, nh * hd)
+            h = h + a @ dense["o_proj"].t()
+            x = norm(h, layer.post_attention_layernorm)
+            m = torch.nn.functional.silu(x @ dense["gate_proj"].t()) * (x @ dense["up_proj"].t())
+            h = h + m @ dense["down_proj"].t()
+        return (norm(h, self.norm) @ self.lm_head.t()).float()

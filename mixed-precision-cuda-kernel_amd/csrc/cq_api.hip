@@ -197,4 +197,48 @@ int cherryq_unpack_f16(int w_bits, const uint8_t *qweight, const void *cherry_we
                                   reinterpret_cast<hipStream_t>(stream));
 }
 
+// ---- decode-step glue (see include/cherryq.h) ----------------------------------------------
+
+int cherryq_decode_add_rmsnorm_f16(void *hidden, const void *delta, const void *weight, void *normed,
+                                   int hidden_size, float eps, void *stream) {
+    if (!hidden || !weight || !normed) return CHERRYQ_E_NULL;
+    if (hidden_size <= 0) return CHERRYQ_E_SHAPE;
+    return (int)cq::launch_add_rmsnorm(reinterpret_cast<__half *>(hidden), reinterpret_cast<const __half *>(delta),
+                                       reinterpret_cast<const __half *>(weight), reinterpret_cast<__half *>(normed),
+                                       hidden_size, eps, reinterpret_cast<hipStream_t>(stream));
+}
+
+int cherryq_decode_rope_cache_f16(void *q, const void *k, const void *v, void *k_cache, void *v_cache,
+                                  const int *position, int n_heads, int n_kv_heads, int head_dim, int max_len,
+                                  float theta, void *stream) {
+    if (!q || !k || !v || !k_cache || !v_cache || !position) return CHERRYQ_E_NULL;
+    if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads || head_dim <= 0 || head_dim % 2 ||
+        head_dim > 2048 || max_len <= 0)
+        return CHERRYQ_E_SHAPE;
+    return (int)cq::launch_rope_cache(reinterpret_cast<__half *>(q), reinterpret_cast<const __half *>(k),
+                                      reinterpret_cast<const __half *>(v), reinterpret_cast<__half *>(k_cache),
+                                      reinterpret_cast<__half *>(v_cache), position, n_heads, n_kv_heads, head_dim,
+                                      max_len, theta, reinterpret_cast<hipStream_t>(stream));
+}
+
+int cherryq_decode_attention_f16(const void *q, const void *k_cache, const void *v_cache, void *out,
+                                 const int *position, int n_heads, int n_kv_heads, int head_dim, int max_len,
+                                 void *stream) {
+    if (!q || !k_cache || !v_cache || !out || !position) return CHERRYQ_E_NULL;
+    if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads || max_len <= 0 || max_len > cq::attn_max_len())
+        return CHERRYQ_E_SHAPE;
+    if (head_dim != 128) return CHERRYQ_E_UNSUPPORTED;
+    return (int)cq::launch_attn_decode(reinterpret_cast<const __half *>(q), reinterpret_cast<const __half *>(k_cache),
+                                       reinterpret_cast<const __half *>(v_cache), reinterpret_cast<__half *>(out),
+                                       position, n_heads, n_kv_heads, max_len, 1.0f / sqrtf((float)head_dim),
+                                       reinterpret_cast<hipStream_t>(stream));
+}
+
+int cherryq_decode_silu_mul_f16(const void *gate, const void *up, void *out, int n, void *stream) {
+    if (!gate || !up || !out) return CHERRYQ_E_NULL;
+    if (n <= 0) return CHERRYQ_E_SHAPE;
+    return (int)cq::launch_silu_mul(reinterpret_cast<const __half *>(gate), reinterpret_cast<const __half *>(up),
+                                    reinterpret_cast<__half *>(out), n, reinterpret_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

@@ -1,0 +1,187 @@
+// Batch-1 decode-step glue for a LLaMA-shaped decoder around the CherryQ linears: the operations
+// between two fused matvecs, each as ONE launch so that a token step is a short chain of kernels
+// (captured in a HIP graph by the caller) instead of dozens of element-wise launches.
+//
+// Semantics follow the reference's model code (llama/modeling_llama_quant.py): RMSNorm :75-89,
+// rotary embedding :95-147 and apply_rotary_pos_emb :179-210, attention with KV cache :391-402 /
+// :671-696, SiLU-gated MLP :251.  fp16 storage, fp32 arithmetic inside a kernel, roundings at the
+// points where the reference's fp16 tensors are materialised.
+#include "cq_common.cuh"
+#include "cq_kernels.h"
+
+namespace cq {
+
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+__device__ inline float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+
+// h <- h + delta (skipped when delta is null);  y <- weight * fp16(h * rsqrt(mean(h^2) + eps))
+__global__ __launch_bounds__(1024) void add_rmsnorm_kernel(__half *__restrict__ h, const __half *__restrict__ delta,
+                                                           const __half *__restrict__ weight, __half *__restrict__ y,
+                                                           int H, float eps) {
+    __shared__ float s_part[16];
+    const int t = threadIdx.x;
+    float ss = 0.f;
+    for (int i = t; i < H; i += 1024) {
+        float v = __half2float(h[i]);
+        if (delta) {
+            v = __half2float(__float2half_rn(v + __half2float(delta[i])));
+            h[i] = __float2half_rn(v);
+        }
+        ss += v * v;
+    }
+    ss = wave_sum(ss);
+    if ((t & 63) == 0) s_part[t >> 6] = ss;
+    __syncthreads();
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < 16; w++) tot += s_part[w];
+    const float rs = rsqrtf(tot / (float)H + eps);
+    for (int i = t; i < H; i += 1024) {
+        const float n = __half2float(__float2half_rn(__half2float(h[i]) * rs));
+        y[i] = __float2half_rn(__half2float(weight[i]) * n);
+    }
+}
+
+// Rotary embedding of q (in place) and k, and the KV-cache write at position *pos.
+// One workgroup per head (q heads first, then kv heads), head_dim / 2 threads.
+// Cache layout: [kv_head][max_len][head_dim].
+__global__ void rope_cache_kernel(__half *__restrict__ q, const __half *__restrict__ k, const __half *__restrict__ v,
+                                  __half *__restrict__ k_cache, __half *__restrict__ v_cache,
+                                  const int *__restrict__ pos_ptr, int n_heads, int n_kv_heads, int head_dim,
+                                  int max_len, float theta) {
+    const int pos = *pos_ptr;
+    const int head = blockIdx.x, i = threadIdx.x, half_dim = head_dim / 2;
+    if (i >= half_dim || pos >= max_len) return;
+    const float inv_freq = powf(theta, -2.0f * (float)i / (float)head_dim);
+    float sn, cs;
+    sincosf((float)pos * inv_freq, &sn, &cs);
+    const float c = __half2float(__float2half_rn(cs)), s = __half2float(__float2half_rn(sn));
+    auto rot = [&](float x1, float x2, __half &o1, __half &o2) {
+        // x * cos + rotate_half(x) * sin with every product and the sum rounded to fp16
+        const float a1 = __half2float(__float2half_rn(x1 * c)), b1 = __half2float(__float2half_rn(-x2 * s));
+        const float a2 = __half2float(__float2half_rn(x2 * c)), b2 = __half2float(__float2half_rn(x1 * s));
+        o1 = __float2half_rn(a1 + b1);
+        o2 = __float2half_rn(a2 + b2);
+    };
+    if (head < n_heads) {
+        __half *qh = q + (size_t)head * head_dim;
+        __half o1, o2;
+        rot(__half2float(qh[i]), __half2float(qh[i + half_dim]), o1, o2);
+        qh[i] = o1;
+        qh[i + half_dim] = o2;
+    } else {
+        const int kh = head - n_heads;
+        const __half *ksrc = k + (size_t)kh * head_dim;
+        const __half *vsrc = v + (size_t)kh * head_dim;
+        __half *kd = k_cache + ((size_t)kh * max_len + pos) * head_dim;
+        __half *vd = v_cache + ((size_t)kh * max_len + pos) * head_dim;
+        __half o1, o2;
+        rot(__half2float(ksrc[i]), __half2float(ksrc[i + half_dim]), o1, o2);
+        kd[i] = o1;
+        kd[i + half_dim] = o2;
+        vd[i] = vsrc[i];
+        vd[i + half_dim] = vsrc[i + half_dim];
+    }
+}
+
+// Single-query attention over the cache positions 0 .. *pos, one workgroup (256 threads) per head.
+// softmax in fp32, probabilities rounded to fp16 before the value product (as the eager path of
+// the reference does), fp32 accumulation.  head_dim must be 128, max_len <= kMaxAttnLen.
+constexpr int kMaxAttnLen = 4096;
+__global__ __launch_bounds__(256) void attn_decode_kernel(const __half *__restrict__ q,
+                                                          const __half *__restrict__ k_cache,
+                                                          const __half *__restrict__ v_cache,
+                                                          __half *__restrict__ out, const int *__restrict__ pos_ptr,
+                                                          int n_heads, int n_kv_heads, int max_len, float scale) {
+    __shared__ float s_score[kMaxAttnLen];
+    __shared__ float s_red[8];
+    __shared__ float s_acc[2][128];
+    const int head = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int kvh = head / (n_heads / n_kv_heads);
+    const int len = min(*pos_ptr + 1, max_len);
+    const __half *kb = k_cache + (size_t)kvh * max_len * 128;
+    const __half *vb = v_cache + (size_t)kvh * max_len * 128;
+    const __half2 q2 = reinterpret_cast<const __half2 *>(q + (size_t)head * 128)[lane];
+    const float qx = __low2float(q2), qy = __high2float(q2);
+    for (int j = wave; j < len; j += 4) {
+        const __half2 k2 = reinterpret_cast<const __half2 *>(kb + (size_t)j * 128)[lane];
+        const float d = wave_sum(qx * __low2float(k2) + qy * __high2float(k2));
+        if (lane == 0) s_score[j] = __half2float(__float2half_rn(d)) * scale;  // fp16 q k^T, then / sqrt(d)
+    }
+    __syncthreads();
+    float m = -INFINITY;
+    for (int j = t; j < len; j += 256) m = fmaxf(m, s_score[j]);
+    m = wave_max(m);
+    if (lane == 0) s_red[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+    float sum = 0.f;
+    for (int j = t; j < len; j += 256) {
+        const float e = __expf(s_score[j] - m);
+        s_score[j] = e;
+        sum += e;
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) s_red[4 + wave] = sum;
+    __syncthreads();
+    const float inv = 1.f / (s_red[4] + s_red[5] + s_red[6] + s_red[7]);
+    const int d = t & 127, part = t >> 7;
+    float acc = 0.f;
+    for (int j = part; j < len; j += 2) {
+        const float p = __half2float(__float2half_rn(s_score[j] * inv));
+        acc += p * __half2float(vb[(size_t)j * 128 + d]);
+    }
+    s_acc[part][d] = acc;
+    __syncthreads();
+    if (t < 128) out[(size_t)head * 128 + t] = __float2half_rn(s_acc[0][t] + s_acc[1][t]);
+}
+
+// out <- fp16(silu(gate)) * up
+__global__ __launch_bounds__(256) void silu_mul_kernel(const __half *__restrict__ gate, const __half *__restrict__ up,
+                                                       __half *__restrict__ out, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float g = __half2float(gate[i]);
+    const float a = __half2float(__float2half_rn(g / (1.f + __expf(-g))));
+    out[i] = __float2half_rn(a * __half2float(up[i]));
+}
+
+hipError_t launch_add_rmsnorm(__half *h, const __half *delta, const __half *weight, __half *y, int H, float eps,
+                              hipStream_t stream) {
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(1024), 0, stream, h, delta, weight, y, H, eps);
+    return hipGetLastError();
+}
+
+hipError_t launch_rope_cache(__half *q, const __half *k, const __half *v, __half *k_cache, __half *v_cache,
+                             const int *pos, int n_heads, int n_kv_heads, int head_dim, int max_len, float theta,
+                             hipStream_t stream) {
+    hipLaunchKernelGGL(rope_cache_kernel, dim3(n_heads + n_kv_heads), dim3(head_dim / 2), 0, stream, q, k, v, k_cache,
+                       v_cache, pos, n_heads, n_kv_heads, head_dim, max_len, theta);
+    return hipGetLastError();
+}
+
+hipError_t launch_attn_decode(const __half *q, const __half *k_cache, const __half *v_cache, __half *out,
+                              const int *pos, int n_heads, int n_kv_heads, int max_len, float scale,
+                              hipStream_t stream) {
+    hipLaunchKernelGGL(attn_decode_kernel, dim3(n_heads), dim3(256), 0, stream, q, k_cache, v_cache, out, pos, n_heads,
+                       n_kv_heads, max_len, scale);
+    return hipGetLastError();
+}
+
+hipError_t launch_silu_mul(const __half *gate, const __half *up, __half *out, int n, hipStream_t stream) {
+    hipLaunchKernelGGL(silu_mul_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, stream, gate, up, out, n);
+    return hipGetLastError();
+}
+
+int attn_max_len() { return kMaxAttnLen; }
+
+}  // namespace cq

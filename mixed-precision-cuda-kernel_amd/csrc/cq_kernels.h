@@ -39,4 +39,16 @@ hipError_t launch_batch(int bits, const __half *vec, const uint8_t *qweight, con
                         int C, int G, int accumulate, void *workspace, void *scratch, hipStream_t stream);
 size_t scratch_bytes(int B, int K, int N, int C);
 
+// cq_decode.hip: batch-1 decode-step glue kernels.
+hipError_t launch_add_rmsnorm(__half *h, const __half *delta, const __half *weight, __half *y, int H, float eps,
+                              hipStream_t stream);
+hipError_t launch_rope_cache(__half *q, const __half *k, const __half *v, __half *k_cache, __half *v_cache,
+                             const int *pos, int n_heads, int n_kv_heads, int head_dim, int max_len, float theta,
+                             hipStream_t stream);
+hipError_t launch_attn_decode(const __half *q, const __half *k_cache, const __half *v_cache, __half *out,
+                              const int *pos, int n_heads, int n_kv_heads, int max_len, float scale,
+                              hipStream_t stream);
+hipError_t launch_silu_mul(const __half *gate, const __half *up, __half *out, int n, hipStream_t stream);
+int attn_max_len();
+
 }  // namespace cq

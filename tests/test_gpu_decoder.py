@@ -1,0 +1,138 @@
+"""Decode-step glue kernels and the 7B-shaped decoder built from them (MI355X only)."""
+import ctypes
+import math
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dec():
+    assert torch.cuda.is_available()
+    import cherryq_decoder
+    return cherryq_decoder
+
+
+def rel(a, b):
+    a, b = a.double(), b.double()
+    return float((a - b).norm() / b.norm())
+
+
+def stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def test_add_rmsnorm_kernel(dec):
+    print("[case] add_rmsnorm", flush=True)
+    lib = dec._lib
+    torch.manual_seed(0)
+    for H in (4096, 256, 5120):
+        h = torch.randn(1, H, device="cuda").half()
+        d = torch.randn(1, H, device="cuda").half()
+        w = (torch.rand(H, device="cuda") + 0.5).half()
+        y = torch.empty_like(h)
+        h2 = h.clone()
+        assert lib.cherryq_decode_add_rmsnorm_f16(h2.data_ptr(), d.data_ptr(), w.data_ptr(), y.data_ptr(), H, 1e-6,
+                                                  stream()) == 0
+        torch.cuda.synchronize()
+        hs = h + d
+        xf = hs.float()
+        want = w * (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6)).half()
+        assert torch.equal(h2, hs)
+        assert rel(y, want) < 1e-3
+        h3 = h.clone()
+        assert lib.cherryq_decode_add_rmsnorm_f16(h3.data_ptr(), None, w.data_ptr(), y.data_ptr(), H, 1e-6, stream()) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(h3, h)
+
+
+def test_rope_cache_and_attention_kernels(dec):
+    print("[case] rope/attention", flush=True)
+    lib = dec._lib
+    torch.manual_seed(1)
+    nh, nkv, hd, ml = 8, 4, 128, 64
+    kc = torch.zeros(nkv, ml, hd, device="cuda").half()
+    vc = torch.zeros_like(kc)
+    pos = torch.zeros(1, dtype=torch.int32, device="cuda")
+    inv = 1.0 / (10000.0 ** (torch.arange(0, hd, 2, device="cuda").float() / hd))
+
+    def rope(x, p):
+        fr = p * inv
+        emb = torch.cat([fr, fr])
+        c, s = emb.cos().half(), emb.sin().half()
+        x1, x2 = x[..., :hd // 2], x[..., hd // 2:]
+        return x * c + torch.cat([-x2, x1], -1) * s
+
+    ks, vs = [], []
+    for p in range(20):
+        q = torch.randn(nh, hd, device="cuda").half()
+        k = torch.randn(nkv, hd, device="cuda").half()
+        v = torch.randn(nkv, hd, device="cuda").half()
+        pos.fill_(p)
+        q2 = q.clone()
+        assert lib.cherryq_decode_rope_cache_f16(q2.data_ptr(), k.data_ptr(), v.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+                                                 pos.data_ptr(), nh, nkv, hd, ml, 10000.0, stream()) == 0
+        out = torch.empty(nh, hd, device="cuda").half()
+        assert lib.cherryq_decode_attention_f16(q2.data_ptr(), kc.data_ptr(), vc.data_ptr(), out.data_ptr(),
+                                                pos.data_ptr(), nh, nkv, hd, ml, stream()) == 0
+        torch.cuda.synchronize()
+        qr, kr = rope(q, float(p)), rope(k, float(p))
+        ks.append(kr)
+        vs.append(v)
+        assert rel(q2, qr) < 2e-3
+        assert rel(kc[:, p], kr) < 2e-3 and torch.equal(vc[:, p], v)
+        K = torch.stack(ks, 1).repeat_interleave(nh // nkv, 0).float()   # (nh, p+1, hd)
+        V = torch.stack(vs, 1).repeat_interleave(nh // nkv, 0).float()
+        att = torch.softmax(torch.einsum("hd,hjd->hj", qr.float(), K) / math.sqrt(hd), -1)
+        want = torch.einsum("hj,hjd->hd", att, V)
+        assert rel(out, want) < 5e-3, p
+
+
+def test_silu_mul_kernel(dec):
+    print("[case] silu_mul", flush=True)
+    lib = dec._lib
+    g = torch.randn(11008, device="cuda").half() * 3
+    u = torch.randn(11008, device="cuda").half()
+    o = torch.empty_like(g)
+    assert lib.cherryq_decode_silu_mul_f16(g.data_ptr(), u.data_ptr(), o.data_ptr(), 11008, stream()) == 0
+    torch.cuda.synchronize()
+    assert rel(o, torch.nn.functional.silu(g) * u) < 1e-3
+
+
+def test_decode_validation(dec):
+    lib = dec._lib
+    assert lib.cherryq_decode_add_rmsnorm_f16(None, None, None, None, 4096, 1e-6, None) == -1
+    assert lib.cherryq_decode_attention_f16(1 << 12, 1 << 12, 1 << 12, 1 << 12, 1 << 12, 32, 32, 64, 256, None) == -7
+    assert lib.cherryq_decode_attention_f16(1 << 12, 1 << 12, 1 << 12, 1 << 12, 1 << 12, 32, 5, 128, 256, None) == -2
+    assert lib.cherryq_decode_silu_mul_f16(1 << 12, 1 << 12, 1 << 12, 0, None) == -2
+
+
+@pytest.mark.parametrize("bits", [4, 3])
+def test_small_decoder_matches_dense_reference(dec, bits):
+    """Two-layer decoder with real packed linears: the fused token step agrees with the same model
+    on dequantised weights and plain torch ops, eagerly and as a replayed HIP graph."""
+    print("[case] small decoder", bits, flush=True)
+    cfg = dec.DecoderConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=2,
+                            num_key_value_heads=2, vocab_size=512, max_position_embeddings=32, w_bits=bits,
+                            group_size=128, cherry_fraction=1 / 16)
+    model = dec.CherryLlamaDecoder(cfg, seed=3)
+    ids = torch.randint(0, cfg.vocab_size, (12,), generator=torch.Generator().manual_seed(0))
+    want = model.reference_logits(ids)
+    eager = model.step_logits(ids, use_graph=False)
+    for t in range(ids.numel()):
+        assert rel(eager[t], want[t]) < 2e-2, t
+    # several replays with eager work between them, each checked against the eager result
+    for fork in (False, True):
+        model._graph = None
+        graph = model.step_logits(ids, use_graph=True, fork=fork)
+        torch.cuda.synchronize()
+        _ = model.reference_logits(ids[:4])  # unrelated eager work between replays
+        graph2 = model.step_logits(ids, use_graph=True, fork=fork)
+        assert torch.equal(graph, eager) and torch.equal(graph2, eager), fork
+    out, times, total = model.generate(ids[:4], 8, use_graph=True)
+    out2, _, _ = model.generate(ids[:4], 8, use_graph=False)
+    assert torch.equal(out, out2) and out.numel() == 8
