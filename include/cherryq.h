@@ -136,6 +136,31 @@ int cherryq_unpack_f16(int w_bits, const uint8_t *qweight, const void *cherry_we
  * `position` is a device pointer to the current token position (so a captured graph can be
  * replayed while the caller increments it); caches are [kv_head][max_len][head_dim].
  */
+/*
+ * One batch-1 launch over 1..4 packed layers that read the SAME activation vector and share
+ * in_features, num_cherries, group_size and w_bits: q/k/v_proj (llama/modeling_llama_quant.py
+ * :346-348 of the reference) or gate/up_proj (:251).  Arithmetic per layer is that of
+ * cherryq_vecquant{3,4}matmul_f16 at batch 1; the point is that the layers' weight streams
+ * overlap inside one grid instead of running as short launches one after another.
+ * When vec_gate is non-NULL the activations are fp16(fp16(silu(vec_gate)) * vec), the
+ * gated-MLP product that feeds down_proj (:251), formed while the kernel stages its activations.
+ * workspace: zero-kept like the matmul workspace, cherryq_group_workspace_bytes() bytes.
+ * Returns CHERRYQ_E_UNSUPPORTED for vec_gate with shapes the streaming kernel does not take.
+ */
+typedef struct cherryq_layer {
+    const uint8_t *qweight;
+    const void *cherry_weight;
+    const int16_t *cherry_indices;
+    const void *scales;
+    void *mul;
+    int out_features;
+} cherryq_layer;
+size_t cherryq_group_workspace_bytes(int n_layers, const int *out_features);
+int cherryq_decode_matvec_group_f16(int w_bits, const void *vec, const void *vec_gate /* may be NULL */,
+                                    const cherryq_layer *layers, int n_layers, int in_features,
+                                    int num_cherries, int group_size, int accumulate, void *workspace,
+                                    size_t workspace_bytes, void *stream);
+
 int cherryq_decode_add_rmsnorm_f16(void *hidden, const void *delta /* may be NULL */, const void *weight,
                                    void *normed, int hidden_size, float eps, void *stream);
 int cherryq_decode_rope_cache_f16(void *q, const void *k, const void *v, void *k_cache, void *v_cache,

@@ -9,8 +9,12 @@ its HF-transformers scaffolding, and the per-token timing loop of benchmark_perp
 Every projection is a `llama.qlinear.QuantLinear` (the reference's buffer schema); a token step
 calls the fused kernels through `quant_cuda`, and the operations between them (residual +
 RMSNorm, rotary + cache write, single-query attention, SiLU * up) through the decode entry points
-of libcherryq.  The whole step is captured once in a HIP graph and replayed per token; q/k/v and
-gate/up, which do not depend on each other, are captured on forked streams.
+of libcherryq.  The whole step is captured once in a HIP graph and replayed per token.  q/k/v and
+gate/up do not depend on each other: by default each set runs as ONE grouped launch
+(`matvec_group`), the residual additions are the accumulate mode of o_proj / down_proj, and
+SiLU * up is formed inside down_proj.  `grouped=False` keeps one launch per operation;
+`fork=True` captures the independent projections of that variant on forked streams, which on this
+ROCm stack costs more in cross-stream edges than the overlap gains.
 """
 from __future__ import annotations
 
@@ -34,6 +38,49 @@ _lib.cherryq_decode_silu_mul_f16.argtypes = [_vp, _vp, _vp, _int, _vp]
 for _n in ("cherryq_decode_add_rmsnorm_f16", "cherryq_decode_rope_cache_f16", "cherryq_decode_attention_f16",
            "cherryq_decode_silu_mul_f16"):
     getattr(_lib, _n).restype = _int
+
+
+class _Layer(ctypes.Structure):
+    """struct cherryq_layer of include/cherryq.h"""
+    _fields_ = [("qweight", _vp), ("cherry_weight", _vp), ("cherry_indices", _vp), ("scales", _vp), ("mul", _vp),
+                ("out_features", _int)]
+
+
+_lib.cherryq_group_workspace_bytes.argtypes = [_int, ctypes.POINTER(_int)]
+_lib.cherryq_group_workspace_bytes.restype = ctypes.c_size_t
+_lib.cherryq_decode_matvec_group_f16.argtypes = [_int, _vp, _vp, ctypes.POINTER(_Layer), _int, _int, _int, _int, _int,
+                                                 _vp, ctypes.c_size_t, _vp]
+_lib.cherryq_decode_matvec_group_f16.restype = _int
+
+
+def matvec_group(mods, vec, outs, vec_gate=None, accumulate=False):
+    """outs[i] (+)= act @ W_i^T for 1..4 QuantLinear modules that read the same (1, K) activation
+    row, in ONE launch; act = vec, or fp16(fp16(silu(vec_gate)) * vec) when vec_gate is given."""
+    m0 = mods[0]
+    k, c = vec.shape[1], m0.cherry_indices.shape[0]
+    for m, o in zip(mods, outs):
+        if (m.w_bits, m.group_size, m.cherry_indices.shape[0], m.in_features) != (m0.w_bits, m0.group_size, c, k):
+            raise RuntimeError("matvec_group: the layers must share w_bits, group_size, num_cherries and in_features")
+        for t, dt in ((m.qweight, torch.uint8), (m.scales, torch.float16), (m.cherry_weight, torch.float16),
+                      (m.cherry_indices, torch.int16), (o, torch.float16)):
+            if not t.is_cuda or t.dtype != dt or not t.is_contiguous() or t.device != vec.device:
+                raise RuntimeError("matvec_group: contiguous GPU tensors of the packed schema's dtypes expected")
+        if tuple(o.shape) != (1, m.out_features) or m.qweight.shape != ((k - c) // 8 * m.w_bits, m.out_features):
+            raise RuntimeError("matvec_group: buffer shapes do not match the layer")
+    if tuple(vec.shape) != (1, k) or vec.dtype != torch.float16 or not vec.is_cuda or not vec.is_contiguous():
+        raise RuntimeError("matvec_group: vec must be a contiguous (1, in_features) fp16 GPU tensor")
+    if vec_gate is not None and (vec_gate.shape != vec.shape or vec_gate.dtype != torch.float16
+                                 or not vec_gate.is_cuda or not vec_gate.is_contiguous()):
+        raise RuntimeError("matvec_group: vec_gate must match vec")
+    arr = (_Layer * len(mods))(*[_Layer(m.qweight.data_ptr(), quant_cuda._ptr(m.cherry_weight),
+                                        quant_cuda._ptr(m.cherry_indices), m.scales.data_ptr(), o.data_ptr(),
+                                        m.out_features) for m, o in zip(mods, outs)])
+    ns = (_int * len(mods))(*[m.out_features for m in mods])
+    stream = _stream()
+    ws = quant_cuda._workspace(vec.device, stream, _lib.cherryq_group_workspace_bytes(len(mods), ns))
+    _ok(_lib.cherryq_decode_matvec_group_f16(m0.w_bits, vec.data_ptr(), None if vec_gate is None else vec_gate.data_ptr(),
+                                             arr, len(mods), k, c, m0.group_size, 1 if accumulate else 0,
+                                             ws.data_ptr(), ws.numel(), stream), "matvec_group")
 
 
 def _ok(rc, what):
@@ -156,8 +203,47 @@ class CherryLlamaDecoder(nn.Module):
         for st in self._side[:len(fns) - 1]:
             main.wait_stream(st)
 
-    def _step(self, fork=True):
-        """One token: self.token at position self.pos -> self.logits, self.next_token; pos += 1."""
+    def _norm(self, weight, delta=None):
+        cfg = self.cfg
+        _ok(_lib.cherryq_decode_add_rmsnorm_f16(self.hid.data_ptr(), delta, weight.data_ptr(), self.normed.data_ptr(),
+                                                cfg.hidden_size, cfg.rms_norm_eps, _stream()), "add_rmsnorm")
+
+    def _step_grouped(self):
+        """The token step with 9 launches per layer: q/k/v in one grid, gate/up in one grid, the
+        residual additions folded into o_proj and down_proj (they accumulate into the hidden
+        state, rounded once from fp32), SiLU * up folded into down_proj's activation staging."""
+        cfg = self.cfg
+        nh, nkv, hd, ml = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.max_position_embeddings
+        torch.index_select(self.embed_tokens, 0, self.token, out=self.hid)
+        for li, layer in enumerate(self.layers):
+            self._norm(layer.input_layernorm)
+            matvec_group([layer.q_proj, layer.k_proj, layer.v_proj], self.normed, [self.q, self.k, self.v])
+            _ok(_lib.cherryq_decode_rope_cache_f16(self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(),
+                                                   self.k_cache[li].data_ptr(), self.v_cache[li].data_ptr(),
+                                                   self.pos.data_ptr(), nh, nkv, hd, ml, cfg.rope_theta, _stream()),
+                "rope_cache")
+            _ok(_lib.cherryq_decode_attention_f16(self.q.data_ptr(), self.k_cache[li].data_ptr(),
+                                                  self.v_cache[li].data_ptr(), self.attn.data_ptr(),
+                                                  self.pos.data_ptr(), nh, nkv, hd, ml, _stream()), "attention")
+            matvec_group([layer.o_proj], self.attn, [self.hid], accumulate=True)
+            self._norm(layer.post_attention_layernorm)
+            matvec_group([layer.gate_proj, layer.up_proj], self.normed, [self.gate, self.up])
+            matvec_group([layer.down_proj], self.up, [self.hid], vec_gate=self.gate, accumulate=True)
+        self._norm(self.norm)
+        self._head()
+
+    def _head(self):
+        torch.matmul(self.normed, self.lm_head_t, out=self.logits16)  # unquantised fp16 head
+        self.logits.copy_(self.logits16)
+        torch.argmax(self.logits, dim=-1, out=self.next_token)
+        self.pos.add_(1)
+
+    def _step(self, fork=False, grouped=True):
+        """One token: self.token at position self.pos -> self.logits, self.next_token; pos += 1.
+        grouped=False runs every projection and every element-wise operation as its own launch
+        (12 per layer), the literal sequence of the reference's decoder layer."""
+        if grouped and not fork:
+            return self._step_grouped()
         cfg = self.cfg
         nh, nkv, hd, ml = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.max_position_embeddings
         torch.index_select(self.embed_tokens, 0, self.token, out=self.hid)
@@ -199,28 +285,25 @@ class CherryLlamaDecoder(nn.Module):
         _ok(_lib.cherryq_decode_add_rmsnorm_f16(self.hid.data_ptr(), delta, self.norm.data_ptr(),
                                                 self.normed.data_ptr(), cfg.hidden_size, cfg.rms_norm_eps, _stream()),
             "final norm")
-        torch.matmul(self.normed, self.lm_head_t, out=self.logits16)  # unquantised fp16 head
-        self.logits.copy_(self.logits16)
-        torch.argmax(self.logits, dim=-1, out=self.next_token)
-        self.pos.add_(1)
+        self._head()
 
     def reset(self):
         self.pos.zero_()
         self.k_cache.zero_()
         self.v_cache.zero_()
 
-    def capture(self, fork=True):
+    def capture(self, fork=False, grouped=True):
         """Warm up (allocates the per-stream workspaces) and capture one token step."""
         self.reset()
         s = torch.cuda.Stream(device=self.device_)
         s.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(s):
             for _ in range(2):
-                self._step(fork)
+                self._step(fork, grouped)
             s.synchronize()
             self._graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(self._graph, stream=s):
-                self._step(fork)
+                self._step(fork, grouped)
         torch.cuda.current_stream().wait_stream(s)
         self.reset()
 
@@ -255,10 +338,10 @@ class CherryLlamaDecoder(nn.Module):
         return out, times, time.perf_counter() - t0
 
     @torch.inference_mode()
-    def step_logits(self, ids: torch.Tensor, use_graph=False, fork=False) -> torch.Tensor:
+    def step_logits(self, ids: torch.Tensor, use_graph=False, fork=False, grouped=True) -> torch.Tensor:
         """Logits after each token of `ids`, produced by the token step (teacher forcing)."""
         if use_graph and self._graph is None:
-            self.capture(fork)
+            self.capture(fork, grouped)
         self.reset()
         ids = ids.to(self.device_)
         rows = []
@@ -267,7 +350,7 @@ class CherryLlamaDecoder(nn.Module):
             if use_graph:
                 self._graph.replay()
             else:
-                self._step(fork)
+                self._step(fork, grouped)
             rows.append(self.logits.clone())
         torch.cuda.synchronize()
         return torch.cat(rows, dim=0)

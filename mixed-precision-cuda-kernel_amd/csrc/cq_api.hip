@@ -199,10 +199,64 @@ int cherryq_unpack_f16(int w_bits, const uint8_t *qweight, const void *cherry_we
 
 // ---- decode-step glue (see include/cherryq.h) ----------------------------------------------
 
+size_t cherryq_group_workspace_bytes(int n_layers, const int *out_features) {
+    size_t bytes = 0;
+    for (int i = 0; i < n_layers; i++) {
+        const int n = out_features && out_features[i] > 0 ? out_features[i] : 8;
+        bytes += (size_t)((n + 255) / 256) * 256 * sizeof(unsigned long long);
+    }
+    return bytes;
+}
+
+int cherryq_decode_matvec_group_f16(int w_bits, const void *vec, const void *vec_gate, const cherryq_layer *layers,
+                                    int n_layers, int in_features, int num_cherries, int group_size,
+                                    int accumulate, void *workspace, size_t workspace_bytes, void *stream) {
+    using namespace cq;
+    if (w_bits != 3 && w_bits != 4) return CHERRYQ_E_BITS;
+    if (!layers) return CHERRYQ_E_NULL;
+    if (n_layers < 1 || n_layers > kMaxGroup) return CHERRYQ_E_SHAPE;
+    const int K = in_features, C = num_cherries, G = group_size;
+    int outs[kMaxGroup];
+    for (int i = 0; i < n_layers; i++) outs[i] = layers[i].out_features;
+    if (workspace_bytes < cherryq_group_workspace_bytes(n_layers, outs)) return CHERRYQ_E_WORKSPACE;
+    if (vec_gate && !aligned(vec_gate, 4)) return CHERRYQ_E_ALIGN;
+    bool fast = !force_generic();
+    MatvecMember members[kMaxGroup];
+    for (int i = 0; i < n_layers; i++) {
+        const cherryq_layer &l = layers[i];
+        int rc = check_common(vec, l.qweight, l.cherry_weight, l.cherry_indices, l.scales, l.mul, 1, K,
+                              l.out_features, C, G, workspace, workspace_bytes, nullptr, 0);
+        if (rc) return rc;
+        fast = fast && matvec_supported(w_bits, 1, K, l.out_features, C, G);
+        members[i] = {l.qweight, reinterpret_cast<const __half *>(l.cherry_weight), l.cherry_indices,
+                      reinterpret_cast<const __half *>(l.scales), reinterpret_cast<__half *>(l.mul), l.out_features, 0};
+    }
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (fast)
+        return (int)launch_matvec_group(w_bits, reinterpret_cast<const __half *>(vec),
+                                        reinterpret_cast<const __half *>(vec_gate), members, n_layers, K, C, G,
+                                        accumulate, workspace, s);
+    // shapes the streaming kernel does not take: one launch per layer, no fused activation
+    if (vec_gate) return CHERRYQ_E_UNSUPPORTED;
+    for (int i = 0; i < n_layers; i++) {
+        const cherryq_layer &l = layers[i];
+        int rc = w_bits == 4 ? matmul_f16<4>(vec, l.qweight, l.cherry_weight, l.cherry_indices, l.scales, l.mul, 1, K,
+                                             l.out_features, C, G, accumulate, workspace, workspace_bytes, nullptr,
+                                             0, stream)
+                             : matmul_f16<3>(vec, l.qweight, l.cherry_weight, l.cherry_indices, l.scales, l.mul, 1, K,
+                                             l.out_features, C, G, accumulate, workspace, workspace_bytes, nullptr,
+                                             0, stream);
+        if (rc) return rc;
+    }
+    return CHERRYQ_OK;
+}
+
 int cherryq_decode_add_rmsnorm_f16(void *hidden, const void *delta, const void *weight, void *normed,
                                    int hidden_size, float eps, void *stream) {
     if (!hidden || !weight || !normed) return CHERRYQ_E_NULL;
-    if (hidden_size <= 0) return CHERRYQ_E_SHAPE;
+    if (hidden_size <= 0 || hidden_size % 4) return CHERRYQ_E_SHAPE;
+    if (!cq::aligned(hidden, 8) || !cq::aligned(weight, 8) || !cq::aligned(normed, 8) || (delta && !cq::aligned(delta, 8)))
+        return CHERRYQ_E_ALIGN;
     return (int)cq::launch_add_rmsnorm(reinterpret_cast<__half *>(hidden), reinterpret_cast<const __half *>(delta),
                                        reinterpret_cast<const __half *>(weight), reinterpret_cast<__half *>(normed),
                                        hidden_size, eps, reinterpret_cast<hipStream_t>(stream));

@@ -24,19 +24,31 @@ __device__ inline float wave_max(float v) {
 }
 
 // h <- h + delta (skipped when delta is null);  y <- weight * fp16(h * rsqrt(mean(h^2) + eps))
+// One workgroup; a thread takes 4 consecutive elements (one 8-byte access) per pass.  H % 4 == 0.
 __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(__half *__restrict__ h, const __half *__restrict__ delta,
                                                            const __half *__restrict__ weight, __half *__restrict__ y,
                                                            int H, float eps) {
     __shared__ float s_part[16];
     const int t = threadIdx.x;
     float ss = 0.f;
-    for (int i = t; i < H; i += 1024) {
-        float v = __half2float(h[i]);
+    for (int i = 4 * t; i < H; i += 4096) {
+        const uint2 raw = *reinterpret_cast<const uint2 *>(h + i);
+        float v[4] = {__half2float(__ushort_as_half(raw.x & 0xffff)), __half2float(__ushort_as_half(raw.x >> 16)),
+                      __half2float(__ushort_as_half(raw.y & 0xffff)), __half2float(__ushort_as_half(raw.y >> 16))};
         if (delta) {
-            v = __half2float(__float2half_rn(v + __half2float(delta[i])));
-            h[i] = __float2half_rn(v);
+            const uint2 dr = *reinterpret_cast<const uint2 *>(delta + i);
+            const float d[4] = {__half2float(__ushort_as_half(dr.x & 0xffff)), __half2float(__ushort_as_half(dr.x >> 16)),
+                                __half2float(__ushort_as_half(dr.y & 0xffff)), __half2float(__ushort_as_half(dr.y >> 16))};
+            unsigned short o[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                o[e] = __half_as_ushort(__float2half_rn(v[e] + d[e]));
+                v[e] = __half2float(__ushort_as_half(o[e]));
+            }
+            *reinterpret_cast<uint2 *>(h + i) = make_uint2(o[0] | (uint32_t)o[1] << 16, o[2] | (uint32_t)o[3] << 16);
         }
-        ss += v * v;
+#pragma unroll
+        for (int e = 0; e < 4; e++) ss += v[e] * v[e];
     }
     ss = wave_sum(ss);
     if ((t & 63) == 0) s_part[t >> 6] = ss;
@@ -45,9 +57,18 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(__half *__restrict__ 
 #pragma unroll
     for (int w = 0; w < 16; w++) tot += s_part[w];
     const float rs = rsqrtf(tot / (float)H + eps);
-    for (int i = t; i < H; i += 1024) {
-        const float n = __half2float(__float2half_rn(__half2float(h[i]) * rs));
-        y[i] = __float2half_rn(__half2float(weight[i]) * n);
+    for (int i = 4 * t; i < H; i += 4096) {
+        const uint2 raw = *reinterpret_cast<const uint2 *>(h + i);
+        const uint2 wr = *reinterpret_cast<const uint2 *>(weight + i);
+        const uint32_t hv[4] = {raw.x & 0xffff, raw.x >> 16, raw.y & 0xffff, raw.y >> 16};
+        const uint32_t wv[4] = {wr.x & 0xffff, wr.x >> 16, wr.y & 0xffff, wr.y >> 16};
+        unsigned short o[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const float n = __half2float(__float2half_rn(__half2float(__ushort_as_half(hv[e])) * rs));
+            o[e] = __half_as_ushort(__float2half_rn(__half2float(__ushort_as_half(wv[e])) * n));
+        }
+        *reinterpret_cast<uint2 *>(y + i) = make_uint2(o[0] | (uint32_t)o[1] << 16, o[2] | (uint32_t)o[3] << 16);
     }
 }
 
@@ -94,9 +115,27 @@ __global__ void rope_cache_kernel(__half *__restrict__ q, const __half *__restri
 }
 
 // Single-query attention over the cache positions 0 .. *pos, one workgroup (256 threads) per head.
+// The 256 threads form 16 rows of 16 lanes; a row takes one cache position at a time, each lane
+// 8 of the 128 dimensions (one 16-byte load), so 16 positions are in flight per iteration.
 // softmax in fp32, probabilities rounded to fp16 before the value product (as the eager path of
 // the reference does), fp32 accumulation.  head_dim must be 128, max_len <= kMaxAttnLen.
 constexpr int kMaxAttnLen = 4096;
+
+__device__ inline float row16_sum(float v) {
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 16);
+    return v;
+}
+
+__device__ inline void unpack8(const uint4 &u, float (&f)[8]) {
+    const __half2 *h = reinterpret_cast<const __half2 *>(&u);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        f[2 * i] = __low2float(h[i]);
+        f[2 * i + 1] = __high2float(h[i]);
+    }
+}
+
 __global__ __launch_bounds__(256) void attn_decode_kernel(const __half *__restrict__ q,
                                                           const __half *__restrict__ k_cache,
                                                           const __half *__restrict__ v_cache,
@@ -104,18 +143,23 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const __half *__restri
                                                           int n_heads, int n_kv_heads, int max_len, float scale) {
     __shared__ float s_score[kMaxAttnLen];
     __shared__ float s_red[8];
-    __shared__ float s_acc[2][128];
+    __shared__ float s_acc[16][128];
     const int head = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int row = t >> 4, l16 = t & 15;
     const int kvh = head / (n_heads / n_kv_heads);
     const int len = min(*pos_ptr + 1, max_len);
-    const __half *kb = k_cache + (size_t)kvh * max_len * 128;
-    const __half *vb = v_cache + (size_t)kvh * max_len * 128;
-    const __half2 q2 = reinterpret_cast<const __half2 *>(q + (size_t)head * 128)[lane];
-    const float qx = __low2float(q2), qy = __high2float(q2);
-    for (int j = wave; j < len; j += 4) {
-        const __half2 k2 = reinterpret_cast<const __half2 *>(kb + (size_t)j * 128)[lane];
-        const float d = wave_sum(qx * __low2float(k2) + qy * __high2float(k2));
-        if (lane == 0) s_score[j] = __half2float(__float2half_rn(d)) * scale;  // fp16 q k^T, then / sqrt(d)
+    const uint4 *kb = reinterpret_cast<const uint4 *>(k_cache + (size_t)kvh * max_len * 128);
+    const uint4 *vb = reinterpret_cast<const uint4 *>(v_cache + (size_t)kvh * max_len * 128);
+    float qf[8];
+    unpack8(reinterpret_cast<const uint4 *>(q + (size_t)head * 128)[l16], qf);
+    for (int j = row; j < len; j += 16) {
+        float kf[8];
+        unpack8(kb[(size_t)j * 16 + l16], kf);
+        float d = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) d += qf[i] * kf[i];
+        d = row16_sum(d);
+        if (l16 == 0) s_score[j] = __half2float(__float2half_rn(d)) * scale;  // fp16 q k^T, then / sqrt(d)
     }
     __syncthreads();
     float m = -INFINITY;
@@ -134,15 +178,25 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const __half *__restri
     if (lane == 0) s_red[4 + wave] = sum;
     __syncthreads();
     const float inv = 1.f / (s_red[4] + s_red[5] + s_red[6] + s_red[7]);
-    const int d = t & 127, part = t >> 7;
-    float acc = 0.f;
-    for (int j = part; j < len; j += 2) {
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = 0.f;
+    for (int j = row; j < len; j += 16) {
         const float p = __half2float(__float2half_rn(s_score[j] * inv));
-        acc += p * __half2float(vb[(size_t)j * 128 + d]);
+        float vf[8];
+        unpack8(vb[(size_t)j * 16 + l16], vf);
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[i] += p * vf[i];
     }
-    s_acc[part][d] = acc;
+#pragma unroll
+    for (int i = 0; i < 8; i++) s_acc[row][8 * l16 + i] = acc[i];
     __syncthreads();
-    if (t < 128) out[(size_t)head * 128 + t] = __float2half_rn(s_acc[0][t] + s_acc[1][t]);
+    if (t < 128) {
+        float o = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) o += s_acc[r][t];
+        out[(size_t)head * 128 + t] = __float2half_rn(o);
+    }
 }
 
 // out <- fp16(silu(gate)) * up

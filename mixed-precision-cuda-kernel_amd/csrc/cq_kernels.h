@@ -27,6 +27,28 @@ hipError_t launch_matvec(int bits, const __half *vec, const uint8_t *qweight, co
                          const int16_t *cherry_indices, const __half *scales, __half *mul, int K, int N,
                          int C, int G, int accumulate, void *workspace, hipStream_t stream);
 
+// One launch over up to kMaxGroup layers that share the activation vector, K, C and G (q/k/v or
+// gate/up of a decoder block).  vec_gate, when non-null, makes the activations
+// fp16(fp16(silu(vec_gate)) * vec).  The zero-kept workspace needs 8 bytes per column of every
+// member, each member's columns rounded up to a multiple of 256.
+constexpr int kMaxGroup = 4;
+struct MatvecMember {
+    const uint8_t *qweight;
+    const __half *cherry_weight;
+    const int16_t *cherry_indices;
+    const __half *scales;
+    __half *mul;
+    int N;
+    int tile_begin;  // filled in by the launcher
+};
+struct MatvecGroup {
+    MatvecMember m[kMaxGroup];
+    int count;
+};
+hipError_t launch_matvec_group(int bits, const __half *vec, const __half *vec_gate, const MatvecMember *members,
+                               int count, int K, int C, int G, int accumulate, void *workspace,
+                               hipStream_t stream);
+
 // cq_batch.hip: 2..16 batch rows per pass on the matrix cores.
 struct BatchWorkspace {
     size_t tickets, workspace_total;                       // zero-kept workspace: offset, size

@@ -57,6 +57,21 @@ __device__ inline float fdot2(uint32_t a, uint32_t b, float c) {
     return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a), __builtin_bit_cast(half2_t, b), c, false);
 }
 
+// fp16 pair (silu(gate) rounded to fp16) * up, rounded to fp16: the gated-MLP activation the
+// reference materialises between its up/gate and down projections, applied while the down
+// projection stages its activations.
+__device__ inline uint32_t silu_mul_pair(uint32_t gate, uint32_t up) {
+    uint32_t r = 0;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const float g = __half2float(__ushort_as_half((unsigned short)(gate >> (16 * i))));
+        const float u = __half2float(__ushort_as_half((unsigned short)(up >> (16 * i))));
+        const float a = __half2float(__float2half_rn(g / (1.f + __expf(-g))));
+        r |= (uint32_t)__half_as_ushort(__float2half_rn(a * u)) << (16 * i);
+    }
+    return r;
+}
+
 // all-reduce over the 16 lanes of a DPP row by rotations 8, 4, 2, 1
 __device__ inline float row_sum(float v) {
     v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
@@ -109,9 +124,8 @@ struct Geo {
 // that larger workgroups would leave CUs without work.
 template <int BITS, int NW, int KPL>
 __global__ __launch_bounds__(64 * NW) void matvec_kernel(
-    const __half *__restrict__ x, const uint8_t *__restrict__ qweight, const __half *__restrict__ cherry_weight,
-    const int16_t *__restrict__ cherry_indices, const __half *__restrict__ scales, __half *__restrict__ mul,
-    unsigned long long *__restrict__ acc_words, int K, int N, int C, int G, int accumulate, Plan plan) {
+    const __half *__restrict__ x, const __half *__restrict__ x_gate, MatvecGroup grp,
+    unsigned long long *__restrict__ acc_words, int K, int C, int G, int accumulate, Plan plan) {
     using G_ = Geo<BITS, KPL>;
     constexpr int R = G_::kRowsPerLaneGroup;
     constexpr int UK = G_::kUnit;
@@ -124,8 +138,22 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
     // Consecutive workgroups take neighbouring column tiles of the same rows, so that the
     // workgroups in flight at any moment read whole byte rows (DRAM page locality); walking one
     // 256-byte strip down the rows instead costs ~40 % of the bandwidth on square layers.
-    const int tile = blockIdx.x % plan.tiles;
+    // A launch covers up to kMaxGroup layers that share the activation vector (q/k/v, gate/up):
+    // plan.tiles counts the column tiles of all of them and a workgroup picks its layer by tile.
+    const int gtile = blockIdx.x % plan.tiles;
     const int split = blockIdx.x / plan.tiles;
+    MatvecMember mm = grp.m[0];
+#pragma unroll
+    for (int i = 1; i < kMaxGroup; i++)
+        if (i < grp.count && gtile >= grp.m[i].tile_begin) mm = grp.m[i];
+    const uint8_t *__restrict__ qweight = mm.qweight;
+    const __half *__restrict__ cherry_weight = mm.cherry_weight;
+    const int16_t *__restrict__ cherry_indices = mm.cherry_indices;
+    const __half *__restrict__ scales = mm.scales;
+    __half *__restrict__ mul = mm.mul;
+    const int N = mm.N;
+    const int tile = gtile - mm.tile_begin;
+    acc_words += (size_t)mm.tile_begin * kTileCols;
     const int u = split * NW + wave;
     const int n0 = tile * kTileCols + nl * 16;
     const bool col_ok = n0 < N;
@@ -152,9 +180,15 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
 #ifdef CQ_EXP_NOWIN
         const uint32_t win0 = 0x3c003c00u + lane, win1 = 0x3c003c00u;
 #else
-        const uint32_t win0 = __builtin_amdgcn_raw_buffer_load_b32(rx, (ubase + 2 * lane) * 2, 0, 0);
-        const uint32_t win1 = __builtin_amdgcn_raw_buffer_load_b32(rx, (ubase + 128 + 2 * lane) * 2, 0, 0);
+        uint32_t win0 = __builtin_amdgcn_raw_buffer_load_b32(rx, (ubase + 2 * lane) * 2, 0, 0);
+        uint32_t win1 = __builtin_amdgcn_raw_buffer_load_b32(rx, (ubase + 128 + 2 * lane) * 2, 0, 0);
 #endif
+        uint32_t gat0 = 0, gat1 = 0;
+        if (x_gate) {
+            const __amdgpu_buffer_rsrc_t rg = __builtin_amdgcn_make_buffer_rsrc((void *)x_gate, 0, K * 2, kRsrcFlags);
+            gat0 = __builtin_amdgcn_raw_buffer_load_b32(rg, (ubase + 2 * lane) * 2, 0, 0);
+            gat1 = __builtin_amdgcn_raw_buffer_load_b32(rg, (ubase + 128 + 2 * lane) * 2, 0, 0);
+        }
         const int ng = ceil_div(Kn, G);
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)scales, 0, ng * N * 2, kRsrcFlags);
         const int g = (ubase + KPL * kq) / G;
@@ -182,6 +216,10 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
         // t[m] = idx[m] - m is non-decreasing; position k sits after every m with t[m] <= k
         const int t0 = lane < C ? i0 - lane : 0x7fffffff;
         const int t1 = lane + 64 < C ? i1 - (lane + 64) : 0x7fffffff;
+        if (x_gate) {
+            win0 = silu_mul_pair(gat0, win0);
+            win1 = silu_mul_pair(gat1, win1);
+        }
         s_win[wave][lane] = win0;
         s_win[wave][64 + lane] = win1;
         // positions this lane prepares, relative to the lane group's first position
@@ -323,7 +361,12 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
         const int ci = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(ri, (c0 + (nl & 7)) * 2, 0, 0);
         const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, K * 2, kRsrcFlags);
         const uint32_t xoff = (nl < 8 && c0 + nl < C) ? (uint32_t)ci * 2u : kOob;
-        const uint32_t xraw = __builtin_amdgcn_raw_buffer_load_b16(rx, xoff, 0, 0);
+        uint32_t xraw = __builtin_amdgcn_raw_buffer_load_b16(rx, xoff, 0, 0);
+        if (x_gate) {
+            const __amdgpu_buffer_rsrc_t rg = __builtin_amdgcn_make_buffer_rsrc((void *)x_gate, 0, K * 2, kRsrcFlags);
+            const uint32_t graw = __builtin_amdgcn_raw_buffer_load_b16(rg, xoff, 0, 0);
+            xraw = silu_mul_pair(graw & 0xffffu, xraw & 0xffffu) & 0xffffu;
+        }
         __builtin_amdgcn_sched_barrier(0);  // keep the weight loads behind the gather in the queue
         u32x4 cw[8][2];
 #pragma unroll
@@ -408,13 +451,13 @@ bool matvec_supported(int bits, int B, int K, int N, int C, int G) {
 #endif
 
 template <int BITS, int NW, int KPL>
-static hipError_t launch_matvec_nw(const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
-                                   const int16_t *cherry_indices, const __half *scales, __half *mul, int K, int N,
-                                   int C, int G, int accumulate, void *workspace, hipStream_t stream) {
-    const Plan plan = make_plan(K, N, C, NW, 4 * KPL);
+static hipError_t launch_matvec_nw(const __half *vec, const __half *vec_gate, const MatvecGroup &grp, int tiles,
+                                   int K, int C, int G, int accumulate, void *workspace, hipStream_t stream) {
+    Plan plan = make_plan(K, kTileCols, C, NW, 4 * KPL);
+    plan.tiles = tiles;
     hipLaunchKernelGGL((matvec_kernel<BITS, NW, KPL>), dim3(plan.tiles * plan.splits), dim3(64 * NW), 0, stream,
-                       vec, qweight, cherry_weight, cherry_indices, scales, mul,
-                       reinterpret_cast<unsigned long long *>(workspace), K, N, C, G, accumulate, plan);
+                       vec, vec_gate, grp, reinterpret_cast<unsigned long long *>(workspace), K, C, G, accumulate,
+                       plan);
     return hipGetLastError();
 }
 
@@ -439,14 +482,24 @@ int matvec_waves_per_wg(int K, int N, int C, int kpl) {
     return nw;
 }
 
-hipError_t launch_matvec(int bits, const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
-                         const int16_t *cherry_indices, const __half *scales, __half *mul, int K, int N, int C,
-                         int G, int accumulate, void *workspace, hipStream_t stream) {
-    const int kpl = matvec_kpl(bits, K, N, C);
-    const int nw = matvec_waves_per_wg(K, N, C, kpl);
+hipError_t launch_matvec_group(int bits, const __half *vec, const __half *vec_gate, const MatvecMember *members,
+                               int count, int K, int C, int G, int accumulate, void *workspace,
+                               hipStream_t stream) {
+    MatvecGroup grp = {};
+    grp.count = count;
+    int tiles = 0, n_total = 0;
+    for (int i = 0; i < count; i++) {
+        grp.m[i] = members[i];
+        grp.m[i].tile_begin = tiles;
+        tiles += ceil_div(members[i].N, kTileCols);
+        n_total += members[i].N;
+    }
+    for (int i = count; i < kMaxGroup; i++) grp.m[i] = grp.m[0];
+    // geometry from the group's total size: the launch streams all members' weights together
+    const int kpl = matvec_kpl(bits, K, n_total, C);
+    const int nw = matvec_waves_per_wg(K, n_total, C, kpl);
 #define CQ_LAUNCH(B, W, P)                                                                                   \
-    return launch_matvec_nw<B, W, P>(vec, qweight, cherry_weight, cherry_indices, scales, mul, K, N, C, G,   \
-                                     accumulate, workspace, stream)
+    return launch_matvec_nw<B, W, P>(vec, vec_gate, grp, tiles, K, C, G, accumulate, workspace, stream)
 #define CQ_PICK_NW(B, P)                                                                                     \
     do {                                                                                                     \
         if (nw >= 8 && P == 16) CQ_LAUNCH(B, 8, 16);                                                         \
@@ -462,6 +515,13 @@ hipError_t launch_matvec(int bits, const __half *vec, const uint8_t *qweight, co
     CQ_PICK_NW(3, 32);
 #undef CQ_PICK_NW
 #undef CQ_LAUNCH
+}
+
+hipError_t launch_matvec(int bits, const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
+                         const int16_t *cherry_indices, const __half *scales, __half *mul, int K, int N, int C,
+                         int G, int accumulate, void *workspace, hipStream_t stream) {
+    MatvecMember m = {qweight, cherry_weight, cherry_indices, scales, mul, N, 0};
+    return launch_matvec_group(bits, vec, nullptr, &m, 1, K, C, G, accumulate, workspace, stream);
 }
 
 }  // namespace cq

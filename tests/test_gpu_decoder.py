@@ -112,9 +112,59 @@ def test_decode_validation(dec):
 
 
 @pytest.mark.parametrize("bits", [4, 3])
+def test_matvec_group_matches_single_calls(dec, bits):
+    """One grouped launch over layers of different widths equals the per-layer entry points
+    (which the parity tests pin to the oracle); with a gate vector it equals the per-layer call
+    on silu(gate) * up; accumulate adds into the existing output."""
+    print("[case] matvec_group", bits, flush=True)
+    import quant_cuda
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    for K, widths, frac in ((1024, (768, 256, 520), 1 / 64), (4096, (4096, 1024, 1024), 1 / 256),
+                            (2048, (5504, 5504), 1 / 256), (11008, (4096,), 1 / 256)):
+        cfg = dec.DecoderConfig(w_bits=bits, group_size=128, cherry_fraction=frac)
+        mods = [dec.random_packed_linear(cfg, K, n, gen, "cuda") for n in widths]
+        x = torch.randn(1, K, device="cuda", generator=gen).half()
+        g = torch.randn(1, K, device="cuda", generator=gen).half()
+        want, want_act = [], []
+        act = torch.nn.functional.silu(g) * x
+        for m in mods:
+            for vec, dst in ((x, want), (act, want_act)):
+                o = torch.empty(1, m.out_features, dtype=torch.float16, device="cuda")
+                quant_cuda.matmul_cherryq(bits, vec, m.qweight, m.cherry_weight, m.cherry_indices, m.scales, o, 128)
+                dst.append(o)
+        for rep in range(2):  # the second call finds the workspace as the first one left it
+            outs = [torch.full((1, n), 7.0, dtype=torch.float16, device="cuda") for n in widths]
+            dec.matvec_group(mods, x, outs)
+            for o, w in zip(outs, want):
+                assert rel(o, w) < 1e-3, (K, widths, rep)
+        outs = [torch.full((1, n), 7.0, dtype=torch.float16, device="cuda") for n in widths]
+        dec.matvec_group(mods, x, outs, vec_gate=g)
+        for o, w in zip(outs, want_act):
+            assert rel(o, w) < 1e-3, (K, widths, "gate")
+        base = [torch.randn(1, n, device="cuda", generator=gen).half() for n in widths]
+        outs = [b.clone() for b in base]
+        dec.matvec_group(mods, x, outs, accumulate=True)
+        for o, b, w in zip(outs, base, want):
+            assert rel(o, (b.float() + w.float())) < 2e-3, (K, widths, "accumulate")
+    torch.cuda.synchronize()
+
+
+def test_matvec_group_validation(dec):
+    lib = dec._lib
+    assert lib.cherryq_decode_matvec_group_f16(5, None, None, None, 1, 4096, 16, 128, 0, None, 0, None) == -5
+    assert lib.cherryq_decode_matvec_group_f16(4, None, None, None, 1, 4096, 16, 128, 0, None, 0, None) == -1
+    arr = (dec._Layer * 1)(dec._Layer(1 << 12, 1 << 12, 1 << 12, 1 << 12, 1 << 12, 4096))
+    assert lib.cherryq_decode_matvec_group_f16(4, 1 << 12, None, arr, 5, 4096, 16, 128, 0, 1 << 12, 1 << 20, None) == -2
+    assert lib.cherryq_decode_matvec_group_f16(4, 1 << 12, None, arr, 1, 4096, 16, 128, 0, 1 << 12, 64, None) == -4
+    ns = (ctypes.c_int * 2)(4096, 1000)
+    assert lib.cherryq_group_workspace_bytes(2, ns) == (4096 + 1024) * 8
+
+
+@pytest.mark.parametrize("bits", [4, 3])
 def test_small_decoder_matches_dense_reference(dec, bits):
-    """Two-layer decoder with real packed linears: the fused token step agrees with the same model
-    on dequantised weights and plain torch ops, eagerly and as a replayed HIP graph."""
+    """Two-layer decoder with real packed linears: every variant of the fused token step (grouped
+    launches, one launch per operation, forked streams) agrees with the same model on dequantised
+    weights and plain torch ops, and its replayed HIP graph equals its eager run bit for bit."""
     print("[case] small decoder", bits, flush=True)
     cfg = dec.DecoderConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=2,
                             num_key_value_heads=2, vocab_size=512, max_position_embeddings=32, w_bits=bits,
@@ -122,17 +172,18 @@ def test_small_decoder_matches_dense_reference(dec, bits):
     model = dec.CherryLlamaDecoder(cfg, seed=3)
     ids = torch.randint(0, cfg.vocab_size, (12,), generator=torch.Generator().manual_seed(0))
     want = model.reference_logits(ids)
-    eager = model.step_logits(ids, use_graph=False)
-    for t in range(ids.numel()):
-        assert rel(eager[t], want[t]) < 2e-2, t
-    # several replays with eager work between them, each checked against the eager result
-    for fork in (False, True):
+    for fork, grouped in ((False, True), (False, False), (True, False)):
+        eager = model.step_logits(ids, use_graph=False, fork=fork, grouped=grouped)
+        for t in range(ids.numel()):
+            assert rel(eager[t], want[t]) < 2e-2, (t, fork, grouped)
+        # several replays with eager work between them, each checked against the eager result
         model._graph = None
-        graph = model.step_logits(ids, use_graph=True, fork=fork)
+        graph = model.step_logits(ids, use_graph=True, fork=fork, grouped=grouped)
         torch.cuda.synchronize()
         _ = model.reference_logits(ids[:4])  # unrelated eager work between replays
-        graph2 = model.step_logits(ids, use_graph=True, fork=fork)
-        assert torch.equal(graph, eager) and torch.equal(graph2, eager), fork
+        graph2 = model.step_logits(ids, use_graph=True, fork=fork, grouped=grouped)
+        assert torch.equal(graph, eager) and torch.equal(graph2, eager), (fork, grouped)
+    model._graph = None
     out, times, total = model.generate(ids[:4], 8, use_graph=True)
     out2, _, _ = model.generate(ids[:4], 8, use_graph=False)
     assert torch.equal(out, out2) and out.numel() == 8
