@@ -144,8 +144,12 @@ int cherryq_unpack_f16(int w_bits, const uint8_t *qweight, const void *cherry_we
  * overlap inside one grid instead of running as short launches one after another.
  * When vec_gate is non-NULL the activations are fp16(fp16(silu(vec_gate)) * vec), the
  * gated-MLP product that feeds down_proj (:251), formed while the kernel stages its activations.
+ * When norm_weight is non-NULL, vec is the un-normalised hidden state and the activations are
+ * norm_weight * fp16(vec * rsqrt(mean(vec^2) + eps)), the RMSNorm of :75-89 in front of q/k/v
+ * and gate/up, each workgroup taking the sum of squares itself (vec must be 16-byte aligned).
  * workspace: zero-kept like the matmul workspace, cherryq_group_workspace_bytes() bytes.
- * Returns CHERRYQ_E_UNSUPPORTED for vec_gate with shapes the streaming kernel does not take.
+ * Returns CHERRYQ_E_UNSUPPORTED for vec_gate / norm_weight with shapes the streaming kernel
+ * does not take (the caller then runs the separate decode entry points below).
  */
 typedef struct cherryq_layer {
     const uint8_t *qweight;
@@ -157,6 +161,7 @@ typedef struct cherryq_layer {
 } cherryq_layer;
 size_t cherryq_group_workspace_bytes(int n_layers, const int *out_features);
 int cherryq_decode_matvec_group_f16(int w_bits, const void *vec, const void *vec_gate /* may be NULL */,
+                                    const void *norm_weight /* may be NULL */, float eps,
                                     const cherryq_layer *layers, int n_layers, int in_features,
                                     int num_cherries, int group_size, int accumulate, void *workspace,
                                     size_t workspace_bytes, void *stream);
@@ -169,6 +174,10 @@ int cherryq_decode_rope_cache_f16(void *q, const void *k, const void *v, void *k
 int cherryq_decode_attention_f16(const void *q, const void *k_cache, const void *v_cache, void *out,
                                  const int *position, int n_heads, int n_kv_heads, int head_dim, int max_len,
                                  void *stream);
+/* rope_cache followed by attention for the same token, as one launch (q is not modified). */
+int cherryq_decode_rope_attention_f16(const void *q, const void *k, const void *v, void *k_cache, void *v_cache,
+                                      void *out, const int *position, int n_heads, int n_kv_heads,
+                                      int head_dim, int max_len, float theta, void *stream);
 int cherryq_decode_silu_mul_f16(const void *gate, const void *up, void *out, int n, void *stream);
 
 #ifdef __cplusplus

@@ -11,8 +11,9 @@ calls the fused kernels through `quant_cuda`, and the operations between them (r
 RMSNorm, rotary + cache write, single-query attention, SiLU * up) through the decode entry points
 of libcherryq.  The whole step is captured once in a HIP graph and replayed per token.  q/k/v and
 gate/up do not depend on each other: by default each set runs as ONE grouped launch
-(`matvec_group`), the residual additions are the accumulate mode of o_proj / down_proj, and
-SiLU * up is formed inside down_proj.  `grouped=False` keeps one launch per operation;
+(`matvec_group`) that also applies the RMSNorm in front of it, rotary + cache write + attention
+are one launch, the residual additions are the accumulate mode of o_proj / down_proj, and
+SiLU * up is formed inside down_proj: 5 launches per layer.  `grouped=False` keeps one launch per operation;
 `fork=True` captures the independent projections of that variant on forked streams, which on this
 ROCm stack costs more in cross-stream edges than the overlap gains.
 """
@@ -35,8 +36,9 @@ _lib.cherryq_decode_add_rmsnorm_f16.argtypes = [_vp, _vp, _vp, _vp, _int, _f, _v
 _lib.cherryq_decode_rope_cache_f16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _f, _vp]
 _lib.cherryq_decode_attention_f16.argtypes = [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp]
 _lib.cherryq_decode_silu_mul_f16.argtypes = [_vp, _vp, _vp, _int, _vp]
+_lib.cherryq_decode_rope_attention_f16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _f, _vp]
 for _n in ("cherryq_decode_add_rmsnorm_f16", "cherryq_decode_rope_cache_f16", "cherryq_decode_attention_f16",
-           "cherryq_decode_silu_mul_f16"):
+           "cherryq_decode_silu_mul_f16", "cherryq_decode_rope_attention_f16"):
     getattr(_lib, _n).restype = _int
 
 
@@ -48,14 +50,15 @@ class _Layer(ctypes.Structure):
 
 _lib.cherryq_group_workspace_bytes.argtypes = [_int, ctypes.POINTER(_int)]
 _lib.cherryq_group_workspace_bytes.restype = ctypes.c_size_t
-_lib.cherryq_decode_matvec_group_f16.argtypes = [_int, _vp, _vp, ctypes.POINTER(_Layer), _int, _int, _int, _int, _int,
-                                                 _vp, ctypes.c_size_t, _vp]
+_lib.cherryq_decode_matvec_group_f16.argtypes = [_int, _vp, _vp, _vp, _f, ctypes.POINTER(_Layer), _int, _int, _int,
+                                                 _int, _int, _vp, ctypes.c_size_t, _vp]
 _lib.cherryq_decode_matvec_group_f16.restype = _int
 
 
-def matvec_group(mods, vec, outs, vec_gate=None, accumulate=False):
+def matvec_group(mods, vec, outs, vec_gate=None, accumulate=False, norm_weight=None, eps=1e-6):
     """outs[i] (+)= act @ W_i^T for 1..4 QuantLinear modules that read the same (1, K) activation
-    row, in ONE launch; act = vec, or fp16(fp16(silu(vec_gate)) * vec) when vec_gate is given."""
+    row, in ONE launch; act = vec, or fp16(fp16(silu(vec_gate)) * vec) when vec_gate is given, or
+    norm_weight * fp16(vec * rsqrt(mean(vec^2) + eps)) when norm_weight is given."""
     m0 = mods[0]
     k, c = vec.shape[1], m0.cherry_indices.shape[0]
     for m, o in zip(mods, outs):
@@ -72,6 +75,9 @@ def matvec_group(mods, vec, outs, vec_gate=None, accumulate=False):
     if vec_gate is not None and (vec_gate.shape != vec.shape or vec_gate.dtype != torch.float16
                                  or not vec_gate.is_cuda or not vec_gate.is_contiguous()):
         raise RuntimeError("matvec_group: vec_gate must match vec")
+    if norm_weight is not None and (tuple(norm_weight.shape) != (k,) or norm_weight.dtype != torch.float16
+                                    or not norm_weight.is_cuda or not norm_weight.is_contiguous()):
+        raise RuntimeError("matvec_group: norm_weight must be a contiguous (in_features,) fp16 GPU tensor")
     arr = (_Layer * len(mods))(*[_Layer(m.qweight.data_ptr(), quant_cuda._ptr(m.cherry_weight),
                                         quant_cuda._ptr(m.cherry_indices), m.scales.data_ptr(), o.data_ptr(),
                                         m.out_features) for m, o in zip(mods, outs)])
@@ -79,6 +85,7 @@ def matvec_group(mods, vec, outs, vec_gate=None, accumulate=False):
     stream = _stream()
     ws = quant_cuda._workspace(vec.device, stream, _lib.cherryq_group_workspace_bytes(len(mods), ns))
     _ok(_lib.cherryq_decode_matvec_group_f16(m0.w_bits, vec.data_ptr(), None if vec_gate is None else vec_gate.data_ptr(),
+                                             None if norm_weight is None else norm_weight.data_ptr(), eps,
                                              arr, len(mods), k, c, m0.group_size, 1 if accumulate else 0,
                                              ws.data_ptr(), ws.numel(), stream), "matvec_group")
 
@@ -178,6 +185,7 @@ class CherryLlamaDecoder(nn.Module):
         self.logits = torch.zeros(1, cfg.vocab_size, dtype=torch.float32, device=self.device_)
         self.lm_head_t = self.lm_head.t()
         self._graph = None
+        self.fuse_norm = True
         self._side = [torch.cuda.Stream(device=self.device_) for _ in range(2)]
 
     # ---- packed bytes a token step must read (for the roofline of tokens/s)
@@ -209,25 +217,33 @@ class CherryLlamaDecoder(nn.Module):
                                                 cfg.hidden_size, cfg.rms_norm_eps, _stream()), "add_rmsnorm")
 
     def _step_grouped(self):
-        """The token step with 9 launches per layer: q/k/v in one grid, gate/up in one grid, the
-        residual additions folded into o_proj and down_proj (they accumulate into the hidden
-        state, rounded once from fp32), SiLU * up folded into down_proj's activation staging."""
+        """The token step with 5 launches per layer: RMSNorm + q/k/v in one grid, rotary + cache
+        write + attention in one, o_proj accumulating into the hidden state (the residual add,
+        rounded once from fp32), RMSNorm + gate/up in one grid, down_proj with SiLU * up formed in
+        its activation staging and accumulating into the hidden state.  `self.fuse_norm = False`
+        keeps the two norms as launches of their own (7 per layer)."""
         cfg = self.cfg
         nh, nkv, hd, ml = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.max_position_embeddings
         torch.index_select(self.embed_tokens, 0, self.token, out=self.hid)
         for li, layer in enumerate(self.layers):
-            self._norm(layer.input_layernorm)
-            matvec_group([layer.q_proj, layer.k_proj, layer.v_proj], self.normed, [self.q, self.k, self.v])
-            _ok(_lib.cherryq_decode_rope_cache_f16(self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(),
-                                                   self.k_cache[li].data_ptr(), self.v_cache[li].data_ptr(),
-                                                   self.pos.data_ptr(), nh, nkv, hd, ml, cfg.rope_theta, _stream()),
-                "rope_cache")
-            _ok(_lib.cherryq_decode_attention_f16(self.q.data_ptr(), self.k_cache[li].data_ptr(),
-                                                  self.v_cache[li].data_ptr(), self.attn.data_ptr(),
-                                                  self.pos.data_ptr(), nh, nkv, hd, ml, _stream()), "attention")
+            qkv, gu = [layer.q_proj, layer.k_proj, layer.v_proj], [layer.gate_proj, layer.up_proj]
+            if self.fuse_norm:
+                matvec_group(qkv, self.hid, [self.q, self.k, self.v], norm_weight=layer.input_layernorm,
+                             eps=cfg.rms_norm_eps)
+            else:
+                self._norm(layer.input_layernorm)
+                matvec_group(qkv, self.normed, [self.q, self.k, self.v])
+            _ok(_lib.cherryq_decode_rope_attention_f16(self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(),
+                                                       self.k_cache[li].data_ptr(), self.v_cache[li].data_ptr(),
+                                                       self.attn.data_ptr(), self.pos.data_ptr(), nh, nkv, hd, ml,
+                                                       cfg.rope_theta, _stream()), "rope_attention")
             matvec_group([layer.o_proj], self.attn, [self.hid], accumulate=True)
-            self._norm(layer.post_attention_layernorm)
-            matvec_group([layer.gate_proj, layer.up_proj], self.normed, [self.gate, self.up])
+            if self.fuse_norm:
+                matvec_group(gu, self.hid, [self.gate, self.up], norm_weight=layer.post_attention_layernorm,
+                             eps=cfg.rms_norm_eps)
+            else:
+                self._norm(layer.post_attention_layernorm)
+                matvec_group(gu, self.normed, [self.gate, self.up])
             matvec_group([layer.down_proj], self.up, [self.hid], vec_gate=self.gate, accumulate=True)
         self._norm(self.norm)
         self._head()

@@ -208,9 +208,10 @@ size_t cherryq_group_workspace_bytes(int n_layers, const int *out_features) {
     return bytes;
 }
 
-int cherryq_decode_matvec_group_f16(int w_bits, const void *vec, const void *vec_gate, const cherryq_layer *layers,
-                                    int n_layers, int in_features, int num_cherries, int group_size,
-                                    int accumulate, void *workspace, size_t workspace_bytes, void *stream) {
+int cherryq_decode_matvec_group_f16(int w_bits, const void *vec, const void *vec_gate, const void *norm_weight,
+                                    float eps, const cherryq_layer *layers, int n_layers, int in_features,
+                                    int num_cherries, int group_size, int accumulate, void *workspace,
+                                    size_t workspace_bytes, void *stream) {
     using namespace cq;
     if (w_bits != 3 && w_bits != 4) return CHERRYQ_E_BITS;
     if (!layers) return CHERRYQ_E_NULL;
@@ -220,6 +221,7 @@ int cherryq_decode_matvec_group_f16(int w_bits, const void *vec, const void *vec
     for (int i = 0; i < n_layers; i++) outs[i] = layers[i].out_features;
     if (workspace_bytes < cherryq_group_workspace_bytes(n_layers, outs)) return CHERRYQ_E_WORKSPACE;
     if (vec_gate && !aligned(vec_gate, 4)) return CHERRYQ_E_ALIGN;
+    if (norm_weight && (!aligned(norm_weight, 4) || !aligned(vec, 16))) return CHERRYQ_E_ALIGN;
     bool fast = !force_generic();
     MatvecMember members[kMaxGroup];
     for (int i = 0; i < n_layers; i++) {
@@ -232,10 +234,17 @@ int cherryq_decode_matvec_group_f16(int w_bits, const void *vec, const void *vec
                       reinterpret_cast<const __half *>(l.scales), reinterpret_cast<__half *>(l.mul), l.out_features, 0};
     }
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    if (fast)
-        return (int)launch_matvec_group(w_bits, reinterpret_cast<const __half *>(vec),
-                                        reinterpret_cast<const __half *>(vec_gate), members, n_layers, K, C, G,
-                                        accumulate, workspace, s);
+    if (norm_weight) {
+        int n_total = 0;
+        for (int i = 0; i < n_layers; i++) n_total += outs[i];
+        if (!fast || !matvec_norm_supported(w_bits, K, n_total, C)) return CHERRYQ_E_UNSUPPORTED;
+    }
+    if (fast) {
+        const MatvecPrologue pro = {reinterpret_cast<const __half *>(vec_gate),
+                                    reinterpret_cast<const __half *>(norm_weight), eps};
+        return (int)launch_matvec_group(w_bits, reinterpret_cast<const __half *>(vec), pro, members, n_layers, K, C,
+                                        G, accumulate, workspace, s);
+    }
     // shapes the streaming kernel does not take: one launch per layer, no fused activation
     if (vec_gate) return CHERRYQ_E_UNSUPPORTED;
     for (int i = 0; i < n_layers; i++) {
@@ -286,6 +295,23 @@ int cherryq_decode_attention_f16(const void *q, const void *k_cache, const void 
                                        reinterpret_cast<const __half *>(v_cache), reinterpret_cast<__half *>(out),
                                        position, n_heads, n_kv_heads, max_len, 1.0f / sqrtf((float)head_dim),
                                        reinterpret_cast<hipStream_t>(stream));
+}
+
+int cherryq_decode_rope_attention_f16(const void *q, const void *k, const void *v, void *k_cache, void *v_cache,
+                                      void *out, const int *position, int n_heads, int n_kv_heads, int head_dim,
+                                      int max_len, float theta, void *stream) {
+    if (!q || !k || !v || !k_cache || !v_cache || !out || !position) return CHERRYQ_E_NULL;
+    if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads || max_len <= 0 || max_len > cq::attn_max_len())
+        return CHERRYQ_E_SHAPE;
+    if (head_dim != 128) return CHERRYQ_E_UNSUPPORTED;
+    if (!cq::aligned(q, 16) || !cq::aligned(k, 16) || !cq::aligned(v, 16) || !cq::aligned(k_cache, 16) ||
+        !cq::aligned(v_cache, 16) || !cq::aligned(out, 2))
+        return CHERRYQ_E_ALIGN;
+    return (int)cq::launch_rope_attn_decode(
+        reinterpret_cast<const __half *>(q), reinterpret_cast<const __half *>(k), reinterpret_cast<const __half *>(v),
+        reinterpret_cast<__half *>(k_cache), reinterpret_cast<__half *>(v_cache), reinterpret_cast<__half *>(out),
+        position, n_heads, n_kv_heads, max_len, theta, 1.0f / sqrtf((float)head_dim),
+        reinterpret_cast<hipStream_t>(stream));
 }
 
 int cherryq_decode_silu_mul_f16(const void *gate, const void *up, void *out, int n, void *stream) {

@@ -199,6 +199,162 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const __half *__restri
     }
 }
 
+// Rotary embedding, KV-cache write and single-query attention of one token in ONE launch: one
+// workgroup of 1024 threads (64 rows of 16 lanes) per query head.  The workgroup rotates its own
+// q and its kv head's k in LDS and attends to the new position from there, so no workgroup reads
+// a cache row that another one writes in the same launch; the first query head of each kv group
+// stores the rotated k and the v row into the caches for later tokens.  Arithmetic and rounding
+// points are those of rope_cache_kernel followed by attn_decode_kernel.
+__global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
+    const __half *__restrict__ q, const __half *__restrict__ k, const __half *__restrict__ v,
+    __half *__restrict__ k_cache, __half *__restrict__ v_cache, __half *__restrict__ out,
+    const int *__restrict__ pos_ptr, int n_heads, int n_kv_heads, int max_len, float theta, float scale) {
+    __shared__ float s_score[kMaxAttnLen];
+    __shared__ float s_red[32];
+    __shared__ float s_acc[16][128];
+    __shared__ float s_q[128], s_k[128];
+    const int head = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int row = t >> 4, l16 = t & 15;
+    const int rep = n_heads / n_kv_heads, kvh = head / rep;
+    const int pos = *pos_ptr;
+    if (pos >= max_len) return;
+    if (t < 128) {
+        const int i = t & 63;
+        const bool is_k = t >= 64;
+        const float inv_freq = powf(theta, -2.0f * (float)i / 128.f);
+        float sn, cs;
+        sincosf((float)pos * inv_freq, &sn, &cs);
+        const float c = __half2float(__float2half_rn(cs)), sr = __half2float(__float2half_rn(sn));
+        const __half *src = is_k ? k + (size_t)kvh * 128 : q + (size_t)head * 128;
+        const float x1 = __half2float(src[i]), x2 = __half2float(src[i + 64]);
+        const float a1 = __half2float(__float2half_rn(x1 * c)), b1 = __half2float(__float2half_rn(-x2 * sr));
+        const float a2 = __half2float(__float2half_rn(x2 * c)), b2 = __half2float(__float2half_rn(x1 * sr));
+        const __half o1 = __float2half_rn(a1 + b1), o2 = __float2half_rn(a2 + b2);
+        float *dst = is_k ? s_k : s_q;
+        dst[i] = __half2float(o1);
+        dst[i + 64] = __half2float(o2);
+        if (is_k && head % rep == 0) {
+            __half *kd = k_cache + ((size_t)kvh * max_len + pos) * 128;
+            __half *vd = v_cache + ((size_t)kvh * max_len + pos) * 128;
+            const __half *vs = v + (size_t)kvh * 128;
+            kd[i] = o1;
+            kd[i + 64] = o2;
+            vd[i] = vs[i];
+            vd[i + 64] = vs[i + 64];
+        }
+    }
+    __syncthreads();
+    const uint4 *kb = reinterpret_cast<const uint4 *>(k_cache + (size_t)kvh * max_len * 128);
+    const uint4 *vb = reinterpret_cast<const uint4 *>(v_cache + (size_t)kvh * max_len * 128);
+    float qf[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) qf[i] = s_q[8 * l16 + i];
+    // the value rows of the first pass are requested now, so that their latency overlaps the
+    // score and softmax phases (contexts up to 256 positions need no other value loads)
+    uint4 v_first[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const int j = row + 64 * u;
+        v_first[u] = j < pos ? vb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
+    }
+    // scores of the cached positions 0 .. pos-1, four rows of loads in flight per thread
+    for (int j0 = row; j0 < pos; j0 += 256) {
+        uint4 kk[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int j = j0 + 64 * u;
+            kk[u] = j < pos ? kb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int j = j0 + 64 * u;
+            float kf[8];
+            unpack8(kk[u], kf);
+            float d = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) d += qf[i] * kf[i];
+            d = row16_sum(d);
+            if (l16 == 0 && j < pos) s_score[j] = __half2float(__float2half_rn(d)) * scale;
+        }
+    }
+    if (row == 0) {  // the new position, from LDS
+        float d = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) d += qf[i] * s_k[8 * l16 + i];
+        d = row16_sum(d);
+        if (l16 == 0) s_score[pos] = __half2float(__float2half_rn(d)) * scale;
+    }
+    __syncthreads();
+    const int len = pos + 1;
+    float m = -INFINITY;
+    for (int j = t; j < len; j += 1024) m = fmaxf(m, s_score[j]);
+    m = wave_max(m);
+    if (lane == 0) s_red[wave] = m;
+    __syncthreads();
+    m = s_red[0];
+#pragma unroll
+    for (int w = 1; w < 16; w++) m = fmaxf(m, s_red[w]);
+    float sum = 0.f;
+    for (int j = t; j < len; j += 1024) {
+        const float e = __expf(s_score[j] - m);
+        s_score[j] = e;
+        sum += e;
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) s_red[16 + wave] = sum;
+    __syncthreads();
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < 16; w++) tot += s_red[16 + w];
+    const float inv = 1.f / tot;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = 0.f;
+    for (int j0 = row; j0 < pos; j0 += 256) {
+        uint4 vv[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int j = j0 + 64 * u;
+            if (j0 == row)
+                vv[u] = v_first[u];
+            else
+                vv[u] = j < pos ? vb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int j = j0 + 64 * u;
+            const float p = j < pos ? __half2float(__float2half_rn(s_score[j] * inv)) : 0.f;
+            float vf[8];
+            unpack8(vv[u], vf);
+#pragma unroll
+            for (int i = 0; i < 8; i++) acc[i] += p * vf[i];
+        }
+    }
+    if (row == 0) {
+        const float p = __half2float(__float2half_rn(s_score[pos] * inv));
+        float vf[8];
+        unpack8(reinterpret_cast<const uint4 *>(v + (size_t)kvh * 128)[l16], vf);
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[i] += p * vf[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        acc[i] += __shfl_xor(acc[i], 16);
+        acc[i] += __shfl_xor(acc[i], 32);
+    }
+    if (lane < 16) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) s_acc[wave][8 * l16 + i] = acc[i];
+    }
+    __syncthreads();
+    if (t < 128) {
+        float o = 0.f;
+#pragma unroll
+        for (int w = 0; w < 16; w++) o += s_acc[w][t];
+        out[(size_t)head * 128 + t] = __float2half_rn(o);
+    }
+}
+
 // out <- fp16(silu(gate)) * up
 __global__ __launch_bounds__(256) void silu_mul_kernel(const __half *__restrict__ gate, const __half *__restrict__ up,
                                                        __half *__restrict__ out, int n) {
@@ -228,6 +384,14 @@ hipError_t launch_attn_decode(const __half *q, const __half *k_cache, const __ha
                               hipStream_t stream) {
     hipLaunchKernelGGL(attn_decode_kernel, dim3(n_heads), dim3(256), 0, stream, q, k_cache, v_cache, out, pos, n_heads,
                        n_kv_heads, max_len, scale);
+    return hipGetLastError();
+}
+
+hipError_t launch_rope_attn_decode(const __half *q, const __half *k, const __half *v, __half *k_cache,
+                                   __half *v_cache, __half *out, const int *pos, int n_heads, int n_kv_heads,
+                                   int max_len, float theta, float scale, hipStream_t stream) {
+    hipLaunchKernelGGL(rope_attn_decode_kernel, dim3(n_heads), dim3(1024), 0, stream, q, k, v, k_cache, v_cache, out,
+                       pos, n_heads, n_kv_heads, max_len, theta, scale);
     return hipGetLastError();
 }
 

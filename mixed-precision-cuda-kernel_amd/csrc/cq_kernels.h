@@ -28,8 +28,7 @@ hipError_t launch_matvec(int bits, const __half *vec, const uint8_t *qweight, co
                          int C, int G, int accumulate, void *workspace, hipStream_t stream);
 
 // One launch over up to kMaxGroup layers that share the activation vector, K, C and G (q/k/v or
-// gate/up of a decoder block).  vec_gate, when non-null, makes the activations
-// fp16(fp16(silu(vec_gate)) * vec).  The zero-kept workspace needs 8 bytes per column of every
+// gate/up of a decoder block).  The zero-kept workspace needs 8 bytes per column of every
 // member, each member's columns rounded up to a multiple of 256.
 constexpr int kMaxGroup = 4;
 struct MatvecMember {
@@ -45,7 +44,16 @@ struct MatvecGroup {
     MatvecMember m[kMaxGroup];
     int count;
 };
-hipError_t launch_matvec_group(int bits, const __half *vec, const __half *vec_gate, const MatvecMember *members,
+// What the kernel does to the activation vector while staging it (at most one of the two):
+// gate != null: act = fp16(fp16(silu(gate)) * vec);
+// norm_weight != null: act = norm_weight * fp16(vec * rsqrt(mean(vec^2) + eps)).
+struct MatvecPrologue {
+    const __half *gate;
+    const __half *norm_weight;
+    float eps;
+};
+bool matvec_norm_supported(int bits, int K, int n_total, int C);
+hipError_t launch_matvec_group(int bits, const __half *vec, const MatvecPrologue &pro, const MatvecMember *members,
                                int count, int K, int C, int G, int accumulate, void *workspace,
                                hipStream_t stream);
 
@@ -70,6 +78,9 @@ hipError_t launch_rope_cache(__half *q, const __half *k, const __half *v, __half
 hipError_t launch_attn_decode(const __half *q, const __half *k_cache, const __half *v_cache, __half *out,
                               const int *pos, int n_heads, int n_kv_heads, int max_len, float scale,
                               hipStream_t stream);
+hipError_t launch_rope_attn_decode(const __half *q, const __half *k, const __half *v, __half *k_cache,
+                                   __half *v_cache, __half *out, const int *pos, int n_heads, int n_kv_heads,
+                                   int max_len, float theta, float scale, hipStream_t stream);
 hipError_t launch_silu_mul(const __half *gate, const __half *up, __half *out, int n, hipStream_t stream);
 int attn_max_len();
 

@@ -72,6 +72,49 @@ __device__ inline uint32_t silu_mul_pair(uint32_t gate, uint32_t up) {
     return r;
 }
 
+// weight * fp16(x * rs) per half of a pair: RMSNorm applied while the activations are staged
+__device__ inline uint32_t norm_pair(uint32_t xp, uint32_t wp, float rs) {
+    uint32_t r = 0;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const float xv = __half2float(__ushort_as_half((unsigned short)(xp >> (16 * i))));
+        const float wv = __half2float(__ushort_as_half((unsigned short)(wp >> (16 * i))));
+        const float nv = __half2float(__float2half_rn(xv * rs));
+        r |= (uint32_t)__half_as_ushort(__float2half_rn(wv * nv)) << (16 * i);
+    }
+    return r;
+}
+
+constexpr int kNormLoads = 2;  // 16-byte loads per thread for the fused RMSNorm's sum of squares
+
+// rsqrt(mean(x^2) + eps) from the workgroup's shared pass over x (chunk = this thread's loads).
+// Holds a workgroup barrier: when the fused norm is on, every wavefront of the workgroup calls it
+// exactly once, whichever unit path it is on.  The fences are LDS-only so that the unit's
+// weight loads stay in flight across the barrier.
+template <int NW>
+__device__ inline float norm_scale(const u32x4 (&chunk)[kNormLoads], float *s_ss, int wave, int lane, int K,
+                                   float eps) {
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kNormLoads; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float a = __half2float(__ushort_as_half((unsigned short)(chunk[i][j] & 0xffffu)));
+            const float b = __half2float(__ushort_as_half((unsigned short)(chunk[i][j] >> 16)));
+            ss += a * a + b * b;
+        }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+    if (lane == 0) s_ss[wave] = ss;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    float t = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < NW; wv++) t += s_ss[wv];
+    return rsqrtf(t / (float)K + eps);
+}
+
 // all-reduce over the 16 lanes of a DPP row by rotations 8, 4, 2, 1
 __device__ inline float row_sum(float v) {
     v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
@@ -122,9 +165,9 @@ struct Geo {
 
 // NW = wavefronts (= units) per workgroup: 4 for large layers, 2 or 1 when the layer is so small
 // that larger workgroups would leave CUs without work.
-template <int BITS, int NW, int KPL>
+template <int BITS, int NW, int KPL, bool NORM>
 __global__ __launch_bounds__(64 * NW) void matvec_kernel(
-    const __half *__restrict__ x, const __half *__restrict__ x_gate, MatvecGroup grp,
+    const __half *__restrict__ x, MatvecPrologue pro, MatvecGroup grp,
     unsigned long long *__restrict__ acc_words, int K, int C, int G, int accumulate, Plan plan) {
     using G_ = Geo<BITS, KPL>;
     constexpr int R = G_::kRowsPerLaneGroup;
@@ -133,8 +176,14 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
     __shared__ uint32_t s_pair[NW][64];  // per wave: activation pairs laid out for the dot2 operands
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    // wave-uniform by construction; telling the compiler makes every branch on the unit index a
+    // scalar branch, so a wavefront executes exactly one of the unit paths below
+    const int wave = NORM ? __builtin_amdgcn_readfirstlane(tid >> 6) : tid >> 6;
     const int kq = lane >> 4, nl = lane & 15;
+    const __half *__restrict__ x_gate = pro.gate;
+    // NORM is a template parameter so that the plain kernel does not pay the registers
+    const __half *__restrict__ norm_w = NORM ? pro.norm_weight : nullptr;
     // Consecutive workgroups take neighbouring column tiles of the same rows, so that the
     // workgroups in flight at any moment read whole byte rows (DRAM page locality); walking one
     // 256-byte strip down the rows instead costs ~40 % of the bandwidth on square layers.
@@ -164,6 +213,17 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
     for (int c = 0; c < 16; c++) tot[c] = 0.f;
     CQ_STAMP(0);
 
+    // Fused RMSNorm: the workgroup's threads share one pass over the K activations (16 bytes per
+    // load, reads past the end return 0) for the sum of squares.  The loads are issued here, ahead
+    // of the unit's own loads; they are consumed in norm_scale<NW>(nchunk, s_ss, wave, lane, K, pro.eps) after those have been issued.
+    __shared__ float s_ss[NW];
+    u32x4 nchunk[kNormLoads];
+    if (norm_w) {
+        const __amdgpu_buffer_rsrc_t rn = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, K * 2, kRsrcFlags);
+#pragma unroll
+        for (int i = 0; i < kNormLoads; i++)
+            nchunk[i] = __builtin_amdgcn_raw_buffer_load_b128(rn, (uint32_t)(tid + i * 64 * NW) * 16u, 0, 0);
+    }
     if (u < plan.units_normal) {
         const int ubase = u * UK;
         // ---- small operands first: vmcnt retires in order, so these can be waited on while
@@ -183,6 +243,12 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
         uint32_t win0 = __builtin_amdgcn_raw_buffer_load_b32(rx, (ubase + 2 * lane) * 2, 0, 0);
         uint32_t win1 = __builtin_amdgcn_raw_buffer_load_b32(rx, (ubase + 128 + 2 * lane) * 2, 0, 0);
 #endif
+        uint32_t nw0 = 0, nw1 = 0;
+        if (norm_w) {
+            const __amdgpu_buffer_rsrc_t rnw = __builtin_amdgcn_make_buffer_rsrc((void *)norm_w, 0, K * 2, kRsrcFlags);
+            nw0 = __builtin_amdgcn_raw_buffer_load_b32(rnw, (ubase + 2 * lane) * 2, 0, 0);
+            nw1 = __builtin_amdgcn_raw_buffer_load_b32(rnw, (ubase + 128 + 2 * lane) * 2, 0, 0);
+        }
         uint32_t gat0 = 0, gat1 = 0;
         if (x_gate) {
             const __amdgpu_buffer_rsrc_t rg = __builtin_amdgcn_make_buffer_rsrc((void *)x_gate, 0, K * 2, kRsrcFlags);
@@ -219,6 +285,11 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
         if (x_gate) {
             win0 = silu_mul_pair(gat0, win0);
             win1 = silu_mul_pair(gat1, win1);
+        }
+        if (norm_w) {
+            const float rs = norm_scale<NW>(nchunk, s_ss, wave, lane, K, pro.eps);
+            win0 = norm_pair(win0, nw0, rs);
+            win1 = norm_pair(win1, nw1, rs);
         }
         s_win[wave][lane] = win0;
         s_win[wave][64 + lane] = win1;
@@ -367,6 +438,11 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
             const uint32_t graw = __builtin_amdgcn_raw_buffer_load_b16(rg, xoff, 0, 0);
             xraw = silu_mul_pair(graw & 0xffffu, xraw & 0xffffu) & 0xffffu;
         }
+        uint32_t nwraw = 0;
+        if (norm_w) {
+            const __amdgpu_buffer_rsrc_t rnw = __builtin_amdgcn_make_buffer_rsrc((void *)norm_w, 0, K * 2, kRsrcFlags);
+            nwraw = __builtin_amdgcn_raw_buffer_load_b16(rnw, xoff, 0, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);  // keep the weight loads behind the gather in the queue
         u32x4 cw[8][2];
 #pragma unroll
@@ -374,6 +450,7 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
             cw[r][0] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff + (uint32_t)(r * N * 2), 0, kStreamPolicy);
             cw[r][1] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff + (uint32_t)(r * N * 2) + 16, 0, kStreamPolicy);
         }
+        if (norm_w) xraw = norm_pair(xraw & 0xffffu, nwraw & 0xffffu, norm_scale<NW>(nchunk, s_ss, wave, lane, K, pro.eps)) & 0xffffu;
         s_pair[wave][lane] = __builtin_bit_cast(uint32_t, half_bits_to_float(xraw));
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -388,6 +465,8 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
                 tot[c] += half_bits_to_float((c & 1) ? (ww >> 16) : (ww & 0xffffu)) * xc[r];
             }
         }
+    } else if (norm_w) {
+        (void)norm_scale<NW>(nchunk, s_ss, wave, lane, K, pro.eps);  // a wavefront without a unit still owes the workgroup its barrier
     }
 
     CQ_STAMP(2);
@@ -451,13 +530,20 @@ bool matvec_supported(int bits, int B, int K, int N, int C, int G) {
 #endif
 
 template <int BITS, int NW, int KPL>
-static hipError_t launch_matvec_nw(const __half *vec, const __half *vec_gate, const MatvecGroup &grp, int tiles,
+static hipError_t launch_matvec_nw(const __half *vec, const MatvecPrologue &pro, const MatvecGroup &grp, int tiles,
                                    int K, int C, int G, int accumulate, void *workspace, hipStream_t stream) {
+    // the fused norm reads K activations with kNormLoads 16-byte loads per thread
+    if (pro.norm_weight && K > kNormLoads * 8 * 64 * NW) return hipErrorNotSupported;
     Plan plan = make_plan(K, kTileCols, C, NW, 4 * KPL);
     plan.tiles = tiles;
-    hipLaunchKernelGGL((matvec_kernel<BITS, NW, KPL>), dim3(plan.tiles * plan.splits), dim3(64 * NW), 0, stream,
-                       vec, vec_gate, grp, reinterpret_cast<unsigned long long *>(workspace), K, C, G, accumulate,
-                       plan);
+    if (pro.norm_weight)
+        hipLaunchKernelGGL((matvec_kernel<BITS, NW, KPL, true>), dim3(plan.tiles * plan.splits), dim3(64 * NW), 0,
+                           stream, vec, pro, grp, reinterpret_cast<unsigned long long *>(workspace), K, C, G,
+                           accumulate, plan);
+    else
+        hipLaunchKernelGGL((matvec_kernel<BITS, NW, KPL, false>), dim3(plan.tiles * plan.splits), dim3(64 * NW), 0,
+                           stream, vec, pro, grp, reinterpret_cast<unsigned long long *>(workspace), K, C, G,
+                           accumulate, plan);
     return hipGetLastError();
 }
 
@@ -482,7 +568,12 @@ int matvec_waves_per_wg(int K, int N, int C, int kpl) {
     return nw;
 }
 
-hipError_t launch_matvec_group(int bits, const __half *vec, const __half *vec_gate, const MatvecMember *members,
+bool matvec_norm_supported(int bits, int K, int n_total, int C) {
+    const int kpl = matvec_kpl(bits, K, n_total, C);
+    return K <= kNormLoads * 8 * 64 * matvec_waves_per_wg(K, n_total, C, kpl);
+}
+
+hipError_t launch_matvec_group(int bits, const __half *vec, const MatvecPrologue &pro, const MatvecMember *members,
                                int count, int K, int C, int G, int accumulate, void *workspace,
                                hipStream_t stream) {
     MatvecGroup grp = {};
@@ -499,7 +590,7 @@ hipError_t launch_matvec_group(int bits, const __half *vec, const __half *vec_ga
     const int kpl = matvec_kpl(bits, K, n_total, C);
     const int nw = matvec_waves_per_wg(K, n_total, C, kpl);
 #define CQ_LAUNCH(B, W, P)                                                                                   \
-    return launch_matvec_nw<B, W, P>(vec, vec_gate, grp, tiles, K, C, G, accumulate, workspace, stream)
+    return launch_matvec_nw<B, W, P>(vec, pro, grp, tiles, K, C, G, accumulate, workspace, stream)
 #define CQ_PICK_NW(B, P)                                                                                     \
     do {                                                                                                     \
         if (nw >= 8 && P == 16) CQ_LAUNCH(B, 8, 16);                                                         \
@@ -521,7 +612,8 @@ hipError_t launch_matvec(int bits, const __half *vec, const uint8_t *qweight, co
                          const int16_t *cherry_indices, const __half *scales, __half *mul, int K, int N, int C,
                          int G, int accumulate, void *workspace, hipStream_t stream) {
     MatvecMember m = {qweight, cherry_weight, cherry_indices, scales, mul, N, 0};
-    return launch_matvec_group(bits, vec, nullptr, &m, 1, K, C, G, accumulate, workspace, stream);
+    return launch_matvec_group(bits, vec, MatvecPrologue{nullptr, nullptr, 0.f}, &m, 1, K, C, G, accumulate,
+                               workspace, stream);
 }
 
 }  // namespace cq

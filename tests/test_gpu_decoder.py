@@ -92,6 +92,39 @@ def test_rope_cache_and_attention_kernels(dec):
         assert rel(out, want) < 5e-3, p
 
 
+def test_rope_attention_fused_matches_separate_kernels(dec):
+    """The one-launch rotary + cache write + attention equals rope_cache followed by attention,
+    bit for bit, over a growing cache (grouped-query heads included)."""
+    print("[case] rope_attention fused", flush=True)
+    lib = dec._lib
+    torch.manual_seed(2)
+    for nh, nkv, ml, steps in ((8, 4, 64, 20), (4, 4, 600, 530)):
+        hd = 128
+        kc1 = torch.zeros(nkv, ml, hd, device="cuda").half()
+        vc1 = torch.zeros_like(kc1)
+        kc2, vc2 = torch.zeros_like(kc1), torch.zeros_like(kc1)
+        pos = torch.zeros(1, dtype=torch.int32, device="cuda")
+        for step in range(steps):
+            q = torch.randn(1, nh * hd, device="cuda").half()
+            k = torch.randn(1, nkv * hd, device="cuda").half()
+            v = torch.randn(1, nkv * hd, device="cuda").half()
+            q1, o1, o2 = q.clone(), torch.empty_like(q), torch.empty_like(q)
+            assert lib.cherryq_decode_rope_cache_f16(q1.data_ptr(), k.data_ptr(), v.data_ptr(), kc1.data_ptr(),
+                                                     vc1.data_ptr(), pos.data_ptr(), nh, nkv, hd, ml, 10000.0,
+                                                     stream()) == 0
+            assert lib.cherryq_decode_attention_f16(q1.data_ptr(), kc1.data_ptr(), vc1.data_ptr(), o1.data_ptr(),
+                                                    pos.data_ptr(), nh, nkv, hd, ml, stream()) == 0
+            assert lib.cherryq_decode_rope_attention_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), kc2.data_ptr(),
+                                                         vc2.data_ptr(), o2.data_ptr(), pos.data_ptr(), nh, nkv, hd,
+                                                         ml, 10000.0, stream()) == 0
+            if step % 37 == 0 or step == steps - 1:
+                torch.cuda.synchronize()
+                assert rel(o2, o1) < 1e-3, (nh, nkv, step)
+            pos.add_(1)
+        torch.cuda.synchronize()
+        assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+
+
 def test_silu_mul_kernel(dec):
     print("[case] silu_mul", flush=True)
     lib = dec._lib
@@ -141,6 +174,19 @@ def test_matvec_group_matches_single_calls(dec, bits):
         dec.matvec_group(mods, x, outs, vec_gate=g)
         for o, w in zip(outs, want_act):
             assert rel(o, w) < 1e-3, (K, widths, "gate")
+        if K <= 4096:
+            # fused RMSNorm: equals the per-layer call on the separately normalised vector
+            nw = (torch.rand(K, device="cuda", generator=gen) + 0.5).half()
+            h = (torch.randn(1, K, device="cuda", generator=gen) * 3).half()
+            y = torch.empty_like(h)
+            assert dec._lib.cherryq_decode_add_rmsnorm_f16(h.data_ptr(), None, nw.data_ptr(), y.data_ptr(), K, 1e-6,
+                                                           stream()) == 0
+            outs = [torch.full((1, n), 7.0, dtype=torch.float16, device="cuda") for n in widths]
+            dec.matvec_group(mods, h, outs, norm_weight=nw, eps=1e-6)
+            for m, o in zip(mods, outs):
+                w = torch.empty_like(o)
+                quant_cuda.matmul_cherryq(bits, y, m.qweight, m.cherry_weight, m.cherry_indices, m.scales, w, 128)
+                assert rel(o, w) < 1e-3, (K, widths, "norm")
         base = [torch.randn(1, n, device="cuda", generator=gen).half() for n in widths]
         outs = [b.clone() for b in base]
         dec.matvec_group(mods, x, outs, accumulate=True)
@@ -151,11 +197,11 @@ def test_matvec_group_matches_single_calls(dec, bits):
 
 def test_matvec_group_validation(dec):
     lib = dec._lib
-    assert lib.cherryq_decode_matvec_group_f16(5, None, None, None, 1, 4096, 16, 128, 0, None, 0, None) == -5
-    assert lib.cherryq_decode_matvec_group_f16(4, None, None, None, 1, 4096, 16, 128, 0, None, 0, None) == -1
+    assert lib.cherryq_decode_matvec_group_f16(5, None, None, None, 0.0, None, 1, 4096, 16, 128, 0, None, 0, None) == -5
+    assert lib.cherryq_decode_matvec_group_f16(4, None, None, None, 0.0, None, 1, 4096, 16, 128, 0, None, 0, None) == -1
     arr = (dec._Layer * 1)(dec._Layer(1 << 12, 1 << 12, 1 << 12, 1 << 12, 1 << 12, 4096))
-    assert lib.cherryq_decode_matvec_group_f16(4, 1 << 12, None, arr, 5, 4096, 16, 128, 0, 1 << 12, 1 << 20, None) == -2
-    assert lib.cherryq_decode_matvec_group_f16(4, 1 << 12, None, arr, 1, 4096, 16, 128, 0, 1 << 12, 64, None) == -4
+    assert lib.cherryq_decode_matvec_group_f16(4, 1 << 12, None, None, 0.0, arr, 5, 4096, 16, 128, 0, 1 << 12, 1 << 20, None) == -2
+    assert lib.cherryq_decode_matvec_group_f16(4, 1 << 12, None, None, 0.0, arr, 1, 4096, 16, 128, 0, 1 << 12, 64, None) == -4
     ns = (ctypes.c_int * 2)(4096, 1000)
     assert lib.cherryq_group_workspace_bytes(2, ns) == (4096 + 1024) * 8
 
@@ -172,7 +218,9 @@ def test_small_decoder_matches_dense_reference(dec, bits):
     model = dec.CherryLlamaDecoder(cfg, seed=3)
     ids = torch.randint(0, cfg.vocab_size, (12,), generator=torch.Generator().manual_seed(0))
     want = model.reference_logits(ids)
-    for fork, grouped in ((False, True), (False, False), (True, False)):
+    for fork, grouped, fuse_norm in ((False, True, True), (False, True, False), (False, False, False),
+                                     (True, False, False)):
+        model.fuse_norm = fuse_norm
         eager = model.step_logits(ids, use_graph=False, fork=fork, grouped=grouped)
         for t in range(ids.numel()):
             assert rel(eager[t], want[t]) < 2e-2, (t, fork, grouped)
@@ -184,6 +232,7 @@ def test_small_decoder_matches_dense_reference(dec, bits):
         graph2 = model.step_logits(ids, use_graph=True, fork=fork, grouped=grouped)
         assert torch.equal(graph, eager) and torch.equal(graph2, eager), (fork, grouped)
     model._graph = None
+    model.fuse_norm = True
     out, times, total = model.generate(ids[:4], 8, use_graph=True)
     out2, _, _ = model.generate(ids[:4], 8, use_graph=False)
     assert torch.equal(out, out2) and out.numel() == 8
