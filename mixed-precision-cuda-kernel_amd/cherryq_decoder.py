@@ -157,6 +157,8 @@ class CherryLlamaDecoder(nn.Module):
         super().__init__()
         self.cfg = cfg
         self.device_ = torch.device(device)
+        if cfg.head_dim * cfg.num_attention_heads != cfg.hidden_size:
+            raise ValueError("hidden_size must be num_attention_heads * head_dim")
         gen = torch.Generator(device=self.device_).manual_seed(seed)
         h = cfg.hidden_size
         self.embed_tokens = (torch.randn(cfg.vocab_size, h, device=self.device_, generator=gen) * 0.02).half()
@@ -186,7 +188,45 @@ class CherryLlamaDecoder(nn.Module):
         self.lm_head_t = self.lm_head.t()
         self._graph = None
         self.fuse_norm = True
-        self._side = [torch.cuda.Stream(device=self.device_) for _ in range(2)]
+        self._side = [torch.cuda.Stream(device=self.device_) for _ in range(2)] if self.device_.type == "cuda" else []
+
+    # ---- checkpoint schema of the reference's LlamaForCausalLM (llama/modeling_llama_quant.py:
+    # model.embed_tokens :949, layers.N.self_attn.{q,k,v,o}_proj :299-310, layers.N.mlp.{gate,up,
+    # down}_proj :221-229, the two layer norms :754-775, model.norm :1064, lm_head :1132), with the
+    # packed buffer names of llama/qlinear.py:43-63, as utils.py:99-118 writes it
+    _ATTN = ("q_proj", "k_proj", "v_proj", "o_proj")
+    _MLP = ("gate_proj", "up_proj", "down_proj")
+    _BUFFERS = ("cherry_indices", "cherry_weight", "qweight", "scales")
+
+    def reference_state_dict(self) -> dict:
+        sd = {"model.embed_tokens.weight": self.embed_tokens}
+        for i, layer in enumerate(self.layers):
+            for group, names in (("self_attn", self._ATTN), ("mlp", self._MLP)):
+                for n in names:
+                    m = getattr(layer, n)
+                    for b in self._BUFFERS:
+                        sd[f"model.layers.{i}.{group}.{n}.{b}"] = getattr(m, b)
+            sd[f"model.layers.{i}.input_layernorm.weight"] = layer.input_layernorm.data
+            sd[f"model.layers.{i}.post_attention_layernorm.weight"] = layer.post_attention_layernorm.data
+        sd["model.norm.weight"] = self.norm
+        sd["lm_head.weight"] = self.lm_head
+        return sd
+
+    def load_reference_state_dict(self, sd: dict):
+        """Copy a checkpoint in the reference's schema into this decoder (shapes and dtypes are
+        checked; rotary inv_freq buffers, which older transformers versions persist, are ignored)."""
+        want = self.reference_state_dict()
+        extra = [k for k in sd if k not in want and not k.endswith("rotary_emb.inv_freq")]
+        missing = [k for k in want if k not in sd]
+        if extra or missing:
+            raise KeyError(f"checkpoint does not match the decoder: missing {missing[:4]}, unexpected {extra[:4]}")
+        for k, dst in want.items():
+            src = sd[k]
+            if tuple(src.shape) != tuple(dst.shape) or src.dtype != dst.dtype:
+                raise ValueError(f"{k}: checkpoint has {tuple(src.shape)} {src.dtype}, "
+                                 f"decoder expects {tuple(dst.shape)} {dst.dtype}")
+            dst.copy_(src)
+        self._graph = None
 
     # ---- packed bytes a token step must read (for the roofline of tokens/s)
     def step_bytes(self) -> int:

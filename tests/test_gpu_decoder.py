@@ -236,3 +236,21 @@ def test_small_decoder_matches_dense_reference(dec, bits):
     out, times, total = model.generate(ids[:4], 8, use_graph=True)
     out2, _, _ = model.generate(ids[:4], 8, use_graph=False)
     assert torch.equal(out, out2) and out.numel() == 8
+
+
+def test_saved_checkpoint_reloads_to_identical_logits(dec, tmp_path):
+    """save_quantized -> from_quantized (reference file name and key names) gives a decoder whose
+    token step reproduces the original's logits bit for bit."""
+    print("[case] checkpoint round trip", flush=True)
+    import utils as cq_utils
+    cfg = dec.DecoderConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=2,
+                            num_key_value_heads=1, vocab_size=512, max_position_embeddings=32, w_bits=4,
+                            group_size=128, cherry_fraction=1 / 16)
+    model = dec.CherryLlamaDecoder(cfg, seed=7)
+    ids = torch.randint(0, cfg.vocab_size, (6,), generator=torch.Generator().manual_seed(0))
+    want = model.step_logits(ids)
+    cq_utils.save_quantized(model, str(tmp_path))
+    loaded = cq_utils.from_quantized(str(tmp_path))
+    assert loaded.layers[0].q_proj.qweight.is_cuda
+    assert torch.equal(loaded.step_logits(ids), want)
+    assert rel(want[-1], model.reference_logits(ids)[-1]) < 2e-2
