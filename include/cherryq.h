@@ -137,6 +137,18 @@ int cherryq_unpack_f16(int w_bits, const uint8_t *qweight, const void *cherry_we
  * replayed while the caller increments it); caches are [kv_head][max_len][head_dim].
  */
 /*
+ * pack() on the device: dense fp16 `weight` (out_features, in_features), row-major, and the
+ * ASCENDING cherry channels -> qweight, scales (ceil(Kn/group_size), out_features) and
+ * cherry_weight (num_cherries, out_features), bit for bit what QuantLinear.pack() computes on
+ * the host for fp16 weights (llama/qlinear.py:67-118 with llama/cherry_linear.py:69-75 and
+ * FullSymQuantizer.get_scaling_factor / quantize, llama/quantizer.py:148-158).  cherry_indices
+ * must hold distinct channels in [0, in_features).  No workspace.
+ */
+int cherryq_pack_f16(int w_bits, const void *weight, const int16_t *cherry_indices, uint8_t *qweight,
+                     void *scales, void *cherry_weight, int in_features, int out_features, int num_cherries,
+                     int group_size, void *stream);
+
+/*
  * One batch-1 launch over 1..4 packed layers that read the SAME activation vector and share
  * in_features, num_cherries, group_size and w_bits: q/k/v_proj (llama/modeling_llama_quant.py
  * :346-348 of the reference) or gate/up_proj (:251).  Arithmetic per layer is that of

@@ -199,6 +199,21 @@ int cherryq_unpack_f16(int w_bits, const uint8_t *qweight, const void *cherry_we
 
 // ---- decode-step glue (see include/cherryq.h) ----------------------------------------------
 
+int cherryq_pack_f16(int w_bits, const void *weight, const int16_t *cherry_indices, uint8_t *qweight, void *scales,
+                     void *cherry_weight, int in_features, int out_features, int num_cherries, int group_size,
+                     void *stream) {
+    if (w_bits != 3 && w_bits != 4) return CHERRYQ_E_BITS;
+    const int K = in_features, N = out_features, C = num_cherries;
+    if (K <= 0 || N <= 0 || C < 0 || C > K || K % 8 || C % 8) return CHERRYQ_E_SHAPE;
+    if (group_size <= 0) return CHERRYQ_E_GROUP;
+    if (!weight) return CHERRYQ_E_NULL;
+    if (K - C > 0 && (!qweight || !scales)) return CHERRYQ_E_NULL;
+    if (C > 0 && (!cherry_indices || !cherry_weight)) return CHERRYQ_E_NULL;
+    return (int)cq::launch_pack(w_bits, reinterpret_cast<const __half *>(weight), cherry_indices, qweight,
+                                reinterpret_cast<__half *>(scales), reinterpret_cast<__half *>(cherry_weight), K, N,
+                                C, group_size, reinterpret_cast<hipStream_t>(stream));
+}
+
 size_t cherryq_group_workspace_bytes(int n_layers, const int *out_features) {
     size_t bytes = 0;
     for (int i = 0; i < n_layers; i++) {

@@ -69,6 +69,10 @@ hipError_t launch_batch(int bits, const __half *vec, const uint8_t *qweight, con
                         int C, int G, int accumulate, void *workspace, void *scratch, hipStream_t stream);
 size_t scratch_bytes(int B, int K, int N, int C);
 
+// cq_pack.hip: dense fp16 weight -> packed buffers on the device.
+hipError_t launch_pack(int bits, const __half *w, const int16_t *idx, uint8_t *qweight, __half *scales,
+                       __half *cherry_weight, int K, int N, int C, int G, hipStream_t stream);
+
 // cq_decode.hip: batch-1 decode-step glue kernels.
 hipError_t launch_add_rmsnorm(__half *h, const __half *delta, const __half *weight, __half *y, int H, float eps,
                               hipStream_t stream);

@@ -19,7 +19,7 @@ import torch.nn as nn
 import quant_cuda
 
 from .cherry_linear import QuantLinear as QuantLinearForTraining
-from .quantizer import Quantizer
+from .quantizer import FullSymQuantizer, Quantizer
 
 
 def pack_codes(codes: torch.Tensor, w_bits: int) -> torch.Tensor:
@@ -123,6 +123,16 @@ class QuantLinear(nn.Module):
         if linear.bias is not None:
             self.bias = linear.bias.detach().to(torch.float16).cpu().clone()
         weight = linear.weight
+        if (weight.is_cuda and weight.dtype == torch.float16 and self.w_bits in (3, 4)
+                and linear.quantizer is FullSymQuantizer):
+            # same arithmetic on the device; the buffers stay on the weight's device
+            if self.bias is not None:
+                self.bias = self.bias.to(weight.device)
+            group = linear.group_size if linear.group_size != -1 else weight.shape[1]
+            (self.cherry_indices, self.cherry_weight, self.qweight,
+             self.scales) = quant_cuda.pack_cherryq(self.w_bits, weight.detach().contiguous(),
+                                                    linear.cherry_indices, group)
+            return
         cherry = linear.cherry_indices.sort().values.long()
         self.cherry_indices = cherry.to(dtype=torch.int16).cpu()
         self.cherry_weight = weight.t()[cherry].to(torch.float16).cpu()

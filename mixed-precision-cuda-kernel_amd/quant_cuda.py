@@ -47,6 +47,8 @@ for _name in ("cherryq_dequantize3_normal_f32", "cherryq_dequantize4_normal_f32"
     getattr(_lib, _name).restype = _int
 _lib.cherryq_unpack_f16.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp]
 _lib.cherryq_unpack_f16.restype = _int
+_lib.cherryq_pack_f16.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp]
+_lib.cherryq_pack_f16.restype = _int
 _lib.cherryq_workspace_bytes.argtypes = [_int, _int, _int, _int]
 _lib.cherryq_workspace_bytes.restype = _sz
 _lib.cherryq_scratch_bytes.argtypes = [_int, _int, _int, _int]
@@ -249,3 +251,33 @@ def unpack_cherryq(w_bits, qweight, cherry_weight, cherry_indices, scaling_facto
     if rc != 0:
         _fail(rc, "unpack_cherryq")
     return dense
+
+
+def pack_cherryq(w_bits, weight, cherry_indices, group_size):
+    """pack() on the GPU: dense fp16 `weight` (out, in) and the cherry channels (any order, any
+    integer dtype) -> (cherry_indices int16 ascending, cherry_weight, qweight, scales) in the
+    packed schema, bit for bit what QuantLinear.pack() computes on the host
+    (llama/qlinear.py:67-118).  No counterpart in the reference extension."""
+    _check(weight, "weight", torch.float16, 2)
+    dev = weight.device
+    if w_bits not in (3, 4):
+        raise NotImplementedError(f"{w_bits} bit is not implemented yet.")
+    n, k = weight.shape
+    idx = cherry_indices.to(device=dev).sort().values
+    c = idx.numel()
+    if c and (int(idx[0]) < 0 or int(idx[-1]) >= k or bool((idx[1:] == idx[:-1]).any())):
+        raise RuntimeError("cherry_indices must be distinct channels in [0, in_features)")
+    idx = idx.to(torch.int16).contiguous()
+    group_size = int(group_size) if int(group_size) != -1 else k
+    kn = k - c
+    if k % 8 or c % 8 or group_size <= 0:
+        raise RuntimeError(f"pack_cherryq: in_features={k}, num_cherries={c}, group_size={group_size} not packable")
+    qweight = torch.empty((kn // 8 * w_bits, n), dtype=torch.uint8, device=dev)
+    scales = torch.empty((-(-kn // group_size), n), dtype=torch.float16, device=dev)
+    cherry_weight = torch.empty((c, n), dtype=torch.float16, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.cherryq_pack_f16(w_bits, weight.data_ptr(), _ptr(idx), _ptr(qweight), _ptr(scales),
+                                   _ptr(cherry_weight), k, n, c, group_size, torch.cuda.current_stream(dev).cuda_stream)
+    if rc != 0:
+        _fail(rc, "pack_cherryq")
+    return idx, cherry_weight, qweight, scales

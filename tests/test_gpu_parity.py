@@ -466,3 +466,40 @@ def test_direct_c_abi_call_with_raw_pointers(qc):
     want = c_oracle.fused(x.cpu().numpy(), p, bits, 128)
     assert orc.rel_l2(out.cpu().numpy(), want) <= TOL  # accumulate=0 overwrote the 7.0 fill
     assert int(ws.cpu().sum()) == 0  # every accumulator word is back to zero
+
+
+# ------------------------------------------------------------------------- device-side pack
+@pytest.mark.parametrize("bits", [3, 4])
+def test_device_pack_is_bit_identical_to_host_pack(bits):
+    """cherryq_pack_f16 against QuantLinear.pack() on the host (which the golden fixtures pin to
+    the reference): every packed buffer equal byte for byte, on shapes with short last groups,
+    groups that are not multiples of 128, ties, tiny and zero weights."""
+    print("[case] device pack", bits, flush=True)
+    import quant_cuda
+    from llama.cherry_linear import QuantLinear as TrainLinear
+    from llama.qlinear import QuantLinear
+    gen = torch.Generator().manual_seed(11)
+    for k, n, g, frac in ((256, 64, 128, 1 / 16), (1024, 328, 128, 1 / 64), (4096, 512, 128, 1 / 256),
+                          (512, 136, 64, 1 / 32), (768, 72, 256, 1 / 32), (11008, 256, 128, 1 / 256)):
+        lin = TrainLinear(k, n, bias=False, w_bits=bits, group_size=g, cherryq=True, cherry_fraction=frac).half()
+        w = torch.randn(n, k, generator=gen) * 0.02
+        w[torch.rand(n, k, generator=gen) < 0.01] *= 10
+        w[0, :] = 0                                   # an all-zero row: scale from the 1e-6 floor alone
+        w[1, : k // 2] = 1e-7                         # below fp16 resolution
+        w = w.half()
+        w[2] = (torch.randint(-8, 8, (k,), generator=gen).half() * 0.25)  # exact grid points: rounding ties
+        with torch.no_grad():
+            lin.weight.copy_(w)
+        lin.register_cherry_indices(torch.randperm(k, generator=gen)[:lin.num_cherries])
+        host = QuantLinear(bits, g, lin.quantizer, frac, k, n, bias=False)
+        host.pack(lin)
+        dev = QuantLinear(bits, g, lin.quantizer, frac, k, n, bias=False)
+        dev.pack(lin.cuda())
+        assert dev.qweight.is_cuda
+        for name in ("cherry_indices", "cherry_weight", "scales", "qweight"):
+            a, b = getattr(host, name), getattr(dev, name).cpu()
+            assert a.dtype == b.dtype and a.shape == b.shape, (name, k, n, g)
+            assert torch.equal(a, b), (name, k, n, g, int((a != b).sum()))
+    with pytest.raises(RuntimeError):
+        quant_cuda.pack_cherryq(bits, torch.zeros(8, 64, dtype=torch.float16, device="cuda"),
+                                torch.tensor([1, 1, 2, 3, 4, 5, 6, 7]), 64)
