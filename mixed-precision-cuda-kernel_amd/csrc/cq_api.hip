@@ -190,7 +190,7 @@ int cherryq_unpack_f16(int w_bits, const uint8_t *qweight, const void *cherry_we
     if (!dense) return CHERRYQ_E_NULL;
     if (K - C > 0 && (!qweight || !scales)) return CHERRYQ_E_NULL;
     if (C > 0 && (!cherry_weight || !cherry_indices)) return CHERRYQ_E_NULL;
-    if (!cq::aligned(qweight, 4) || !cq::aligned(scales, 2) || !cq::aligned(dense, 2)) return CHERRYQ_E_ALIGN;
+    if (!cq::aligned(qweight, 4) || !cq::aligned(scales, 8) || !cq::aligned(dense, 16)) return CHERRYQ_E_ALIGN;
     return (int)cq::launch_unpack(w_bits, qweight, reinterpret_cast<const __half *>(cherry_weight),
                                   cherry_indices, reinterpret_cast<const __half *>(scales),
                                   reinterpret_cast<__half *>(dense), K, N, C, group_size,

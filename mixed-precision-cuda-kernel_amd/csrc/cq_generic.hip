@@ -212,84 +212,108 @@ hipError_t launch_dequant_normal(int bits, const uint8_t *qweight, const float *
     return hipGetLastError();
 }
 
-// ---- QuantLinear.unpack(): dense (N, K) fp16 -----------------------------------------------
-// llama/qlinear.py:120-162.  A workgroup dequantises a 64-position x 64-column block, turns it
-// through LDS and writes 128-byte row segments of the transposed (N, K) result.  Normal
-// positions scatter to their original columns normal[k] = k + gather_offset(k); the cherry
-// columns are copied by the trailing blocks of the grid.
+// Dense (N, K) fp16 weight, bit for bit what QuantLinear.unpack() computes on the host,
+// llama/qlinear.py:120-162.  A workgroup owns 128 consecutive columns of the DENSE weight and 64
+// of its rows: it decodes the (at most 17) packed 8-position units whose normal columns fall
+// into that range into LDS, stages the cherry rows of the range next to them, and writes every
+// dense row as 16-byte stores, 256 bytes contiguous per row.  Column d of the dense weight is
+// cherry c when idx[c] == d, else normal position d - #{idx < d}.
+constexpr int kUnpackCols = 128;
+constexpr int kUnpackRows = 64;
+constexpr int kUnpackUnits = kUnpackCols / 8 + 1;
+
+template <typename IDX>
+__device__ inline int cherries_below(const IDX *__restrict__ idx, int C, int d) {
+    int lo = 0, hi = C;
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if ((int)idx[mid] < d) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+
 template <int BITS>
 __global__ __launch_bounds__(256) void unpack_kernel(const uint8_t *__restrict__ qweight,
                                                      const __half *__restrict__ cherry_weight,
                                                      const int16_t *__restrict__ cherry_indices,
                                                      const __half *__restrict__ scales,
-                                                     __half *__restrict__ dense, int K, int N, int C, int G,
-                                                     int kblocks) {
-    __shared__ __half tile[64][64 + 2];
-    __shared__ int dst[64];
+                                                     __half *__restrict__ dense, int K, int N, int C, int G) {
+    __shared__ unsigned short s_norm[kUnpackRows][kUnpackUnits * 8 + 2];
+    __shared__ unsigned short s_ch[kUnpackCols][kUnpackRows];
+    __shared__ short s_src[kUnpackCols];
     const int Kn = K - C;
-    const int nb = blockIdx.x * 64;
+    const int d0 = blockIdx.x * kUnpackCols, d1 = min(d0 + kUnpackCols, K);
+    const int n0 = blockIdx.y * kUnpackRows;
     const int t = threadIdx.x;
-    if ((int)blockIdx.y < kblocks) {
-        const int kb = blockIdx.y * 64;
-        if (t < 64) {
-            int k = kb + t;
-            dst[t] = (k < Kn) ? k + gather_offset(cherry_indices, C, k) : -1;
+    const int c_lo = cherries_below(cherry_indices, C, d0), c_hi = cherries_below(cherry_indices, C, d1);
+    const int k_lo = d0 - c_lo, k_hi = d1 - c_hi;  // normal positions of this column range
+    const int ku0 = k_lo & ~7;
+    const int units = k_hi > k_lo ? ceil_div(k_hi - ku0, 8) : 0;
+    if (t < kUnpackCols) {
+        const int d = d0 + t;
+        short src = 0;
+        if (d < d1) {
+            const int c = cherries_below(cherry_indices, C, d);
+            src = (c < C && (int)cherry_indices[c] == d) ? (short)(-1 - (c - c_lo)) : (short)(d - c - ku0);
         }
-        // 8 units of 8 positions x 16 column quads = 128 work items, two per pass of 256 threads
-        if (t < 128) {
-            const int unit = t >> 4, quad = t & 15;
-            const int k0 = kb + unit * 8, n0 = nb + quad * 4;
-            if (k0 < Kn && n0 < N) {
-                uint32_t w[BITS];
+        s_src[t] = src;
+    }
+    for (int e = t; e < (c_hi - c_lo) * kUnpackRows; e += 256) {
+        const int c = e / kUnpackRows, nl = e % kUnpackRows;
+        s_ch[c][nl] = n0 + nl < N ? __half_as_ushort(cherry_weight[(size_t)(c_lo + c) * N + n0 + nl]) : 0;
+    }
+    for (int e = t; e < units * 16; e += 256) {
+        const int u = e >> 4, quad = e & 15;
+        const int k0 = ku0 + 8 * u, nq = n0 + 4 * quad;
+        if (k0 >= Kn || nq >= N) continue;
+        uint32_t w[BITS];
 #pragma unroll
-                for (int r = 0; r < BITS; r++)
-                    w[r] = *reinterpret_cast<const uint32_t *>(qweight + (size_t)(k0 / 8 * BITS + r) * N + n0);
-                const __half *sp = scales + (size_t)(k0 / G) * N + n0;
+        for (int r = 0; r < BITS; r++)
+            w[r] = *reinterpret_cast<const uint32_t *>(qweight + (size_t)(k0 / 8 * BITS + r) * N + nq);
+        const uint2 sraw = *reinterpret_cast<const uint2 *>(scales + (size_t)(k0 / G) * N + nq);
+        const uint32_t sbits[4] = {sraw.x & 0xffffu, sraw.x >> 16, sraw.y & 0xffffu, sraw.y >> 16};
 #pragma unroll
-                for (int c = 0; c < 4; c++) {
-                    float v[8];
-                    decode8<BITS>(w, c, v);
-                    // (code - c_b) has 4 significant bits and the fp16 scale 11: the float
-                    // product is exact, so this is the single rounding the reference performs
-                    float s = __half2float(sp[c]);
+        for (int c = 0; c < 4; c++) {
+            float v[8];
+            decode8<BITS>(w, c, v);
+            // (code - c_b) has 4 significant bits and the fp16 scale 11: the float product is
+            // exact, so this is the single rounding the reference performs
+            const float sc = __half2float(__ushort_as_half((unsigned short)sbits[c]));
 #pragma unroll
-                    for (int i = 0; i < 8; i++) tile[quad * 4 + c][unit * 8 + i] = __float2half_rn(v[i] * s);
-                }
-            }
+            for (int i = 0; i < 8; i++) s_norm[4 * quad + c][8 * u + i] = __half_as_ushort(__float2half_rn(v[i] * sc));
         }
-        __syncthreads();
-        // thread -> (row n = t / 4 .. , 16 consecutive positions)
-        const int nl = t >> 2, seg = (t & 3) * 16;
-        if (nb + nl < N) {
-            __half *row = dense + (size_t)(nb + nl) * K;
-            for (int j = 0; j < 16; j++) {
-                int d = dst[seg + j];
-                if (d >= 0) row[d] = tile[nl][seg + j];
-            }
+    }
+    __syncthreads();
+    for (int e = t; e < kUnpackRows * (kUnpackCols / 8); e += 256) {
+        const int seg = e & 15, nl = e >> 4;
+        const int d = d0 + 8 * seg;
+        if (d >= d1 || n0 + nl >= N) continue;
+        unsigned short h[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int src = s_src[8 * seg + j];
+            h[j] = src >= 0 ? s_norm[nl][src] : s_ch[-1 - src][nl];
         }
-    } else {
-        // cherry columns: dense[n, idx[c]] = cherry_weight[c, n]
-        const int cblk = blockIdx.y - kblocks;
-        for (int i = t; i < 64 * 64; i += 256) {
-            int c = cblk * 64 + (i >> 6), n = nb + (i & 63);
-            if (c < C && n < N) dense[(size_t)n * K + (int)cherry_indices[c]] = cherry_weight[(size_t)c * N + n];
-        }
+        uint4 out;
+        out.x = h[0] | (uint32_t)h[1] << 16;
+        out.y = h[2] | (uint32_t)h[3] << 16;
+        out.z = h[4] | (uint32_t)h[5] << 16;
+        out.w = h[6] | (uint32_t)h[7] << 16;
+        *reinterpret_cast<uint4 *>(dense + (size_t)(n0 + nl) * K + d) = out;
     }
 }
 
 hipError_t launch_unpack(int bits, const uint8_t *qweight, const __half *cherry_weight,
                          const int16_t *cherry_indices, const __half *scales, __half *dense, int K, int N,
                          int C, int G, hipStream_t stream) {
-    const int Kn = K - C;
-    const int kblocks = ceil_div(Kn, 64);
-    dim3 grid(ceil_div(N, 64), kblocks + ceil_div(C, 64));
+    dim3 grid(ceil_div(K, kUnpackCols), ceil_div(N, kUnpackRows));
     if (grid.x == 0 || grid.y == 0) return hipSuccess;
     if (bits == 4)
         hipLaunchKernelGGL(unpack_kernel<4>, grid, dim3(256), 0, stream, qweight, cherry_weight, cherry_indices,
-                           scales, dense, K, N, C, G, kblocks);
+                           scales, dense, K, N, C, G);
     else
         hipLaunchKernelGGL(unpack_kernel<3>, grid, dim3(256), 0, stream, qweight, cherry_weight, cherry_indices,
-                           scales, dense, K, N, C, G, kblocks);
+                           scales, dense, K, N, C, G);
     return hipGetLastError();
 }
 

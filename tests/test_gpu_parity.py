@@ -503,3 +503,29 @@ def test_device_pack_is_bit_identical_to_host_pack(bits):
     with pytest.raises(RuntimeError):
         quant_cuda.pack_cherryq(bits, torch.zeros(8, 64, dtype=torch.float16, device="cuda"),
                                 torch.tensor([1, 1, 2, 3, 4, 5, 6, 7]), 64)
+
+
+# ------------------------------------------------------------------------- prompt-sized batches
+@pytest.mark.parametrize("bits,k,n,rows", [(4, 4096, 1024, 64), (3, 4096, 1024, 128), (4, 11008, 520, 96)])
+def test_prefill_rows_dequantise_once_then_gemm(qc, bits, k, n, rows):
+    """QuantLinear.forward with >= prefill_rows rows (dense GEMM on the bit-exact dequantised
+    weight) against the oracle's dequantised product, and against the fused path just below
+    the threshold."""
+    announce("prefill", bits, k, n, rows)
+    from llama.qlinear import QuantLinear as PackedLinear
+    from llama.quantizer import FullSymQuantizer
+    p = orc.synthetic_packed_fast(k, n, bits, 128, seed=rows)
+    q = PackedLinear(bits, 128, FullSymQuantizer, 1 / 256, k, n, bias=False)
+    for name in NAMES:
+        setattr(q, name, torch.from_numpy(p[name]).cuda())
+    x = np.random.default_rng(rows).standard_normal((rows, k)).astype(np.float16)
+    y = q(torch.from_numpy(x).cuda())
+    assert y.shape == (rows, n) and y.dtype == torch.float16
+    dense, y_deq, _ = oracle_outputs(bits, x, p, 128)
+    assert orc.rel_l2(y.cpu().numpy(), y_deq) <= TOL
+    saved, PackedLinear.prefill_rows = PackedLinear.prefill_rows, 1 << 30
+    try:
+        y_fused = q(torch.from_numpy(x).cuda())
+    finally:
+        PackedLinear.prefill_rows = saved
+    assert orc.rel_l2(y.cpu().numpy(), y_fused.cpu().numpy().astype(np.float64)) <= 2 * TOL
