@@ -549,15 +549,15 @@ static hipError_t launch_matvec_nw(const __half *vec, const MatvecPrologue &pro,
 
 // Positions per lane group.  Small layers are latency bound: 64-position units (8 KB per wave)
 // put twice the wavefronts in flight and halve the compute each one still has to do when its
-// data lands.  Large layers are throughput bound and prefer 128-position units (fewer waves,
-// less fixed work per byte).  Measured crossover on MI355X: about 64 MB of packed weights.
+// data lands.  Larger layers prefer 128-position units (half the wavefronts, split-K atomics and
+// fixed work per byte).  Measured crossover on MI355X: between 10 MB and 17 MB of packed weights.
 int matvec_kpl(int bits, int K, int N, int C) {
 #ifdef CQ_KPL
     (void)bits; (void)K; (void)N; (void)C;
     return CQ_KPL;
 #else
     const long long bytes = (long long)(K - C) / 8 * bits * N;
-    return bytes < (64ll << 20) ? 16 : 32;
+    return bytes < (14ll << 20) ? 16 : 32;
 #endif
 }
 
