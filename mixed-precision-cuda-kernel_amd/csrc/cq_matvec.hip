@@ -562,8 +562,14 @@ int matvec_kpl(int bits, int K, int N, int C) {
 }
 
 int matvec_waves_per_wg(int K, int N, int C, int kpl) {
-    const int max_waves = kpl == 16 ? 8 : 4;
-    int nw = choose_units_per_wg(K, N, C, max_waves, CQ_MIN_WGS, 4 * kpl);
+    const int max_waves = 8;
+    int nw = choose_units_per_wg(K, N, C, kpl == 16 ? 8 : 4, CQ_MIN_WGS, 4 * kpl);
+    // 128-position units: 8 waves per workgroup (half the split-K atomics) pay off only while the
+    // grid still has about three workgroups per CU
+    if (kpl == 32 && nw == 4) {
+        const Plan p8 = make_plan(K, N, C, 8, 4 * kpl);
+        if (p8.tiles * p8.splits >= 768) nw = 8;
+    }
     while (nw < max_waves && make_plan(K, N, C, nw, 4 * kpl).splits > kMaxSplits) nw <<= 1;
     return nw;
 }
@@ -593,7 +599,7 @@ hipError_t launch_matvec_group(int bits, const __half *vec, const MatvecPrologue
     return launch_matvec_nw<B, W, P>(vec, pro, grp, tiles, K, C, G, accumulate, workspace, stream)
 #define CQ_PICK_NW(B, P)                                                                                     \
     do {                                                                                                     \
-        if (nw >= 8 && P == 16) CQ_LAUNCH(B, 8, 16);                                                         \
+        if (nw >= 8) CQ_LAUNCH(B, 8, P);                                                                   \
         if (nw >= 4) CQ_LAUNCH(B, 4, P);                                                                     \
         if (nw == 2) CQ_LAUNCH(B, 2, P);                                                                     \
         CQ_LAUNCH(B, 1, P);                                                                                  \
