@@ -180,8 +180,7 @@ __global__ __launch_bounds__(256) void batch_prep_kernel(const __half *__restric
 }
 
 // ---- main kernel -------------------------------------------------------------------------------
-// Everything one unit needs from memory; two of these alternate so that the loads of the next
-// unit are in flight while the matrix cores work on the current one.
+// Everything one unit needs from memory.
 struct UnitRegs {
     u32x4 w[16];    // 16 (12) byte rows x 16 columns
     u32x4 sc0, sc1; // 16 group scales (fp16)
@@ -317,9 +316,6 @@ __global__ __launch_bounds__(64 * kBatchWaves) __attribute__((amdgpu_waves_per_e
 #pragma unroll
     for (int c = 0; c < 16; c++) tot[c] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-    // this wave's units: u0, u0 + 4, u0 + 8, ...  (the 4 waves interleave).  Two units per round:
-    // both sets of loads are issued before the first unit is consumed, so the second unit's
-    // 16 KB arrive while the matrix cores work on the first.
     // this wave's units: u0, u0 + 4, u0 + 8, ...  (the 4 waves interleave).  One register set per
     // wave keeps the kernel at two waves per SIMD, which overlap each other's loads and MFMAs.
     CQB_STAMP(0);

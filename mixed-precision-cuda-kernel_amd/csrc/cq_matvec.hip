@@ -48,10 +48,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kMaxFastCherries = 128;  // two 64-lane chunks of cherry indices
 constexpr uint32_t kRsrcFlags = 0x00020000u;
 constexpr uint32_t kOob = 0x80000000u;  // byte offset beyond any buffer this kernel accepts
-#ifndef CQ_STREAM_POLICY
-#define CQ_STREAM_POLICY 2
-#endif
-constexpr int kStreamPolicy = CQ_STREAM_POLICY;  // cache policy of the weight stream: 2 = nt (read once)
+constexpr int kStreamPolicy = 2;  // cache policy of the weight stream: nt (read once)
 
 __device__ inline float fdot2(uint32_t a, uint32_t b, float c) {
     return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a), __builtin_bit_cast(half2_t, b), c, false);
@@ -230,19 +227,11 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
         // the weight loads issued after them are still in flight
         const __amdgpu_buffer_rsrc_t ri =
             __builtin_amdgcn_make_buffer_rsrc((void *)cherry_indices, 0, C * 2, kRsrcFlags);
-#ifdef CQ_EXP_NOIDX
-        const int i0 = 16000 + lane, i1 = 17000 + lane;
-#else
         const int i0 = (short)__builtin_amdgcn_raw_buffer_load_b16(ri, lane * 2, 0, 0);
         const int i1 = (short)__builtin_amdgcn_raw_buffer_load_b16(ri, (lane + 64) * 2, 0, 0);
-#endif
         const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, K * 2, kRsrcFlags);
-#ifdef CQ_EXP_NOWIN
-        const uint32_t win0 = 0x3c003c00u + lane, win1 = 0x3c003c00u;
-#else
         uint32_t win0 = __builtin_amdgcn_raw_buffer_load_b32(rx, (ubase + 2 * lane) * 2, 0, 0);
         uint32_t win1 = __builtin_amdgcn_raw_buffer_load_b32(rx, (ubase + 128 + 2 * lane) * 2, 0, 0);
-#endif
         uint32_t nw0 = 0, nw1 = 0;
         if (norm_w) {
             const __amdgpu_buffer_rsrc_t rnw = __builtin_amdgcn_make_buffer_rsrc((void *)norm_w, 0, K * 2, kRsrcFlags);
@@ -259,16 +248,9 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)scales, 0, ng * N * 2, kRsrcFlags);
         const int g = (ubase + KPL * kq) / G;
         const uint32_t soff = col_ok ? (uint32_t)(g * N + n0) * 2u : kOob;
-#ifdef CQ_EXP_NOSCALE
-        const u32x4 sc0 = {0x20002000u + soff, 0x20002000u, 0x20002000u, 0x20002000u}, sc1 = sc0;
-#else
         const u32x4 sc0 = __builtin_amdgcn_raw_buffer_load_b128(rs, soff, 0, 0);
         const u32x4 sc1 = __builtin_amdgcn_raw_buffer_load_b128(rs, soff + 16, 0, 0);
-#endif
 
-#ifdef CQ_EXP_WAIT_SMALL
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#endif
         // ---- the weight stream: R byte rows x 16 columns per lane, rows past the end read 0
         const int qrows = Kn / 8 * BITS;
         const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void *)qweight, 0, qrows * N, kRsrcFlags);
@@ -351,17 +333,7 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
             xq[i] = *reinterpret_cast<const u32x4 *>(&s_pair[wave][16 * kq + 4 * i]);
         CQ_STAMP(1);
 
-#ifdef CQ_EXP_NOCOMPUTE
-        {
-            uint32_t acc_x = 0;
-#pragma unroll
-            for (int r = 0; r < R; r++) acc_x ^= w[r][0] ^ w[r][1] ^ w[r][2] ^ w[r][3];
-            tot[0] = __builtin_bit_cast(float, (acc_x & 0xffu) | xq[0][0]) * xsum;
-        }
-        if (false) {
-#else
         if (BITS == 4) {
-#endif
             float lo[16], hi[16];
 #pragma unroll
             for (int c = 0; c < 16; c++) lo[c] = hi[c] = 0.f;
@@ -479,11 +451,7 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
     if (NW == 1) {
         const int n = n0 + 4 * kq;
         CQ_STAMP(3);
-#ifdef CQ_EXP_NOEPILOGUE
-        if (n < N && q4[0][0] == 123.f) mul[n] = __float2half(q4[0][1]);
-#else
         splitk_finish<__half, 1, 4>(q4, 1, N, n, n < N, plan.splits, acc_words, mul, accumulate);
-#endif
         CQ_STAMP(4);
     } else {
         // ---- across the workgroup's wavefronts through LDS, then 4 / NW columns per thread
@@ -501,12 +469,8 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
         }
         const int n = tile * kTileCols + tid * CPT;
         CQ_STAMP(3);
-#ifdef CQ_EXP_NOEPILOGUE
-        if (n < N && vals[0][0] == 123.f) mul[n] = __float2half(vals[0][0]);
-#else
         splitk_finish<__half, 1, CPT>(vals, 1, N, n, n < N && tid * CPT < kTileCols, plan.splits, acc_words, mul,
                                       accumulate);
-#endif
         CQ_STAMP(4);
     }
 }
@@ -525,9 +489,7 @@ bool matvec_supported(int bits, int B, int K, int N, int C, int G) {
     return K - C > 0;
 }
 
-#ifndef CQ_MIN_WGS
-#define CQ_MIN_WGS 256
-#endif
+constexpr int kMinWorkgroups = 256;  // one per CU at least
 
 template <int BITS, int NW, int KPL>
 static hipError_t launch_matvec_nw(const __half *vec, const MatvecPrologue &pro, const MatvecGroup &grp, int tiles,
@@ -552,18 +514,13 @@ static hipError_t launch_matvec_nw(const __half *vec, const MatvecPrologue &pro,
 // data lands.  Larger layers prefer 128-position units (half the wavefronts, split-K atomics and
 // fixed work per byte).  Measured crossover on MI355X: between 10 MB and 17 MB of packed weights.
 int matvec_kpl(int bits, int K, int N, int C) {
-#ifdef CQ_KPL
-    (void)bits; (void)K; (void)N; (void)C;
-    return CQ_KPL;
-#else
     const long long bytes = (long long)(K - C) / 8 * bits * N;
     return bytes < (14ll << 20) ? 16 : 32;
-#endif
 }
 
 int matvec_waves_per_wg(int K, int N, int C, int kpl) {
     const int max_waves = 8;
-    int nw = choose_units_per_wg(K, N, C, kpl == 16 ? 8 : 4, CQ_MIN_WGS, 4 * kpl);
+    int nw = choose_units_per_wg(K, N, C, kpl == 16 ? 8 : 4, kMinWorkgroups, 4 * kpl);
     // 128-position units: 8 waves per workgroup (half the split-K atomics) pay off only while the
     // grid still has about three workgroups per CU
     if (kpl == 32 && nw == 4) {
