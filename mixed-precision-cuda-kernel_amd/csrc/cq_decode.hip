@@ -9,6 +9,10 @@
 #include "cq_common.cuh"
 #include "cq_kernels.h"
 
+// The rotary embedding rounds every product and every sum to fp16 separately, as the reference's
+// fp16 tensor operations do; contraction would merge a product and a sum into one rounding.
+#pragma clang fp contract(off)
+
 namespace cq {
 
 __device__ inline float wave_sum(float v) {
@@ -216,6 +220,31 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
     const int head = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int row = t >> 4, l16 = t & 15;
     const int rep = n_heads / n_kv_heads, kvh = head / rep;
+    const uint4 *kb = reinterpret_cast<const uint4 *>(k_cache + (size_t)kvh * max_len * 128);
+    const uint4 *vb = reinterpret_cast<const uint4 *>(v_cache + (size_t)kvh * max_len * 128);
+    // The cache rows of the first pass are requested before the position is known (rows up to
+    // max_len exist; those at or beyond the position are ignored below), so that the position,
+    // q/k/v and the cache rows travel together: one memory round trip in front of the arithmetic.
+    uint4 k_first[4], v_first[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const int j = row + 64 * u;
+        k_first[u] = j < max_len ? kb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
+        v_first[u] = j < max_len ? vb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
+    }
+    // likewise the new token's q (threads 0..63), k and v (threads 64..127)
+    float x1 = 0.f, x2 = 0.f;
+    __half v1 = __float2half(0.f), v2 = v1;
+    if (t < 128) {
+        const int i = t & 63;
+        const __half *src = t >= 64 ? k + (size_t)kvh * 128 : q + (size_t)head * 128;
+        x1 = __half2float(src[i]);
+        x2 = __half2float(src[i + 64]);
+        if (t >= 64) {
+            v1 = v[(size_t)kvh * 128 + i];
+            v2 = v[(size_t)kvh * 128 + i + 64];
+        }
+    }
     const int pos = *pos_ptr;
     if (pos >= max_len) return;
     if (t < 128) {
@@ -225,8 +254,6 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
         float sn, cs;
         sincosf((float)pos * inv_freq, &sn, &cs);
         const float c = __half2float(__float2half_rn(cs)), sr = __half2float(__float2half_rn(sn));
-        const __half *src = is_k ? k + (size_t)kvh * 128 : q + (size_t)head * 128;
-        const float x1 = __half2float(src[i]), x2 = __half2float(src[i + 64]);
         const float a1 = __half2float(__float2half_rn(x1 * c)), b1 = __half2float(__float2half_rn(-x2 * sr));
         const float a2 = __half2float(__float2half_rn(x2 * c)), b2 = __half2float(__float2half_rn(x1 * sr));
         const __half o1 = __float2half_rn(a1 + b1), o2 = __float2half_rn(a2 + b2);
@@ -236,34 +263,26 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
         if (is_k && head % rep == 0) {
             __half *kd = k_cache + ((size_t)kvh * max_len + pos) * 128;
             __half *vd = v_cache + ((size_t)kvh * max_len + pos) * 128;
-            const __half *vs = v + (size_t)kvh * 128;
             kd[i] = o1;
             kd[i + 64] = o2;
-            vd[i] = vs[i];
-            vd[i + 64] = vs[i + 64];
+            vd[i] = v1;
+            vd[i + 64] = v2;
         }
     }
     __syncthreads();
-    const uint4 *kb = reinterpret_cast<const uint4 *>(k_cache + (size_t)kvh * max_len * 128);
-    const uint4 *vb = reinterpret_cast<const uint4 *>(v_cache + (size_t)kvh * max_len * 128);
     float qf[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) qf[i] = s_q[8 * l16 + i];
-    // the value rows of the first pass are requested now, so that their latency overlaps the
-    // score and softmax phases (contexts up to 256 positions need no other value loads)
-    uint4 v_first[4];
-#pragma unroll
-    for (int u = 0; u < 4; u++) {
-        const int j = row + 64 * u;
-        v_first[u] = j < pos ? vb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
-    }
     // scores of the cached positions 0 .. pos-1, four rows of loads in flight per thread
     for (int j0 = row; j0 < pos; j0 += 256) {
         uint4 kk[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             const int j = j0 + 64 * u;
-            kk[u] = j < pos ? kb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
+            if (j0 == row)
+                kk[u] = k_first[u];
+            else
+                kk[u] = j < pos ? kb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int u = 0; u < 4; u++) {
@@ -316,7 +335,7 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
         for (int u = 0; u < 4; u++) {
             const int j = j0 + 64 * u;
             if (j0 == row)
-                vv[u] = v_first[u];
+                vv[u] = j < pos ? v_first[u] : make_uint4(0, 0, 0, 0);  // rows past the position may hold anything
             else
                 vv[u] = j < pos ? vb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
         }
