@@ -134,6 +134,49 @@ def time_gpu(bits, k, n, group, steps, warmup, batch=1, use_graph=True):
     return dev_us, wall_us, base, x, out, copies
 
 
+def roofline_reference(copies, steps):
+    """What the GPU does with the same packed bytes when a kernel only reads them (the library's
+    stream-read probe over each copy's qweight, same rotation, same graph replay), and the cost
+    of an empty launch.  Puts the fused kernel's time in proportion."""
+    import ctypes
+    import torch
+    import quant_cuda
+    lib = quant_cuda._lib
+    lib.cherryq_probe_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p]
+    lib.cherryq_probe_empty_launch.argtypes = [ctypes.c_void_p]
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+    nbytes = copies[0]["qweight"].numel()
+    stream = torch.cuda.Stream()
+    out = {}
+    with torch.cuda.stream(stream):
+        for name in ("plain_read", "empty_launch"):
+            def step(i):
+                if name == "plain_read":
+                    rc = lib.cherryq_probe_stream_read(copies[i % len(copies)]["qweight"].data_ptr(), nbytes,
+                                                       sink.data_ptr(), stream.cuda_stream)
+                else:
+                    rc = lib.cherryq_probe_empty_launch(stream.cuda_stream)
+                assert rc == 0, rc
+            for i in range(20):
+                step(i)
+            stream.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for i in range(steps):
+                    step(i)
+            graph.replay()
+            stream.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            graph.replay()
+            e1.record(stream)
+            stream.synchronize()
+            out[name] = e0.elapsed_time(e1) * 1e3 / steps
+    return {"plain_read_us": round(out["plain_read"], 3), "plain_read_bytes": nbytes,
+            "plain_read_gbs": round(nbytes / out["plain_read"] / 1e3, 1),
+            "empty_launch_us": round(out["empty_launch"], 3)}
+
+
 def cpu_baseline(bits, k, n, group, base, x_np):
     """The reference CPU path -- QuantLinear.unpack() then linear -- restated in C (oracle),
     timed on this host: cold = unpack + matvec, cached = matvec on the dense fp16 weight."""
@@ -273,6 +316,8 @@ def main():
                      "kernel": f"cq::matvec_kernel<{bits}>" if args.batch == 1 else
                                f"cq::batch_prep_kernel<{bits}> + cq::batch_kernel<{bits}>"},
     }
+    if args.batch == 1:
+        result["roofline"]["reference"] = roofline_reference(copies, args.steps)
     if not args.no_decode:
         del copies, x, out
         torch.cuda.empty_cache()

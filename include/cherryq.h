@@ -137,6 +137,15 @@ int cherryq_unpack_f16(int w_bits, const uint8_t *qweight, const void *cherry_we
  * replayed while the caller increments it); caches are [kv_head][max_len][head_dim].
  */
 /*
+ * Roofline reference launches for measurement scripts; no counterpart in the reference and no
+ * part in the product path.  cherryq_probe_stream_read reads `bytes` (< 2 GiB) of `buf` once with
+ * the access shape of the weight stream and nothing else (sink: 4 writable bytes, never written
+ * in practice); cherryq_probe_empty_launch launches an empty kernel.
+ */
+int cherryq_probe_stream_read(const void *buf, size_t bytes, void *sink, void *stream);
+int cherryq_probe_empty_launch(void *stream);
+
+/*
  * pack() on the device: dense fp16 `weight` (out_features, in_features), row-major, and the
  * ASCENDING cherry channels -> qweight, scales (ceil(Kn/group_size), out_features) and
  * cherry_weight (num_cherries, out_features), bit for bit what QuantLinear.pack() computes on

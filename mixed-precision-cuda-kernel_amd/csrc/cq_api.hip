@@ -214,6 +214,15 @@ int cherryq_pack_f16(int w_bits, const void *weight, const int16_t *cherry_indic
                                 C, group_size, reinterpret_cast<hipStream_t>(stream));
 }
 
+int cherryq_probe_stream_read(const void *buf, size_t bytes, void *sink, void *stream) {
+    if (!buf || !sink) return CHERRYQ_E_NULL;
+    if (bytes >= 0x7fff0000ull) return CHERRYQ_E_SHAPE;
+    if (!cq::aligned(buf, 16) || !cq::aligned(sink, 4)) return CHERRYQ_E_ALIGN;
+    return (int)cq::launch_probe_read(buf, bytes, sink, reinterpret_cast<hipStream_t>(stream));
+}
+
+int cherryq_probe_empty_launch(void *stream) { return (int)cq::launch_probe_empty(reinterpret_cast<hipStream_t>(stream)); }
+
 size_t cherryq_group_workspace_bytes(int n_layers, const int *out_features) {
     size_t bytes = 0;
     for (int i = 0; i < n_layers; i++) {

@@ -73,6 +73,10 @@ size_t scratch_bytes(int B, int K, int N, int C);
 hipError_t launch_pack(int bits, const __half *w, const int16_t *idx, uint8_t *qweight, __half *scales,
                        __half *cherry_weight, int K, int N, int C, int G, hipStream_t stream);
 
+// cq_probe.hip: roofline reference kernels for the measurement script.
+hipError_t launch_probe_read(const void *buf, size_t bytes, void *sink, hipStream_t stream);
+hipError_t launch_probe_empty(hipStream_t stream);
+
 // cq_decode.hip: batch-1 decode-step glue kernels.
 hipError_t launch_add_rmsnorm(__half *h, const __half *delta, const __half *weight, __half *y, int H, float eps,
                               hipStream_t stream);
