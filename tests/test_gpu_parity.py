@@ -529,3 +529,22 @@ def test_prefill_rows_dequantise_once_then_gemm(qc, bits, k, n, rows):
     finally:
         PackedLinear.prefill_rows = saved
     assert orc.rel_l2(y.cpu().numpy(), y_fused.cpu().numpy().astype(np.float64)) <= 2 * TOL
+
+
+def test_empty_batch_is_a_no_op(qc):
+    """Zero activation rows: nothing is launched, through the entry point and through the module."""
+    announce("empty batch")
+    from llama.qlinear import QuantLinear as PackedLinear
+    from llama.quantizer import FullSymQuantizer
+    k, n = 1024, 256
+    p = orc.synthetic_packed_fast(k, n, 4, 128, seed=3)
+    d = dev(p)
+    x = torch.zeros(0, k, dtype=torch.float16, device="cuda")
+    out = torch.zeros(0, n, dtype=torch.float16, device="cuda")
+    qc.vecquant4matmul_cherryq(x, d["qweight"], d["cherry_weight"], d["cherry_indices"], d["scales"], out, 128)
+    q = PackedLinear(4, 128, FullSymQuantizer, 1 / 256, k, n, bias=False)
+    for name in NAMES:
+        setattr(q, name, d[name])
+    y = q(torch.zeros(2, 0, k, dtype=torch.float16, device="cuda"))
+    assert y.shape == (2, 0, n)
+    torch.cuda.synchronize()
