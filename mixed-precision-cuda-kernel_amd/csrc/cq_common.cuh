@@ -34,15 +34,6 @@ __host__ __device__ inline Plan make_plan(int K, int N, int C, int units_per_wg,
     return p;
 }
 
-// Units per workgroup for the streaming kernels: as many as possible (fewer split-K atomics on
-// the same word, which serialise at roughly 80 ns each) while the grid still has at least
-// `min_wgs` workgroups to cover the 256 CUs.
-inline int choose_units_per_wg(int K, int N, int C, int max_units, int min_wgs, int unit_k = kUnitK) {
-    int u = max_units;
-    while (u > 1 && make_plan(K, N, C, u, unit_k).tiles * make_plan(K, N, C, u, unit_k).splits < min_wgs) u >>= 1;
-    return u;
-}
-
 // Workgroups are dealt to the 8 XCDs round-robin by their linear id.  Renumber so that
 // consecutive logical ids (all K-splits of one column tile) run on the same XCD and share
 // its L2 for the activation vector, the scales and the split-K partials.

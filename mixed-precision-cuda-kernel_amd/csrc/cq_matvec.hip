@@ -82,7 +82,7 @@ __device__ inline uint32_t norm_pair(uint32_t xp, uint32_t wp, float rs) {
     return r;
 }
 
-constexpr int kNormLoads = 2;  // 16-byte loads per thread for the fused RMSNorm's sum of squares
+constexpr int kNormLoads = 4;  // 16-byte loads per thread for the fused RMSNorm's sum of squares
 
 // rsqrt(mean(x^2) + eps) from the workgroup's shared pass over x (chunk = this thread's loads).
 // Holds a workgroup barrier: when the fused norm is on, every wavefront of the workgroup calls it
@@ -160,7 +160,7 @@ struct Geo {
     static constexpr int kPairs = KPL / 2;  // activation pair dwords per lane group
 };
 
-// NW = wavefronts (= units) per workgroup: 4 for large layers, 2 or 1 when the layer is so small
+// NW = wavefronts (= units) per workgroup: 4, or 2 or 1 when the layer is so small
 // that larger workgroups would leave CUs without work.
 template <int BITS, int NW, int KPL, bool NORM>
 __global__ __launch_bounds__(64 * NW) void matvec_kernel(
@@ -458,7 +458,7 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
         __shared__ float s_red[NW][kTileCols];
         *reinterpret_cast<float4 *>(&s_red[wave][16 * nl + 4 * kq]) = make_float4(q4[0][0], q4[0][1], q4[0][2], q4[0][3]);
         __syncthreads();
-        constexpr int CPT = NW <= 4 ? 4 / NW : 1;  // columns per thread; 8 waves: first 256 threads
+        constexpr int CPT = 4 / NW;  // columns per thread
         float vals[1][CPT];
 #pragma unroll
         for (int c = 0; c < CPT; c++) {
@@ -485,11 +485,10 @@ bool matvec_supported(int bits, int B, int K, int N, int C, int G) {
     const long long cbytes = (long long)C * N * 2;
     const long long sbytes = (long long)ceil_div(K - C, G) * N * 2;
     if (wbytes >= 0x7fff0000ll || cbytes >= 0x7fff0000ll || sbytes >= 0x7fff0000ll) return false;
-    if (make_plan(K, N, C, 8, 64).splits > kMaxSplits) return false;
+    if (make_plan(K, N, C, 4, 128).splits > kMaxSplits) return false;
     return K - C > 0;
 }
 
-constexpr int kMinWorkgroups = 256;  // one per CU at least
 
 template <int BITS, int NW, int KPL>
 static hipError_t launch_matvec_nw(const __half *vec, const MatvecPrologue &pro, const MatvecGroup &grp, int tiles,
@@ -509,25 +508,26 @@ static hipError_t launch_matvec_nw(const __half *vec, const MatvecPrologue &pro,
     return hipGetLastError();
 }
 
-// Positions per lane group.  Small layers are latency bound: 64-position units (8 KB per wave)
-// put twice the wavefronts in flight and halve the compute each one still has to do when its
-// data lands.  Larger layers prefer 128-position units (half the wavefronts, split-K atomics and
-// fixed work per byte).  Measured crossover on MI355X: between 10 MB and 17 MB of packed weights.
+// Geometry, from sweeps over the LLaMA-7B/13B/70B layer shapes on MI355X (3- and 4-bit, single and
+// grouped launches): 64-position units (8 KB per wave: more wavefronts in flight, half the
+// decode left to do when a wave's data lands) up to 28 MB of packed weights, 128-position units
+// (half the wavefronts and split-K atomics) above; four wavefronts per workgroup throughout --
+// eight make the workgroup barrier and the per-CU placement coarser and were slower nearly
+// everywhere, fewer multiply the split-K atomics.  Only layers too small to give every second
+// CU a workgroup use fewer wavefronts per workgroup.
 int matvec_kpl(int bits, int K, int N, int C) {
     const long long bytes = (long long)(K - C) / 8 * bits * N;
-    return bytes < (14ll << 20) ? 16 : 32;
+    return bytes < (28ll << 20) ? 16 : 32;
 }
 
 int matvec_waves_per_wg(int K, int N, int C, int kpl) {
-    const int max_waves = 8;
-    int nw = choose_units_per_wg(K, N, C, kpl == 16 ? 8 : 4, kMinWorkgroups, 4 * kpl);
-    // 128-position units: 8 waves per workgroup (half the split-K atomics) pay off only while the
-    // grid still has about three workgroups per CU
-    if (kpl == 32 && nw == 4) {
-        const Plan p8 = make_plan(K, N, C, 8, 4 * kpl);
-        if (p8.tiles * p8.splits >= 768) nw = 8;
+    int nw = 4;
+    while (nw > 1) {
+        const Plan p = make_plan(K, N, C, nw, 4 * kpl);
+        if (p.tiles * p.splits >= 128) break;
+        nw >>= 1;
     }
-    while (nw < max_waves && make_plan(K, N, C, nw, 4 * kpl).splits > kMaxSplits) nw <<= 1;
+    while (nw < 4 && make_plan(K, N, C, nw, 4 * kpl).splits > kMaxSplits) nw <<= 1;
     return nw;
 }
 
@@ -556,7 +556,6 @@ hipError_t launch_matvec_group(int bits, const __half *vec, const MatvecPrologue
     return launch_matvec_nw<B, W, P>(vec, pro, grp, tiles, K, C, G, accumulate, workspace, stream)
 #define CQ_PICK_NW(B, P)                                                                                     \
     do {                                                                                                     \
-        if (nw >= 8) CQ_LAUNCH(B, 8, P);                                                                   \
         if (nw >= 4) CQ_LAUNCH(B, 4, P);                                                                     \
         if (nw == 2) CQ_LAUNCH(B, 2, P);                                                                     \
         CQ_LAUNCH(B, 1, P);                                                                                  \
