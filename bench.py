@@ -47,7 +47,7 @@ WORKLOADS = {
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, each
 # counter scaled by its reading for a 256 MiB device copy (x2.000 and x1.000); the counters
 # cannot be read while timing, so the figure is recorded here for the workloads measured.
-MEASURED_TRAFFIC = {("llama7b_gate_up_w4", 1): 24648200}
+MEASURED_TRAFFIC = {("llama7b_gate_up_w4", 1): 25320960}
 
 
 def algorithmic_bytes(bits, k, n, batch=1, group=128):
