@@ -16,7 +16,7 @@ static bool force_generic() {
     return e && e[0] == '1';
 }
 
-// One 64-bit accumulator word per output element of the largest batch chunk a kernel handles.
+// Size queries answer for any arguments; nonsensical ones are clamped, not rejected.
 static void clamp_dims(int &B, int &K, int &N, int &C) {
     if (B < 1) B = 1;
     if (K < 8) K = 8;
@@ -197,7 +197,7 @@ int cherryq_unpack_f16(int w_bits, const uint8_t *qweight, const void *cherry_we
                                   reinterpret_cast<hipStream_t>(stream));
 }
 
-// ---- decode-step glue (see include/cherryq.h) ----------------------------------------------
+// ---- device-side pack, measurement probes ----------------------------------------------------
 
 int cherryq_pack_f16(int w_bits, const void *weight, const int16_t *cherry_indices, uint8_t *qweight, void *scales,
                      void *cherry_weight, int in_features, int out_features, int num_cherries, int group_size,
@@ -222,6 +222,8 @@ int cherryq_probe_stream_read(const void *buf, size_t bytes, void *sink, void *s
 }
 
 int cherryq_probe_empty_launch(void *stream) { return (int)cq::launch_probe_empty(reinterpret_cast<hipStream_t>(stream)); }
+
+// ---- decode-step entry points (see include/cherryq.h) ------------------------------------------
 
 size_t cherryq_group_workspace_bytes(int n_layers, const int *out_features) {
     size_t bytes = 0;

@@ -212,7 +212,7 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
 
     // Fused RMSNorm: the workgroup's threads share one pass over the K activations (16 bytes per
     // load, reads past the end return 0) for the sum of squares.  The loads are issued here, ahead
-    // of the unit's own loads; they are consumed in norm_scale<NW>(nchunk, s_ss, wave, lane, K, pro.eps) after those have been issued.
+    // of the unit's own loads; they are consumed in norm_scale() after those have been issued.
     __shared__ float s_ss[NW];
     u32x4 nchunk[kNormLoads];
     if (norm_w) {
@@ -422,7 +422,10 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
             cw[r][0] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff + (uint32_t)(r * N * 2), 0, kStreamPolicy);
             cw[r][1] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff + (uint32_t)(r * N * 2) + 16, 0, kStreamPolicy);
         }
-        if (norm_w) xraw = norm_pair(xraw & 0xffffu, nwraw & 0xffffu, norm_scale<NW>(nchunk, s_ss, wave, lane, K, pro.eps)) & 0xffffu;
+        if (norm_w) {
+            const float rs = norm_scale<NW>(nchunk, s_ss, wave, lane, K, pro.eps);
+            xraw = norm_pair(xraw & 0xffffu, nwraw & 0xffffu, rs) & 0xffffu;
+        }
         s_pair[wave][lane] = __builtin_bit_cast(uint32_t, half_bits_to_float(xraw));
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -438,7 +441,8 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
             }
         }
     } else if (norm_w) {
-        (void)norm_scale<NW>(nchunk, s_ss, wave, lane, K, pro.eps);  // a wavefront without a unit still owes the workgroup its barrier
+        // a wavefront without a unit still owes the workgroup its barrier
+        (void)norm_scale<NW>(nchunk, s_ss, wave, lane, K, pro.eps);
     }
 
     CQ_STAMP(2);

@@ -36,7 +36,8 @@ __global__ __launch_bounds__(256) void pack_scales_kernel(const __half *__restri
     const int g = (int)(item / N), n = (int)(item % N);
     const int k0 = g * G, k1 = min(k0 + G, Kn);
     float mx = 0.f;
-    for (int k = k0 + lane; k < k1; k += 64) mx = fmaxf(mx, fabsf(__half2float(w[(size_t)n * K + normal_source(idx, C, k)])));
+    for (int k = k0 + lane; k < k1; k += 64)
+        mx = fmaxf(mx, fabsf(__half2float(w[(size_t)n * K + normal_source(idx, C, k)])));
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
     if (lane == 0) {
