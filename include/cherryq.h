@@ -199,6 +199,15 @@ int cherryq_decode_attention_f16(const void *q, const void *k_cache, const void 
 int cherryq_decode_rope_attention_f16(const void *q, const void *k, const void *v, void *k_cache, void *v_cache,
                                       void *out, const int *position, int n_heads, int n_kv_heads,
                                       int head_dim, int max_len, float theta, void *stream);
+/*
+ * Tail of a greedy step: *next_token = argmax(logits[0..vocab)) (lowest index among equal maxima),
+ * history[*position] = that token when history is non-NULL and the position lies below
+ * history_len, hidden_out[0..hidden) = embed[token] (the next step's input), *position += 1.
+ * The host side of the reference's generation loop (benchmark_perplexity.py:92-109).
+ */
+int cherryq_decode_argmax_embed_f16(const void *logits, int vocab, const void *embed, int hidden,
+                                    void *hidden_out, long long *next_token, long long *history /* may be NULL */,
+                                    int history_len, int *position, void *stream);
 int cherryq_decode_silu_mul_f16(const void *gate, const void *up, void *out, int n, void *stream);
 
 #ifdef __cplusplus

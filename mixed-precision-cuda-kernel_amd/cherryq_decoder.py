@@ -36,6 +36,8 @@ _lib.cherryq_decode_add_rmsnorm_f16.argtypes = [_vp, _vp, _vp, _vp, _int, _f, _v
 _lib.cherryq_decode_rope_cache_f16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _f, _vp]
 _lib.cherryq_decode_attention_f16.argtypes = [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp]
 _lib.cherryq_decode_silu_mul_f16.argtypes = [_vp, _vp, _vp, _int, _vp]
+_lib.cherryq_decode_argmax_embed_f16.argtypes = [_vp, _int, _vp, _int, _vp, _vp, _vp, _int, _vp, _vp]
+_lib.cherryq_decode_argmax_embed_f16.restype = _int
 _lib.cherryq_decode_rope_attention_f16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _f, _vp]
 for _n in ("cherryq_decode_add_rmsnorm_f16", "cherryq_decode_rope_cache_f16", "cherryq_decode_attention_f16",
            "cherryq_decode_silu_mul_f16", "cherryq_decode_rope_attention_f16"):
@@ -184,7 +186,7 @@ class CherryLlamaDecoder(nn.Module):
         self.up = torch.zeros(1, cfg.intermediate_size, **f16)
         self.act = torch.zeros(1, cfg.intermediate_size, **f16)
         self.logits16 = torch.zeros(1, cfg.vocab_size, **f16)
-        self.logits = torch.zeros(1, cfg.vocab_size, dtype=torch.float32, device=self.device_)
+        self.history = torch.zeros(ml, dtype=torch.int64, device=self.device_)  # history[p]: token predicted at position p
         self.lm_head_t = self.lm_head.t()
         self._graph = None
         self.fuse_norm = True
@@ -264,7 +266,6 @@ class CherryLlamaDecoder(nn.Module):
         keeps the two norms as launches of their own (7 per layer)."""
         cfg = self.cfg
         nh, nkv, hd, ml = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.max_position_embeddings
-        torch.index_select(self.embed_tokens, 0, self.token, out=self.hid)
         for li, layer in enumerate(self.layers):
             qkv, gu = [layer.q_proj, layer.k_proj, layer.v_proj], [layer.gate_proj, layer.up_proj]
             if self.fuse_norm:
@@ -289,20 +290,34 @@ class CherryLlamaDecoder(nn.Module):
         self._head()
 
     def _head(self):
-        torch.matmul(self.normed, self.lm_head_t, out=self.logits16)  # unquantised fp16 head
-        self.logits.copy_(self.logits16)
-        torch.argmax(self.logits, dim=-1, out=self.next_token)
-        self.pos.add_(1)
+        """Unquantised fp16 head, then the greedy tail on the device: next_token = argmax, recorded
+        in history[pos]; its embedding becomes the next step's hidden state; pos += 1."""
+        cfg = self.cfg
+        torch.matmul(self.normed, self.lm_head_t, out=self.logits16)
+        _ok(_lib.cherryq_decode_argmax_embed_f16(self.logits16.data_ptr(), cfg.vocab_size, self.embed_tokens.data_ptr(),
+                                                 cfg.hidden_size, self.hid.data_ptr(), self.next_token.data_ptr(),
+                                                 self.history.data_ptr(), self.history.numel(), self.pos.data_ptr(),
+                                                 _stream()), "argmax_embed")
+
+    @property
+    def logits(self):
+        return self.logits16.float()
+
+    def embed(self):
+        """hid <- embedding of self.token.  A step reads its input from `hid`: after a step `hid`
+        already holds the embedding of the token that step predicted, so free-running greedy
+        decoding needs no call here; feeding a given token (prompt, teacher forcing) does."""
+        torch.index_select(self.embed_tokens, 0, self.token, out=self.hid)
 
     def _step(self, fork=False, grouped=True):
-        """One token: self.token at position self.pos -> self.logits, self.next_token; pos += 1.
+        """One token: the embedding in self.hid at position self.pos -> self.logits16, self.next_token,
+        the next input in self.hid; pos += 1.
         grouped=False runs every projection and every element-wise operation as its own launch
         (12 per layer), the literal sequence of the reference's decoder layer."""
         if grouped and not fork:
             return self._step_grouped()
         cfg = self.cfg
         nh, nkv, hd, ml = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.max_position_embeddings
-        torch.index_select(self.embed_tokens, 0, self.token, out=self.hid)
         delta = None
         for li, layer in enumerate(self.layers):
             _ok(_lib.cherryq_decode_add_rmsnorm_f16(self.hid.data_ptr(), delta, layer.input_layernorm.data_ptr(),
@@ -375,23 +390,26 @@ class CherryLlamaDecoder(nn.Module):
         self.reset()
         run = self._graph.replay if use_graph else self._step
         prompt_ids = prompt_ids.to(self.device_)
-        for i in range(prompt_ids.numel()):
+        n_prompt = prompt_ids.numel()
+        for i in range(n_prompt):
             self.token.copy_(prompt_ids[i:i + 1])
+            self.embed()
             run()
-        out = torch.zeros(max_new_tokens, dtype=torch.int64, device=self.device_)
         torch.cuda.synchronize()
         times = []
         t0 = time.perf_counter()
         for i in range(max_new_tokens):
             tick = time.perf_counter()
-            self.token.copy_(self.next_token)
-            out[i:i + 1].copy_(self.next_token)
-            run()
+            run()  # consumes the token the previous step predicted; nothing for the host to do
             if sync_each_token:
                 torch.cuda.synchronize()
                 times.append(time.perf_counter() - tick)
         torch.cuda.synchronize()
-        return out, times, time.perf_counter() - t0
+        total = time.perf_counter() - t0
+        # history[p] is the token predicted at position p: the first generated token was predicted
+        # by the last prompt step
+        out = self.history[n_prompt - 1:n_prompt - 1 + max_new_tokens].clone()
+        return out, times, total
 
     @torch.inference_mode()
     def step_logits(self, ids: torch.Tensor, use_graph=False, fork=False, grouped=True) -> torch.Tensor:
@@ -403,11 +421,12 @@ class CherryLlamaDecoder(nn.Module):
         rows = []
         for i in range(ids.numel()):
             self.token.copy_(ids[i:i + 1])
+            self.embed()
             if use_graph:
                 self._graph.replay()
             else:
                 self._step(fork, grouped)
-            rows.append(self.logits.clone())
+            rows.append(self.logits)
         torch.cuda.synchronize()
         return torch.cat(rows, dim=0)
 

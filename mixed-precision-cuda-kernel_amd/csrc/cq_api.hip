@@ -340,6 +340,20 @@ int cherryq_decode_rope_attention_f16(const void *q, const void *k, const void *
         reinterpret_cast<hipStream_t>(stream));
 }
 
+int cherryq_decode_argmax_embed_f16(const void *logits, int vocab, const void *embed, int hidden, void *hidden_out,
+                                    long long *next_token, long long *history, int history_len, int *position,
+                                    void *stream) {
+    if (!logits || !embed || !hidden_out || !next_token || !position) return CHERRYQ_E_NULL;
+    if (vocab <= 0 || hidden <= 0 || history_len < 0) return CHERRYQ_E_SHAPE;
+    if (!cq::aligned(logits, 16) || !cq::aligned(embed, 2) || !cq::aligned(hidden_out, 2) ||
+        !cq::aligned(next_token, 8) || !cq::aligned(history, 8))
+        return CHERRYQ_E_ALIGN;
+    return (int)cq::launch_argmax_embed(reinterpret_cast<const __half *>(logits), vocab,
+                                        reinterpret_cast<const __half *>(embed), hidden,
+                                        reinterpret_cast<__half *>(hidden_out), next_token, history, history_len,
+                                        position, reinterpret_cast<hipStream_t>(stream));
+}
+
 int cherryq_decode_silu_mul_f16(const void *gate, const void *up, void *out, int n, void *stream) {
     if (!gate || !up || !out) return CHERRYQ_E_NULL;
     if (n <= 0) return CHERRYQ_E_SHAPE;

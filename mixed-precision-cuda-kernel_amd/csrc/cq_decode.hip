@@ -384,6 +384,81 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const __half *__restrict_
     out[i] = __float2half_rn(a * __half2float(up[i]));
 }
 
+// Tail of a greedy decoding step, one workgroup: next = argmax(logits) (lowest index among equal
+// maxima), recorded in *next_token and history[*pos]; the next token's embedding row becomes the
+// hidden state of the following step; *pos += 1.  What the reference's generation loop does on
+// the host between two forward passes (benchmark_perplexity.py:92-109), kept on the device so
+// that a replayed graph needs no host work per token.
+__global__ __launch_bounds__(1024) void argmax_embed_kernel(const __half *__restrict__ logits, int vocab,
+                                                            const __half *__restrict__ embed, int hidden,
+                                                            __half *__restrict__ hid, long long *__restrict__ next_token,
+                                                            long long *__restrict__ history, int history_len,
+                                                            int *__restrict__ pos_ptr) {
+    __shared__ float s_val[16];
+    __shared__ int s_idx[16];
+    __shared__ int s_best;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    // 8 logits per 16-byte load; the tail that is not a multiple of 8 is read element-wise
+    const int vec_end = vocab & ~7;
+    for (int i = 8 * t; i < vec_end; i += 8 * 1024) {
+        float f[8];
+        unpack8(*reinterpret_cast<const uint4 *>(logits + i), f);
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+            if (f[e] > best) {
+                best = f[e];
+                best_i = i + e;
+            }
+    }
+    for (int i = vec_end + t; i < vocab; i += 1024) {
+        const float f = __half2float(logits[i]);
+        if (f > best) {
+            best = f;
+            best_i = i;
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o);
+        const int oi = __shfl_xor(best_i, o);
+        if (ov > best || (ov == best && oi < best_i)) {
+            best = ov;
+            best_i = oi;
+        }
+    }
+    if (lane == 0) {
+        s_val[wave] = best;
+        s_idx[wave] = best_i;
+    }
+    __syncthreads();
+    if (t == 0) {
+        for (int w = 1; w < 16; w++)
+            if (s_val[w] > best || (s_val[w] == best && s_idx[w] < best_i)) {
+                best = s_val[w];
+                best_i = s_idx[w];
+            }
+        if (best_i >= vocab) best_i = 0;  // every logit was NaN or -inf
+        s_best = best_i;
+        const int pos = *pos_ptr;
+        *next_token = best_i;
+        if (history && pos >= 0 && pos < history_len) history[pos] = best_i;
+        *pos_ptr = pos + 1;
+    }
+    __syncthreads();
+    const __half *row = embed + (size_t)s_best * hidden;
+    for (int i = t; i < hidden; i += 1024) hid[i] = row[i];
+}
+
+hipError_t launch_argmax_embed(const __half *logits, int vocab, const __half *embed, int hidden, __half *hid,
+                               long long *next_token, long long *history, int history_len, int *pos,
+                               hipStream_t stream) {
+    hipLaunchKernelGGL(argmax_embed_kernel, dim3(1), dim3(1024), 0, stream, logits, vocab, embed, hidden, hid,
+                       next_token, history, history_len, pos);
+    return hipGetLastError();
+}
+
 hipError_t launch_add_rmsnorm(__half *h, const __half *delta, const __half *weight, __half *y, int H, float eps,
                               hipStream_t stream) {
     hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(1024), 0, stream, h, delta, weight, y, H, eps);

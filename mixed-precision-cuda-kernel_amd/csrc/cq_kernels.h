@@ -89,6 +89,9 @@ hipError_t launch_attn_decode(const __half *q, const __half *k_cache, const __ha
 hipError_t launch_rope_attn_decode(const __half *q, const __half *k, const __half *v, __half *k_cache,
                                    __half *v_cache, __half *out, const int *pos, int n_heads, int n_kv_heads,
                                    int max_len, float theta, float scale, hipStream_t stream);
+hipError_t launch_argmax_embed(const __half *logits, int vocab, const __half *embed, int hidden, __half *hid,
+                               long long *next_token, long long *history, int history_len, int *pos,
+                               hipStream_t stream);
 hipError_t launch_silu_mul(const __half *gate, const __half *up, __half *out, int n, hipStream_t stream);
 int attn_max_len();
 

@@ -254,3 +254,35 @@ def test_saved_checkpoint_reloads_to_identical_logits(dec, tmp_path):
     assert loaded.layers[0].q_proj.qweight.is_cuda
     assert torch.equal(loaded.step_logits(ids), want)
     assert rel(want[-1], model.reference_logits(ids)[-1]) < 2e-2
+
+
+def test_argmax_embed_tail_kernel(dec):
+    """Greedy tail: argmax with the lowest index among equal maxima, history entry, embedding of
+    the chosen token as next hidden state, position increment; odd vocabulary sizes included."""
+    print("[case] argmax_embed", flush=True)
+    lib = dec._lib
+    torch.manual_seed(4)
+    for vocab, hidden in ((32000, 4096), (517, 256), (8, 64)):
+        embed = torch.randn(vocab, hidden, device="cuda").half()
+        hid = torch.zeros(1, hidden, device="cuda").half()
+        nxt = torch.full((1,), -1, dtype=torch.int64, device="cuda")
+        hist = torch.full((16,), -1, dtype=torch.int64, device="cuda")
+        pos = torch.tensor([3], dtype=torch.int32, device="cuda")
+        for trial in range(4):
+            logits = torch.randn(1, vocab, device="cuda").half()
+            if trial == 1:  # a tie: the same maximum at two places
+                logits[0, vocab - 1] = 9.0
+                logits[0, vocab // 3] = 9.0
+            if trial == 2:
+                logits[0, 0] = 11.0
+            lf = logits.float()[0]
+            want = int((lf == lf.max()).nonzero()[0])  # lowest index among equal maxima
+            p0 = int(pos)
+            assert lib.cherryq_decode_argmax_embed_f16(logits.data_ptr(), vocab, embed.data_ptr(), hidden, hid.data_ptr(),
+                                                       nxt.data_ptr(), hist.data_ptr(), hist.numel(), pos.data_ptr(),
+                                                       stream()) == 0
+            torch.cuda.synchronize()
+            assert int(nxt) == want, (vocab, trial)
+            assert int(pos) == p0 + 1 and int(hist[p0]) == want
+            assert torch.equal(hid[0], embed[want])
+    assert lib.cherryq_decode_argmax_embed_f16(None, 8, None, 8, None, None, None, 0, None, None) == -1
