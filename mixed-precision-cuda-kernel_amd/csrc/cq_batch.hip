@@ -21,9 +21,10 @@
 //   costs nothing; per unit the fp32 tile is scaled by the group scale and added to the totals.
 //
 // Cherry rows (dense fp16) run through the same MFMA with operands packed by v_perm_b32.
-// Across workgroups the K splits meet in per-split partial tiles plus one ticket per column tile
-// (agent-scope sc1 stores / loads, no cache-wide fences); the last workgroup adds the partials in
-// split order, so results are deterministic.
+// Across workgroups the K splits meet, for calls with few outputs, in one 64-bit fixed-point atomic
+// per output element (cq_common.cuh), and for larger ones in per-split partial tiles plus one
+// ticket per column tile (agent-scope sc1 stores / loads, no cache-wide fences; the last
+// workgroup adds the partials in split order).  Both are independent of arrival order.
 //
 // Arithmetic contract: csrc/quant_cuda_kernel.cu:797-834 (the reference loops its batch-1 body
 // over the batch rows, re-reading the weights for every row); fp32 accumulation, one rounding.
@@ -50,6 +51,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kBatchRows = 16;        // MFMA M dimension; smaller batches are zero padded
 constexpr int kBatchWaves = 4;        // wavefronts per workgroup
+constexpr int kBatchAtomicOutputs = 8 * 14336;  // calls with at most this many outputs use the atomic split-K epilogue
 constexpr int kBatchMaxSplits = 8;    // bounds the partial-tile scratch and the last workgroup's reads
 constexpr uint32_t kRsrcFlagsB = 0x00020000u;
 constexpr uint32_t kOobB = 0x80000000u;
@@ -288,8 +290,8 @@ __global__ __launch_bounds__(64 * kBatchWaves) __attribute__((amdgpu_waves_per_e
     const uint8_t *__restrict__ qweight, const __half *__restrict__ cherry_weight,
     const __half *__restrict__ scales, __half *__restrict__ mul, const uint4 *__restrict__ xa,
     const float *__restrict__ rowsum, const int *__restrict__ rowshift, float *__restrict__ partial,
-    unsigned *__restrict__ tickets, int B, int K, int N, int C, int G, int accumulate, Plan plan,
-    int units_per_wave) {
+    unsigned *__restrict__ tickets, unsigned long long *__restrict__ acc_words, int atomic_epilogue, int B, int K,
+    int N, int C, int G, int accumulate, Plan plan, int units_per_wave) {
     __shared__ float s_red[kBatchWaves][kBatchRows][kTileCols];  // 64 KB
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -355,6 +357,16 @@ __global__ __launch_bounds__(64 * kBatchWaves) __attribute__((amdgpu_waves_per_e
     // per output element, as in the batch-1 kernel, is slower here: 16 rows make 16x the atomics.)
     // Partials travel as agent-scope sc1 stores / loads, no cache-wide fences; see cq_common.cuh.
     CQB_STAMP(2);
+    if (atomic_epilogue) {
+        // few enough outputs: one 64-bit fixed-point atomic per output element, as in the batch-1
+        // kernel (order-independent, leaves the words zero), instead of partial tiles + ticket
+        float v2[kBatchRows][1];
+#pragma unroll
+        for (int b = 0; b < kBatchRows; b++) v2[b][0] = vals[b];
+        splitk_finish<__half, kBatchRows, 1>(v2, B, N, n, active, plan.splits, acc_words, mul, accumulate);
+        CQB_STAMP(4);
+        return;
+    }
     if (plan.splits > 1) {
         if (active)
 #pragma unroll
@@ -433,20 +445,33 @@ static hipError_t launch_batch_bits(const __half *vec, const uint8_t *qweight, c
     float *partial = reinterpret_cast<float *>(base + ws.partial);
     unsigned *tickets = reinterpret_cast<unsigned *>(reinterpret_cast<char *>(workspace) + ws.tickets);
     const Plan unit_plan = make_plan(K, N, C, 1, kUnitK);
-    // units per wave: one if the split count then fits the partial workspace (every wave's loads
-    // go out at once and the kernel is one memory latency deep); more only for very long K, or
-    // when the grid would otherwise exceed ~4 workgroups per CU (less split-K traffic)
-    int upv = 1;
-    while (ceil_div(unit_plan.units_total, kBatchWaves * upv) > kBatchMaxSplits) upv++;
-    while (upv < 8 && unit_plan.tiles * ceil_div(unit_plan.units_total, kBatchWaves * (upv + 1)) >= 1024) upv++;
-    const Plan plan = make_plan(K, N, C, kBatchWaves * upv, kUnitK);
     for (int b0 = 0; b0 < B; b0 += kBatchRows) {
         const int nb = min(kBatchRows, B - b0);
+        // Split-K epilogue.  Up to ~115k outputs (8 rows of a 13B MLP layer, 16 rows of a 5120-wide
+        // one): one fixed-point atomic per output element, as in the batch-1 kernel (measured
+        // 5-25 % faster there than the alternative, and up to 15 % slower above).  More outputs:
+        // per-split partial tiles + a ticket, the last workgroup of a tile adds them.
+        const int atomic_epilogue = (long long)nb * N <= kBatchAtomicOutputs;
+        // Units per wave.  Atomic epilogue: as few as keep the grid within one resident round
+        // (two workgroups per CU), so that nearly every wave's loads go out at once.  Partial
+        // tiles: as few as keep the split count within the partial workspace; more only when the
+        // grid would otherwise exceed ~4 workgroups per CU (less split-K traffic).
+        int upv = 1;
+        if (atomic_epilogue) {
+            while (upv < 64 && (unit_plan.tiles * ceil_div(unit_plan.units_total, kBatchWaves * upv) > 512 ||
+                                ceil_div(unit_plan.units_total, kBatchWaves * upv) > kMaxSplits))
+                upv++;
+        } else {
+            while (ceil_div(unit_plan.units_total, kBatchWaves * upv) > kBatchMaxSplits) upv++;
+            while (upv < 8 && unit_plan.tiles * ceil_div(unit_plan.units_total, kBatchWaves * (upv + 1)) >= 1024) upv++;
+        }
+        const Plan plan = make_plan(K, N, C, kBatchWaves * upv, kUnitK);
         hipLaunchKernelGGL(batch_prep_kernel<BITS>, dim3(plan.units_total), dim3(256), 0, stream, vec + (size_t)b0 * K,
                            cherry_indices, xa, rowsum, rowshift, nb, K, C, plan.units_normal);
         hipLaunchKernelGGL(batch_kernel<BITS>, dim3(plan.tiles * plan.splits), dim3(64 * kBatchWaves), 0, stream,
                            qweight, cherry_weight, scales, mul + (size_t)b0 * N, xa, rowsum, rowshift, partial, tickets,
-                           nb, K, N, C, G, accumulate, plan, upv);
+                           reinterpret_cast<unsigned long long *>(workspace), atomic_epilogue, nb, K, N, C, G,
+                           accumulate, plan, upv);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
