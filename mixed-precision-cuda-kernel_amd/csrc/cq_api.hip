@@ -34,13 +34,22 @@ size_t workspace_bytes(int B, int K, int N, int C) {
         size_t b2 = batch_workspace(K, N, C).workspace_total;
         if (b2 > bytes) bytes = b2;
     }
+    if (B >= kGemmMinRows) {
+        size_t b3 = gemm_plan(B, K, N, C).workspace_bytes;
+        if (b3 > bytes) bytes = b3;
+    }
     return bytes;
 }
 
 // uninitialised: partial tiles and prepared activations of the matrix-core path
 size_t scratch_bytes(int B, int K, int N, int C) {
     clamp_dims(B, K, N, C);
-    return B >= 2 ? batch_workspace(K, N, C).scratch_total : 0;
+    size_t bytes = B >= 2 ? batch_workspace(K, N, C).scratch_total : 0;
+    if (B >= kGemmMinRows) {
+        size_t b3 = gemm_plan(B, K, N, C).scratch_bytes;
+        if (b3 > bytes) bytes = b3;
+    }
+    return bytes;
 }
 
 static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
@@ -83,6 +92,8 @@ static int matmul_f16(const void *vec, const uint8_t *qweight, const void *cherr
     hipError_t e;
     if (!force_generic() && B == 1 && matvec_supported(BITS, B, K, N, C, G)) {
         e = launch_matvec(BITS, x, qweight, cw, cherry_indices, sc, y, K, N, C, G, accumulate, workspace, s);
+    } else if (!force_generic() && B >= kGemmMinRows && gemm_supported(BITS, B, K, N, C, G)) {
+        e = launch_gemm(BITS, x, qweight, cw, cherry_indices, sc, y, B, K, N, C, G, accumulate, workspace, scratch, s);
     } else if (!force_generic() && batch_supported(BITS, B, K, N, C, G)) {
         e = launch_batch(BITS, x, qweight, cw, cherry_indices, sc, y, B, K, N, C, G, accumulate, workspace, scratch, s);
     } else {

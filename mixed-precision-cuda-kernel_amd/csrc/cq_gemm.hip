@@ -1,0 +1,456 @@
+// Prompt-sized batches (more than 16 rows): fused dequantise + GEMM on the gfx950 matrix cores.
+//
+//   Y[M, N] (+)= Xn[M, Kn] * Wn[Kn, N] + Xc[M, C] * Wc[C, N]
+//
+// Wn are the packed codes, Wc the fp16 cherry rows; Xn / Xc are the activations gathered at the
+// normal / cherry input channels.  A workgroup (4 wavefronts, 2 x 2) owns a 128 x 128 output tile
+// and walks K in steps of 64 positions.  Per step
+//   * the weights of the step (64 positions x 128 columns, 4 KB at 4 bits) are loaded as one
+//     dword per byte row and thread (4 adjacent columns; 8 positions = 4 or 3 byte rows),
+//     dequantised in registers to exactly the fp16 values of the dense weight
+//     (llama/qlinear.py:120-162: RN16((u - c_b) * s)) and written to LDS in the matrix cores'
+//     operand order: v_perm_b32 interleaves a column's bytes of two byte rows, a mask cuts out a
+//     pair of codes, OR-ing 0x6400 into each half makes them the fp16 numbers 1024 + u * 2^p,
+//     one packed fp16 fma turns that into u - c_b (exact) and one packed multiply applies the
+//     group scale (one rounding, the reference's);
+//   * the activations of the step (128 rows x 64 positions) come from a compacted copy made by a
+//     small kernel in front (gathered around the cherry channels, zero padded to whole tiles, in
+//     the same position order inside every group of 8 as the code pairs above);
+//   * every wavefront runs 16 v_mfma_f32_32x32x16_f16 on its 64 x 64 quarter, operands read from
+//     LDS with ds_read_b128 (rows padded to 144 bytes: conflict free).
+// LDS is double buffered: the next step's global loads are in flight during the MFMAs, its
+// dequantisation follows them, one barrier per step.  Cherry rows are further steps whose B
+// operands are the fp16 rows themselves.
+//
+// K splits (when the tiles alone would leave CUs idle) meet in per-split fp32 partial tiles and
+// one ticket per output tile; the last workgroup adds the partials in split order, so the result
+// does not depend on arrival order.
+//
+// Arithmetic contract: csrc/quant_cuda_kernel.cu:797-834 (the reference loops its batch-1 body
+// over the rows); here fp16 weights as the dense path's (qlinear.py:183-195), fp32 accumulation,
+// one final rounding.
+#include "cq_common.cuh"
+#include "cq_kernels.h"
+
+namespace cq {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kGemmTM = 128, kGemmTN = 128, kGemmTK = 64;
+constexpr int kGemmPitch = kGemmTK * 2 + 16;               // bytes per LDS row
+constexpr int kGemmStageBytes = kGemmTM * kGemmPitch;      // one operand, one stage
+constexpr int kGemmLdsBytes = 4 * kGemmStageBytes;         // A and B, two stages
+constexpr int kGemmMaxSplits = 8;
+constexpr uint32_t kRsrcFlagsG = 0x00020000u;
+constexpr uint32_t kOobG = 0x80000000u;
+
+// position order inside a group of 8 and the bit position of each code's field in its 16-bit
+// half, as produced by the perm / mask sequence in dequant_step
+//   4-bit: ord = {0, 2, 1, 3, 4, 6, 5, 7}   p = {0, 0, 4, 4, 0, 0, 4, 4}
+//   3-bit: ord = {0, 3, 1, 4, 5, 6, 2, 7}   p = {0, 1, 3, 4, 7, 2, 6, 5}
+template <int BITS>
+__host__ __device__ constexpr int gemm_ord(int kk) {
+    return BITS == 4 ? ((kk & 4) | ((kk & 1) << 1) | ((kk >> 1) & 1)) : (int)((0x72654130u >> (4 * kk)) & 7u);
+}
+template <int BITS>
+__host__ __device__ constexpr int gemm_pos(int kk) {
+    return BITS == 4 ? ((kk & 2) ? 4 : 0) : (int)((0x56274310u >> (4 * kk)) & 7u);
+}
+
+GemmPlan gemm_plan(int M, int K, int N, int C) {
+    GemmPlan p;
+    p.mtiles = ceil_div(M, kGemmTM);
+    p.ntiles = ceil_div(N, kGemmTN);
+    p.steps_normal = ceil_div(K - C, kGemmTK);
+    p.steps_total = p.steps_normal + ceil_div(C, kGemmTK);
+    p.Kp = p.steps_total * kGemmTK;
+    p.Mp = p.mtiles * kGemmTM;
+    // K splits: enough workgroups for two per CU, at least 8 steps each
+    int splits = 1;
+    const int tiles = p.mtiles * p.ntiles;
+    while (splits < kGemmMaxSplits && tiles * splits < 512 && p.steps_total / (splits + 1) >= 8) splits++;
+    p.steps_per_split = ceil_div(p.steps_total, splits);
+    p.splits = ceil_div(p.steps_total, p.steps_per_split);
+    // zero-kept workspace: one ticket per output tile
+    p.workspace_bytes = ((size_t)tiles * sizeof(unsigned) + 255) / 256 * 256;
+    // scratch: compacted activations, then the partial tiles
+    p.a_bytes = ((size_t)p.Mp * p.Kp * sizeof(__half) + 255) / 256 * 256;
+    p.partial_bytes = p.splits > 1 ? (size_t)p.splits * tiles * kGemmTM * kGemmTN * sizeof(float) : 0;
+    p.scratch_bytes = p.a_bytes + (p.partial_bytes + 255) / 256 * 256;
+    return p;
+}
+
+// ---- activation compaction -----------------------------------------------------------------------
+// One thread per (row, group of 8 positions): A[row][8 g + kk] = x[row][normal(8 g + ord[kk])] in
+// the normal part, x[row][idx[c]] in the cherry part, 0 in the padding (rows >= M, positions past
+// the end).
+template <int BITS>
+__global__ __launch_bounds__(256) void gemm_prep_kernel(const __half *__restrict__ x,
+                                                        const int16_t *__restrict__ cherry_indices,
+                                                        uint4 *__restrict__ a, int M, int K, int C, int Kp,
+                                                        int groups_normal) {
+    const int g = blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
+    if (g >= Kp / 8) return;
+    const int Kn = K - C;
+    unsigned short h[8];
+#pragma unroll
+    for (int kk = 0; kk < 8; kk++) h[kk] = 0;
+    if (row < M) {
+        const __half *xr = x + (size_t)row * K;
+        if (g < groups_normal) {
+            const int kb = 8 * g;
+            int lows[8];
+            int lo = gather_offset(cherry_indices, C, kb);
+            lows[0] = lo;
+#pragma unroll
+            for (int j = 1; j < 8; j++) {
+                while (lo < C && (int)cherry_indices[lo] - lo <= kb + j) lo++;
+                lows[j] = lo;
+            }
+#pragma unroll
+            for (int kk = 0; kk < 8; kk++) {
+                const int j = gemm_ord<BITS>(kk);
+                if (kb + j < Kn) h[kk] = __half_as_ushort(xr[kb + j + lows[j]]);
+            }
+        } else {
+            const int c0 = (g - groups_normal) * 8;
+#pragma unroll
+            for (int kk = 0; kk < 8; kk++)
+                if (c0 + kk < C) h[kk] = __half_as_ushort(xr[(int)cherry_indices[c0 + kk]]);
+        }
+    }
+    a[(size_t)row * (Kp / 8) + g] =
+        make_uint4(h[0] | h[1] << 16, h[2] | h[3] << 16, h[4] | h[5] << 16, h[6] | h[7] << 16);
+}
+
+// ---- main kernel ---------------------------------------------------------------------------------
+// What a thread holds of one K step between the global loads and the LDS writes.
+struct GemmStepRegs {
+    uint32_t w[4];  // 4 (3) byte rows x 4 columns
+    uint32_t sc0, sc1;  // the 4 columns' group scales
+    u32x4 a[4];     // 4 rows x 8 positions of activations
+};
+struct GemmCherryRegs {
+    u32x2 w[8];     // 8 cherry rows x 4 columns of fp16
+    u32x4 a[4];
+};
+
+// Packed fp16 constants per output dword d (low half: kk = 2 d, high half: kk = 2 d + 1).  With
+// x = 1024 + u * 2^p:  x * 2^-p - 1024 * 2^-p = u, then u - c_b; every intermediate is exact.  When
+// both fields sit at p >= 1 the constant 1024 * 2^-p + c_b is itself an fp16 number and one fma does
+// it; 1024 + c_b is not, so a dword with a field at p = 0 takes the subtraction of c_b separately.
+template <int BITS>
+struct GemmConst {
+    static constexpr float kGrid = BITS == 4 ? 7.5f : 3.5f;
+    static __host__ __device__ constexpr bool fused(int d) {
+        return gemm_pos<BITS>(2 * d) >= 1 && gemm_pos<BITS>(2 * d + 1) >= 1;
+    }
+    static __device__ __forceinline__ half2_t mul(int d) {
+        return (half2_t){(_Float16)(1.0f / (float)(1 << gemm_pos<BITS>(2 * d))),
+                         (_Float16)(1.0f / (float)(1 << gemm_pos<BITS>(2 * d + 1)))};
+    }
+    static __device__ __forceinline__ half2_t add(int d) {
+        const float c = fused(d) ? kGrid : 0.f;
+        return (half2_t){(_Float16)(-(1024.0f / (float)(1 << gemm_pos<BITS>(2 * d)) + c)),
+                         (_Float16)(-(1024.0f / (float)(1 << gemm_pos<BITS>(2 * d + 1)) + c))};
+    }
+};
+
+template <int BITS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_kernel(
+    const uint8_t *__restrict__ qweight, const __half *__restrict__ cherry_weight,
+    const __half *__restrict__ scales, __half *__restrict__ out, const __half *__restrict__ a_compact,
+    float *__restrict__ partial, unsigned *__restrict__ tickets, int M, int K, int N, int C, int G,
+    int accumulate, GemmPlan plan) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char s_lds[];
+    unsigned char *const s_a = s_lds;                         // [2][128][pitch]
+    unsigned char *const s_b = s_lds + 2 * kGemmStageBytes;   // [2][128][pitch]
+
+    constexpr int R = BITS == 4 ? 4 : 3;  // byte rows per 8 positions
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int ntile = blockIdx.x % plan.ntiles, mtile = blockIdx.x / plan.ntiles, split = blockIdx.y;
+    const int m0 = mtile * kGemmTM, n0 = ntile * kGemmTN;
+    const int Kn = K - C;
+    // staging roles: B -- column quad cq, position group kg; A -- row ar (+32 i), chunk ac
+    const int cq = tid & 31, kg = tid >> 5;
+    const int ar = tid >> 3, ac = tid & 7;
+    const bool col_ok = n0 + 4 * cq < N;
+
+    const __amdgpu_buffer_rsrc_t rw =
+        __builtin_amdgcn_make_buffer_rsrc((void *)qweight, 0, Kn / 8 * BITS * N, kRsrcFlagsG);
+    const __amdgpu_buffer_rsrc_t rs =
+        __builtin_amdgcn_make_buffer_rsrc((void *)scales, 0, ceil_div(Kn, G) * N * 2, kRsrcFlagsG);
+    const __amdgpu_buffer_rsrc_t rc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)cherry_weight, 0, C * N * 2, kRsrcFlagsG);
+    const u32x4 *arow = reinterpret_cast<const u32x4 *>(a_compact) + (size_t)(m0 + ar) * (plan.Kp / 8) + ac;
+
+    auto load_a = [=](u32x4 (&av)[4], int st) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) av[i] = arow[(size_t)(32 * i) * (plan.Kp / 8) + st * 8];
+    };
+    auto store_a = [=](const u32x4 (&av)[4], int buf) {
+        unsigned char *sa = s_a + buf * kGemmStageBytes;
+#pragma unroll
+        for (int i = 0; i < 4; i++) *reinterpret_cast<u32x4 *>(sa + (ar + 32 * i) * kGemmPitch + ac * 16) = av[i];
+    };
+    auto load_step = [=](GemmStepRegs &r, int st) {
+        load_a(r.a, st);
+        const uint32_t woff = col_ok ? (uint32_t)((st * 8 + kg) * R * N + n0 + 4 * cq) : kOobG;
+#pragma unroll
+        for (int i = 0; i < R; i++) r.w[i] = __builtin_amdgcn_raw_buffer_load_b32(rw, woff + (uint32_t)(i * N), 0, 0);
+        const int g = (st * kGemmTK) / G;
+        const uint32_t soff = col_ok ? (uint32_t)(g * N + n0 + 4 * cq) * 2u : kOobG;
+        const u32x2 sv = __builtin_amdgcn_raw_buffer_load_b64(rs, soff, 0, 0);
+        r.sc0 = sv[0];
+        r.sc1 = sv[1];
+    };
+    auto load_cherry = [=](GemmCherryRegs &r, int st) {
+        load_a(r.a, st);
+        const int c0 = (st - plan.steps_normal) * kGemmTK + 8 * kg;
+        const uint32_t coff = col_ok ? (uint32_t)(c0 * N + n0 + 4 * cq) * 2u : kOobG;
+#pragma unroll
+        for (int i = 0; i < 8; i++) r.w[i] = __builtin_amdgcn_raw_buffer_load_b64(rc, coff + (uint32_t)(i * N * 2), 0, 0);
+    };
+    auto store_cherry = [=](const GemmCherryRegs &r, int buf) {
+        store_a(r.a, buf);
+        unsigned char *sb = s_b + buf * kGemmStageBytes;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;  // (row r half, row r + 1 half)
+            u32x4 o;
+#pragma unroll
+            for (int d = 0; d < 4; d++) o[d] = __builtin_amdgcn_perm(r.w[2 * d + 1][j >> 1], r.w[2 * d][j >> 1], sel);
+            *reinterpret_cast<u32x4 *>(sb + (4 * cq + j) * kGemmPitch + kg * 16) = o;
+        }
+    };
+
+    // registers -> LDS stage `buf`
+    auto store_step = [=](const GemmStepRegs &r, int buf) {
+        store_a(r.a, buf);
+        unsigned char *sb = s_b + buf * kGemmStageBytes;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint32_t f[4];
+            if (BITS == 4) {
+                const uint32_t sel = 0x0c000c00u | (uint32_t)(j << 16) | (uint32_t)(4 + j);
+                const uint32_t p0 = __builtin_amdgcn_perm(r.w[0], r.w[1], sel);
+                const uint32_t p1 = __builtin_amdgcn_perm(r.w[2], r.w[3], sel);
+                f[0] = p0 & 0x000f000fu;
+                f[1] = p0 & 0x00f000f0u;
+                f[2] = p1 & 0x000f000fu;
+                f[3] = p1 & 0x00f000f0u;
+            } else {
+                const uint32_t sel = 0x0c000000u | (uint32_t)(j << 16) | (uint32_t)(j << 8) | (uint32_t)(4 + j);
+                const uint32_t p1 = __builtin_amdgcn_perm(r.w[0], r.w[1], sel);
+                const uint32_t p2 = __builtin_amdgcn_perm(r.w[1], r.w[2], sel);
+                f[0] = p1 & 0x000e0007u;
+                f[1] = p1 & 0x00700038u;
+                f[2] = p2 & 0x001c0380u;
+                f[3] = (p1 & 0x000001c0u) | (p2 & 0x00e00000u);
+            }
+            const uint32_t sw = j < 2 ? r.sc0 : r.sc1;
+            const uint32_t s2 = (j & 1) ? __builtin_amdgcn_perm(sw, sw, 0x03020302u)
+                                        : __builtin_amdgcn_perm(sw, sw, 0x01000100u);
+            const half2_t sv = __builtin_bit_cast(half2_t, s2);
+            u32x4 o;
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                const half2_t x = __builtin_bit_cast(half2_t, f[d] | 0x64006400u);
+                half2_t y = x * GemmConst<BITS>::mul(d) + GemmConst<BITS>::add(d);
+                if (!GemmConst<BITS>::fused(d))
+                    y = y - (half2_t){(_Float16)GemmConst<BITS>::kGrid, (_Float16)GemmConst<BITS>::kGrid};
+                o[d] = __builtin_bit_cast(uint32_t, y * sv);
+            }
+            *reinterpret_cast<u32x4 *>(sb + (4 * cq + j) * kGemmPitch + kg * 16) = o;
+        }
+    };
+
+    float16_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+
+    const int st_begin = split * plan.steps_per_split;
+    const int st_end = min(st_begin + plan.steps_per_split, plan.steps_total);
+    const int frag_row = lane & 31, frag_k = (lane >> 5) * 16;  // byte offset of the lane's 8 positions
+
+    const unsigned char *sa0 = s_a + (wm * 64 + frag_row) * kGemmPitch + frag_k;
+    const unsigned char *sb0 = s_b + (wn * 64 + frag_row) * kGemmPitch + frag_k;
+    auto compute = [&](int buf) {
+        const unsigned char *sa = sa0 + buf * kGemmStageBytes;
+        const unsigned char *sb = sb0 + buf * kGemmStageBytes;
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            half8_t af[2], bf[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                af[i] = *reinterpret_cast<const half8_t *>(sa + i * 32 * kGemmPitch + ks * 32);
+                bf[i] = *reinterpret_cast<const half8_t *>(sb + i * 32 * kGemmPitch + ks * 32);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+    };
+    // Packed steps.  Ring of kRing register sets: the global loads of step st + kRing - 1 are issued
+    // while step st is computed, so a load has kRing - 2 whole steps to arrive before its
+    // dequantisation.
+    {
+        constexpr int kRing = 4;
+        const int n_end = min(st_end, plan.steps_normal);
+        GemmStepRegs regs[kRing];
+#pragma unroll
+        for (int i = 0; i < kRing - 1; i++)
+            if (st_begin + i < n_end) load_step(regs[i], st_begin + i);
+        if (st_begin < n_end) store_step(regs[0], 0);
+        __syncthreads();
+        for (int base = st_begin; base < n_end; base += kRing) {
+#pragma unroll
+            for (int r = 0; r < kRing; r++) {
+                const int st = base + r;
+                if (st < n_end) {  // uniform
+                    const int buf = r & 1;
+                    if (st + kRing - 1 < n_end) load_step(regs[(r + kRing - 1) % kRing], st + kRing - 1);
+                    compute(buf);
+                    if (st + 1 < n_end) store_step(regs[(r + 1) % kRing], buf ^ 1);
+                    __syncthreads();
+                }
+            }
+        }
+    }
+    // Cherry steps (one or two per call): plain load, stage, compute.
+    for (int st = max(st_begin, plan.steps_normal); st < st_end; st++) {
+        GemmCherryRegs cr;
+        load_cherry(cr, st);
+        store_cherry(cr, 0);
+        __syncthreads();
+        compute(0);
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane holds column (lane & 31), rows 8 blk + 4 (lane >> 5) + r of each 32 x 32 tile
+    const int col_l = lane & 31, row_l = 4 * (lane >> 5);
+    if (plan.splits > 1) {
+        // partial tiles in the accumulators' own order: element q of a lane at [q][lane], so that
+        // every store and load instruction covers 256 contiguous bytes
+        const size_t tile_elems = (size_t)kGemmTM * kGemmTN;
+        const size_t tiles = (size_t)plan.mtiles * plan.ntiles;
+        float *mine = partial + ((size_t)split * tiles + blockIdx.x) * tile_elems + wave * 4096 + lane;
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int e = 0; e < 16; e++)
+                    __hip_atomic_store(mine + ((i * 2 + j) * 16 + e) * 64, acc[i][j][e], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+        int *s_last = reinterpret_cast<int *>(s_lds);  // the stages have been consumed
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        if (tid == 0) {
+            unsigned old = __hip_atomic_fetch_add(&tickets[blockIdx.x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *s_last = (old == (unsigned)(plan.splits - 1));
+        }
+        __syncthreads();
+        if (!*s_last) return;
+        if (tid == 0) __hip_atomic_store(&tickets[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+        for (int s = 0; s < plan.splits; s++) {  // split order: independent of arrival order
+            const float *theirs = partial + ((size_t)s * tiles + blockIdx.x) * tile_elems + wave * 4096 + lane;
+            float v[64];
+#pragma unroll
+            for (int q = 0; q < 64; q++)
+                v[q] = __hip_atomic_load(theirs + q * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+#pragma unroll
+                    for (int e = 0; e < 16; e++) acc[i][j][e] += v[(i * 2 + j) * 16 + e];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int n = n0 + wn * 64 + j * 32 + col_l;
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + row_l + (e & 3);
+                if (n < N && m < M) {
+                    __half *o = out + (size_t)m * N + n;
+                    float v = acc[i][j][e];
+                    if (accumulate) v += __half2float(*o);
+                    *o = __float2half_rn(v);
+                }
+            }
+        }
+}
+
+bool gemm_supported(int bits, int M, int K, int N, int C, int G) {
+    (void)bits;
+    if (M < 2) return false;
+    if (G % kGemmTK) return false;  // a step must not straddle a group
+    if (K - C <= 0) return false;
+    const long long wbytes = (long long)(K - C) / 8 * 4 * N;
+    const long long cbytes = (long long)C * N * 2;
+    const long long sbytes = (long long)ceil_div(K - C, G) * N * 2;
+    if (wbytes >= 0x7fff0000ll || cbytes >= 0x7fff0000ll || sbytes >= 0x7fff0000ll) return false;
+    return true;
+}
+
+template <int BITS>
+static hipError_t launch_gemm_bits(const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
+                                   const int16_t *cherry_indices, const __half *scales, __half *mul, int M, int K,
+                                   int N, int C, int G, int accumulate, void *workspace, void *scratch,
+                                   hipStream_t stream) {
+    const GemmPlan plan = gemm_plan(M, K, N, C);
+    __half *a = reinterpret_cast<__half *>(scratch);
+    float *partial = reinterpret_cast<float *>(reinterpret_cast<char *>(scratch) + plan.a_bytes);
+    unsigned *tickets = reinterpret_cast<unsigned *>(workspace);
+    // more than 64 KB of LDS per workgroup has to be requested once per device
+    static bool lds_set[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= 64 || !lds_set[dev]) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<BITS>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes);
+        if (e != hipSuccess) return e;
+        if (dev >= 0 && dev < 64) lds_set[dev] = true;
+    }
+    hipLaunchKernelGGL(gemm_prep_kernel<BITS>, dim3(ceil_div(plan.Kp / 8, 256), plan.Mp), dim3(256), 0, stream, vec,
+                       cherry_indices, reinterpret_cast<uint4 *>(a), M, K, C, plan.Kp, plan.steps_normal * 8);
+    hipLaunchKernelGGL(gemm_kernel<BITS>, dim3(plan.mtiles * plan.ntiles, plan.splits), dim3(256), kGemmLdsBytes,
+                       stream, qweight, cherry_weight, scales, mul, a, partial, tickets, M, K, N, C, G, accumulate,
+                       plan);
+    return hipGetLastError();
+}
+
+hipError_t launch_gemm(int bits, const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
+                       const int16_t *cherry_indices, const __half *scales, __half *mul, int M, int K, int N, int C,
+                       int G, int accumulate, void *workspace, void *scratch, hipStream_t stream) {
+    if (bits == 4)
+        return launch_gemm_bits<4>(vec, qweight, cherry_weight, cherry_indices, scales, mul, M, K, N, C, G, accumulate,
+                                   workspace, scratch, stream);
+    return launch_gemm_bits<3>(vec, qweight, cherry_weight, cherry_indices, scales, mul, M, K, N, C, G, accumulate,
+                               workspace, scratch, stream);
+}
+
+}  // namespace cq

@@ -69,6 +69,23 @@ hipError_t launch_batch(int bits, const __half *vec, const uint8_t *qweight, con
                         int C, int G, int accumulate, void *workspace, void *scratch, hipStream_t stream);
 size_t scratch_bytes(int B, int K, int N, int C);
 
+// cq_gemm.hip: more than 16 rows (prompt processing) -- dequantise into LDS, fp16 MFMA tiles.
+struct GemmPlan {
+    int mtiles, ntiles;               // 128 x 128 output tiles
+    int steps_normal, steps_total;    // K steps of 64 positions: packed part, then the cherry rows
+    int Kp, Mp;                       // padded sizes of the compacted activation copy
+    int splits, steps_per_split;      // K splits (grid.y)
+    size_t workspace_bytes;           // zero-kept: one ticket per output tile
+    size_t a_bytes, partial_bytes;    // scratch: compacted activations, then the per-split partial tiles
+    size_t scratch_bytes;
+};
+constexpr int kGemmMinRows = 17;  // fewer rows go through the 16-row kernel
+GemmPlan gemm_plan(int M, int K, int N, int C);
+bool gemm_supported(int bits, int M, int K, int N, int C, int G);
+hipError_t launch_gemm(int bits, const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
+                       const int16_t *cherry_indices, const __half *scales, __half *mul, int M, int K, int N, int C,
+                       int G, int accumulate, void *workspace, void *scratch, hipStream_t stream);
+
 // cq_pack.hip: dense fp16 weight -> packed buffers on the device.
 hipError_t launch_pack(int bits, const __half *w, const int16_t *idx, uint8_t *qweight, __half *scales,
                        __half *cherry_weight, int K, int N, int C, int G, hipStream_t stream);
