@@ -57,9 +57,12 @@ const char *cherryq_status_string(int status);
  *   and one arrival ticket per 256-column tile.  At least cherryq_workspace_bytes() bytes,
  *   256-byte aligned.  It must be all zero before the first call; every call leaves it all zero
  *   again, whatever the shapes of earlier calls were.
- * scratch: uninitialised memory for the batched path (batch >= 2): per-split partial tiles and
+ * scratch: uninitialised memory for the batched paths (batch >= 2): per-split partial tiles and
  *   the activations laid out in matrix-core operand order.  At least cherryq_scratch_bytes()
  *   bytes (0 for batch 1, then it may be NULL), 256-byte aligned.
+ * Both sizes depend on the batch: up to 16 rows run in the small-batch kernel, more (prompt
+ * processing) in the tiled GEMM kernel, whose compacted copy of the activations and partial
+ * tiles grow with the number of rows.  Size the buffers for the largest batch that will be passed.
  * Calls that may overlap in time (different streams) must use different workspace and scratch.
  */
 size_t cherryq_workspace_bytes(int batch, int in_features, int out_features, int num_cherries);

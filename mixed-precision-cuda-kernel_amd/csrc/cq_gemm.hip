@@ -18,9 +18,10 @@
 //     the same position order inside every group of 8 as the code pairs above);
 //   * every wavefront runs 16 v_mfma_f32_32x32x16_f16 on its 64 x 64 quarter, operands read from
 //     LDS with ds_read_b128 (rows padded to 144 bytes: conflict free).
-// LDS is double buffered: the next step's global loads are in flight during the MFMAs, its
-// dequantisation follows them, one barrier per step.  Cherry rows are further steps whose B
-// operands are the fp16 rows themselves.
+// LDS is double buffered and a ring of four register sets keeps the global loads three steps
+// ahead of their dequantisation; one barrier per step.  Cherry rows are further steps whose B
+// operands are the fp16 rows themselves.  The kernel is bound by LDS traffic (each 32 x 32 x 16
+// MFMA needs one 1 KB operand read on average), not by the matrix cores.
 //
 // K splits (when the tiles alone would leave CUs idle) meet in per-split fp32 partial tiles and
 // one ticket per output tile; the last workgroup adds the partials in split order, so the result
@@ -40,11 +41,15 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kGemmTM = 128, kGemmTN = 128, kGemmTK = 64;
+// Output tile: 128 rows x 64 * WN columns, WN wave columns (2 x WN wavefronts); the library
+// instantiates WN = 2.
+constexpr int kGemmTM = 128, kGemmTK = 64;
 constexpr int kGemmPitch = kGemmTK * 2 + 16;               // bytes per LDS row
-constexpr int kGemmStageBytes = kGemmTM * kGemmPitch;      // one operand, one stage
-constexpr int kGemmLdsBytes = 4 * kGemmStageBytes;         // A and B, two stages
+constexpr int kGemmStageA = kGemmTM * kGemmPitch;          // activations, one stage
+constexpr int gemm_stage_b(int wn) { return 64 * wn * kGemmPitch; }
+constexpr int gemm_lds_bytes(int wn) { return 2 * (kGemmStageA + gemm_stage_b(wn)); }
 constexpr int kGemmMaxSplits = 8;
+constexpr int kGemmResidentWgs = 512;  // 256 CUs x 2 workgroups (LDS: 72 KB each)
 constexpr uint32_t kRsrcFlagsG = 0x00020000u;
 constexpr uint32_t kOobG = 0x80000000u;
 
@@ -64,7 +69,8 @@ __host__ __device__ constexpr int gemm_pos(int kk) {
 GemmPlan gemm_plan(int M, int K, int N, int C) {
     GemmPlan p;
     p.mtiles = ceil_div(M, kGemmTM);
-    p.ntiles = ceil_div(N, kGemmTN);
+    p.wn = 2;  // 256-column tiles (wn = 4, one workgroup of eight waves per CU) measured 0-10 % slower
+    p.ntiles = ceil_div(N, 64 * p.wn);
     p.steps_normal = ceil_div(K - C, kGemmTK);
     p.steps_total = p.steps_normal + ceil_div(C, kGemmTK);
     p.Kp = p.steps_total * kGemmTK;
@@ -72,14 +78,17 @@ GemmPlan gemm_plan(int M, int K, int N, int C) {
     // K splits: enough workgroups for two per CU, at least 8 steps each
     int splits = 1;
     const int tiles = p.mtiles * p.ntiles;
-    while (splits < kGemmMaxSplits && tiles * splits < 512 && p.steps_total / (splits + 1) >= 8) splits++;
+    // as many splits as still give ONE resident round of workgroups (two per CU; a few workgroups
+    // more start a second round and double the time), at least 8 steps each
+    while (splits < kGemmMaxSplits && tiles * (splits + 1) <= kGemmResidentWgs && p.steps_total / (splits + 1) >= 8)
+        splits++;
     p.steps_per_split = ceil_div(p.steps_total, splits);
     p.splits = ceil_div(p.steps_total, p.steps_per_split);
     // zero-kept workspace: one ticket per output tile
     p.workspace_bytes = ((size_t)tiles * sizeof(unsigned) + 255) / 256 * 256;
     // scratch: compacted activations, then the partial tiles
     p.a_bytes = ((size_t)p.Mp * p.Kp * sizeof(__half) + 255) / 256 * 256;
-    p.partial_bytes = p.splits > 1 ? (size_t)p.splits * tiles * kGemmTM * kGemmTN * sizeof(float) : 0;
+    p.partial_bytes = p.splits > 1 ? (size_t)p.splits * tiles * kGemmTM * 64 * p.wn * sizeof(float) : 0;
     p.scratch_bytes = p.a_bytes + (p.partial_bytes + 255) / 256 * 256;
     return p;
 }
@@ -132,7 +141,7 @@ __global__ __launch_bounds__(256) void gemm_prep_kernel(const __half *__restrict
 struct GemmStepRegs {
     uint32_t w[4];  // 4 (3) byte rows x 4 columns
     uint32_t sc0, sc1;  // the 4 columns' group scales
-    u32x4 a[4];     // 4 rows x 8 positions of activations
+    u32x4 a[4];     // 8 / WN rows x 8 positions of activations
 };
 struct GemmCherryRegs {
     u32x2 w[8];     // 8 cherry rows x 4 columns of fp16
@@ -160,24 +169,29 @@ struct GemmConst {
     }
 };
 
-template <int BITS>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_kernel(
+template <int BITS, int WN>
+__global__ __launch_bounds__(128 * WN) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_kernel(
     const uint8_t *__restrict__ qweight, const __half *__restrict__ cherry_weight,
     const __half *__restrict__ scales, __half *__restrict__ out, const __half *__restrict__ a_compact,
     float *__restrict__ partial, unsigned *__restrict__ tickets, int M, int K, int N, int C, int G,
     int accumulate, GemmPlan plan) {
     extern __shared__ __attribute__((aligned(16))) unsigned char s_lds[];
+    constexpr int kStageB = gemm_stage_b(WN);
+    constexpr int TN = 64 * WN;
+    constexpr int APT = 8 / WN;                               // activation chunks per thread and step
     unsigned char *const s_a = s_lds;                         // [2][128][pitch]
-    unsigned char *const s_b = s_lds + 2 * kGemmStageBytes;   // [2][128][pitch]
+    unsigned char *const s_b = s_lds + 2 * kGemmStageA;       // [2][TN][pitch]
 
     constexpr int R = BITS == 4 ? 4 : 3;  // byte rows per 8 positions
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
     const int ntile = blockIdx.x % plan.ntiles, mtile = blockIdx.x / plan.ntiles, split = blockIdx.y;
-    const int m0 = mtile * kGemmTM, n0 = ntile * kGemmTN;
+    const int m0 = mtile * kGemmTM, n0 = ntile * TN;
     const int Kn = K - C;
     // staging roles: B -- column quad cq, position group kg; A -- row ar (+32 i), chunk ac
-    const int cq = tid & 31, kg = tid >> 5;
+    // (16 consecutive lanes = 4 column quads x 4 position groups: their 16-byte LDS writes, 144
+    // bytes apart per row, then fall into 16 different bank groups)
+    const int cq = (wave % WN) * 16 + (lane >> 4) * 4 + (lane & 3), kg = (wave / WN) * 4 + ((lane >> 2) & 3);
     const int ar = tid >> 3, ac = tid & 7;
     const bool col_ok = n0 + 4 * cq < N;
 
@@ -191,12 +205,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     auto load_a = [=](u32x4 (&av)[4], int st) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) av[i] = arow[(size_t)(32 * i) * (plan.Kp / 8) + st * 8];
+        for (int i = 0; i < APT; i++) av[i] = arow[(size_t)(16 * WN * i) * (plan.Kp / 8) + st * 8];
     };
     auto store_a = [=](const u32x4 (&av)[4], int buf) {
-        unsigned char *sa = s_a + buf * kGemmStageBytes;
+        unsigned char *sa = s_a + buf * kGemmStageA;
 #pragma unroll
-        for (int i = 0; i < 4; i++) *reinterpret_cast<u32x4 *>(sa + (ar + 32 * i) * kGemmPitch + ac * 16) = av[i];
+        for (int i = 0; i < APT; i++)
+            *reinterpret_cast<u32x4 *>(sa + (ar + 16 * WN * i) * kGemmPitch + ac * 16) = av[i];
     };
     auto load_step = [=](GemmStepRegs &r, int st) {
         load_a(r.a, st);
@@ -218,7 +233,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     };
     auto store_cherry = [=](const GemmCherryRegs &r, int buf) {
         store_a(r.a, buf);
-        unsigned char *sb = s_b + buf * kGemmStageBytes;
+        unsigned char *sb = s_b + buf * kStageB;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;  // (row r half, row r + 1 half)
@@ -232,7 +247,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // registers -> LDS stage `buf`
     auto store_step = [=](const GemmStepRegs &r, int buf) {
         store_a(r.a, buf);
-        unsigned char *sb = s_b + buf * kGemmStageBytes;
+        unsigned char *sb = s_b + buf * kStageB;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             uint32_t f[4];
@@ -285,8 +300,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const unsigned char *sa0 = s_a + (wm * 64 + frag_row) * kGemmPitch + frag_k;
     const unsigned char *sb0 = s_b + (wn * 64 + frag_row) * kGemmPitch + frag_k;
     auto compute = [&](int buf) {
-        const unsigned char *sa = sa0 + buf * kGemmStageBytes;
-        const unsigned char *sb = sb0 + buf * kGemmStageBytes;
+        const unsigned char *sa = sa0 + buf * kGemmStageA;
+        const unsigned char *sb = sb0 + buf * kStageB;
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
             half8_t af[2], bf[2];
@@ -343,7 +358,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (plan.splits > 1) {
         // partial tiles in the accumulators' own order: element q of a lane at [q][lane], so that
         // every store and load instruction covers 256 contiguous bytes
-        const size_t tile_elems = (size_t)kGemmTM * kGemmTN;
+        const size_t tile_elems = (size_t)kGemmTM * TN;
         const size_t tiles = (size_t)plan.mtiles * plan.ntiles;
         float *mine = partial + ((size_t)split * tiles + blockIdx.x) * tile_elems + wave * 4096 + lane;
 #pragma unroll
@@ -371,18 +386,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             for (int j = 0; j < 2; j++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
-        for (int s = 0; s < plan.splits; s++) {  // split order: independent of arrival order
-            const float *theirs = partial + ((size_t)s * tiles + blockIdx.x) * tile_elems + wave * 4096 + lane;
-            float v[64];
+        // two splits (128 loads) in flight at a time, added in split order: independent of arrival order
+        for (int s0 = 0; s0 < plan.splits; s0 += 2) {
+            float v[2][64];
 #pragma unroll
-            for (int q = 0; q < 64; q++)
-                v[q] = __hip_atomic_load(theirs + q * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int ds = 0; ds < 2; ds++) {
+                const int sx = min(s0 + ds, plan.splits - 1);
+                const float *theirs = partial + ((size_t)sx * tiles + blockIdx.x) * tile_elems + wave * 4096 + lane;
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+                for (int q = 0; q < 64; q++)
+                    v[ds][q] = __hip_atomic_load(theirs + q * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
 #pragma unroll
-                for (int j = 0; j < 2; j++)
+            for (int ds = 0; ds < 2; ds++)
+                if (s0 + ds < plan.splits) {
 #pragma unroll
-                    for (int e = 0; e < 16; e++) acc[i][j][e] += v[(i * 2 + j) * 16 + e];
+                    for (int i = 0; i < 2; i++)
+#pragma unroll
+                        for (int j = 0; j < 2; j++)
+#pragma unroll
+                            for (int e = 0; e < 16; e++) acc[i][j][e] += v[ds][(i * 2 + j) * 16 + e];
+                }
         }
     }
 #pragma unroll
@@ -415,7 +439,7 @@ bool gemm_supported(int bits, int M, int K, int N, int C, int G) {
     return true;
 }
 
-template <int BITS>
+template <int BITS, int WN>
 static hipError_t launch_gemm_bits(const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
                                    const int16_t *cherry_indices, const __half *scales, __half *mul, int M, int K,
                                    int N, int C, int G, int accumulate, void *workspace, void *scratch,
@@ -430,16 +454,16 @@ static hipError_t launch_gemm_bits(const __half *vec, const uint8_t *qweight, co
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 64 || !lds_set[dev]) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<BITS>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes);
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<BITS, WN>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, gemm_lds_bytes(WN));
         if (e != hipSuccess) return e;
         if (dev >= 0 && dev < 64) lds_set[dev] = true;
     }
     hipLaunchKernelGGL(gemm_prep_kernel<BITS>, dim3(ceil_div(plan.Kp / 8, 256), plan.Mp), dim3(256), 0, stream, vec,
                        cherry_indices, reinterpret_cast<uint4 *>(a), M, K, C, plan.Kp, plan.steps_normal * 8);
-    hipLaunchKernelGGL(gemm_kernel<BITS>, dim3(plan.mtiles * plan.ntiles, plan.splits), dim3(256), kGemmLdsBytes,
-                       stream, qweight, cherry_weight, scales, mul, a, partial, tickets, M, K, N, C, G, accumulate,
-                       plan);
+    hipLaunchKernelGGL((gemm_kernel<BITS, WN>), dim3(plan.mtiles * plan.ntiles, plan.splits), dim3(128 * WN),
+                       gemm_lds_bytes(WN), stream, qweight, cherry_weight, scales, mul, a, partial, tickets, M, K, N,
+                       C, G, accumulate, plan);
     return hipGetLastError();
 }
 
@@ -447,10 +471,10 @@ hipError_t launch_gemm(int bits, const __half *vec, const uint8_t *qweight, cons
                        const int16_t *cherry_indices, const __half *scales, __half *mul, int M, int K, int N, int C,
                        int G, int accumulate, void *workspace, void *scratch, hipStream_t stream) {
     if (bits == 4)
-        return launch_gemm_bits<4>(vec, qweight, cherry_weight, cherry_indices, scales, mul, M, K, N, C, G, accumulate,
-                                   workspace, scratch, stream);
-    return launch_gemm_bits<3>(vec, qweight, cherry_weight, cherry_indices, scales, mul, M, K, N, C, G, accumulate,
-                               workspace, scratch, stream);
+        return launch_gemm_bits<4, 2>(vec, qweight, cherry_weight, cherry_indices, scales, mul, M, K, N, C, G,
+                                      accumulate, workspace, scratch, stream);
+    return launch_gemm_bits<3, 2>(vec, qweight, cherry_weight, cherry_indices, scales, mul, M, K, N, C, G, accumulate,
+                                  workspace, scratch, stream);
 }
 
 }  // namespace cq

@@ -506,11 +506,94 @@ def test_device_pack_is_bit_identical_to_host_pack(bits):
 
 
 # ------------------------------------------------------------------------- prompt-sized batches
+def column_sample(p, rng, count):
+    n = p["qweight"].shape[1]
+    cols = np.sort(rng.choice(n, size=min(count, n), replace=False))
+    sub = {"cherry_indices": p["cherry_indices"], "cherry_weight": np.ascontiguousarray(p["cherry_weight"][:, cols]),
+           "qweight": np.ascontiguousarray(p["qweight"][:, cols]), "scales": np.ascontiguousarray(p["scales"][:, cols])}
+    return cols, sub
+
+
+@pytest.mark.parametrize("bits,gs,k,n,rows", [
+    (4, 128, 4096, 1024, 17),      # one row tile, 8 K splits
+    (3, 128, 4096, 1024, 128),
+    (4, 128, 11008, 520, 96),      # N % 128 != 0, Kn % 64 != 0
+    (3, 128, 1160, 264, 33),       # short K: few steps, ragged everything
+    (3, 64, 2048, 256, 40),        # 3-bit with 64-wide groups
+    (4, 256, 4096, 512, 70),       # groups of two steps... of four steps
+    (4, 128, 28672, 512, 20),      # 112 cherry rows: two cherry steps
+    (4, 128, 2048, 4096, 1100),    # nine row tiles, no K split
+    (3, 128, 4096, 11008, 200),    # 7B gate/up, two row tiles
+])
+def test_gemm_rows_against_oracle(qc, bits, gs, k, n, rows):
+    """More than 16 rows: the tiled dequantise + MFMA kernel against the C oracle (a column sample
+    for the large shapes), every row on its own as well."""
+    announce("gemm", bits, gs, k, n, rows)
+    p = orc.synthetic_packed_fast(k, n, bits, gs, seed=rows)
+    rng = np.random.default_rng(rows)
+    x = rng.standard_normal((rows, k)).astype(np.float16)
+    y = run_fused(qc, bits, x, p, gs)
+    cols, sub = column_sample(p, rng, 256)
+    want = c_oracle.fused(x, sub, bits, gs)
+    assert orc.rel_l2(y[:, cols], want) <= TOL
+    for r in (0, 1, 15, 16, rows // 2, rows - 1):
+        assert orc.rel_l2(y[r, cols], want[r]) <= TOL, r
+    # against the dense path on the dequantised weight (fp16 weights, as this kernel uses them)
+    dense = c_oracle.unpack(sub, bits, gs, k)
+    assert orc.rel_l2(y[:, cols], c_oracle.linear(x, dense, want_f64=True)[1]) <= TOL
+
+
+@pytest.mark.parametrize("bits,k,n", [(4, 4096, 1024), (3, 4096, 1024), (4, 11008, 520), (3, 1160, 264)])
+def test_gemm_one_hot_rows_are_bit_exact(qc, bits, k, n):
+    """One-hot activation rows through the tiled kernel: row i returns the dequantised weight
+    column j_i bit for bit (field extraction, the exact u - c_b, the single rounding of the scale
+    product, the position order shared by the A and B operands, the cherry steps)."""
+    announce("gemm one-hot", bits, k, n)
+    w, p = orc.synthetic_layer(k, n, bits, 128, seed=9)
+    dense = c_oracle.unpack(p, bits, 128, k)
+    idx = p["cherry_indices"].astype(np.int64)
+    nidx = orc.normal_indices(k, idx)
+    picks = [0, 1, 2, 3, 4, 5, 6, 7, 8, 31, 32, 63, 64, 65, 127, 128, len(nidx) - 1, len(nidx) - 2, len(nidx) - 9,
+             len(nidx) // 2]
+    cols = [int(nidx[i]) for i in picks] + [int(i) for i in idx]
+    rng = np.random.default_rng(1)
+    cols += [int(c) for c in rng.choice(k, size=150 - len(cols), replace=False)]   # spans two row tiles
+    x = np.zeros((len(cols), k), dtype=np.float16)
+    x[np.arange(len(cols)), cols] = 1
+    y = run_fused(qc, bits, x, p, 128)
+    np.testing.assert_array_equal(y, dense[:, cols].T)
+
+
+def test_gemm_accumulate_linearity_and_determinism(qc):
+    announce("gemm accumulate")
+    bits, k, n, rows = 4, 4096, 2048, 150
+    p = orc.synthetic_packed_fast(k, n, bits, 128, seed=2)
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((rows, k)).astype(np.float16)
+    y1 = run_fused(qc, bits, x, p, 128)
+    y1b = run_fused(qc, bits, x, p, 128)
+    np.testing.assert_array_equal(y1, y1b)                    # split-K partials are added in split order
+    base = rng.standard_normal((rows, n)).astype(np.float16)
+    y2 = run_fused(qc, bits, x, p, 128, mul=base.copy())     # the reference's accumulate-in-place contract
+    cols, sub = column_sample(p, rng, 256)
+    want = c_oracle.fused(x, sub, bits, 128)
+    assert orc.rel_l2(y2[:, cols], want + base[:, cols].astype(np.float64)) <= TOL
+    # f(2 x) == 2 f(x) exactly: powers of two commute with every rounding involved
+    y4 = run_fused(qc, bits, (x * np.float16(2)).astype(np.float16), p, 128)
+    np.testing.assert_array_equal(y4, (y1.astype(np.float32) * 2).astype(np.float16))
+    # rows do not interact: a row gives the same bits alone in a 17-row call padded with zeros
+    x17 = np.zeros((17, k), dtype=np.float16)
+    x17[3] = x[77]
+    y17 = run_fused(qc, bits, x17, p, 128)
+    assert not y17[[i for i in range(17) if i != 3]].any()
+    assert orc.rel_l2(y17[3], y1[77].astype(np.float64)) <= 1e-3   # different split count: same contract
+
+
 @pytest.mark.parametrize("bits,k,n,rows", [(4, 4096, 1024, 64), (3, 4096, 1024, 128), (4, 11008, 520, 96)])
 def test_prefill_rows_dequantise_once_then_gemm(qc, bits, k, n, rows):
-    """QuantLinear.forward with >= prefill_rows rows (dense GEMM on the bit-exact dequantised
-    weight) against the oracle's dequantised product, and against the fused path just below
-    the threshold."""
+    """QuantLinear.forward at and above prefill_rows (dense library GEMM on the bit-exact dequantised
+    weight) against the oracle's dequantised product, and against the fused kernel below the
+    threshold."""
     announce("prefill", bits, k, n, rows)
     from llama.qlinear import QuantLinear as PackedLinear
     from llama.quantizer import FullSymQuantizer
@@ -519,15 +602,18 @@ def test_prefill_rows_dequantise_once_then_gemm(qc, bits, k, n, rows):
     for name in NAMES:
         setattr(q, name, torch.from_numpy(p[name]).cuda())
     x = np.random.default_rng(rows).standard_normal((rows, k)).astype(np.float16)
-    y = q(torch.from_numpy(x).cuda())
-    assert y.shape == (rows, n) and y.dtype == torch.float16
-    dense, y_deq, _ = oracle_outputs(bits, x, p, 128)
-    assert orc.rel_l2(y.cpu().numpy(), y_deq) <= TOL
-    saved, PackedLinear.prefill_rows = PackedLinear.prefill_rows, 1 << 30
+    saved = PackedLinear.prefill_rows
     try:
+        PackedLinear.prefill_rows = 32
+        y = q(torch.from_numpy(x).cuda())
+        PackedLinear.prefill_rows = 1 << 30
         y_fused = q(torch.from_numpy(x).cuda())
     finally:
         PackedLinear.prefill_rows = saved
+    assert y.shape == (rows, n) and y.dtype == torch.float16
+    dense, y_deq, _ = oracle_outputs(bits, x, p, 128)
+    assert orc.rel_l2(y.cpu().numpy(), y_deq) <= TOL
+    assert orc.rel_l2(y_fused.cpu().numpy(), y_deq) <= TOL
     assert orc.rel_l2(y.cpu().numpy(), y_fused.cpu().numpy().astype(np.float64)) <= 2 * TOL
 
 
