@@ -218,6 +218,19 @@ def decode_benchmark(prompt_len=128, new_tokens=128, w_bits=4, seed=0):
     model.generate(prompt, 8)                                   # warm-up
     out, _, total = model.generate(prompt, new_tokens)          # throughput: one sync at the end
     _, times, _ = model.generate(prompt, new_tokens, sync_each_token=True)  # latency per token
+    # prompt processing: token by token through the captured step, and in one batched pass
+    def timed(fn, reps=3):
+        best = float("inf")
+        for _ in range(reps):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            best = min(best, time.perf_counter() - t0)
+        return best
+    model.prefill(prompt)                                        # warm-up (workspaces for 128 rows)
+    prefill_batched = timed(lambda: model.prefill(prompt))
+    prefill_steps = timed(lambda: model.generate(prompt, 0), reps=1)
     bytes_per_token = model.step_bytes()
     tok_s = new_tokens / total
     res = {"model": "llama7b-shape random init", "w_bits": w_bits, "prompt_tokens": prompt_len,
@@ -227,6 +240,8 @@ def decode_benchmark(prompt_len=128, new_tokens=128, w_bits=4, seed=0):
            "hbm_gbs": round(bytes_per_token * tok_s / 1e9, 1),
            "frac_of_hbm_peak": round(bytes_per_token * tok_s / 1e9 / HBM_PEAK_GBS, 4),
            "launch": "one single-stream HIP graph per token",
+           "prefill_ms_batched": round(prefill_batched * 1e3, 2),
+           "prefill_ms_token_steps": round(prefill_steps * 1e3, 2),
            "first_tokens": out[:8].tolist()}
     del model
     torch.cuda.empty_cache()
@@ -240,7 +255,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default="llama7b_gate_up_w4", choices=sorted(WORKLOADS))
     ap.add_argument("--group", type=int, default=128)
-    ap.add_argument("--batch", type=int, default=1, help="activation rows per call (2..16: matrix-core path)")
+    ap.add_argument("--batch", type=int, default=1, help="activation rows per call (2..16: small-batch matrix-core kernel, more: tiled GEMM kernel)")
     ap.add_argument("--all", action="store_true", help="also print a table of every workload to stderr")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the 7B-shape decode measurement")
@@ -283,6 +298,19 @@ def main():
                   f"({fl / us / 1e6 / 2500 * 100:4.1f}% of fp16 MFMA peak; prep + main kernel)",
                   file=sys.stderr, flush=True)
             torch.cuda.empty_cache()
+        # prompt-sized batches: the tiled dequantise + MFMA GEMM kernel
+        for name, b in (("llama7b_attn_w4", 128), ("llama7b_gate_up_w4", 32), ("llama7b_gate_up_w4", 128),
+                        ("llama7b_gate_up_w3", 128), ("llama7b_down_w4", 128), ("llama7b_gate_up_w4", 512),
+                        ("llama7b_gate_up_w4", 2048), ("llama70b_gate_up_w4", 128), ("llama70b_down_w4", 128)):
+            bits, k, n = WORKLOADS[name]
+            us, wall_us, *_ = time_gpu(bits, k, n, args.group, 100, 10, batch=b, use_graph=not args.no_graph)
+            ab = algorithmic_bytes(bits, k, n, b, args.group)
+            fl = 2.0 * b * k * n
+            print(f"{name:24s} {bits}-bit {k:5d}->{n:5d} rows {b:4d}: {us:7.2f} us  {fl / us / 1e6:6.1f} TFLOP/s "
+                  f"({fl / us / 1e6 / 2500 * 100:4.1f}% of fp16 MFMA peak)  {ab / us / 1e3:7.1f} GB/s "
+                  f"({ab / us / 1e3 / HBM_PEAK_GBS * 100:4.1f}% of 8 TB/s; prep + main kernel)",
+                  file=sys.stderr, flush=True)
+            torch.cuda.empty_cache()
         for name, (bits, k, n) in WORKLOADS.items():
             us, wall_us, *_ = time_gpu(bits, k, n, args.group, max(200, args.steps // 4), args.warmup,
                                       use_graph=not args.no_graph)
@@ -314,7 +342,8 @@ def main():
                      "traffic": MEASURED_TRAFFIC.get((args.workload, args.batch)),
                      "algorithmic_bytes_per_launch": ab,
                      "kernel": f"cq::matvec_kernel<{bits}>" if args.batch == 1 else
-                               f"cq::batch_prep_kernel<{bits}> + cq::batch_kernel<{bits}>"},
+                               f"cq::batch_prep_kernel<{bits}> + cq::batch_kernel<{bits}>" if args.batch <= 16 else
+                               f"cq::gemm_prep_kernel<{bits}> + cq::gemm_kernel<{bits}, 2>"},
     }
     if args.batch == 1:
         result["roofline"]["reference"] = roofline_reference(copies, args.steps)

@@ -379,10 +379,63 @@ class CherryLlamaDecoder(nn.Module):
         self.reset()
 
     @torch.inference_mode()
-    def generate(self, prompt_ids: torch.Tensor, max_new_tokens: int, use_graph=True, sync_each_token=False):
-        """Greedy decoding.  The prompt is fed token by token through the same step (prefill is
-        not timed separately here).  Returns (generated ids, per-token seconds of the decode part
-        when sync_each_token, total decode seconds)."""
+    def prefill(self, prompt_ids: torch.Tensor) -> torch.Tensor:
+        """The whole prompt in one batched pass, as the reference's model processes it
+        (llama/modeling_llama_quant.py:1009-1100): every linear sees all T rows at once (the tiled
+        GEMM kernel from 17 rows, the small-batch kernel below), RMSNorm / rotary / causal attention
+        are torch operations with the reference's rounding points.  Fills the KV caches for
+        positions 0..T-1, leaves the decoder exactly where T token steps would (position T, the
+        first generated token predicted and embedded) and returns the last position's logits."""
+        cfg = self.cfg
+        ids = prompt_ids.to(self.device_)
+        T, nh, nkv, hd = ids.numel(), cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+        assert ids.dim() == 1 and 1 <= T <= cfg.max_position_embeddings
+
+        def norm(x, w):
+            xf = x.float()
+            return w * (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + cfg.rms_norm_eps)).half()
+
+        pos = torch.arange(T, device=self.device_, dtype=torch.float32)
+        inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, hd, 2, device=self.device_, dtype=torch.float32) / hd))
+        fr = torch.outer(pos, inv)
+        emb = torch.cat([fr, fr], dim=-1)
+        cos, sin = emb.cos().half()[None], emb.sin().half()[None]  # (1, T, hd)
+
+        def rot(x):
+            return torch.cat([-x[..., hd // 2:], x[..., :hd // 2]], dim=-1)
+
+        self.reset()
+        h = self.embed_tokens[ids]
+        mask = torch.full((T, T), float("-inf"), device=self.device_).triu(1)
+        rep = nh // nkv
+        for li, layer in enumerate(self.layers):
+            x = norm(h, layer.input_layernorm)
+            q = layer.q_proj(x).view(T, nh, hd).transpose(0, 1)
+            k = layer.k_proj(x).view(T, nkv, hd).transpose(0, 1)
+            v = layer.v_proj(x).view(T, nkv, hd).transpose(0, 1)
+            q = q * cos + rot(q) * sin
+            k = k * cos + rot(k) * sin
+            self.k_cache[li, :, :T].copy_(k)
+            self.v_cache[li, :, :T].copy_(v)
+            kk, vv = k.repeat_interleave(rep, 0), v.repeat_interleave(rep, 0)
+            att = (q @ kk.transpose(1, 2)) / math.sqrt(hd)
+            att = torch.softmax(att.float() + mask, dim=-1).half()
+            a = (att @ vv).transpose(0, 1).reshape(T, nh * hd)
+            h = h + layer.o_proj(a)
+            x = norm(h, layer.post_attention_layernorm)
+            h = h + layer.down_proj(torch.nn.functional.silu(layer.gate_proj(x)) * layer.up_proj(x))
+        self.normed.copy_(norm(h[T - 1:T], self.norm))
+        self.pos.fill_(T - 1)
+        self._head()  # logits of the last prompt position; greedy tail: history[T-1], next embedding, pos = T
+        return self.logits
+
+    @torch.inference_mode()
+    def generate(self, prompt_ids: torch.Tensor, max_new_tokens: int, use_graph=True, sync_each_token=False,
+                 batched_prefill=False):
+        """Greedy decoding.  The prompt is fed token by token through the same step, or, with
+        batched_prefill, in one pass over all prompt rows (prefill is not part of the timed
+        region either way).  Returns (generated ids, per-token seconds of the decode part when
+        sync_each_token, total decode seconds)."""
         import time
         assert prompt_ids.dim() == 1 and prompt_ids.numel() + max_new_tokens <= self.cfg.max_position_embeddings
         if use_graph and self._graph is None:
@@ -391,10 +444,13 @@ class CherryLlamaDecoder(nn.Module):
         run = self._graph.replay if use_graph else self._step
         prompt_ids = prompt_ids.to(self.device_)
         n_prompt = prompt_ids.numel()
-        for i in range(n_prompt):
-            self.token.copy_(prompt_ids[i:i + 1])
-            self.embed()
-            run()
+        if batched_prefill:
+            self.prefill(prompt_ids)
+        else:
+            for i in range(n_prompt):
+                self.token.copy_(prompt_ids[i:i + 1])
+                self.embed()
+                run()
         torch.cuda.synchronize()
         times = []
         t0 = time.perf_counter()

@@ -238,6 +238,37 @@ def test_small_decoder_matches_dense_reference(dec, bits):
     assert torch.equal(out, out2) and out.numel() == 8
 
 
+@pytest.mark.parametrize("bits,prompt_len", [(4, 24), (3, 7)])
+def test_batched_prefill_matches_token_steps(dec, bits, prompt_len):
+    """The prompt in one batched pass (tiled GEMM kernel at 24 rows, small-batch kernel at 7): last
+    position's logits against the dense reference and against feeding the prompt token by
+    token; the KV caches agree with the step path's; decoding continues from the prefilled state."""
+    print("[case] batched prefill", bits, prompt_len, flush=True)
+    cfg = dec.DecoderConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=2,
+                            num_key_value_heads=1, vocab_size=512, max_position_embeddings=48, w_bits=bits,
+                            group_size=128, cherry_fraction=1 / 16)
+    model = dec.CherryLlamaDecoder(cfg, seed=5)
+    ids = torch.randint(0, cfg.vocab_size, (prompt_len,), generator=torch.Generator().manual_seed(1))
+    want = model.reference_logits(ids)[-1]
+    stepped = model.step_logits(ids)[-1]
+    k_step, v_step = model.k_cache.clone(), model.v_cache.clone()
+    got = model.prefill(ids)[0]
+    assert rel(got, want) < 2e-2 and rel(got, stepped) < 2e-2
+    assert int(model.pos.item()) == prompt_len
+    assert int(model.history[prompt_len - 1].item()) == int(got.argmax().item())
+    assert rel(model.k_cache[:, :, :prompt_len], k_step[:, :, :prompt_len]) < 1e-2
+    assert rel(model.v_cache[:, :, :prompt_len], v_step[:, :, :prompt_len]) < 1e-2
+    assert not model.k_cache[:, :, prompt_len:].any()
+    # the step that follows consumes the predicted token: teacher-forced reference on prompt + that token
+    nxt = model.history[prompt_len - 1:prompt_len]
+    model._step()
+    want2 = model.reference_logits(torch.cat([ids.to(nxt.device), nxt]))[-1]
+    assert rel(model.logits[0], want2) < 2e-2
+    out, _, _ = model.generate(ids, 6, use_graph=True, batched_prefill=True)
+    out2, _, _ = model.generate(ids, 6, use_graph=False, batched_prefill=True)
+    assert out.numel() == 6 and torch.equal(out, out2) and int(out[0]) == int(nxt[0])
+
+
 def test_saved_checkpoint_reloads_to_identical_logits(dec, tmp_path):
     """save_quantized -> from_quantized (reference file name and key names) gives a decoder whose
     token step reproduces the original's logits bit for bit."""
