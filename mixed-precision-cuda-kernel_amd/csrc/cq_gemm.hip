@@ -319,7 +319,9 @@ __global__ __launch_bounds__(128 * WN) __attribute__((amdgpu_waves_per_eu(2, 2))
     };
     // Packed steps.  Ring of kRing register sets: the global loads of step st + kRing - 1 are issued
     // while step st is computed, so a load has kRing - 2 whole steps to arrive before its
-    // dequantisation.
+    // dequantisation.  The steady-state loop has no branches inside (four steps per trip, every
+    // load and store unconditional): only then does the compiler's wait-count bookkeeping let
+    // the younger loads stay in flight instead of draining the queue in every step.
     {
         constexpr int kRing = 4;
         const int n_end = min(st_end, plan.steps_normal);
@@ -329,15 +331,24 @@ __global__ __launch_bounds__(128 * WN) __attribute__((amdgpu_waves_per_eu(2, 2))
             if (st_begin + i < n_end) load_step(regs[i], st_begin + i);
         if (st_begin < n_end) store_step(regs[0], 0);
         __syncthreads();
-        for (int base = st_begin; base < n_end; base += kRing) {
+        int base = st_begin;
+        for (; base + 2 * kRing - 1 <= n_end; base += kRing) {  // all of st + kRing - 1 < n_end
+#pragma unroll
+            for (int r = 0; r < kRing; r++) {
+                load_step(regs[(r + kRing - 1) % kRing], base + r + kRing - 1);
+                compute(r & 1);
+                store_step(regs[(r + 1) % kRing], (r & 1) ^ 1);
+                __syncthreads();
+            }
+        }
+        for (; base < n_end; base += kRing) {  // the last steps, guarded
 #pragma unroll
             for (int r = 0; r < kRing; r++) {
                 const int st = base + r;
                 if (st < n_end) {  // uniform
-                    const int buf = r & 1;
                     if (st + kRing - 1 < n_end) load_step(regs[(r + kRing - 1) % kRing], st + kRing - 1);
-                    compute(buf);
-                    if (st + 1 < n_end) store_step(regs[(r + 1) % kRing], buf ^ 1);
+                    compute(r & 1);
+                    if (st + 1 < n_end) store_step(regs[(r + 1) % kRing], (r & 1) ^ 1);
                     __syncthreads();
                 }
             }
