@@ -64,6 +64,68 @@ __device__ inline int gather_offset(const IDX *__restrict__ idx, int C, int k) {
     return lo;
 }
 
+// ---- cross-lane reductions without LDS ---------------------------------------------------------
+// all-reduce over the 16 lanes of a DPP row by rotations 8, 4, 2, 1
+__device__ inline float row_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x122, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xf, 0xf, false));
+    return v;
+}
+
+__device__ inline int row_max(int v) {
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x128, 0xf, 0xf, false));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x124, 0xf, 0xf, false));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x122, 0xf, 0xf, false));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x121, 0xf, 0xf, false));
+    return v;
+}
+
+// v_permlane32_swap_b32 exchanges lanes 32..63 of its first operand with lanes 0..31 of its
+// second; v_permlane16_swap_b32 exchanges the odd 16-lane rows of the first with the even rows
+// of the second.  Written as inline assembly because the compiler builtin of this toolchain
+// returns the first result twice; the s_nop pad the VALU->permlane-swap data hazards that the
+// compiler cannot see through an asm statement.
+//
+// swap32_add: lanes < 32 return a[l] + a[l+32], lanes >= 32 return b[l-32] + b[l].
+__device__ inline float swap32_add(float a, float b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return a + b;
+}
+
+// swap16_add: even rows return a[row] + a[row+1], odd rows return b[row-1] + b[row].
+__device__ inline float swap16_add(float a, float b) {
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return a + b;
+}
+
+// all lanes of the wavefront receive the sum / maximum over its 64 lanes
+__device__ inline float wave_sum_all(float v) {
+    v = row_sum(v);
+    v = swap16_add(v, v);
+    return swap32_add(v, v);
+}
+
+__device__ inline float row_max_f(float v) {
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false)));
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false)));
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x122, 0xf, 0xf, false)));
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xf, 0xf, false)));
+    return v;
+}
+
+__device__ inline float wave_max_all(float v) {
+    v = row_max_f(v);
+    float a = v, b = v;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    v = fmaxf(a, b);
+    a = v;
+    b = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return fmaxf(a, b);
+}
+
 // Split-K epilogue: one 64-bit atomic per output element.
 //
 // Each output element owns a 64-bit accumulator word in the workspace:

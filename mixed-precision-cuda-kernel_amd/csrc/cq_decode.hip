@@ -13,6 +13,17 @@
 // fp16 tensor operations do; contraction would merge a product and a sum into one rounding.
 #pragma clang fp contract(off)
 
+// Optional per-workgroup phase timestamps for a profiling harness; compiled out in the library.
+#ifdef CQ_TRACE
+extern __device__ unsigned long long *g_cq_trace;
+#define CQD_STAMP(slot)                                                                                      \
+    do {                                                                                                     \
+        if (g_cq_trace && threadIdx.x == 0) g_cq_trace[(size_t)blockIdx.x * 8 + (slot)] = wall_clock64();    \
+    } while (0)
+#else
+#define CQD_STAMP(slot) do { } while (0)
+#endif
+
 namespace cq {
 
 __device__ inline float wave_sum(float v) {
@@ -76,17 +87,48 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(__half *__restrict__ 
     }
 }
 
+// theta^(-2 i / head_dim), the rotary frequency of dimension pair i.  The library routine powf is a
+// call of several hundred instructions on the critical path of every decode step.  For a
+// power-of-two head_dim the exponent x = (2 i / head_dim) * log2(theta) is split into an integer
+// and a fraction in [-0.5, 0.5] without rounding error beyond that of log2(theta), which the host
+// passes as an unevaluated sum of two floats; 2^-fraction is one v_exp_f32 (about 1 ulp), so the
+// result is within about 2 ulp of the exact value, like powf's.  Other head dims use powf.
+struct RopeBase {
+    float theta, log2_hi, log2_lo;
+};
+
+static RopeBase rope_base(float theta) {
+    const double l = log2((double)theta);
+    RopeBase b;
+    b.theta = theta;
+    b.log2_hi = (float)l;
+    b.log2_lo = (float)(l - (double)b.log2_hi);
+    return b;
+}
+
+__device__ inline float rope_inv_freq(int i, int head_dim, const RopeBase &b) {
+    if (head_dim & (head_dim - 1)) return powf(b.theta, -2.0f * (float)i / (float)head_dim);
+    const float fi = (float)(2 * i);                 // exact
+    const float p = fi * b.log2_hi;
+    const float e = fmaf(fi, b.log2_hi, -p);         // exact error of the product
+    const float inv_hd = 1.0f / (float)head_dim;     // exact: a power of two
+    const float ps = p * inv_hd;                     // exact scaling
+    const float n = rintf(ps);
+    const float frac = (ps - n) + (e + fi * b.log2_lo) * inv_hd;  // ps - n is exact
+    return ldexpf(__builtin_amdgcn_exp2f(-frac), -(int)n);
+}
+
 // Rotary embedding of q (in place) and k, and the KV-cache write at position *pos.
 // One workgroup per head (q heads first, then kv heads), head_dim / 2 threads.
 // Cache layout: [kv_head][max_len][head_dim].
 __global__ void rope_cache_kernel(__half *__restrict__ q, const __half *__restrict__ k, const __half *__restrict__ v,
                                   __half *__restrict__ k_cache, __half *__restrict__ v_cache,
                                   const int *__restrict__ pos_ptr, int n_heads, int n_kv_heads, int head_dim,
-                                  int max_len, float theta) {
+                                  int max_len, RopeBase base) {
     const int pos = *pos_ptr;
     const int head = blockIdx.x, i = threadIdx.x, half_dim = head_dim / 2;
     if (i >= half_dim || pos >= max_len) return;
-    const float inv_freq = powf(theta, -2.0f * (float)i / (float)head_dim);
+    const float inv_freq = rope_inv_freq(i, head_dim, base);
     float sn, cs;
     sincosf((float)pos * inv_freq, &sn, &cs);
     const float c = __half2float(__float2half_rn(cs)), s = __half2float(__float2half_rn(sn));
@@ -212,12 +254,14 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const __half *__restri
 __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
     const __half *__restrict__ q, const __half *__restrict__ k, const __half *__restrict__ v,
     __half *__restrict__ k_cache, __half *__restrict__ v_cache, __half *__restrict__ out,
-    const int *__restrict__ pos_ptr, int n_heads, int n_kv_heads, int max_len, float theta, float scale) {
+    const int *__restrict__ pos_ptr, int n_heads, int n_kv_heads, int max_len, RopeBase base, float scale) {
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
     __shared__ float s_score[kMaxAttnLen];
     __shared__ float s_red[32];
     __shared__ float s_acc[16][128];
-    __shared__ float s_q[128], s_k[128];
+    __shared__ __attribute__((aligned(16))) unsigned short s_qh[128], s_kh[128];  // rotated q, k as fp16
     const int head = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    CQD_STAMP(0);
     const int row = t >> 4, l16 = t & 15;
     const int rep = n_heads / n_kv_heads, kvh = head / rep;
     const uint4 *kb = reinterpret_cast<const uint4 *>(k_cache + (size_t)kvh * max_len * 128);
@@ -233,7 +277,7 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
         v_first[u] = j < max_len ? vb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
     }
     // likewise the new token's q (threads 0..63), k and v (threads 64..127)
-    float x1 = 0.f, x2 = 0.f;
+    float x1 = 0.f, x2 = 0.f, inv_freq = 0.f;
     __half v1 = __float2half(0.f), v2 = v1;
     if (t < 128) {
         const int i = t & 63;
@@ -244,22 +288,23 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
             v1 = v[(size_t)kvh * 128 + i];
             v2 = v[(size_t)kvh * 128 + i + 64];
         }
+        inv_freq = rope_inv_freq(i, 128, base);  // does not need the position
     }
     const int pos = *pos_ptr;
     if (pos >= max_len) return;
+    CQD_STAMP(1);
     if (t < 128) {
         const int i = t & 63;
         const bool is_k = t >= 64;
-        const float inv_freq = powf(theta, -2.0f * (float)i / 128.f);
         float sn, cs;
         sincosf((float)pos * inv_freq, &sn, &cs);
         const float c = __half2float(__float2half_rn(cs)), sr = __half2float(__float2half_rn(sn));
         const float a1 = __half2float(__float2half_rn(x1 * c)), b1 = __half2float(__float2half_rn(-x2 * sr));
         const float a2 = __half2float(__float2half_rn(x2 * c)), b2 = __half2float(__float2half_rn(x1 * sr));
         const __half o1 = __float2half_rn(a1 + b1), o2 = __float2half_rn(a2 + b2);
-        float *dst = is_k ? s_k : s_q;
-        dst[i] = __half2float(o1);
-        dst[i + 64] = __half2float(o2);
+        unsigned short *dst = is_k ? s_kh : s_qh;
+        dst[i] = __half_as_ushort(o1);
+        dst[i + 64] = __half_as_ushort(o2);
         if (is_k && head % rep == 0) {
             __half *kd = k_cache + ((size_t)kvh * max_len + pos) * 128;
             __half *vd = v_cache + ((size_t)kvh * max_len + pos) * 128;
@@ -270,10 +315,20 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
         }
     }
     __syncthreads();
-    float qf[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) qf[i] = s_q[8 * l16 + i];
-    // scores of the cached positions 0 .. pos-1, four rows of loads in flight per thread
+    CQD_STAMP(2);
+    // q . k over the lane's 8 dimensions as four packed fp16 dot products (fp32 accumulation), the 16
+    // lanes of a row then add up with DPP rotations
+    const uint4 qv = *reinterpret_cast<const uint4 *>(&s_qh[8 * l16]);
+    auto dot8 = [&](const uint4 &kv) {
+        float d = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, kv.x), __builtin_bit_cast(half2_t, qv.x), 0.f, false);
+        d = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, kv.y), __builtin_bit_cast(half2_t, qv.y), d, false);
+        d = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, kv.z), __builtin_bit_cast(half2_t, qv.z), d, false);
+        d = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, kv.w), __builtin_bit_cast(half2_t, qv.w), d, false);
+        return row_sum(d);
+    };
+    // scores of the cached positions 0 .. pos-1, four rows of loads in flight per thread; the running
+    // maximum rides along, so that the softmax needs no pass of its own for it
+    float m = -INFINITY;
     for (int j0 = row; j0 < pos; j0 += 256) {
         uint4 kk[4];
 #pragma unroll
@@ -287,29 +342,23 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             const int j = j0 + 64 * u;
-            float kf[8];
-            unpack8(kk[u], kf);
-            float d = 0.f;
-#pragma unroll
-            for (int i = 0; i < 8; i++) d += qf[i] * kf[i];
-            d = row16_sum(d);
-            if (l16 == 0 && j < pos) s_score[j] = __half2float(__float2half_rn(d)) * scale;
+            const float sc = __half2float(__float2half_rn(dot8(kk[u]))) * scale;  // fp16 q k^T, then / sqrt(d)
+            if (j < pos) {
+                m = fmaxf(m, sc);
+                if (l16 == 0) s_score[j] = sc;
+            }
         }
     }
     if (row == 0) {  // the new position, from LDS
-        float d = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; i++) d += qf[i] * s_k[8 * l16 + i];
-        d = row16_sum(d);
-        if (l16 == 0) s_score[pos] = __half2float(__float2half_rn(d)) * scale;
+        const float sc = __half2float(__float2half_rn(dot8(*reinterpret_cast<const uint4 *>(&s_kh[8 * l16])))) * scale;
+        m = fmaxf(m, sc);
+        if (l16 == 0) s_score[pos] = sc;
     }
-    __syncthreads();
-    const int len = pos + 1;
-    float m = -INFINITY;
-    for (int j = t; j < len; j += 1024) m = fmaxf(m, s_score[j]);
-    m = wave_max(m);
+    m = wave_max_all(m);
     if (lane == 0) s_red[wave] = m;
     __syncthreads();
+    CQD_STAMP(3);
+    const int len = pos + 1;
     m = s_red[0];
 #pragma unroll
     for (int w = 1; w < 16; w++) m = fmaxf(m, s_red[w]);
@@ -319,9 +368,10 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
         s_score[j] = e;
         sum += e;
     }
-    sum = wave_sum(sum);
+    sum = wave_sum_all(sum);
     if (lane == 0) s_red[16 + wave] = sum;
     __syncthreads();
+    CQD_STAMP(4);
     float tot = 0.f;
 #pragma unroll
     for (int w = 0; w < 16; w++) tot += s_red[16 + w];
@@ -346,7 +396,7 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
             float vf[8];
             unpack8(vv[u], vf);
 #pragma unroll
-            for (int i = 0; i < 8; i++) acc[i] += p * vf[i];
+            for (int i = 0; i < 8; i++) acc[i] = fmaf(p, vf[i], acc[i]);
         }
     }
     if (row == 0) {
@@ -354,24 +404,30 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
         float vf[8];
         unpack8(reinterpret_cast<const uint4 *>(v + (size_t)kvh * 128)[l16], vf);
 #pragma unroll
-        for (int i = 0; i < 8; i++) acc[i] += p * vf[i];
+        for (int i = 0; i < 8; i++) acc[i] = fmaf(p, vf[i], acc[i]);
     }
+    CQD_STAMP(5);
+    // the four 16-lane rows of a wavefront hold partial sums for the same 128 dimensions: two
+    // halving exchanges leave every lane with 2 of its 8 dimensions summed over the four rows
+    {
+        float h4[4], q2[2];
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        acc[i] += __shfl_xor(acc[i], 16);
-        acc[i] += __shfl_xor(acc[i], 32);
-    }
-    if (lane < 16) {
+        for (int i = 0; i < 4; i++) h4[i] = swap32_add(acc[i], acc[4 + i]);  // lanes >= 32: dimensions 4..7
 #pragma unroll
-        for (int i = 0; i < 8; i++) s_acc[wave][8 * l16 + i] = acc[i];
+        for (int i = 0; i < 2; i++) q2[i] = swap16_add(h4[i], h4[2 + i]);    // odd rows: + 2
+        const int d0 = 8 * l16 + 4 * (lane >> 5) + 2 * ((lane >> 4) & 1);
+        s_acc[wave][d0] = q2[0];
+        s_acc[wave][d0 + 1] = q2[1];
     }
     __syncthreads();
+    CQD_STAMP(6);
     if (t < 128) {
         float o = 0.f;
 #pragma unroll
         for (int w = 0; w < 16; w++) o += s_acc[w][t];
         out[(size_t)head * 128 + t] = __float2half_rn(o);
     }
+    CQD_STAMP(7);
 }
 
 // out <- fp16(silu(gate)) * up
@@ -469,7 +525,7 @@ hipError_t launch_rope_cache(__half *q, const __half *k, const __half *v, __half
                              const int *pos, int n_heads, int n_kv_heads, int head_dim, int max_len, float theta,
                              hipStream_t stream) {
     hipLaunchKernelGGL(rope_cache_kernel, dim3(n_heads + n_kv_heads), dim3(head_dim / 2), 0, stream, q, k, v, k_cache,
-                       v_cache, pos, n_heads, n_kv_heads, head_dim, max_len, theta);
+                       v_cache, pos, n_heads, n_kv_heads, head_dim, max_len, rope_base(theta));
     return hipGetLastError();
 }
 
@@ -485,7 +541,7 @@ hipError_t launch_rope_attn_decode(const __half *q, const __half *k, const __hal
                                    __half *v_cache, __half *out, const int *pos, int n_heads, int n_kv_heads,
                                    int max_len, float theta, float scale, hipStream_t stream) {
     hipLaunchKernelGGL(rope_attn_decode_kernel, dim3(n_heads), dim3(1024), 0, stream, q, k, v, k_cache, v_cache, out,
-                       pos, n_heads, n_kv_heads, max_len, theta, scale);
+                       pos, n_heads, n_kv_heads, max_len, rope_base(theta), scale);
     return hipGetLastError();
 }
 

@@ -112,43 +112,8 @@ __device__ inline float norm_scale(const u32x4 (&chunk)[kNormLoads], float *s_ss
     return rsqrtf(t / (float)K + eps);
 }
 
-// all-reduce over the 16 lanes of a DPP row by rotations 8, 4, 2, 1
-__device__ inline float row_sum(float v) {
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false));
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x122, 0xf, 0xf, false));
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xf, 0xf, false));
-    return v;
-}
-
-__device__ inline int row_max(int v) {
-    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x128, 0xf, 0xf, false));
-    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x124, 0xf, 0xf, false));
-    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x122, 0xf, 0xf, false));
-    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x121, 0xf, 0xf, false));
-    return v;
-}
-
 __device__ inline float half_bits_to_float(uint32_t h) {
     return __half2float(__ushort_as_half((unsigned short)h));
-}
-
-// v_permlane32_swap_b32 exchanges lanes 32..63 of its first operand with lanes 0..31 of its
-// second; v_permlane16_swap_b32 exchanges the odd 16-lane rows of the first with the even rows
-// of the second.  Written as inline assembly because the compiler builtin of this toolchain
-// returns the first result twice; the s_nop pad the VALU->permlane-swap data hazards that the
-// compiler cannot see through an asm statement.
-//
-// swap32_add: lanes < 32 return a[l] + a[l+32], lanes >= 32 return b[l-32] + b[l].
-__device__ inline float swap32_add(float a, float b) {
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-    return a + b;
-}
-
-// swap16_add: even rows return a[row] + a[row+1], odd rows return b[row-1] + b[row].
-__device__ inline float swap16_add(float a, float b) {
-    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-    return a + b;
 }
 
 // KPL = compacted positions per lane group (16 or 32); a unit is 4 * KPL positions.
