@@ -26,17 +26,9 @@ extern __device__ unsigned long long *g_cq_trace;
 
 namespace cq {
 
-__device__ inline float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    return v;
-}
-
-__device__ inline float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
-    return v;
-}
+// wavefront-wide sum / maximum, delivered to every lane (DPP rotations and permlane swaps, no LDS)
+__device__ inline float wave_sum(float v) { return wave_sum_all(v); }
+__device__ inline float wave_max(float v) { return wave_max_all(v); }
 
 // h <- h + delta (skipped when delta is null);  y <- weight * fp16(h * rsqrt(mean(h^2) + eps))
 // One workgroup; a thread takes 4 consecutive elements (one 8-byte access) per pass.  H % 4 == 0.
@@ -167,11 +159,7 @@ __global__ void rope_cache_kernel(__half *__restrict__ q, const __half *__restri
 // the reference does), fp32 accumulation.  head_dim must be 128, max_len <= kMaxAttnLen.
 constexpr int kMaxAttnLen = 4096;
 
-__device__ inline float row16_sum(float v) {
-#pragma unroll
-    for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 16);
-    return v;
-}
+__device__ inline float row16_sum(float v) { return row_sum(v); }
 
 __device__ inline void unpack8(const uint4 &u, float (&f)[8]) {
     const __half2 *h = reinterpret_cast<const __half2 *>(&u);

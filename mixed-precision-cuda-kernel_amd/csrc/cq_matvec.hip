@@ -100,8 +100,7 @@ __device__ inline float norm_scale(const u32x4 (&chunk)[kNormLoads], float *s_ss
             const float b = __half2float(__ushort_as_half((unsigned short)(chunk[i][j] >> 16)));
             ss += a * a + b * b;
         }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+    ss = wave_sum_all(ss);
     if (lane == 0) s_ss[wave] = ss;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
