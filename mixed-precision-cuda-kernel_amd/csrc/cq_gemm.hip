@@ -13,15 +13,19 @@
 //     pair of codes, OR-ing 0x6400 into each half makes them the fp16 numbers 1024 + u * 2^p,
 //     one packed fp16 fma turns that into u - c_b (exact) and one packed multiply applies the
 //     group scale (one rounding, the reference's);
-//   * the activations of the step (128 rows x 64 positions) come from a compacted copy made by a
-//     small kernel in front (gathered around the cherry channels, zero padded to whole tiles, in
-//     the same position order inside every group of 8 as the code pairs above);
-//   * every wavefront runs 16 v_mfma_f32_32x32x16_f16 on its 64 x 64 quarter, operands read from
-//     LDS with ds_read_b128 (rows padded to 144 bytes: conflict free).
-// LDS is double buffered and a ring of four register sets keeps the global loads three steps
-// ahead of their dequantisation; one barrier per step.  Cherry rows are further steps whose B
-// operands are the fp16 rows themselves.  The kernel is bound by LDS traffic (each 32 x 32 x 16
-// MFMA needs one 1 KB operand read on average), not by the matrix cores.
+//   * the activations never pass through LDS: a small kernel in front writes a compacted copy
+//     (gathered around the cherry channels, zero padded to whole tiles, same position order inside
+//     every group of 8 as the code pairs above) in the matrix cores' A-fragment order, one
+//     contiguous 1 KB block per (32 rows, 16 positions), and every wavefront loads its fragments
+//     from there straight into registers (the two wavefronts that share rows hit the same lines
+//     in the CU's vector cache);
+//   * every wavefront runs 16 v_mfma_f32_32x32x16_f16 on its 64 x 64 quarter, B operands read
+//     from LDS with ds_read_b128 (rows padded to 144 bytes: conflict free).
+// The B tile is double buffered in LDS and rings of three register sets keep the global loads
+// (fragments and packed codes) two steps ahead of their use; one barrier per step.  Cherry rows
+// are further steps whose B operands are the fp16 rows themselves.  With both operands in LDS the
+// kernel was bound by LDS bandwidth (about 64 bytes per clock and CU for 16-byte accesses);
+// keeping A out of it halves that traffic.
 //
 // K splits (when the tiles alone would leave CUs idle) meet in per-split fp32 partial tiles and
 // one ticket per output tile; the last workgroup adds the partials in split order, so the result
@@ -41,15 +45,11 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-// Output tile: 128 rows x 64 * WN columns, WN wave columns (2 x WN wavefronts); the library
-// instantiates WN = 2.
-constexpr int kGemmTM = 128, kGemmTK = 64;
+constexpr int kGemmTM = 128, kGemmTN = 128, kGemmTK = 64;
 constexpr int kGemmPitch = kGemmTK * 2 + 16;               // bytes per LDS row
-constexpr int kGemmStageA = kGemmTM * kGemmPitch;          // activations, one stage
-constexpr int gemm_stage_b(int wn) { return 64 * wn * kGemmPitch; }
-constexpr int gemm_lds_bytes(int wn) { return 2 * (kGemmStageA + gemm_stage_b(wn)); }
+constexpr int kGemmStageB = kGemmTN * kGemmPitch;          // dequantised weights, one stage
 constexpr int kGemmMaxSplits = 8;
-constexpr int kGemmResidentWgs = 512;  // 256 CUs x 2 workgroups (LDS: 72 KB each)
+constexpr int kGemmResidentWgs = 512;  // 256 CUs x 2 workgroups (two waves per SIMD at this register count)
 constexpr uint32_t kRsrcFlagsG = 0x00020000u;
 constexpr uint32_t kOobG = 0x80000000u;
 
@@ -69,8 +69,7 @@ __host__ __device__ constexpr int gemm_pos(int kk) {
 GemmPlan gemm_plan(int M, int K, int N, int C) {
     GemmPlan p;
     p.mtiles = ceil_div(M, kGemmTM);
-    p.wn = 2;  // 256-column tiles (wn = 4, one workgroup of eight waves per CU) measured 0-10 % slower
-    p.ntiles = ceil_div(N, 64 * p.wn);
+    p.ntiles = ceil_div(N, kGemmTN);
     p.steps_normal = ceil_div(K - C, kGemmTK);
     p.steps_total = p.steps_normal + ceil_div(C, kGemmTK);
     p.Kp = p.steps_total * kGemmTK;
@@ -88,15 +87,16 @@ GemmPlan gemm_plan(int M, int K, int N, int C) {
     p.workspace_bytes = ((size_t)tiles * sizeof(unsigned) + 255) / 256 * 256;
     // scratch: compacted activations, then the partial tiles
     p.a_bytes = ((size_t)p.Mp * p.Kp * sizeof(__half) + 255) / 256 * 256;
-    p.partial_bytes = p.splits > 1 ? (size_t)p.splits * tiles * kGemmTM * 64 * p.wn * sizeof(float) : 0;
+    p.partial_bytes = p.splits > 1 ? (size_t)p.splits * tiles * kGemmTM * kGemmTN * sizeof(float) : 0;
     p.scratch_bytes = p.a_bytes + (p.partial_bytes + 255) / 256 * 256;
     return p;
 }
 
 // ---- activation compaction -----------------------------------------------------------------------
-// One thread per (row, group of 8 positions): A[row][8 g + kk] = x[row][normal(8 g + ord[kk])] in
-// the normal part, x[row][idx[c]] in the cherry part, 0 in the padding (rows >= M, positions past
-// the end).
+// One thread per (row, group of 8 positions): x[row][normal(8 g + ord[kk])] in the normal part,
+// x[row][idx[c]] in the cherry part, 0 in the padding (rows >= M, positions past the end).  The 16
+// bytes go where the matrix core wants them: block (row / 32, g / 2) of 1 KB, lane (g % 2) * 32 +
+// row % 32 -- the A fragment of v_mfma_f32_32x32x16_f16 for 32 rows x 16 positions.
 template <int BITS>
 __global__ __launch_bounds__(256) void gemm_prep_kernel(const __half *__restrict__ x,
                                                         const int16_t *__restrict__ cherry_indices,
@@ -132,20 +132,17 @@ __global__ __launch_bounds__(256) void gemm_prep_kernel(const __half *__restrict
                 if (c0 + kk < C) h[kk] = __half_as_ushort(xr[(int)cherry_indices[c0 + kk]]);
         }
     }
-    a[(size_t)row * (Kp / 8) + g] =
+    const size_t block = (size_t)(row >> 5) * (Kp / 16) + (g >> 1);
+    a[block * 64 + (g & 1) * 32 + (row & 31)] =
         make_uint4(h[0] | h[1] << 16, h[2] | h[3] << 16, h[4] | h[5] << 16, h[6] | h[7] << 16);
 }
 
 // ---- main kernel ---------------------------------------------------------------------------------
-// What a thread holds of one K step between the global loads and the LDS writes.
+// What a thread holds of one K step between the global loads and their use.
 struct GemmStepRegs {
-    uint32_t w[4];  // 4 (3) byte rows x 4 columns
+    uint32_t w[4];      // 4 (3) byte rows x 4 columns of packed codes
     uint32_t sc0, sc1;  // the 4 columns' group scales
-    u32x4 a[4];     // 8 / WN rows x 8 positions of activations
-};
-struct GemmCherryRegs {
-    u32x2 w[8];     // 8 cherry rows x 4 columns of fp16
-    u32x4 a[4];
+    u32x4 a[2][4];      // A fragments: 2 row tiles of 32 x 4 sub-steps of 16 positions
 };
 
 // Packed fp16 constants per output dword d (low half: kk = 2 d, high half: kk = 2 d + 1).  With
@@ -169,30 +166,24 @@ struct GemmConst {
     }
 };
 
-template <int BITS, int WN>
-__global__ __launch_bounds__(128 * WN) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_kernel(
+template <int BITS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_kernel(
     const uint8_t *__restrict__ qweight, const __half *__restrict__ cherry_weight,
-    const __half *__restrict__ scales, __half *__restrict__ out, const __half *__restrict__ a_compact,
+    const __half *__restrict__ scales, __half *__restrict__ out, const __half *__restrict__ a_frag,
     float *__restrict__ partial, unsigned *__restrict__ tickets, int M, int K, int N, int C, int G,
     int accumulate, GemmPlan plan) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char s_lds[];
-    constexpr int kStageB = gemm_stage_b(WN);
-    constexpr int TN = 64 * WN;
-    constexpr int APT = 8 / WN;                               // activation chunks per thread and step
-    unsigned char *const s_a = s_lds;                         // [2][128][pitch]
-    unsigned char *const s_b = s_lds + 2 * kGemmStageA;       // [2][TN][pitch]
+    __shared__ __attribute__((aligned(16))) unsigned char s_b[2 * kGemmStageB];  // [2][128 columns][pitch]
 
     constexpr int R = BITS == 4 ? 4 : 3;  // byte rows per 8 positions
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WN, wn = wave % WN;
+    const int wm = wave >> 1, wn = wave & 1;
     const int ntile = blockIdx.x % plan.ntiles, mtile = blockIdx.x / plan.ntiles, split = blockIdx.y;
-    const int m0 = mtile * kGemmTM, n0 = ntile * TN;
+    const int m0 = mtile * kGemmTM, n0 = ntile * kGemmTN;
     const int Kn = K - C;
-    // staging roles: B -- column quad cq, position group kg; A -- row ar (+32 i), chunk ac
-    // (16 consecutive lanes = 4 column quads x 4 position groups: their 16-byte LDS writes, 144
-    // bytes apart per row, then fall into 16 different bank groups)
-    const int cq = (wave % WN) * 16 + (lane >> 4) * 4 + (lane & 3), kg = (wave / WN) * 4 + ((lane >> 2) & 3);
-    const int ar = tid >> 3, ac = tid & 7;
+    // B staging roles: column quad cq, position group kg.  16 consecutive lanes = 4 column quads x 4
+    // position groups: their 16-byte LDS writes, 144 bytes apart per row, then fall into 16
+    // different bank groups.
+    const int cq = wn * 16 + (lane >> 4) * 4 + (lane & 3), kg = wm * 4 + ((lane >> 2) & 3);
     const bool col_ok = n0 + 4 * cq < N;
 
     const __amdgpu_buffer_rsrc_t rw =
@@ -201,20 +192,18 @@ __global__ __launch_bounds__(128 * WN) __attribute__((amdgpu_waves_per_eu(2, 2))
         __builtin_amdgcn_make_buffer_rsrc((void *)scales, 0, ceil_div(Kn, G) * N * 2, kRsrcFlagsG);
     const __amdgpu_buffer_rsrc_t rc =
         __builtin_amdgcn_make_buffer_rsrc((void *)cherry_weight, 0, C * N * 2, kRsrcFlagsG);
-    const u32x4 *arow = reinterpret_cast<const u32x4 *>(a_compact) + (size_t)(m0 + ar) * (plan.Kp / 8) + ac;
+    // this wave's A fragments: row tiles (m0 / 32 + 2 wm + i), blocks of 64 lanes x 16 bytes
+    const u32x4 *afrag = reinterpret_cast<const u32x4 *>(a_frag) +
+                         ((size_t)(m0 / 32 + 2 * wm) * (plan.Kp / 16)) * 64 + lane;
+    const size_t afrag_tile = (size_t)(plan.Kp / 16) * 64;
 
-    auto load_a = [=](u32x4 (&av)[4], int st) {
+    auto load_a = [=](u32x4 (&av)[2][4], int st) {
 #pragma unroll
-        for (int i = 0; i < APT; i++) av[i] = arow[(size_t)(16 * WN * i) * (plan.Kp / 8) + st * 8];
-    };
-    auto store_a = [=](const u32x4 (&av)[4], int buf) {
-        unsigned char *sa = s_a + buf * kGemmStageA;
+        for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int i = 0; i < APT; i++)
-            *reinterpret_cast<u32x4 *>(sa + (ar + 16 * WN * i) * kGemmPitch + ac * 16) = av[i];
+            for (int ks = 0; ks < 4; ks++) av[i][ks] = afrag[i * afrag_tile + (size_t)(st * 4 + ks) * 64];
     };
     auto load_step = [=](GemmStepRegs &r, int st) {
-        load_a(r.a, st);
         const uint32_t woff = col_ok ? (uint32_t)((st * 8 + kg) * R * N + n0 + 4 * cq) : kOobG;
 #pragma unroll
         for (int i = 0; i < R; i++) r.w[i] = __builtin_amdgcn_raw_buffer_load_b32(rw, woff + (uint32_t)(i * N), 0, 0);
@@ -223,31 +212,11 @@ __global__ __launch_bounds__(128 * WN) __attribute__((amdgpu_waves_per_eu(2, 2))
         const u32x2 sv = __builtin_amdgcn_raw_buffer_load_b64(rs, soff, 0, 0);
         r.sc0 = sv[0];
         r.sc1 = sv[1];
-    };
-    auto load_cherry = [=](GemmCherryRegs &r, int st) {
         load_a(r.a, st);
-        const int c0 = (st - plan.steps_normal) * kGemmTK + 8 * kg;
-        const uint32_t coff = col_ok ? (uint32_t)(c0 * N + n0 + 4 * cq) * 2u : kOobG;
-#pragma unroll
-        for (int i = 0; i < 8; i++) r.w[i] = __builtin_amdgcn_raw_buffer_load_b64(rc, coff + (uint32_t)(i * N * 2), 0, 0);
     };
-    auto store_cherry = [=](const GemmCherryRegs &r, int buf) {
-        store_a(r.a, buf);
-        unsigned char *sb = s_b + buf * kStageB;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;  // (row r half, row r + 1 half)
-            u32x4 o;
-#pragma unroll
-            for (int d = 0; d < 4; d++) o[d] = __builtin_amdgcn_perm(r.w[2 * d + 1][j >> 1], r.w[2 * d][j >> 1], sel);
-            *reinterpret_cast<u32x4 *>(sb + (4 * cq + j) * kGemmPitch + kg * 16) = o;
-        }
-    };
-
-    // registers -> LDS stage `buf`
+    // packed codes -> fp16 weights -> LDS stage `buf`
     auto store_step = [=](const GemmStepRegs &r, int buf) {
-        store_a(r.a, buf);
-        unsigned char *sb = s_b + buf * kStageB;
+        unsigned char *sb = s_b + buf * kGemmStageB;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             uint32_t f[4];
@@ -295,35 +264,28 @@ __global__ __launch_bounds__(128 * WN) __attribute__((amdgpu_waves_per_eu(2, 2))
 
     const int st_begin = split * plan.steps_per_split;
     const int st_end = min(st_begin + plan.steps_per_split, plan.steps_total);
-    const int frag_row = lane & 31, frag_k = (lane >> 5) * 16;  // byte offset of the lane's 8 positions
-
-    const unsigned char *sa0 = s_a + (wm * 64 + frag_row) * kGemmPitch + frag_k;
-    const unsigned char *sb0 = s_b + (wn * 64 + frag_row) * kGemmPitch + frag_k;
-    auto compute = [&](int buf) {
-        const unsigned char *sa = sa0 + buf * kGemmStageA;
-        const unsigned char *sb = sb0 + buf * kStageB;
+    const unsigned char *sb0 = s_b + (wn * 64 + (lane & 31)) * kGemmPitch + (lane >> 5) * 16;
+    auto compute = [&](const u32x4 (&av)[2][4], int buf) {
+        const unsigned char *sb = sb0 + buf * kGemmStageB;
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
-            half8_t af[2], bf[2];
+            half8_t bf[2];
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                af[i] = *reinterpret_cast<const half8_t *>(sa + i * 32 * kGemmPitch + ks * 32);
-                bf[i] = *reinterpret_cast<const half8_t *>(sb + i * 32 * kGemmPitch + ks * 32);
-            }
+            for (int j = 0; j < 2; j++) bf[j] = *reinterpret_cast<const half8_t *>(sb + j * 32 * kGemmPitch + ks * 32);
 #pragma unroll
             for (int i = 0; i < 2; i++)
 #pragma unroll
                 for (int j = 0; j < 2; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, av[i][ks]), bf[j],
+                                                                      acc[i][j], 0, 0, 0);
         }
     };
     // Packed steps.  Ring of kRing register sets: the global loads of step st + kRing - 1 are issued
-    // while step st is computed, so a load has kRing - 2 whole steps to arrive before its
-    // dequantisation.  The steady-state loop has no branches inside (four steps per trip, every
-    // load and store unconditional): only then does the compiler's wait-count bookkeeping let
-    // the younger loads stay in flight instead of draining the queue in every step.
+    // while step st is computed.  The steady-state loop has no branches inside (kRing * 2 steps per
+    // trip, every load and store unconditional): only then does the compiler's wait-count
+    // bookkeeping let the younger loads stay in flight instead of draining the queue in every step.
     {
-        constexpr int kRing = 4;
+        constexpr int kRing = 3;
         const int n_end = min(st_end, plan.steps_normal);
         GemmStepRegs regs[kRing];
 #pragma unroll
@@ -332,22 +294,22 @@ __global__ __launch_bounds__(128 * WN) __attribute__((amdgpu_waves_per_eu(2, 2))
         if (st_begin < n_end) store_step(regs[0], 0);
         __syncthreads();
         int base = st_begin;
-        for (; base + 2 * kRing - 1 <= n_end; base += kRing) {  // all of st + kRing - 1 < n_end
+        for (; base + 3 * kRing - 1 <= n_end; base += 2 * kRing) {  // all of st + kRing - 1 < n_end
 #pragma unroll
-            for (int r = 0; r < kRing; r++) {
+            for (int r = 0; r < 2 * kRing; r++) {
                 load_step(regs[(r + kRing - 1) % kRing], base + r + kRing - 1);
-                compute(r & 1);
+                compute(regs[r % kRing].a, r & 1);
                 store_step(regs[(r + 1) % kRing], (r & 1) ^ 1);
                 __syncthreads();
             }
         }
-        for (; base < n_end; base += kRing) {  // the last steps, guarded
+        for (; base < n_end; base += 2 * kRing) {  // the last steps, guarded
 #pragma unroll
-            for (int r = 0; r < kRing; r++) {
+            for (int r = 0; r < 2 * kRing; r++) {
                 const int st = base + r;
                 if (st < n_end) {  // uniform
                     if (st + kRing - 1 < n_end) load_step(regs[(r + kRing - 1) % kRing], st + kRing - 1);
-                    compute(r & 1);
+                    compute(regs[r % kRing].a, r & 1);
                     if (st + 1 < n_end) store_step(regs[(r + 1) % kRing], (r & 1) ^ 1);
                     __syncthreads();
                 }
@@ -356,11 +318,23 @@ __global__ __launch_bounds__(128 * WN) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     // Cherry steps (one or two per call): plain load, stage, compute.
     for (int st = max(st_begin, plan.steps_normal); st < st_end; st++) {
-        GemmCherryRegs cr;
-        load_cherry(cr, st);
-        store_cherry(cr, 0);
+        u32x4 av[2][4];
+        u32x2 cw[8];  // 8 cherry rows x 4 columns of fp16
+        load_a(av, st);
+        const int c0 = (st - plan.steps_normal) * kGemmTK + 8 * kg;
+        const uint32_t coff = col_ok ? (uint32_t)(c0 * N + n0 + 4 * cq) * 2u : kOobG;
+#pragma unroll
+        for (int i = 0; i < 8; i++) cw[i] = __builtin_amdgcn_raw_buffer_load_b64(rc, coff + (uint32_t)(i * N * 2), 0, 0);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;  // (row r half, row r + 1 half)
+            u32x4 o;
+#pragma unroll
+            for (int d = 0; d < 4; d++) o[d] = __builtin_amdgcn_perm(cw[2 * d + 1][j >> 1], cw[2 * d][j >> 1], sel);
+            *reinterpret_cast<u32x4 *>(s_b + (4 * cq + j) * kGemmPitch + kg * 16) = o;
+        }
         __syncthreads();
-        compute(0);
+        compute(av, 0);
         __syncthreads();
     }
 
@@ -369,7 +343,7 @@ __global__ __launch_bounds__(128 * WN) __attribute__((amdgpu_waves_per_eu(2, 2))
     if (plan.splits > 1) {
         // partial tiles in the accumulators' own order: element q of a lane at [q][lane], so that
         // every store and load instruction covers 256 contiguous bytes
-        const size_t tile_elems = (size_t)kGemmTM * TN;
+        const size_t tile_elems = (size_t)kGemmTM * kGemmTN;
         const size_t tiles = (size_t)plan.mtiles * plan.ntiles;
         float *mine = partial + ((size_t)split * tiles + blockIdx.x) * tile_elems + wave * 4096 + lane;
 #pragma unroll
@@ -380,7 +354,7 @@ __global__ __launch_bounds__(128 * WN) __attribute__((amdgpu_waves_per_eu(2, 2))
                 for (int e = 0; e < 16; e++)
                     __hip_atomic_store(mine + ((i * 2 + j) * 16 + e) * 64, acc[i][j][e], __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
-        int *s_last = reinterpret_cast<int *>(s_lds);  // the stages have been consumed
+        int *s_last = reinterpret_cast<int *>(s_b);  // the stages have been consumed
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
@@ -450,7 +424,7 @@ bool gemm_supported(int bits, int M, int K, int N, int C, int G) {
     return true;
 }
 
-template <int BITS, int WN>
+template <int BITS>
 static hipError_t launch_gemm_bits(const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
                                    const int16_t *cherry_indices, const __half *scales, __half *mul, int M, int K,
                                    int N, int C, int G, int accumulate, void *workspace, void *scratch,
@@ -459,22 +433,10 @@ static hipError_t launch_gemm_bits(const __half *vec, const uint8_t *qweight, co
     __half *a = reinterpret_cast<__half *>(scratch);
     float *partial = reinterpret_cast<float *>(reinterpret_cast<char *>(scratch) + plan.a_bytes);
     unsigned *tickets = reinterpret_cast<unsigned *>(workspace);
-    // more than 64 KB of LDS per workgroup has to be requested once per device
-    static bool lds_set[64] = {};
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    if (dev < 0 || dev >= 64 || !lds_set[dev]) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<BITS, WN>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, gemm_lds_bytes(WN));
-        if (e != hipSuccess) return e;
-        if (dev >= 0 && dev < 64) lds_set[dev] = true;
-    }
     hipLaunchKernelGGL(gemm_prep_kernel<BITS>, dim3(ceil_div(plan.Kp / 8, 256), plan.Mp), dim3(256), 0, stream, vec,
                        cherry_indices, reinterpret_cast<uint4 *>(a), M, K, C, plan.Kp, plan.steps_normal * 8);
-    hipLaunchKernelGGL((gemm_kernel<BITS, WN>), dim3(plan.mtiles * plan.ntiles, plan.splits), dim3(128 * WN),
-                       gemm_lds_bytes(WN), stream, qweight, cherry_weight, scales, mul, a, partial, tickets, M, K, N,
-                       C, G, accumulate, plan);
+    hipLaunchKernelGGL(gemm_kernel<BITS>, dim3(plan.mtiles * plan.ntiles, plan.splits), dim3(256), 0, stream, qweight,
+                       cherry_weight, scales, mul, a, partial, tickets, M, K, N, C, G, accumulate, plan);
     return hipGetLastError();
 }
 
@@ -482,10 +444,10 @@ hipError_t launch_gemm(int bits, const __half *vec, const uint8_t *qweight, cons
                        const int16_t *cherry_indices, const __half *scales, __half *mul, int M, int K, int N, int C,
                        int G, int accumulate, void *workspace, void *scratch, hipStream_t stream) {
     if (bits == 4)
-        return launch_gemm_bits<4, 2>(vec, qweight, cherry_weight, cherry_indices, scales, mul, M, K, N, C, G,
-                                      accumulate, workspace, scratch, stream);
-    return launch_gemm_bits<3, 2>(vec, qweight, cherry_weight, cherry_indices, scales, mul, M, K, N, C, G, accumulate,
-                                  workspace, scratch, stream);
+        return launch_gemm_bits<4>(vec, qweight, cherry_weight, cherry_indices, scales, mul, M, K, N, C, G, accumulate,
+                                   workspace, scratch, stream);
+    return launch_gemm_bits<3>(vec, qweight, cherry_weight, cherry_indices, scales, mul, M, K, N, C, G, accumulate,
+                               workspace, scratch, stream);
 }
 
 }  // namespace cq

@@ -71,7 +71,7 @@ size_t scratch_bytes(int B, int K, int N, int C);
 
 // cq_gemm.hip: more than 16 rows (prompt processing) -- dequantise into LDS, fp16 MFMA tiles.
 struct GemmPlan {
-    int mtiles, ntiles, wn;           // output tiles of 128 rows x 64 * wn columns
+    int mtiles, ntiles;               // 128 x 128 output tiles
     int steps_normal, steps_total;    // K steps of 64 positions: packed part, then the cherry rows
     int Kp, Mp;                       // padded sizes of the compacted activation copy
     int splits, steps_per_split;      // K splits (grid.y)
