@@ -617,6 +617,39 @@ def test_prefill_rows_dequantise_once_then_gemm(qc, bits, k, n, rows):
     assert orc.rel_l2(y.cpu().numpy(), y_fused.cpu().numpy().astype(np.float64)) <= 2 * TOL
 
 
+def test_gemm_buffers_are_checked_through_the_c_abi(qc):
+    """Raw C-ABI call with 64 rows: buffers sized for 16 rows are refused (nothing is launched), the
+    sizes the library asks for are accepted."""
+    announce("gemm c-abi buffers")
+    lib = qc._lib
+    bits, k, n, rows = 4, 2048, 512, 64
+    p = orc.synthetic_packed_fast(k, n, bits, 128, seed=5)
+    d = dev(p)
+    c = d["cherry_indices"].numel()
+    x = torch.randn(rows, k, device="cuda").half()
+    out = torch.full((rows, n), 5.0, dtype=torch.float16, device="cuda")
+    small_ws, small_sc = lib.cherryq_workspace_bytes(16, k, n, c), lib.cherryq_scratch_bytes(16, k, n, c)
+    ws_b, sc_b = lib.cherryq_workspace_bytes(rows, k, n, c), lib.cherryq_scratch_bytes(rows, k, n, c)
+    assert sc_b > small_sc and ws_b >= small_ws
+    ws = torch.zeros(ws_b, dtype=torch.uint8, device="cuda")
+    sc = torch.empty(sc_b, dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def call(scratch_bytes):
+        return lib.cherryq_vecquant4matmul_f16(x.data_ptr(), d["qweight"].data_ptr(), d["cherry_weight"].data_ptr(),
+                                               d["cherry_indices"].data_ptr(), d["scales"].data_ptr(), out.data_ptr(),
+                                               rows, k, n, c, 128, 0, ws.data_ptr(), ws_b, sc.data_ptr(),
+                                               scratch_bytes, stream)
+    assert call(small_sc) == -4
+    torch.cuda.synchronize()
+    assert bool((out == 5.0).all())
+    assert call(sc_b) == 0
+    torch.cuda.synchronize()
+    cols, sub = column_sample(p, np.random.default_rng(0), 256)
+    assert orc.rel_l2(out.cpu().numpy()[:, cols], c_oracle.fused(x.cpu().numpy(), sub, bits, 128)) <= TOL
+    assert not ws.any()   # the workspace is left zeroed
+
+
 def test_empty_batch_is_a_no_op(qc):
     """Zero activation rows: nothing is launched, through the entry point and through the module."""
     announce("empty batch")
