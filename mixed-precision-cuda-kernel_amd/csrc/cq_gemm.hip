@@ -81,7 +81,10 @@ GemmPlan gemm_plan(int M, int K, int N, int C) {
     // more start a second round and double the time), at least 8 steps each
     while (splits < kGemmMaxSplits && tiles * (splits + 1) <= kGemmResidentWgs && p.steps_total / (splits + 1) >= 8)
         splits++;
+    // steps per split: 2 + 6 k, the trip structure of the kernel's branch-free loop (two steps of
+    // lead-in, six per trip); only the last split may be ragged
     p.steps_per_split = ceil_div(p.steps_total, splits);
+    if (splits > 1) p.steps_per_split = 2 + 6 * ceil_div(max(p.steps_per_split - 2, 1), 6);
     p.splits = ceil_div(p.steps_total, p.steps_per_split);
     // zero-kept workspace: one ticket per output tile
     p.workspace_bytes = ((size_t)tiles * sizeof(unsigned) + 255) / 256 * 256;
@@ -303,7 +306,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 __syncthreads();
             }
         }
-        for (; base < n_end; base += 2 * kRing) {  // the last steps, guarded
+        if (n_end - base == 2) {  // the usual remainder: two steps whose operands are already loaded
+            compute(regs[0].a, 0);
+            store_step(regs[1], 1);
+            __syncthreads();
+            compute(regs[1].a, 1);
+            __syncthreads();
+            base = n_end;
+        }
+        for (; base < n_end; base += 2 * kRing) {  // any other remainder, guarded
 #pragma unroll
             for (int r = 0; r < 2 * kRing; r++) {
                 const int st = base + r;
