@@ -578,9 +578,12 @@ def test_gemm_accumulate_linearity_and_determinism(qc):
     cols, sub = column_sample(p, rng, 256)
     want = c_oracle.fused(x, sub, bits, 128)
     assert orc.rel_l2(y2[:, cols], want + base[:, cols].astype(np.float64)) <= TOL
-    # f(2 x) == 2 f(x) exactly: powers of two commute with every rounding involved
+    # f(2 x) == 2 f(x) exactly: powers of two commute with every rounding involved, except where
+    # f(x) is an fp16 subnormal (its last bit is lost before the doubling)
     y4 = run_fused(qc, bits, (x * np.float16(2)).astype(np.float16), p, 128)
-    np.testing.assert_array_equal(y4, (y1.astype(np.float32) * 2).astype(np.float16))
+    normal = np.abs(y1.astype(np.float32)) >= 2.0 ** -14
+    np.testing.assert_array_equal(y4[normal], (y1.astype(np.float32) * 2).astype(np.float16)[normal])
+    assert np.abs(y4.astype(np.float32) - 2 * y1.astype(np.float32))[~normal].max(initial=0.0) <= 2.0 ** -23
     # rows do not interact: a row gives the same bits alone in a 17-row call padded with zeros
     x17 = np.zeros((17, k), dtype=np.float16)
     x17[3] = x[77]
