@@ -241,11 +241,21 @@ __global__ __launch_bounds__(256) void unpack_kernel(const uint8_t *__restrict__
     __shared__ unsigned short s_norm[kUnpackRows][kUnpackUnits * 8 + 2];
     __shared__ unsigned short s_ch[kUnpackCols][kUnpackRows];
     __shared__ short s_src[kUnpackCols];
+    // the index list is searched several times per thread: from LDS when it fits (a search in global
+    // memory is a chain of dependent loads in front of everything else the workgroup does)
+    constexpr int kIdxCap = 2048;
+    __shared__ int16_t s_idx[kIdxCap];
     const int Kn = K - C;
     const int d0 = blockIdx.x * kUnpackCols, d1 = min(d0 + kUnpackCols, K);
     const int n0 = blockIdx.y * kUnpackRows;
     const int t = threadIdx.x;
-    const int c_lo = cherries_below(cherry_indices, C, d0), c_hi = cherries_below(cherry_indices, C, d1);
+    const int16_t *idx = cherry_indices;
+    if (C <= kIdxCap) {
+        for (int i = t; i < C; i += 256) s_idx[i] = cherry_indices[i];
+        __syncthreads();
+        idx = s_idx;
+    }
+    const int c_lo = cherries_below(idx, C, d0), c_hi = cherries_below(idx, C, d1);
     const int k_lo = d0 - c_lo, k_hi = d1 - c_hi;  // normal positions of this column range
     const int ku0 = k_lo & ~7;
     const int units = k_hi > k_lo ? ceil_div(k_hi - ku0, 8) : 0;
@@ -253,8 +263,8 @@ __global__ __launch_bounds__(256) void unpack_kernel(const uint8_t *__restrict__
         const int d = d0 + t;
         short src = 0;
         if (d < d1) {
-            const int c = cherries_below(cherry_indices, C, d);
-            src = (c < C && (int)cherry_indices[c] == d) ? (short)(-1 - (c - c_lo)) : (short)(d - c - ku0);
+            const int c = cherries_below(idx, C, d);
+            src = (c < C && (int)idx[c] == d) ? (short)(-1 - (c - c_lo)) : (short)(d - c - ku0);
         }
         s_src[t] = src;
     }
