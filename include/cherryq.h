@@ -161,6 +161,27 @@ int cherryq_pack_f16(int w_bits, const void *weight, const int16_t *cherry_indic
                      int group_size, void *stream);
 
 /*
+ * The training-side forward's weight (QuantLinear._adjust_weight, llama/cherry_linear.py:77-99
+ * of the reference): `out` = `weight` (out_features, in_features), row-major, with every
+ * NON-cherry input channel replaced by FullSymQuantizer.transform of it
+ * (llama/quantizer.py:165-170) under per-row scales of `group_size` consecutive compacted normal
+ * channels (llama/cherry_linear.py:69-75, llama/quantizer.py:148-152), every operation rounded
+ * to the weight's dtype as torch does: bit for bit the reference's result for fp16 and fp32
+ * weights.  ste != 0 gives the straight-through form the training branch feeds to the matmul,
+ * (q - w) + w evaluated in the weight dtype on every channel (:97-98); ste == 0 is what
+ * prepare_weight_for_inference stores (:48-61).  w_bits 2..4.  cherry_indices (int32, as the
+ * QAT module keeps them) need be neither sorted nor distinct; entries outside
+ * [0, in_features) are ignored.  `out` may be `weight` itself.  No workspace.  Returns
+ * CHERRYQ_E_UNSUPPORTED beyond 65536 input channels or 4096 groups per row.
+ */
+int cherryq_fake_quant_f16(int w_bits, const void *weight, const int32_t *cherry_indices, void *out,
+                           int in_features, int out_features, int num_cherries, int group_size, int ste,
+                           void *stream);
+int cherryq_fake_quant_f32(int w_bits, const void *weight, const int32_t *cherry_indices, void *out,
+                           int in_features, int out_features, int num_cherries, int group_size, int ste,
+                           void *stream);
+
+/*
  * One batch-1 launch over 1..4 packed layers that read the SAME activation vector and share
  * in_features, num_cherries, group_size and w_bits: q/k/v_proj (llama/modeling_llama_quant.py
  * :346-348 of the reference) or gate/up_proj (:251).  Arithmetic per layer is that of

@@ -225,6 +225,32 @@ int cherryq_pack_f16(int w_bits, const void *weight, const int16_t *cherry_indic
                                 C, group_size, reinterpret_cast<hipStream_t>(stream));
 }
 
+static int fake_quant_entry(bool fp32, int w_bits, const void *weight, const int32_t *cherry_indices, void *out,
+                            int in_features, int out_features, int num_cherries, int group_size, int ste,
+                            void *stream) {
+    if (w_bits < 2 || w_bits > 4) return CHERRYQ_E_BITS;
+    const int K = in_features, N = out_features, C = num_cherries;
+    if (K <= 0 || N <= 0 || C < 0) return CHERRYQ_E_SHAPE;
+    if (group_size <= 0) return CHERRYQ_E_GROUP;
+    if (!weight || !out || (C > 0 && !cherry_indices)) return CHERRYQ_E_NULL;
+    if (!cq::aligned(weight, fp32 ? 4 : 2) || !cq::aligned(out, fp32 ? 4 : 2)) return CHERRYQ_E_ALIGN;
+    if (!cq::fake_quant_supported(K, C, group_size)) return CHERRYQ_E_UNSUPPORTED;
+    return (int)cq::launch_fake_quant(w_bits, fp32, weight, cherry_indices, out, K, N, C, group_size, ste,
+                                      reinterpret_cast<hipStream_t>(stream));
+}
+
+int cherryq_fake_quant_f16(int w_bits, const void *weight, const int32_t *cherry_indices, void *out, int in_features,
+                           int out_features, int num_cherries, int group_size, int ste, void *stream) {
+    return fake_quant_entry(false, w_bits, weight, cherry_indices, out, in_features, out_features, num_cherries,
+                            group_size, ste, stream);
+}
+
+int cherryq_fake_quant_f32(int w_bits, const void *weight, const int32_t *cherry_indices, void *out, int in_features,
+                           int out_features, int num_cherries, int group_size, int ste, void *stream) {
+    return fake_quant_entry(true, w_bits, weight, cherry_indices, out, in_features, out_features, num_cherries,
+                            group_size, ste, stream);
+}
+
 int cherryq_probe_stream_read(const void *buf, size_t bytes, void *sink, void *stream) {
     if (!buf || !sink) return CHERRYQ_E_NULL;
     if (bytes >= 0x7fff0000ull) return CHERRYQ_E_SHAPE;

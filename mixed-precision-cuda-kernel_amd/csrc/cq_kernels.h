@@ -90,6 +90,11 @@ hipError_t launch_gemm(int bits, const __half *vec, const uint8_t *qweight, cons
 hipError_t launch_pack(int bits, const __half *w, const int16_t *idx, uint8_t *qweight, __half *scales,
                        __half *cherry_weight, int K, int N, int C, int G, hipStream_t stream);
 
+// cq_fakequant.hip: training-side quantise-dequantise of the non-cherry columns, fp16 or fp32.
+bool fake_quant_supported(int K, int C, int G);
+hipError_t launch_fake_quant(int bits, bool fp32, const void *w, const int32_t *idx, void *out, int K, int N, int C,
+                             int G, int ste, hipStream_t stream);
+
 // cq_probe.hip: roofline reference kernels for the measurement script.
 hipError_t launch_probe_read(const void *buf, size_t bytes, void *sink, hipStream_t stream);
 hipError_t launch_probe_empty(hipStream_t stream);

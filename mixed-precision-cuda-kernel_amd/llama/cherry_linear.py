@@ -1,8 +1,11 @@
-"""Training-time / fake-quant CherryQ linear (host side, plain torch).
+"""Training-time / fake-quant CherryQ linear.
 
 Same surface as the reference's llama/cherry_linear.py: an `nn.Linear` whose weight is fake
 quantised group-wise on the fly, except for the `cherry_indices` input channels, which stay in
-full precision.  It is what `llama.qlinear.QuantLinear.pack()` consumes.
+full precision.  It is what `llama.qlinear.QuantLinear.pack()` consumes.  For fp16 and fp32
+weights on a GPU the fake quantisation is one fused kernel of the HIP library (bit-identical to
+the torch operations it replaces); other dtypes, layer-wise scales and CPU tensors go through
+the torch operations.
 """
 import math
 
@@ -10,6 +13,22 @@ import torch
 import torch.nn as nn
 
 from .quantizer import FullSymQuantizer, RestrictedSymQuantizer
+
+
+class _FakeQuantSTE(torch.autograd.Function):
+    """Fused fake quantisation in the straight-through form  (q - w) + w  of
+    llama/cherry_linear.py:97-98: the forward value is that expression evaluated in the weight
+    dtype, the gradient with respect to the weight is the incoming gradient."""
+
+    @staticmethod
+    def forward(ctx, weight, cherry_indices, w_bits, group_size):
+        import quant_cuda
+        return quant_cuda.fake_quant_cherryq(w_bits, weight.detach().contiguous(), cherry_indices, group_size,
+                                             ste=True)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return grad_output, None, None, None
 
 
 class QuantLinear(nn.Linear):
@@ -60,11 +79,27 @@ class QuantLinear(nn.Linear):
         keep[self.cherry_indices.long()] = False
         return keep.nonzero().squeeze(1)
 
+    def _fused_fake_quant(self, weight) -> bool:
+        """Whether the HIP kernel computes this weight's fake quantisation: GPU tensor, fp16 or
+        fp32, per-row group scales of the full-range quantiser, registered channels."""
+        if not weight.is_cuda or self.quantizer is not FullSymQuantizer or self.weight_layerwise:
+            return False
+        if not getattr(self, "cherry_indices_registered", False):
+            return False  # the torch operations raise on the placeholder indices, as the reference does
+        import quant_cuda
+        return quant_cuda.fake_quant_supported(weight, self.w_bits, self.group_size)
+
     def _adjust_weight(self, weight: torch.Tensor, ste=True):
         """Weight with every non-cherry column fake quantised (groups run over the compacted
         normal columns); with `ste` the result carries the straight-through gradient.
         No clipping is applied (llama/cherry_linear.py:77-99)."""
         assert not self.training or self.cherry_indices_registered, "`cherry_indices` is not registered yet."
+        if self._fused_fake_quant(weight):
+            if ste:
+                return _FakeQuantSTE.apply(weight, self.cherry_indices, self.w_bits, self.group_size)
+            import quant_cuda
+            return quant_cuda.fake_quant_cherryq(self.w_bits, weight.detach().contiguous(), self.cherry_indices,
+                                                 self.group_size, ste=False)
         cols = self._normal_columns(weight.shape[1], weight.device)
         normal = weight.detach().index_select(-1, cols)
         s = self._expand_scaling_factors(self._get_scaling_factors(normal), normal)

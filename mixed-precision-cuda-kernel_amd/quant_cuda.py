@@ -49,6 +49,9 @@ _lib.cherryq_unpack_f16.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _int, _int, _
 _lib.cherryq_unpack_f16.restype = _int
 _lib.cherryq_pack_f16.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp]
 _lib.cherryq_pack_f16.restype = _int
+for _name in ("cherryq_fake_quant_f16", "cherryq_fake_quant_f32"):
+    getattr(_lib, _name).argtypes = [_int, _vp, _vp, _vp, _int, _int, _int, _int, _int, _vp]
+    getattr(_lib, _name).restype = _int
 _lib.cherryq_workspace_bytes.argtypes = [_int, _int, _int, _int]
 _lib.cherryq_workspace_bytes.restype = _sz
 _lib.cherryq_scratch_bytes.argtypes = [_int, _int, _int, _int]
@@ -281,3 +284,51 @@ def pack_cherryq(w_bits, weight, cherry_indices, group_size):
     if rc != 0:
         _fail(rc, "pack_cherryq")
     return idx, cherry_weight, qweight, scales
+
+
+FAKE_QUANT_MAX_IN_FEATURES = 65536
+FAKE_QUANT_MAX_GROUPS = 4096
+
+
+def fake_quant_supported(weight, w_bits, group_size) -> bool:
+    """Whether fake_quant_cherryq takes this weight (GPU, fp16 or fp32, 2-D, 2..4 bits, within
+    the kernel's channel and group limits)."""
+    if not (isinstance(weight, torch.Tensor) and weight.is_cuda and weight.dim() == 2):
+        return False
+    if weight.dtype not in (torch.float16, torch.float32) or w_bits not in (2, 3, 4):
+        return False
+    k = weight.shape[1]
+    g = int(group_size) if int(group_size) > 0 else k
+    return 0 < k <= FAKE_QUANT_MAX_IN_FEATURES and -(-k // g) <= FAKE_QUANT_MAX_GROUPS
+
+
+def fake_quant_cherryq(w_bits, weight, cherry_indices, group_size, ste=False, out=None):
+    """The weight the training-side QuantLinear multiplies with: every non-cherry input channel of
+    `weight` (out, in; fp16 or fp32) replaced by its group-wise quantise-dequantise value, bit
+    for bit what QuantLinear._adjust_weight computes with torch operations
+    (llama/cherry_linear.py:77-99, llama/quantizer.py:148-152 and 165-170), in one pass over the
+    matrix.  `ste` selects the straight-through arithmetic form (q - w) + w; the gradient is
+    the caller's business.  No counterpart in the reference extension."""
+    if not isinstance(weight, torch.Tensor) or weight.dtype not in (torch.float16, torch.float32):
+        raise RuntimeError("fake_quant_cherryq: weight must be an fp16 or fp32 tensor")
+    _check(weight, "weight", weight.dtype, 2)
+    dev = weight.device
+    n, k = weight.shape
+    if cherry_indices is None:
+        idx = torch.empty(0, dtype=torch.int32, device=dev)
+    else:
+        idx = cherry_indices.to(device=dev, dtype=torch.int32).contiguous()
+    if out is None:
+        out = torch.empty_like(weight)
+    else:
+        _check(out, "out", weight.dtype, 2, dev)
+        if out.shape != weight.shape:
+            raise RuntimeError("fake_quant_cherryq: out must have the weight's shape")
+    g = int(group_size) if int(group_size) > 0 else k
+    fn = _lib.cherryq_fake_quant_f16 if weight.dtype == torch.float16 else _lib.cherryq_fake_quant_f32
+    with torch.cuda.device(dev):
+        rc = fn(int(w_bits), weight.data_ptr(), _ptr(idx), out.data_ptr(), k, n, idx.numel(), g, int(bool(ste)),
+                torch.cuda.current_stream(dev).cuda_stream)
+    if rc != 0:
+        _fail(rc, "fake_quant_cherryq")
+    return out

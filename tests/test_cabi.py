@@ -122,3 +122,25 @@ def test_python_binding_fails_loudly_without_gpu_tensors():
         quant_cuda.vecquant4matmul_cherryq(z, z, z, z, z, z, 64)
     with pytest.raises(RuntimeError, match="dtype"):
         quant_cuda.vecquant3matmul_cherryq(z.float(), z, z, z, z, z, 128, True)
+
+
+def test_fake_quant_validation(lib):
+    """cherryq_fake_quant_f16 / _f32 reject bad arguments before anything is launched."""
+    E_NULL, E_SHAPE, E_GROUP, E_BITS, E_UNSUPPORTED = -1, -2, -3, -5, -7
+    vp, i = ctypes.c_void_p, ctypes.c_int
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.addressof(buf)
+    for name in ("cherryq_fake_quant_f16", "cherryq_fake_quant_f32"):
+        fn = getattr(lib, name)
+        fn.argtypes = [i, vp, vp, vp, i, i, i, i, i, vp]
+        fn.restype = i
+        assert fn(5, p, p, p, 64, 4, 8, 32, 0, None) == E_BITS
+        assert fn(1, p, p, p, 64, 4, 8, 32, 0, None) == E_BITS
+        assert fn(4, p, p, p, 0, 4, 0, 32, 0, None) == E_SHAPE
+        assert fn(4, p, p, p, 64, 4, -1, 32, 0, None) == E_SHAPE
+        assert fn(4, p, p, p, 64, 4, 8, 0, 0, None) == E_GROUP
+        assert fn(4, None, p, p, 64, 4, 8, 32, 0, None) == E_NULL
+        assert fn(4, p, None, p, 64, 4, 8, 32, 0, None) == E_NULL
+        assert fn(4, p, p, None, 64, 4, 8, 32, 0, None) == E_NULL
+        assert fn(4, p, p, p, 65536 + 8, 4, 8, 128, 0, None) == E_UNSUPPORTED
+        assert fn(4, p, p, p, 65536, 4, 8, 8, 0, None) == E_UNSUPPORTED  # 8192 groups per row
