@@ -180,3 +180,39 @@ def test_full_size_layer_against_device_pack_and_unpack(qc, bits):
     assert float((err / s).max()) <= 0.52           # half a grid step, plus the fp16 roundings
     step = (fq[:, keep].float() - dense[:, keep].float()).abs()
     assert bool((step <= s * 1.01).all())
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_every_fp16_weight_under_every_fp16_group_maximum(qc, bits):
+    """Exhaustive over (group maximum, weight): one row per positive finite fp16 maximum M, holding
+    every fp16 bit pattern of magnitude <= M.  The fp16 kernel replaces the division by a
+    reciprocal and one correction step; here every quotient it can ever form is compared with
+    torch's own fp16 operations on the device, and sampled rows with the numpy oracle."""
+    announce("fake-quant exhaustive fp16", bits)
+    from llama.quantizer import FullSymQuantizer
+    k = 65536
+    pats = torch.arange(k, dtype=torch.int32, device="cuda").to(torch.int16)           # every bit pattern
+    vals = pats.view(torch.float16)
+    mags = (pats.to(torch.int32) & 0x7fff)
+    none = torch.empty(0, dtype=torch.int32, device="cuda")
+    rng = np.random.default_rng(bits)
+    sampled = set(rng.choice(np.arange(1, 0x7c00), 24, replace=False).tolist()) | {1, 2, 0x03ff, 0x0400, 0x7bff}
+    for m0 in range(1, 0x7c00, 1024):
+        m1 = min(m0 + 1024, 0x7c00)
+        mx_pat = torch.arange(m0, m1, dtype=torch.int32, device="cuda")                # (rows,)
+        mx = mx_pat.to(torch.int16).view(torch.float16)
+        w = torch.where(mags[None, :] <= mx_pat[:, None], vals[None, :], mx[:, None]).contiguous()
+        got = qc.fake_quant_cherryq(bits, w, none, k)
+        s = FullSymQuantizer.get_scaling_factor(w, None, bits, False)
+        want = FullSymQuantizer.transform(w, s, bits)
+        same = got.view(torch.int16) == want.view(torch.int16)
+        if not bool(same.all()):
+            r, c = (~same).nonzero()[0].tolist()
+            raise AssertionError(f"max pattern {m0 + r:#x}, weight pattern {c:#x}: kernel "
+                                 f"{got[r, c].item()!r}, torch {want[r, c].item()!r}")
+        for m in sorted(sampled):
+            if m0 <= m < m1:
+                row = w[m - m0:m - m0 + 1].cpu().numpy()
+                np.testing.assert_array_equal(bits_of(got[m - m0:m - m0 + 1].cpu().numpy()),
+                                              bits_of(orc.adjust_weight(row, np.empty(0, np.int64), bits, k)))
+        del w, got, s, want, same
