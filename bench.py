@@ -311,6 +311,37 @@ def main():
                   f"({ab / us / 1e3 / HBM_PEAK_GBS * 100:4.1f}% of 8 TB/s; prep + main kernel)",
                   file=sys.stderr, flush=True)
             torch.cuda.empty_cache()
+        # training side: the fused fake quantisation of a whole weight, against the torch operations it replaces
+        import quant_cuda
+        from llama.cherry_linear import QuantLinear as TrainLinear
+        for dtype in (torch.float16, torch.float32):
+            for k, n in ((4096, 11008), (11008, 4096), (4096, 4096)):
+                lin = TrainLinear(k, n, bias=False, w_bits=4, group_size=args.group, cherryq=True).to(dtype).cuda()
+                lin.weight.data.normal_(0, 0.02)
+                lin.register_cherry_indices(torch.randperm(k)[:lin.num_cherries])
+                dst = torch.empty_like(lin.weight)
+                wsrc = lin.weight.detach()
+
+                def timed(fn, reps):
+                    for _ in range(3):
+                        fn()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    for _ in range(reps):
+                        fn()
+                    e1.record()
+                    torch.cuda.synchronize()
+                    return e0.elapsed_time(e1) / reps * 1e3
+
+                us = timed(lambda: quant_cuda.fake_quant_cherryq(4, wsrc, lin.cherry_indices, args.group, out=dst), 50)
+                lin._fused_fake_quant = lambda weight: False
+                us_torch = timed(lambda: lin._adjust_weight(wsrc, ste=False), 5)
+                ab = 2.0 * k * n * wsrc.element_size()
+                print(f"fake-quant {str(dtype)[6:]:8s} {k:5d}->{n:5d}: {us:7.2f} us  {ab / us / 1e3:7.1f} GB/s "
+                      f"({ab / us / 1e3 / HBM_PEAK_GBS * 100:4.1f}% of 8 TB/s; one read + one write of the weight)  "
+                      f"torch operations {us_torch:8.1f} us", file=sys.stderr, flush=True)
+                del lin, dst, wsrc
+                torch.cuda.empty_cache()
         for name, (bits, k, n) in WORKLOADS.items():
             us, wall_us, *_ = time_gpu(bits, k, n, args.group, max(200, args.steps // 4), args.warmup,
                                       use_graph=not args.no_graph)
