@@ -19,6 +19,9 @@
  *   mul            (B, N)            fp16, accumulated into (mul += x W^T) when
  *                                    `accumulate` != 0, overwritten otherwise
  *
+ * K, N and C are multiples of 8 (rows of whole 16-byte pieces); with int16 indices and C > 0,
+ * K is at most 32768.
+ *
  * Return value: 0 on success; negative = rejected argument (CHERRYQ_E_*); positive = a
  * hipError_t reported by the launch.  cherryq_status_string() names either.
  */

@@ -60,7 +60,6 @@ static int check_common(const void *vec, const void *qweight, const void *cherry
                         size_t scratch_bytes_given) {
     if (B < 0 || K <= 0 || N <= 0 || C < 0 || C > K) return CHERRYQ_E_SHAPE;
     if (K % 8 || N % 8 || C % 8) return CHERRYQ_E_SHAPE;
-    if (K - C <= 0 && C == 0) return CHERRYQ_E_SHAPE;
     if (G <= 0 || G % 32) return CHERRYQ_E_GROUP;
     if (!vec || !mul) return CHERRYQ_E_NULL;
     if (K - C > 0 && (!qweight || !scales)) return CHERRYQ_E_NULL;
@@ -83,6 +82,7 @@ static int matmul_f16(const void *vec, const uint8_t *qweight, const void *cherr
     int rc = check_common(vec, qweight, cherry_weight, cherry_indices, scales, mul, B, K, N, C, G, workspace,
                           wsb, scratch, scb);
     if (rc) return rc;
+    if (C > 0 && K > 32768) return CHERRYQ_E_SHAPE;  // int16 channel indices cannot name the columns
     if (B == 0) return CHERRYQ_OK;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     const __half *x = reinterpret_cast<const __half *>(vec);

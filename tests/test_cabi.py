@@ -90,6 +90,7 @@ def test_argument_validation_rejects_before_launch(lib):
     assert _call(f4, b=4) == -4           # batches need scratch
     assert _call(f4, b=4, scr=0x2000, scrb=1024) == -4
     assert _call(f4, b=-1) == -2
+    assert _call(f4, k=32768 + 8, c=16) == -2   # int16 channel indices end at 32767
     assert _call(f4, b=0) == 0            # empty batch: nothing to do, nothing launched
 
 
