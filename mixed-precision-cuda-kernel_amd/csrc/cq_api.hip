@@ -45,6 +45,7 @@ size_t workspace_bytes(int B, int K, int N, int C) {
 size_t scratch_bytes(int B, int K, int N, int C) {
     clamp_dims(B, K, N, C);
     size_t bytes = B >= 2 ? batch_workspace(K, N, C).scratch_total : 0;
+    if (B >= 2 && f32_scratch_bytes(K, C) > bytes) bytes = f32_scratch_bytes(K, C);  // fp32-tensor variant
     if (B >= kGemmMinRows) {
         size_t b3 = gemm_plan(B, K, N, C).scratch_bytes;
         if (b3 > bytes) bytes = b3;
@@ -164,6 +165,11 @@ int cherryq_vecquant3matmul_f32(const float *vec, const uint8_t *qweight, const 
                               scratch_bytes);
     if (rc) return rc;
     if (batch == 0) return CHERRYQ_OK;
+    if (!cq::force_generic() && batch >= 2 &&
+        cq::f32_supported(batch, in_features, out_features, num_cherries, group_size))
+        return (int)cq::launch_f32(vec, qweight, cherry_weight, cherry_indices, scales, mul, batch, in_features,
+                                   out_features, num_cherries, group_size, accumulate, workspace, scratch,
+                                   reinterpret_cast<hipStream_t>(stream));
     return (int)cq::launch_generic<3, float, int32_t>(vec, qweight, cherry_weight, cherry_indices, scales, mul,
                                                       batch, in_features, out_features, num_cherries,
                                                       group_size, accumulate, workspace,

@@ -90,6 +90,13 @@ hipError_t launch_gemm(int bits, const __half *vec, const uint8_t *qweight, cons
 hipError_t launch_pack(int bits, const __half *w, const int16_t *idx, uint8_t *qweight, __half *scales,
                        __half *cherry_weight, int K, int N, int C, int G, hipStream_t stream);
 
+// cq_f32.hip: the 3-bit fp32-tensor variant on the fp32 matrix-core instruction, 2 rows and more.
+bool f32_supported(int B, int K, int N, int C, int G);
+size_t f32_scratch_bytes(int K, int C);
+hipError_t launch_f32(const float *vec, const uint8_t *qweight, const float *cherry_weight,
+                      const int32_t *cherry_indices, const float *scales, float *mul, int B, int K, int N, int C,
+                      int G, int accumulate, void *workspace, void *scratch, hipStream_t stream);
+
 // cq_fakequant.hip: training-side quantise-dequantise of the non-cherry columns, fp16 or fp32.
 bool fake_quant_supported(int K, int C, int G);
 hipError_t launch_fake_quant(int bits, bool fp32, const void *w, const int32_t *idx, void *out, int K, int N, int C,

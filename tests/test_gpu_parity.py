@@ -349,6 +349,79 @@ def test_fp32_entry_point_benchmark_speed_shape(qc):
     np.testing.assert_allclose(mul.cpu().numpy(), want, rtol=2e-5, atol=2e-3)
 
 
+F32_CASES = [
+    # b, k, n, cherries, group
+    (16, 4096, 1728, 16, 128),     # the benchmark_speed.py call shape (columns / 8)
+    (2, 1024, 256, 8, 128), (5, 1024, 264, 0, 128),        # N % 16 == 8, no cherries
+    (16, 2048 + 40, 520, 40, 128),                          # ragged last unit, two cherry units, N % 256 != 0
+    (17, 1024, 512, 8, 256), (40, 2048, 256, 32, 1024),     # more than one pass of 16 rows; wide groups
+    (3, 1024, 256, 8, 64), (1, 1024, 256, 8, 128),          # group 64 and batch 1 stay on the generic kernel
+]
+
+
+@pytest.mark.parametrize("b,k,n,c,g", F32_CASES, ids=[f"b{v[0]}-k{v[1]}-n{v[2]}-c{v[3]}-g{v[4]}" for v in F32_CASES])
+def test_fp32_variant_against_float64(qc, b, k, n, c, g):
+    """fp32 tensors, int32 indices: the matrix-core kernel (2 rows and more, groups of whole units)
+    and the generic kernel against a float64 evaluation, and against each other."""
+    announce("fp32 variant", b, k, n, c, g)
+    rng = np.random.default_rng(1000 * b + k + n + c)
+    kn = k - c
+    vec = rng.standard_normal((b, k)).astype(np.float32)
+    qweight = rng.integers(0, 256, size=(kn // 8 * 3, n), dtype=np.uint8)
+    cw = rng.standard_normal((c, n)).astype(np.float32)
+    idx = np.sort(rng.choice(k, c, replace=False)).astype(np.int32)
+    scales = (rng.random((-(-kn // g), n)) * 0.01 + 0.005).astype(np.float32)
+    init = rng.standard_normal((b, n)).astype(np.float32)
+    u = orc.unpack_codes(qweight, 3).astype(np.float64) - 3.5
+    wn = u * np.repeat(scales.astype(np.float64), g, axis=0)[:kn]
+    nidx = orc.normal_indices(k, idx)
+    want = init + vec[:, nidx].astype(np.float64) @ wn + vec[:, idx].astype(np.float64) @ cw.astype(np.float64)
+    args = [torch.from_numpy(a).cuda() for a in (vec, qweight, cw, idx, scales)]
+
+    def run():
+        mul = torch.from_numpy(init.copy()).cuda()
+        qc.vecquant3matmul_cherryq(*args, mul, g, False)
+        torch.cuda.synchronize()
+        return mul.cpu().numpy()
+
+    got = run()
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= 2e-6 * scale * np.sqrt(k / 1024)
+    np.testing.assert_array_equal(got, run())           # order-independent accumulation
+    os.environ["CHERRYQ_FORCE_GENERIC"] = "1"
+    try:
+        generic = run()
+    finally:
+        os.environ["CHERRYQ_FORCE_GENERIC"] = "0"
+    assert np.abs(generic - want).max() <= 2e-6 * scale * np.sqrt(k / 1024)
+
+
+def test_fp32_variant_one_hot_rows_read_the_weights_back(qc):
+    """One-hot activations through the fp32 matrix-core kernel return (code - 3.5) * scale and the
+    cherry rows: every product is exact and every sum has one non-zero term, so the only
+    deviation left is the split-K accumulator's fixed-point step of 2^-34."""
+    announce("fp32 one-hot")
+    k, n, c, g = 1024, 512, 8, 128
+    rng = np.random.default_rng(7)
+    kn = k - c
+    qweight = rng.integers(0, 256, size=(kn // 8 * 3, n), dtype=np.uint8)
+    cw = rng.standard_normal((c, n)).astype(np.float32)
+    idx = np.sort(rng.choice(k, c, replace=False)).astype(np.int32)
+    scales = (rng.random((kn // g + (kn % g > 0), n)) * 0.01 + 0.005).astype(np.float32)
+    dense = np.zeros((k, n), np.float32)
+    u = orc.unpack_codes(qweight, 3).astype(np.float32) - np.float32(3.5)
+    dense[orc.normal_indices(k, idx)] = u * np.repeat(scales, g, axis=0)[:kn]
+    dense[idx] = cw
+    args = [torch.from_numpy(a).cuda() for a in (qweight, cw, idx, scales)]
+    cols = np.concatenate([rng.choice(k, 13, replace=False), idx[:3]])
+    x = np.zeros((16, k), np.float32)
+    x[np.arange(16), cols] = 1.0
+    mul = torch.zeros(16, n, device="cuda")
+    qc.vecquant3matmul_cherryq(torch.from_numpy(x).cuda(), *args, mul, g, False)
+    torch.cuda.synchronize()
+    assert np.abs(mul.cpu().numpy().astype(np.float64) - dense[cols]).max() <= 2.0 ** -34
+
+
 def test_unsupported_requests_raise(qc):
     announce("errors")
     k, n = 1024, 256
