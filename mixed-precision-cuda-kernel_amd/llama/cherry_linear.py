@@ -31,6 +31,21 @@ class _FakeQuantSTE(torch.autograd.Function):
         return grad_output, None, None, None
 
 
+class _FakeQuantPlain(torch.autograd.Function):
+    """Group-wise fake quantisation of the whole weight (no cherry channels) for the plain QAT
+    branch: the value of FullSymQuantizer.forward without clipping (llama/quantizer.py:172-184),
+    whose backward hands the gradient through unchanged (:120-133)."""
+
+    @staticmethod
+    def forward(ctx, weight, w_bits, group_size):
+        import quant_cuda
+        return quant_cuda.fake_quant_cherryq(w_bits, weight.detach().contiguous(), None, group_size, ste=False)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return grad_output, None, None
+
+
 class QuantLinear(nn.Linear):
     def __init__(self, *args, bias=False, w_bits=16, weight_layerwise=False, group_size=-1,
                  cherryq=False, cherry_fraction=1 / 256):
@@ -89,6 +104,16 @@ class QuantLinear(nn.Linear):
         import quant_cuda
         return quant_cuda.fake_quant_supported(weight, self.w_bits, self.group_size)
 
+    def _fused_plain(self, weight) -> bool:
+        """The same for the branch without cherry channels (groups must tile the row, as the
+        reference's reshape demands)."""
+        if not weight.is_cuda or self.quantizer is not FullSymQuantizer or self.weight_layerwise:
+            return False
+        if self.group_size <= 0 or weight.shape[1] % self.group_size:
+            return False
+        import quant_cuda
+        return quant_cuda.fake_quant_supported(weight, self.w_bits, self.group_size)
+
     def _adjust_weight(self, weight: torch.Tensor, ste=True):
         """Weight with every non-cherry column fake quantised (groups run over the compacted
         normal columns); with `ste` the result carries the straight-through gradient.
@@ -136,6 +161,8 @@ class QuantLinear(nn.Linear):
                     weight = self._adjust_weight(weight)
                 elif not self.dequantized:
                     weight = self.prepare_weight_for_inference(weight)
+            elif self.training and self._fused_plain(weight):
+                weight = _FakeQuantPlain.apply(weight, self.w_bits, self.group_size)
             elif self.training:
                 # plain QAT: group-wise fake quantisation through the autograd function
                 grouped = weight.reshape(weight.shape[0], -1, self.group_size)

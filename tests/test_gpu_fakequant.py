@@ -158,6 +158,36 @@ def test_training_module_uses_the_kernel_and_matches_the_torch_operations(qc, dt
     assert torch.equal(g_fused, g_torch)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_plain_qat_branch_uses_the_kernel_and_matches_the_torch_operations(qc, dtype):
+    """cherryq=False in training mode: whole-row groups through the kernel (no cherry channels)
+    against the quantiser's autograd function, value and weight gradient."""
+    announce("fake-quant plain QAT", dtype)
+    from llama.cherry_linear import QuantLinear as TrainLinear
+    torch.manual_seed(5)
+    k, n = 1024, 64
+    lin = TrainLinear(k, n, bias=False, w_bits=4, group_size=128, cherryq=False).to(dtype).cuda()
+    lin.weight.data.normal_(0, 0.02)
+    lin.train()
+    assert lin._fused_plain(lin.weight)
+    x = torch.randn(3, k, dtype=dtype, device="cuda")
+
+    def step():
+        lin.weight.grad = None
+        y = lin(x)
+        y.float().square().sum().backward()
+        return y.detach().clone(), lin.weight.grad.detach().clone()
+
+    y_fused, g_fused = step()
+    lin._fused_plain = lambda weight: False
+    y_torch, g_torch = step()
+    assert torch.equal(y_fused, y_torch)
+    assert torch.equal(g_fused, g_torch)
+    want = orc.adjust_weight(lin.weight.detach().cpu().numpy(), np.empty(0, np.int64), 4, 128)
+    got = qc.fake_quant_cherryq(4, lin.weight.detach(), None, 128)
+    np.testing.assert_array_equal(bits_of(got.cpu().numpy()), bits_of(want))
+
+
 @pytest.mark.parametrize("bits", [3, 4])
 def test_full_size_layer_against_device_pack_and_unpack(qc, bits):
     """4096 -> 11008 in fp16: the kernel agrees with unpack(pack(w)) (two other kernels) except
