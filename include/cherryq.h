@@ -67,9 +67,13 @@ const char *cherryq_status_string(int status);
  * processing) in the tiled GEMM kernel, whose compacted copy of the activations and partial
  * tiles grow with the number of rows.  Size the buffers for the largest batch that will be passed.
  * Calls that may overlap in time (different streams) must use different workspace and scratch.
+ * cherryq_scratch_bytes_f32() is the scratch size for the fp32-tensor entry point, which is not 0
+ * at batch 1: with such a buffer one row runs on the matrix-core kernel too, without (NULL) on a
+ * slower general one.
  */
 size_t cherryq_workspace_bytes(int batch, int in_features, int out_features, int num_cherries);
 size_t cherryq_scratch_bytes(int batch, int in_features, int out_features, int num_cherries);
+size_t cherryq_scratch_bytes_f32(int batch, int in_features, int out_features, int num_cherries);
 
 /*
  * Replaces quant_cuda.vecquant4matmul_cherryq (csrc/quant_cuda.cpp:56-69,

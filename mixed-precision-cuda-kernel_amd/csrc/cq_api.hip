@@ -134,6 +134,14 @@ size_t cherryq_scratch_bytes(int batch, int in_features, int out_features, int n
     return cq::scratch_bytes(batch, in_features, out_features, num_cherries);
 }
 
+size_t cherryq_scratch_bytes_f32(int batch, int in_features, int out_features, int num_cherries) {
+    int B = batch, K = in_features, N = out_features, C = num_cherries;
+    cq::clamp_dims(B, K, N, C);
+    const size_t f32 = cq::f32_scratch_bytes(K, C);
+    const size_t common = cq::scratch_bytes(B, K, N, C);
+    return f32 > common ? f32 : common;
+}
+
 int cherryq_vecquant4matmul_f16(const void *vec, const uint8_t *qweight, const void *cherry_weight,
                                 const int16_t *cherry_indices, const void *scales, void *mul, int batch,
                                 int in_features, int out_features, int num_cherries, int group_size,
@@ -165,7 +173,10 @@ int cherryq_vecquant3matmul_f32(const float *vec, const uint8_t *qweight, const 
                               scratch_bytes);
     if (rc) return rc;
     if (batch == 0) return CHERRYQ_OK;
-    if (!cq::force_generic() && batch >= 2 &&
+    // one row: the matrix-core kernel when the caller brought its scratch buffer, else the generic one
+    const bool has_scratch = scratch && cq::aligned(scratch, 256) &&
+                             scratch_bytes >= cq::f32_scratch_bytes(in_features, num_cherries);
+    if (!cq::force_generic() && (batch >= 2 || has_scratch) &&
         cq::f32_supported(batch, in_features, out_features, num_cherries, group_size))
         return (int)cq::launch_f32(vec, qweight, cherry_weight, cherry_indices, scales, mul, batch, in_features,
                                    out_features, num_cherries, group_size, accumulate, workspace, scratch,

@@ -56,6 +56,8 @@ _lib.cherryq_workspace_bytes.argtypes = [_int, _int, _int, _int]
 _lib.cherryq_workspace_bytes.restype = _sz
 _lib.cherryq_scratch_bytes.argtypes = [_int, _int, _int, _int]
 _lib.cherryq_scratch_bytes.restype = _sz
+_lib.cherryq_scratch_bytes_f32.argtypes = [_int, _int, _int, _int]
+_lib.cherryq_scratch_bytes_f32.restype = _sz
 _lib.cherryq_status_string.argtypes = [_int]
 _lib.cherryq_status_string.restype = ctypes.c_char_p
 _lib.cherryq_version.restype = _int
@@ -147,7 +149,10 @@ def _matmul(fn, what, vec, qweight, cherry_weight, cherry_indices, scales, mul, 
                            w_bits, io_dtype, idx_dtype, accumulate)
     stream = torch.cuda.current_stream().cuda_stream
     ws = _workspace(dev, stream, _lib.cherryq_workspace_bytes(batch, k, n, c))
-    sc = _scratch(dev, stream, _lib.cherryq_scratch_bytes(batch, k, n, c)) if batch > 1 else None
+    if io_dtype == torch.float32:
+        sc = _scratch(dev, stream, _lib.cherryq_scratch_bytes_f32(batch, k, n, c))
+    else:
+        sc = _scratch(dev, stream, _lib.cherryq_scratch_bytes(batch, k, n, c)) if batch > 1 else None
     rc = fn(_ptr(vec), _ptr(qweight), _ptr(cherry_weight), _ptr(cherry_indices), _ptr(scales), _ptr(mul),
             batch, k, n, c, group_size, 1 if accumulate else 0, ws.data_ptr(), ws.numel(),
             sc.data_ptr() if sc is not None else None, sc.numel() if sc is not None else 0, stream)

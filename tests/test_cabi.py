@@ -59,6 +59,9 @@ def test_workspace_sizes(lib):
     lib.cherryq_scratch_bytes.restype = ctypes.c_size_t
     assert lib.cherryq_scratch_bytes(1, 4096, 11008, 16) == 0
     assert lib.cherryq_scratch_bytes(2, 4096, 11008, 16) >= 8 * 16 * 11008 * 4 + 33 * 4096
+    lib.cherryq_scratch_bytes_f32.restype = ctypes.c_size_t
+    assert lib.cherryq_scratch_bytes_f32(1, 4096, 13824, 16) >= 33 * 8 * 64 * 16   # operand-order activations
+    assert lib.cherryq_scratch_bytes_f32(16, 4096, 13824, 16) >= lib.cherryq_scratch_bytes(16, 4096, 13824, 16)
 
 
 def _call(fn, *, vec=0x1000, qw=0x1000, cw=0x1000, idx=0x1000, sc=0x1000, mul=0x1000, b=1, k=4096, n=4096,

@@ -355,7 +355,7 @@ F32_CASES = [
     (2, 1024, 256, 8, 128), (5, 1024, 264, 0, 128),        # N % 16 == 8, no cherries
     (16, 2048 + 40, 520, 40, 128),                          # ragged last unit, two cherry units, N % 256 != 0
     (17, 1024, 512, 8, 256), (40, 2048, 256, 32, 1024),     # more than one pass of 16 rows; wide groups
-    (3, 1024, 256, 8, 64), (1, 1024, 256, 8, 128),          # group 64 and batch 1 stay on the generic kernel
+    (3, 1024, 256, 8, 64), (1, 1024, 256, 8, 128),          # group 64: generic kernel; one row: matrix-core kernel
 ]
 
 
@@ -394,6 +394,41 @@ def test_fp32_variant_against_float64(qc, b, k, n, c, g):
     finally:
         os.environ["CHERRYQ_FORCE_GENERIC"] = "0"
     assert np.abs(generic - want).max() <= 2e-6 * scale * np.sqrt(k / 1024)
+
+
+def test_fp32_variant_single_row_with_and_without_scratch_through_the_c_abi(qc):
+    """One fp32 row: without a scratch buffer the call takes the generic kernel, with
+    cherryq_scratch_bytes_f32() bytes the matrix-core kernel; both leave the workspace zeroed."""
+    announce("fp32 c-abi one row")
+    lib = qc._lib
+    k, n, c, g = 2048, 512, 8, 128
+    rng = np.random.default_rng(21)
+    kn = k - c
+    vec = rng.standard_normal((1, k)).astype(np.float32)
+    qweight = rng.integers(0, 256, size=(kn // 8 * 3, n), dtype=np.uint8)
+    cw = rng.standard_normal((c, n)).astype(np.float32)
+    idx = np.sort(rng.choice(k, c, replace=False)).astype(np.int32)
+    scales = (rng.random((-(-kn // g), n)) * 0.01 + 0.005).astype(np.float32)
+    u = orc.unpack_codes(qweight, 3).astype(np.float64) - 3.5
+    want = vec[:, orc.normal_indices(k, idx)].astype(np.float64) @ (u * np.repeat(scales.astype(np.float64), g, axis=0)[:kn]) \
+        + vec[:, idx].astype(np.float64) @ cw.astype(np.float64)
+    t = [torch.from_numpy(a).cuda() for a in (vec, qweight, cw, idx, scales)]
+    ws_b = lib.cherryq_workspace_bytes(1, k, n, c)
+    sc_b = lib.cherryq_scratch_bytes_f32(1, k, n, c)
+    assert lib.cherryq_scratch_bytes(1, k, n, c) == 0 and sc_b > 0
+    ws = torch.zeros(ws_b, dtype=torch.uint8, device="cuda")
+    sc = torch.empty(sc_b, dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    lib.cherryq_vecquant3matmul_f32.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 6 + \
+        [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    for scratch, nbytes in ((None, 0), (sc.data_ptr(), sc_b)):
+        out = torch.zeros(1, n, device="cuda")
+        rc = lib.cherryq_vecquant3matmul_f32(*(a.data_ptr() for a in t), out.data_ptr(), 1, k, n, c, g, 1,
+                                             ws.data_ptr(), ws_b, scratch, nbytes, stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert np.abs(out.cpu().numpy() - want).max() <= 3e-6 * np.abs(want).max()
+        assert not ws.any()
 
 
 def test_fp32_variant_one_hot_rows_read_the_weights_back(qc):
