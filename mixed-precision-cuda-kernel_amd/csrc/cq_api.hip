@@ -93,6 +93,8 @@ static int matmul_f16(const void *vec, const uint8_t *qweight, const void *cherr
     hipError_t e;
     if (!force_generic() && B == 1 && matvec_supported(BITS, B, K, N, C, G)) {
         e = launch_matvec(BITS, x, qweight, cw, cherry_indices, sc, y, K, N, C, G, accumulate, workspace, s);
+    } else if (!force_generic() && matvec_rows_preferred(BITS, B, K, N, C, G)) {
+        e = launch_matvec_rows(BITS, x, qweight, cw, cherry_indices, sc, y, B, K, N, C, G, accumulate, workspace, s);
     } else if (!force_generic() && B >= kGemmMinRows && gemm_supported(BITS, B, K, N, C, G)) {
         e = launch_gemm(BITS, x, qweight, cw, cherry_indices, sc, y, B, K, N, C, G, accumulate, workspace, scratch, s);
     } else if (!force_generic() && batch_supported(BITS, B, K, N, C, G)) {

@@ -21,8 +21,14 @@ hipError_t launch_unpack(int bits, const uint8_t *qweight, const __half *cherry_
                          const int16_t *cherry_indices, const __half *scales, __half *dense, int K, int N,
                          int C, int G, hipStream_t stream);
 
-// cq_matvec.hip: batch-1 HBM-streaming matvec.  Returns false when the shape is not one it takes.
+// cq_matvec.hip: HBM-streaming matvec for 1..kMatvecMaxRows activation rows.  Returns false when
+// the shape is not one it takes.
+constexpr int kMatvecMaxRows = 4;
 bool matvec_supported(int bits, int B, int K, int N, int C, int G);
+bool matvec_rows_preferred(int bits, int B, int K, int N, int C, int G);  // 2..4 rows: this kernel rather than the batch one
+hipError_t launch_matvec_rows(int bits, const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
+                              const int16_t *cherry_indices, const __half *scales, __half *mul, int rows, int K,
+                              int N, int C, int G, int accumulate, void *workspace, hipStream_t stream);
 hipError_t launch_matvec(int bits, const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
                          const int16_t *cherry_indices, const __half *scales, __half *mul, int K, int N,
                          int C, int G, int accumulate, void *workspace, hipStream_t stream);

@@ -126,15 +126,19 @@ struct Geo {
 
 // NW = wavefronts (= units) per workgroup: 4, or 2 or 1 when the layer is so small
 // that larger workgroups would leave CUs without work.
-template <int BITS, int NW, int KPL, bool NORM>
+// ROWS = activation rows handled in the same pass (1, 2 or 4): the codes are decoded once and
+// every row adds its own dot products; `rows` (<= ROWS) of them exist, the others read zeros.
+// The norm / gate prologues exist for one row only.
+template <int BITS, int NW, int KPL, bool NORM, int ROWS>
 __global__ __launch_bounds__(64 * NW) void matvec_kernel(
     const __half *__restrict__ x, MatvecPrologue pro, MatvecGroup grp,
-    unsigned long long *__restrict__ acc_words, int K, int C, int G, int accumulate, Plan plan) {
+    unsigned long long *__restrict__ acc_words, int K, int C, int G, int accumulate, Plan plan, int rows) {
+    static_assert(ROWS == 1 || !NORM, "the fused prologues take one row");
     using G_ = Geo<BITS, KPL>;
     constexpr int R = G_::kRowsPerLaneGroup;
     constexpr int UK = G_::kUnit;
-    __shared__ uint32_t s_win[NW][128];  // per wave: 256 fp16 activations starting at the unit's first position
-    __shared__ uint32_t s_pair[NW][64];  // per wave: activation pairs laid out for the dot2 operands
+    __shared__ uint32_t s_win[NW][ROWS][128];  // per wave and row: 256 fp16 activations starting at the unit's first position
+    __shared__ uint32_t s_pair[NW][ROWS][64];  // per wave and row: activation pairs laid out for the dot2 operands
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -142,7 +146,7 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
     // scalar branch, so a wavefront executes exactly one of the unit paths below
     const int wave = NORM ? __builtin_amdgcn_readfirstlane(tid >> 6) : tid >> 6;
     const int kq = lane >> 4, nl = lane & 15;
-    const __half *__restrict__ x_gate = pro.gate;
+    const __half *__restrict__ x_gate = ROWS == 1 ? pro.gate : nullptr;
     // NORM is a template parameter so that the plain kernel does not pay the registers
     const __half *__restrict__ norm_w = NORM ? pro.norm_weight : nullptr;
     // Consecutive workgroups take neighbouring column tiles of the same rows, so that the
@@ -169,9 +173,11 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
     const bool col_ok = n0 < N;
     const int Kn = K - C;
 
-    float tot[16];
+    float tot[ROWS][16];
 #pragma unroll
-    for (int c = 0; c < 16; c++) tot[c] = 0.f;
+    for (int r = 0; r < ROWS; r++)
+#pragma unroll
+        for (int c = 0; c < 16; c++) tot[r][c] = 0.f;
     CQ_STAMP(0);
 
     // Fused RMSNorm: the workgroup's threads share one pass over the K activations (16 bytes per
@@ -193,9 +199,22 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
             __builtin_amdgcn_make_buffer_rsrc((void *)cherry_indices, 0, C * 2, kRsrcFlags);
         const int i0 = (short)__builtin_amdgcn_raw_buffer_load_b16(ri, lane * 2, 0, 0);
         const int i1 = (short)__builtin_amdgcn_raw_buffer_load_b16(ri, (lane + 64) * 2, 0, 0);
-        const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, K * 2, kRsrcFlags);
-        uint32_t win0 = __builtin_amdgcn_raw_buffer_load_b32(rx, (ubase + 2 * lane) * 2, 0, 0);
-        uint32_t win1 = __builtin_amdgcn_raw_buffer_load_b32(rx, (ubase + 128 + 2 * lane) * 2, 0, 0);
+        // rows beyond `rows` lie outside the descriptor and read as zeros
+        const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, rows * K * 2, kRsrcFlags);
+        uint32_t win0[ROWS], win1[ROWS];
+        if (ROWS == 1) {
+            win0[0] = __builtin_amdgcn_raw_buffer_load_b32(rx, (ubase + 2 * lane) * 2, 0, 0);
+            win1[0] = __builtin_amdgcn_raw_buffer_load_b32(rx, (ubase + 128 + 2 * lane) * 2, 0, 0);
+        } else {
+            // a window that runs past the end of its row must not read the next row's activations
+            const bool in0 = ubase + 2 * lane < K, in1 = ubase + 128 + 2 * lane < K;
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) {
+                const uint32_t roff = (uint32_t)(r * K) * 2u;
+                win0[r] = __builtin_amdgcn_raw_buffer_load_b32(rx, (in0 && r < rows) ? roff + (ubase + 2 * lane) * 2 : kOob, 0, 0);
+                win1[r] = __builtin_amdgcn_raw_buffer_load_b32(rx, (in1 && r < rows) ? roff + (ubase + 128 + 2 * lane) * 2 : kOob, 0, 0);
+            }
+        }
         uint32_t nw0 = 0, nw1 = 0;
         if (norm_w) {
             const __amdgpu_buffer_rsrc_t rnw = __builtin_amdgcn_make_buffer_rsrc((void *)norm_w, 0, K * 2, kRsrcFlags);
@@ -229,16 +248,19 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
         const int t0 = lane < C ? i0 - lane : 0x7fffffff;
         const int t1 = lane + 64 < C ? i1 - (lane + 64) : 0x7fffffff;
         if (x_gate) {
-            win0 = silu_mul_pair(gat0, win0);
-            win1 = silu_mul_pair(gat1, win1);
+            win0[0] = silu_mul_pair(gat0, win0[0]);
+            win1[0] = silu_mul_pair(gat1, win1[0]);
         }
         if (norm_w) {
             const float rs = norm_scale<NW>(nchunk, s_ss, wave, lane, K, pro.eps);
-            win0 = norm_pair(win0, nw0, rs);
-            win1 = norm_pair(win1, nw1, rs);
+            win0[0] = norm_pair(win0[0], nw0, rs);
+            win1[0] = norm_pair(win1[0], nw1, rs);
         }
-        s_win[wave][lane] = win0;
-        s_win[wave][64 + lane] = win1;
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            s_win[wave][r][lane] = win0[r];
+            s_win[wave][r][64 + lane] = win1[r];
+        }
         // positions this lane prepares, relative to the lane group's first position
         int j0, j1, p0 = 0, p1 = 0;
         if (BITS == 4) {
@@ -274,36 +296,44 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        const unsigned short *winh = reinterpret_cast<const unsigned short *>(&s_win[wave][0]);
         const bool prep = nl < G_::kPairs;  // lanes that prepare an activation pair
-        uint32_t h0 = (prep && k0 < Kn) ? winh[(k0 - ubase) + low0] : 0u;
-        uint32_t h1 = (prep && k1 < Kn) ? winh[(k1 - ubase) + low1] : 0u;
-        const float xsum = row_sum(half_bits_to_float(h0) + half_bits_to_float(h1));
-        int sh = 0;
-        if (BITS == 3) {
-            // scale the lane group's activations so that the largest has biased exponent 29;
-            // the per-field factors 2^-p (p <= 7) then stay far inside the fp16 normal range
-            const int e = row_max((int)max(h0 & 0x7fffu, h1 & 0x7fffu)) >> 10;
-            sh = 29 - e;
-            h0 = __half_as_ushort(__float2half_rn(ldexpf(half_bits_to_float(h0), sh - p0)));
-            h1 = __half_as_ushort(__float2half_rn(ldexpf(half_bits_to_float(h1), sh - p1)));
+        float xsum[ROWS];
+        int sh[ROWS];
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            const unsigned short *winh = reinterpret_cast<const unsigned short *>(&s_win[wave][r][0]);
+            uint32_t h0 = (prep && k0 < Kn) ? winh[(k0 - ubase) + low0] : 0u;
+            uint32_t h1 = (prep && k1 < Kn) ? winh[(k1 - ubase) + low1] : 0u;
+            xsum[r] = row_sum(half_bits_to_float(h0) + half_bits_to_float(h1));
+            sh[r] = 0;
+            if (BITS == 3) {
+                // scale the lane group's activations so that the largest has biased exponent 29;
+                // the per-field factors 2^-p (p <= 7) then stay far inside the fp16 normal range
+                const int e = row_max((int)max(h0 & 0x7fffu, h1 & 0x7fffu)) >> 10;
+                sh[r] = 29 - e;
+                h0 = __half_as_ushort(__float2half_rn(ldexpf(half_bits_to_float(h0), sh[r] - p0)));
+                h1 = __half_as_ushort(__float2half_rn(ldexpf(half_bits_to_float(h1), sh[r] - p1)));
+            }
+            s_pair[wave][r][lane] = h0 | (h1 << 16);
         }
-        s_pair[wave][lane] = h0 | (h1 << 16);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        u32x4 xq[G_::kPairs / 4];
+        u32x4 xq[ROWS][G_::kPairs / 4];
 #pragma unroll
-        for (int i = 0; i < G_::kPairs / 4; i++)
-            xq[i] = *reinterpret_cast<const u32x4 *>(&s_pair[wave][16 * kq + 4 * i]);
+        for (int r = 0; r < ROWS; r++)
+#pragma unroll
+            for (int i = 0; i < G_::kPairs / 4; i++)
+                xq[r][i] = *reinterpret_cast<const u32x4 *>(&s_pair[wave][r][16 * kq + 4 * i]);
         CQ_STAMP(1);
 
         if (BITS == 4) {
-            float lo[16], hi[16];
+            float lo[ROWS][16], hi[ROWS][16];
 #pragma unroll
-            for (int c = 0; c < 16; c++) lo[c] = hi[c] = 0.f;
+            for (int r = 0; r < ROWS; r++)
+#pragma unroll
+                for (int c = 0; c < 16; c++) lo[r][c] = hi[r][c] = 0.f;
 #pragma unroll
             for (int p = 0; p < R / 2; p++) {
-                const uint32_t xe = xq[p >> 1][(p & 1) * 2], xo = xq[p >> 1][(p & 1) * 2 + 1];
 #pragma unroll
                 for (int d = 0; d < 4; d++) {
 #pragma unroll
@@ -311,25 +341,33 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
                         // bytes (row 2p col j, 0, row 2p+1 col j, 0)
                         const uint32_t pr = __builtin_amdgcn_perm(w[2 * p][d], w[2 * p + 1][d],
                                                                   0x0c000c00u | (uint32_t)(j << 16) | (uint32_t)(4 + j));
-                        lo[4 * d + j] = fdot2(pr & 0x000f000fu, xe, lo[4 * d + j]);
-                        hi[4 * d + j] = fdot2(pr & 0x00f000f0u, xo, hi[4 * d + j]);
+                        const uint32_t ce = pr & 0x000f000fu, co = pr & 0x00f000f0u;
+#pragma unroll
+                        for (int r = 0; r < ROWS; r++) {
+                            lo[r][4 * d + j] = fdot2(ce, xq[r][p >> 1][(p & 1) * 2], lo[r][4 * d + j]);
+                            hi[r][4 * d + j] = fdot2(co, xq[r][p >> 1][(p & 1) * 2 + 1], hi[r][4 * d + j]);
+                        }
                     }
                 }
             }
-            const float corr = -7.5f * xsum;
 #pragma unroll
-            for (int c = 0; c < 16; c++) {
-                const uint32_t sw = c < 8 ? sc0[c >> 1] : sc1[(c - 8) >> 1];
-                const float s = half_bits_to_float((c & 1) ? (sw >> 16) : (sw & 0xffffu));
-                tot[c] = (lo[c] * 16777216.0f + hi[c] * 1048576.0f + corr) * s;
+            for (int r = 0; r < ROWS; r++) {
+                const float corr = -7.5f * xsum[r];
+#pragma unroll
+                for (int c = 0; c < 16; c++) {
+                    const uint32_t sw = c < 8 ? sc0[c >> 1] : sc1[(c - 8) >> 1];
+                    const float s = half_bits_to_float((c & 1) ? (sw >> 16) : (sw & 0xffffu));
+                    tot[r][c] = (lo[r][c] * 16777216.0f + hi[r][c] * 1048576.0f + corr) * s;
+                }
             }
         } else {
-            float acc[16];
+            float acc[ROWS][16];
 #pragma unroll
-            for (int c = 0; c < 16; c++) acc[c] = 0.f;
+            for (int r = 0; r < ROWS; r++)
+#pragma unroll
+                for (int c = 0; c < 16; c++) acc[r][c] = 0.f;
 #pragma unroll
             for (int t = 0; t < R / 3; t++) {
-                const uint32_t xa = xq[t][0], xb = xq[t][1], xc = xq[t][2], xd = xq[t][3];
 #pragma unroll
                 for (int d = 0; d < 4; d++) {
 #pragma unroll
@@ -339,21 +377,29 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
                         // p2 = bits 8..23 of the unit        | its bits 16..23 in the high half
                         const uint32_t p1 = __builtin_amdgcn_perm(w[3 * t][d], w[3 * t + 1][d], sel);
                         const uint32_t p2 = __builtin_amdgcn_perm(w[3 * t + 1][d], w[3 * t + 2][d], sel);
-                        float a = acc[4 * d + j];
-                        a = fdot2(p1 & 0x000e0007u, xa, a);                            // codes 0 | 3
-                        a = fdot2(p1 & 0x00700038u, xb, a);                            // codes 1 | 4
-                        a = fdot2(p2 & 0x001c0380u, xc, a);                            // codes 5 | 6
-                        a = fdot2((p1 & 0x000001c0u) | (p2 & 0x00e00000u), xd, a);     // codes 2 | 7
-                        acc[4 * d + j] = a;
+                        const uint32_t c03 = p1 & 0x000e0007u, c14 = p1 & 0x00700038u, c56 = p2 & 0x001c0380u;
+                        const uint32_t c27 = (p1 & 0x000001c0u) | (p2 & 0x00e00000u);
+#pragma unroll
+                        for (int r = 0; r < ROWS; r++) {
+                            float a = acc[r][4 * d + j];
+                            a = fdot2(c03, xq[r][t][0], a);  // codes 0 | 3
+                            a = fdot2(c14, xq[r][t][1], a);  // codes 1 | 4
+                            a = fdot2(c56, xq[r][t][2], a);  // codes 5 | 6
+                            a = fdot2(c27, xq[r][t][3], a);  // codes 2 | 7
+                            acc[r][4 * d + j] = a;
+                        }
                     }
                 }
             }
-            const float corr = -3.5f * xsum;
 #pragma unroll
-            for (int c = 0; c < 16; c++) {
-                const uint32_t sw = c < 8 ? sc0[c >> 1] : sc1[(c - 8) >> 1];
-                const float s = half_bits_to_float((c & 1) ? (sw >> 16) : (sw & 0xffffu));
-                tot[c] = (ldexpf(acc[c], 24 - sh) + corr) * s;
+            for (int r = 0; r < ROWS; r++) {
+                const float corr = -3.5f * xsum[r];
+#pragma unroll
+                for (int c = 0; c < 16; c++) {
+                    const uint32_t sw = c < 8 ? sc0[c >> 1] : sc1[(c - 8) >> 1];
+                    const float s = half_bits_to_float((c & 1) ? (sw >> 16) : (sw & 0xffffu));
+                    tot[r][c] = (ldexpf(acc[r][c], 24 - sh[r]) + corr) * s;
+                }
             }
         }
     } else if (u < plan.units_total) {
@@ -366,9 +412,13 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
         const __amdgpu_buffer_rsrc_t ri =
             __builtin_amdgcn_make_buffer_rsrc((void *)cherry_indices, 0, C * 2, kRsrcFlags);
         const int ci = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(ri, (c0 + (nl & 7)) * 2, 0, 0);
-        const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, K * 2, kRsrcFlags);
+        const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, rows * K * 2, kRsrcFlags);
         const uint32_t xoff = (nl < 8 && c0 + nl < C) ? (uint32_t)ci * 2u : kOob;
-        uint32_t xraw = __builtin_amdgcn_raw_buffer_load_b16(rx, xoff, 0, 0);
+        uint32_t xrow[ROWS];
+#pragma unroll
+        for (int r = 0; r < ROWS; r++)
+            xrow[r] = __builtin_amdgcn_raw_buffer_load_b16(rx, (r < rows && xoff != kOob) ? xoff + (uint32_t)(r * K) * 2u : kOob, 0, 0);
+        uint32_t xraw = xrow[0];
         if (x_gate) {
             const __amdgpu_buffer_rsrc_t rg = __builtin_amdgcn_make_buffer_rsrc((void *)x_gate, 0, K * 2, kRsrcFlags);
             const uint32_t graw = __builtin_amdgcn_raw_buffer_load_b16(rg, xoff, 0, 0);
@@ -390,18 +440,24 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
             const float rs = norm_scale<NW>(nchunk, s_ss, wave, lane, K, pro.eps);
             xraw = norm_pair(xraw & 0xffffu, nwraw & 0xffffu, rs) & 0xffffu;
         }
-        s_pair[wave][lane] = __builtin_bit_cast(uint32_t, half_bits_to_float(xraw));
+        xrow[0] = xraw;
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) s_pair[wave][r][lane] = __builtin_bit_cast(uint32_t, half_bits_to_float(xrow[r]));
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        float xc[8];
+        float xc[ROWS][8];
 #pragma unroll
-        for (int r = 0; r < 8; r++) xc[r] = __builtin_bit_cast(float, s_pair[wave][16 * kq + r]);
+        for (int b = 0; b < ROWS; b++)
+#pragma unroll
+            for (int r = 0; r < 8; r++) xc[b][r] = __builtin_bit_cast(float, s_pair[wave][b][16 * kq + r]);
 #pragma unroll
         for (int r = 0; r < 8; r++) {
 #pragma unroll
             for (int c = 0; c < 16; c++) {
                 const uint32_t ww = cw[r][c >> 3][(c & 7) >> 1];
-                tot[c] += half_bits_to_float((c & 1) ? (ww >> 16) : (ww & 0xffffu)) * xc[r];
+                const float wf = half_bits_to_float((c & 1) ? (ww >> 16) : (ww & 0xffffu));
+#pragma unroll
+                for (int b = 0; b < ROWS; b++) tot[b][c] += wf * xc[b][r];
             }
         }
     } else if (norm_w) {
@@ -411,41 +467,49 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
 
     CQ_STAMP(2);
     // ---- reduce over the four lane groups; lane group kq ends up with columns 4kq .. 4kq+3
-    float h8[8], q4[1][4];
+    float q4[ROWS][4];
 #pragma unroll
-    for (int i = 0; i < 8; i++) h8[i] = swap32_add(tot[i], tot[8 + i]);
+    for (int r = 0; r < ROWS; r++) {
+        float h8[8];
 #pragma unroll
-    for (int i = 0; i < 4; i++) q4[0][i] = swap16_add(h8[i], h8[4 + i]);
+        for (int i = 0; i < 8; i++) h8[i] = swap32_add(tot[r][i], tot[r][8 + i]);
+#pragma unroll
+        for (int i = 0; i < 4; i++) q4[r][i] = swap16_add(h8[i], h8[4 + i]);
+    }
     if (NW == 1) {
         const int n = n0 + 4 * kq;
         CQ_STAMP(3);
-        splitk_finish<__half, 1, 4>(q4, 1, N, n, n < N, plan.splits, acc_words, mul, accumulate);
+        splitk_finish<__half, ROWS, 4>(q4, rows, N, n, n < N, plan.splits, acc_words, mul, accumulate);
         CQ_STAMP(4);
     } else {
         // ---- across the workgroup's wavefronts through LDS, then 4 / NW columns per thread
-        __shared__ float s_red[NW][kTileCols];
-        *reinterpret_cast<float4 *>(&s_red[wave][16 * nl + 4 * kq]) = make_float4(q4[0][0], q4[0][1], q4[0][2], q4[0][3]);
+        __shared__ float s_red[NW][ROWS][kTileCols];
+#pragma unroll
+        for (int r = 0; r < ROWS; r++)
+            *reinterpret_cast<float4 *>(&s_red[wave][r][16 * nl + 4 * kq]) = make_float4(q4[r][0], q4[r][1], q4[r][2], q4[r][3]);
         __syncthreads();
         constexpr int CPT = 4 / NW;  // columns per thread
-        float vals[1][CPT];
+        float vals[ROWS][CPT];
 #pragma unroll
-        for (int c = 0; c < CPT; c++) {
-            float v = 0.f;
+        for (int r = 0; r < ROWS; r++)
 #pragma unroll
-            for (int wv = 0; wv < NW; wv++) v += s_red[wv][(tid * CPT + c) & (kTileCols - 1)];
-            vals[0][c] = v;
-        }
+            for (int c = 0; c < CPT; c++) {
+                float v = 0.f;
+#pragma unroll
+                for (int wv = 0; wv < NW; wv++) v += s_red[wv][r][(tid * CPT + c) & (kTileCols - 1)];
+                vals[r][c] = v;
+            }
         const int n = tile * kTileCols + tid * CPT;
         CQ_STAMP(3);
-        splitk_finish<__half, 1, CPT>(vals, 1, N, n, n < N && tid * CPT < kTileCols, plan.splits, acc_words, mul,
-                                      accumulate);
+        splitk_finish<__half, ROWS, CPT>(vals, rows, N, n, n < N && tid * CPT < kTileCols, plan.splits, acc_words, mul,
+                                         accumulate);
         CQ_STAMP(4);
     }
 }
 
 bool matvec_supported(int bits, int B, int K, int N, int C, int G) {
     (void)bits;
-    if (B != 1) return false;
+    if (B < 1 || B > kMatvecMaxRows) return false;
     if (C > kMaxFastCherries) return false;
     if (G % 32) return false;
     // byte offsets are 32-bit and kOob must lie beyond every buffer
@@ -458,21 +522,41 @@ bool matvec_supported(int bits, int B, int K, int N, int C, int G) {
 }
 
 
+// Two rows always take the streaming kernel (9.9 us against 13.6 us for the matrix-core path on
+// the 4096 -> 11008 4-bit layer: no preparation launch, atomics instead of partial tiles).  Three
+// and four rows run the four-row instantiation, whose 2.2 x decode arithmetic and register
+// count only pay while the call is dominated by fixed costs: up to 20 MB of packed weights
+// (4096 x 4096 4-bit: 9.5 us against 11.4; 4096 -> 11008 3-bit: 13.3 against 14.3; 4-bit: 15.5
+// against 14.5, left to the matrix-core path).
+bool matvec_rows_preferred(int bits, int B, int K, int N, int C, int G) {
+    if (B < 2 || !matvec_supported(bits, B, K, N, C, G)) return false;
+    if (B == 2) return true;
+    return (long long)(K - C) / 8 * bits * N <= (20ll << 20);
+}
+
 template <int BITS, int NW, int KPL>
 static hipError_t launch_matvec_nw(const __half *vec, const MatvecPrologue &pro, const MatvecGroup &grp, int tiles,
-                                   int K, int C, int G, int accumulate, void *workspace, hipStream_t stream) {
+                                   int K, int C, int G, int accumulate, void *workspace, hipStream_t stream,
+                                   int rows) {
     // the fused norm reads K activations with kNormLoads 16-byte loads per thread
     if (pro.norm_weight && K > kNormLoads * 8 * 64 * NW) return hipErrorNotSupported;
+    if (rows > 1 && (pro.norm_weight || pro.gate || grp.count != 1)) return hipErrorNotSupported;
     Plan plan = make_plan(K, kTileCols, C, NW, 4 * KPL);
     plan.tiles = tiles;
-    if (pro.norm_weight)
-        hipLaunchKernelGGL((matvec_kernel<BITS, NW, KPL, true>), dim3(plan.tiles * plan.splits), dim3(64 * NW), 0,
-                           stream, vec, pro, grp, reinterpret_cast<unsigned long long *>(workspace), K, C, G,
-                           accumulate, plan);
+    const dim3 grid(plan.tiles * plan.splits), block(64 * NW);
+    unsigned long long *acc = reinterpret_cast<unsigned long long *>(workspace);
+    if (rows > 2)
+        hipLaunchKernelGGL((matvec_kernel<BITS, NW, KPL, false, 4>), grid, block, 0, stream, vec, pro, grp, acc, K, C,
+                           G, accumulate, plan, rows);
+    else if (rows == 2)
+        hipLaunchKernelGGL((matvec_kernel<BITS, NW, KPL, false, 2>), grid, block, 0, stream, vec, pro, grp, acc, K, C,
+                           G, accumulate, plan, rows);
+    else if (pro.norm_weight)
+        hipLaunchKernelGGL((matvec_kernel<BITS, NW, KPL, true, 1>), grid, block, 0, stream, vec, pro, grp, acc, K, C,
+                           G, accumulate, plan, 1);
     else
-        hipLaunchKernelGGL((matvec_kernel<BITS, NW, KPL, false>), dim3(plan.tiles * plan.splits), dim3(64 * NW), 0,
-                           stream, vec, pro, grp, reinterpret_cast<unsigned long long *>(workspace), K, C, G,
-                           accumulate, plan);
+        hipLaunchKernelGGL((matvec_kernel<BITS, NW, KPL, false, 1>), grid, block, 0, stream, vec, pro, grp, acc, K, C,
+                           G, accumulate, plan, 1);
     return hipGetLastError();
 }
 
@@ -504,9 +588,9 @@ bool matvec_norm_supported(int bits, int K, int n_total, int C) {
     return K <= kNormLoads * 8 * 64 * matvec_waves_per_wg(K, n_total, C, kpl);
 }
 
-hipError_t launch_matvec_group(int bits, const __half *vec, const MatvecPrologue &pro, const MatvecMember *members,
-                               int count, int K, int C, int G, int accumulate, void *workspace,
-                               hipStream_t stream) {
+static hipError_t launch_matvec_rows_group(int bits, const __half *vec, const MatvecPrologue &pro,
+                                           const MatvecMember *members, int count, int K, int C, int G,
+                                           int accumulate, void *workspace, hipStream_t stream, int rows) {
     MatvecGroup grp = {};
     grp.count = count;
     int tiles = 0, n_total = 0;
@@ -521,7 +605,7 @@ hipError_t launch_matvec_group(int bits, const __half *vec, const MatvecPrologue
     const int kpl = matvec_kpl(bits, K, n_total, C);
     const int nw = matvec_waves_per_wg(K, n_total, C, kpl);
 #define CQ_LAUNCH(B, W, P)                                                                                   \
-    return launch_matvec_nw<B, W, P>(vec, pro, grp, tiles, K, C, G, accumulate, workspace, stream)
+    return launch_matvec_nw<B, W, P>(vec, pro, grp, tiles, K, C, G, accumulate, workspace, stream, rows)
 #define CQ_PICK_NW(B, P)                                                                                     \
     do {                                                                                                     \
         if (nw >= 4) CQ_LAUNCH(B, 4, P);                                                                     \
@@ -538,12 +622,28 @@ hipError_t launch_matvec_group(int bits, const __half *vec, const MatvecPrologue
 #undef CQ_LAUNCH
 }
 
+hipError_t launch_matvec_group(int bits, const __half *vec, const MatvecPrologue &pro, const MatvecMember *members,
+                               int count, int K, int C, int G, int accumulate, void *workspace,
+                               hipStream_t stream) {
+    return launch_matvec_rows_group(bits, vec, pro, members, count, K, C, G, accumulate, workspace, stream, 1);
+}
+
 hipError_t launch_matvec(int bits, const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
                          const int16_t *cherry_indices, const __half *scales, __half *mul, int K, int N, int C,
                          int G, int accumulate, void *workspace, hipStream_t stream) {
     MatvecMember m = {qweight, cherry_weight, cherry_indices, scales, mul, N, 0};
     return launch_matvec_group(bits, vec, MatvecPrologue{nullptr, nullptr, 0.f}, &m, 1, K, C, G, accumulate,
                                workspace, stream);
+}
+
+// 2..kMatvecMaxRows activation rows (vec (rows, K), mul (rows, N), one accumulator word per
+// output in `workspace`) in one pass over the weights.
+hipError_t launch_matvec_rows(int bits, const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
+                              const int16_t *cherry_indices, const __half *scales, __half *mul, int rows, int K,
+                              int N, int C, int G, int accumulate, void *workspace, hipStream_t stream) {
+    MatvecMember m = {qweight, cherry_weight, cherry_indices, scales, mul, N, 0};
+    return launch_matvec_rows_group(bits, vec, MatvecPrologue{nullptr, nullptr, 0.f}, &m, 1, K, C, G, accumulate,
+                                    workspace, stream, rows);
 }
 
 }  // namespace cq

@@ -294,6 +294,8 @@ def test_batch_accumulate_scale_invariance_and_determinism(qc):
     (4, 128, 4096, 72, 1 / 16, 1), (3, 128, 4096, 72, 1 / 16, 4),     # 256 cherries: beyond the fast path
     (3, 32, 512, 256, 1 / 32, 1), (4, 4096, 4096, 256, 1 / 256, 1),   # group 32; one group for all of K
     (4, 128, 2048 + 8, 256, 1 / 256, 1), (3, 128, 2048 + 8, 256, 1 / 256, 1),  # ragged last unit (8 positions)
+    (4, 128, 2048 + 8, 256, 1 / 256, 2), (3, 128, 2048 + 8, 264, 1 / 256, 4),  # the same with 2 and 4 rows in one pass
+    (4, 128, 1024, 8, 1 / 256, 3), (3, 128, 4096, 1000, 1 / 32, 2),           # rows: tiny N; 128 cherries
 ])
 def test_layout_variants(qc, bits, gs, k, n, frac, b):
     announce("variant", bits, gs, k, n, frac, b)
