@@ -255,7 +255,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default="llama7b_gate_up_w4", choices=sorted(WORKLOADS))
     ap.add_argument("--group", type=int, default=128)
-    ap.add_argument("--batch", type=int, default=1, help="activation rows per call (2..16: small-batch matrix-core kernel, more: tiled GEMM kernel)")
+    ap.add_argument("--batch", type=int, default=1, help="activation rows per call (2..4: streaming kernel with several rows or, like 5..16, the small-batch matrix-core kernel; more: tiled GEMM kernel)")
     ap.add_argument("--all", action="store_true", help="also print a table of every workload to stderr")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the 7B-shape decode measurement")
@@ -285,7 +285,8 @@ def main():
 
     if args.all:
         # the small-batch path (matrix cores) on the 13B and 70B layer shapes
-        for name, b in (("llama13b_attn_w3", 4), ("llama13b_attn_w3", 8), ("llama13b_gate_up_w3", 8),
+        for name, b in (("llama7b_gate_up_w4", 2), ("llama7b_attn_w4", 2), ("llama7b_attn_w4", 4),
+                        ("llama13b_attn_w3", 4), ("llama13b_attn_w3", 8), ("llama13b_gate_up_w3", 8),
                         ("llama13b_down_w3", 8), ("llama70b_attn_w4", 16), ("llama70b_kv_w4", 16),
                         ("llama70b_gate_up_w4", 16), ("llama70b_down_w4", 16), ("llama7b_gate_up_w4", 16)):
             bits, k, n = WORKLOADS[name]
@@ -295,7 +296,7 @@ def main():
             fl = 2.0 * b * k * n
             print(f"{name:24s} {bits}-bit {k:5d}->{n:5d} batch {b:2d}: {us:7.2f} us  {ab / us / 1e3:7.1f} GB/s "
                   f"{ab / us / 1e3 / HBM_PEAK_GBS * 100:5.1f}% of 8 TB/s  {fl / us / 1e6:6.1f} TFLOP/s "
-                  f"({fl / us / 1e6 / 2500 * 100:4.1f}% of fp16 MFMA peak; prep + main kernel)",
+                  f"({fl / us / 1e6 / 2500 * 100:4.1f}% of fp16 MFMA peak; whole call)",
                   file=sys.stderr, flush=True)
             torch.cuda.empty_cache()
         # prompt-sized batches: the tiled dequantise + MFMA GEMM kernel
@@ -373,6 +374,8 @@ def main():
                      "traffic": MEASURED_TRAFFIC.get((args.workload, args.batch)),
                      "algorithmic_bytes_per_launch": ab,
                      "kernel": f"cq::matvec_kernel<{bits}>" if args.batch == 1 else
+                               f"cq::matvec_kernel<{bits}, rows {2 if args.batch == 2 else 4}>"
+                               if args.batch == 2 or (args.batch <= 4 and (k - k // 256 // 8 * 8) // 8 * bits * n <= 20 << 20) else
                                f"cq::batch_prep_kernel<{bits}> + cq::batch_kernel<{bits}>" if args.batch <= 16 else
                                f"cq::gemm_prep_kernel<{bits}> + cq::gemm_kernel<{bits}, 2>"},
     }
