@@ -33,6 +33,8 @@ namespace cq {
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
 
 // Optional per-wave phase timestamps for a profiling harness; compiled out in the library.
 #ifdef CQ_TRACE
@@ -126,9 +128,12 @@ struct Geo {
 
 // NW = wavefronts (= units) per workgroup: 4, or 2 or 1 when the layer is so small
 // that larger workgroups would leave CUs without work.
-// ROWS = activation rows handled in the same pass (1, 2 or 4): the codes are decoded once and
-// every row adds its own dot products; `rows` (<= ROWS) of them exist, the others read zeros.
-// The norm / gate prologues exist for one row only.
+// ROWS = activation rows handled in the same pass (1, 2 or 4); `rows` (<= ROWS) of them exist, the
+// others read zeros.  The codes are decoded once.  ROWS == 2: every row adds its own dot2 products.
+// ROWS == 4: the masked code fields of 4 positions are the B operand and one row's activations
+// the A operand of v_mfma_f32_4x4x4_16B_f16 (16 independent 4 x 4 x 4 products, one per group of
+// four lanes), which costs about what the two dot2 of the one-row kernel cost.  The norm / gate
+// prologues exist for one row only.
 template <int BITS, int NW, int KPL, bool NORM, int ROWS>
 __global__ __launch_bounds__(64 * NW) void matvec_kernel(
     const __half *__restrict__ x, MatvecPrologue pro, MatvecGroup grp,
@@ -266,6 +271,7 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
         if (BITS == 4) {
             j0 = 4 * (nl >> 1) + (nl & 1);  // even lanes: (4p, 4p+2), odd lanes: (4p+1, 4p+3)
             j1 = j0 + 2;
+            if (ROWS == 4) p0 = p1 = 4 * (nl & 1);  // the matrix-core path keeps one accumulator: high nibbles sit at bit 4
         } else {
             const int q = nl & 3, t8 = 8 * (nl >> 2);  // code pairs (0,3) (1,4) (5,6) (2,7) of a unit
             j0 = t8 + ((0x2510 >> (4 * q)) & 15);
@@ -306,7 +312,7 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
             uint32_t h1 = (prep && k1 < Kn) ? winh[(k1 - ubase) + low1] : 0u;
             xsum[r] = row_sum(half_bits_to_float(h0) + half_bits_to_float(h1));
             sh[r] = 0;
-            if (BITS == 3) {
+            if (BITS == 3 || ROWS == 4) {
                 // scale the lane group's activations so that the largest has biased exponent 29;
                 // the per-field factors 2^-p (p <= 7) then stay far inside the fp16 normal range
                 const int e = row_max((int)max(h0 & 0x7fffu, h1 & 0x7fffu)) >> 10;
@@ -318,15 +324,72 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        u32x4 xq[ROWS][G_::kPairs / 4];
+        // ROWS == 4: v_mfma_f32_4x4x4_16B_f16 works on 16 blocks of 4 lanes; lane t of a block feeds
+        // row t's activations (A, 4 positions) and its own column's code fields (B, the same 4
+        // positions) and receives its column's sums for all four rows, so a lane holds the
+        // activations of ONE row, as in the one-row kernel.
+        constexpr int XR = ROWS == 4 ? 1 : ROWS;
+        u32x4 xq[XR][G_::kPairs / 4];
 #pragma unroll
-        for (int r = 0; r < ROWS; r++)
+        for (int r = 0; r < XR; r++)
 #pragma unroll
             for (int i = 0; i < G_::kPairs / 4; i++)
-                xq[r][i] = *reinterpret_cast<const u32x4 *>(&s_pair[wave][r][16 * kq + 4 * i]);
+                xq[r][i] = *reinterpret_cast<const u32x4 *>(&s_pair[wave][ROWS == 4 ? (lane & 3) : r][16 * kq + 4 * i]);
         CQ_STAMP(1);
 
-        if (BITS == 4) {
+        if (ROWS == 4) {
+            // d[c][r]: this lane's column c, activation row r
+            float4_t d[16];
+#pragma unroll
+            for (int c = 0; c < 16; c++) d[c] = (float4_t){0.f, 0.f, 0.f, 0.f};
+            if (BITS == 4) {
+#pragma unroll
+                for (int p = 0; p < R / 2; p++) {
+                    const half4_t av = __builtin_bit_cast(half4_t, (u32x2){xq[0][p >> 1][(p & 1) * 2], xq[0][p >> 1][(p & 1) * 2 + 1]});
+#pragma unroll
+                    for (int dd = 0; dd < 4; dd++) {
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const uint32_t pr = __builtin_amdgcn_perm(w[2 * p][dd], w[2 * p + 1][dd],
+                                                                      0x0c000c00u | (uint32_t)(j << 16) | (uint32_t)(4 + j));
+                            const half4_t bv = __builtin_bit_cast(half4_t, (u32x2){pr & 0x000f000fu, pr & 0x00f000f0u});
+                            d[4 * dd + j] = __builtin_amdgcn_mfma_f32_4x4x4f16(av, bv, d[4 * dd + j], 0, 0, 0);
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < R / 3; t++) {
+                    const half4_t a0 = __builtin_bit_cast(half4_t, (u32x2){xq[0][t][0], xq[0][t][1]});
+                    const half4_t a1 = __builtin_bit_cast(half4_t, (u32x2){xq[0][t][2], xq[0][t][3]});
+#pragma unroll
+                    for (int dd = 0; dd < 4; dd++) {
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const uint32_t sel = 0x0c000000u | (uint32_t)(j << 16) | (uint32_t)(j << 8) | (uint32_t)(4 + j);
+                            const uint32_t p1 = __builtin_amdgcn_perm(w[3 * t][dd], w[3 * t + 1][dd], sel);
+                            const uint32_t p2 = __builtin_amdgcn_perm(w[3 * t + 1][dd], w[3 * t + 2][dd], sel);
+                            const half4_t b0 = __builtin_bit_cast(half4_t, (u32x2){p1 & 0x000e0007u, p1 & 0x00700038u});
+                            const half4_t b1 = __builtin_bit_cast(
+                                half4_t, (u32x2){p2 & 0x001c0380u, (p1 & 0x000001c0u) | (p2 & 0x00e00000u)});
+                            d[4 * dd + j] = __builtin_amdgcn_mfma_f32_4x4x4f16(a0, b0, d[4 * dd + j], 0, 0, 0);
+                            d[4 * dd + j] = __builtin_amdgcn_mfma_f32_4x4x4f16(a1, b1, d[4 * dd + j], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+            constexpr float kGrid = BITS == 4 ? -7.5f : -3.5f;
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) {
+                const float corr = kGrid * xsum[r];
+#pragma unroll
+                for (int c = 0; c < 16; c++) {
+                    const uint32_t sw = c < 8 ? sc0[c >> 1] : sc1[(c - 8) >> 1];
+                    const float s = half_bits_to_float((c & 1) ? (sw >> 16) : (sw & 0xffffu));
+                    tot[r][c] = (ldexpf(d[c][r], 24 - sh[r]) + corr) * s;
+                }
+            }
+        } else if (BITS == 4) {
             float lo[ROWS][16], hi[ROWS][16];
 #pragma unroll
             for (int r = 0; r < ROWS; r++)
@@ -522,16 +585,14 @@ bool matvec_supported(int bits, int B, int K, int N, int C, int G) {
 }
 
 
-// Two rows always take the streaming kernel (9.9 us against 13.6 us for the matrix-core path on
-// the 4096 -> 11008 4-bit layer: no preparation launch, atomics instead of partial tiles).  Three
-// and four rows run the four-row instantiation, whose 2.2 x decode arithmetic and register
-// count only pay while the call is dominated by fixed costs: up to 20 MB of packed weights
-// (4096 x 4096 4-bit: 9.5 us against 11.4; 4096 -> 11008 3-bit: 13.3 against 14.3; 4-bit: 15.5
-// against 14.5, left to the matrix-core path).
+// Two to four rows take this kernel rather than the matrix-core batch path whenever it takes the
+// shape: no preparation launch, atomics instead of partial tiles.  Measured on the 4096 -> 11008
+// 4-bit layer: 2 rows 9.8 us (batch path 13.6), 3 rows 12.3 (14.1), 4 rows 13.2 (14.5); 8192 ->
+// 28672: 28.1 (35.8) and 34.3 (37.6); the one exception found, 5120 -> 13824 3-bit at 4 rows, is
+// 2 % slower (18.1 against 17.6).  Two rows run the dot2 instantiation (the 4 x 4 MFMA one costs
+// 11.4 us there), three and four the MFMA one.
 bool matvec_rows_preferred(int bits, int B, int K, int N, int C, int G) {
-    if (B < 2 || !matvec_supported(bits, B, K, N, C, G)) return false;
-    if (B == 2) return true;
-    return (long long)(K - C) / 8 * bits * N <= (20ll << 20);
+    return B >= 2 && matvec_supported(bits, B, K, N, C, G);
 }
 
 template <int BITS, int NW, int KPL>
