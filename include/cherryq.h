@@ -63,7 +63,7 @@ const char *cherryq_status_string(int status);
  * scratch: uninitialised memory for the batched paths (batch >= 2): per-split partial tiles and
  *   the activations laid out in matrix-core operand order.  At least cherryq_scratch_bytes()
  *   bytes (0 for batch 1, then it may be NULL), 256-byte aligned.
- * Both sizes depend on the batch: up to 16 rows run in the small-batch kernel, more (prompt
+ * Both sizes depend on the batch: up to 16 rows run in the streaming or the small-batch kernel, more (prompt
  * processing) in the tiled GEMM kernel, whose compacted copy of the activations and partial
  * tiles grow with the number of rows.  Size the buffers for the largest batch that will be passed.
  * Calls that may overlap in time (different streams) must use different workspace and scratch.
