@@ -587,10 +587,9 @@ bool matvec_supported(int bits, int B, int K, int N, int C, int G) {
 
 // Two to four rows take this kernel rather than the matrix-core batch path whenever it takes the
 // shape: no preparation launch, atomics instead of partial tiles.  Measured on the 4096 -> 11008
-// 4-bit layer: 2 rows 9.8 us (batch path 13.6), 3 rows 12.3 (14.1), 4 rows 13.2 (14.5); 8192 ->
-// 28672: 28.1 (35.8) and 34.3 (37.6); the one exception found, 5120 -> 13824 3-bit at 4 rows, is
-// 2 % slower (18.1 against 17.6).  Two rows run the dot2 instantiation (the 4 x 4 MFMA one costs
-// 11.4 us there), three and four the MFMA one.
+// 4-bit layer: 2 rows 9.5 us (batch path 13.6), 3 rows 11.0 (14.1), 4 rows 11.5 (14.5); 8192 ->
+// 28672: 28.2 (35.8) and 34.3 (37.6).  Two rows run the dot2 instantiation (the 4 x 4 MFMA one
+// costs 11.4 us there), three and four the MFMA one.
 bool matvec_rows_preferred(int bits, int B, int K, int N, int C, int G) {
     return B >= 2 && matvec_supported(bits, B, K, N, C, G);
 }
@@ -663,7 +662,10 @@ static hipError_t launch_matvec_rows_group(int bits, const __half *vec, const Ma
     }
     for (int i = count; i < kMaxGroup; i++) grp.m[i] = grp.m[0];
     // geometry from the group's total size: the launch streams all members' weights together
-    const int kpl = matvec_kpl(bits, K, n_total, C);
+    // three and four rows: 128-position units whatever the size -- every row multiplies the split-K
+    // atomics (0.85 us per row on the 4096 -> 11008 layer with 64-position units), half as many
+    // splits outweigh the coarser grid (4 rows: 13.1 -> 11.5 us; two rows: 9.5 -> 10.1, left alone)
+    const int kpl = rows > 2 ? 32 : matvec_kpl(bits, K, n_total, C);
     const int nw = matvec_waves_per_wg(K, n_total, C, kpl);
 #define CQ_LAUNCH(B, W, P)                                                                                   \
     return launch_matvec_nw<B, W, P>(vec, pro, grp, tiles, K, C, G, accumulate, workspace, stream, rows)
