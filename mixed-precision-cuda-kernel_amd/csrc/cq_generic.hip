@@ -232,12 +232,15 @@ __device__ inline int cherries_below(const IDX *__restrict__ idx, int C, int d) 
     return lo;
 }
 
+constexpr int kUnpackMaxBlocks = 4;  // row blocks of kUnpackRows a workgroup may walk
+
 template <int BITS>
 __global__ __launch_bounds__(256) void unpack_kernel(const uint8_t *__restrict__ qweight,
                                                      const __half *__restrict__ cherry_weight,
                                                      const int16_t *__restrict__ cherry_indices,
                                                      const __half *__restrict__ scales,
-                                                     __half *__restrict__ dense, int K, int N, int C, int G) {
+                                                     __half *__restrict__ dense, int K, int N, int C, int G,
+                                                     int blocks) {
     __shared__ unsigned short s_norm[kUnpackRows][kUnpackUnits * 8 + 2];
     __shared__ unsigned short s_ch[kUnpackCols][kUnpackRows];
     __shared__ short s_src[kUnpackCols];
@@ -247,7 +250,6 @@ __global__ __launch_bounds__(256) void unpack_kernel(const uint8_t *__restrict__
     __shared__ int16_t s_idx[kIdxCap];
     const int Kn = K - C;
     const int d0 = blockIdx.x * kUnpackCols, d1 = min(d0 + kUnpackCols, K);
-    const int n0 = blockIdx.y * kUnpackRows;
     const int t = threadIdx.x;
     const int16_t *idx = cherry_indices;
     if (C <= kIdxCap) {
@@ -268,62 +270,102 @@ __global__ __launch_bounds__(256) void unpack_kernel(const uint8_t *__restrict__
         }
         s_src[t] = src;
     }
-    for (int e = t; e < (c_hi - c_lo) * kUnpackRows; e += 256) {
-        const int c = e / kUnpackRows, nl = e % kUnpackRows;
-        s_ch[c][nl] = n0 + nl < N ? __half_as_ushort(cherry_weight[(size_t)(c_lo + c) * N + n0 + nl]) : 0;
-    }
-    for (int e = t; e < units * 16; e += 256) {
-        const int u = e >> 4, quad = e & 15;
-        const int k0 = ku0 + 8 * u, nq = n0 + 4 * quad;
-        if (k0 >= Kn || nq >= N) continue;
-        uint32_t w[BITS];
-#pragma unroll
-        for (int r = 0; r < BITS; r++)
-            w[r] = *reinterpret_cast<const uint32_t *>(qweight + (size_t)(k0 / 8 * BITS + r) * N + nq);
-        const uint2 sraw = *reinterpret_cast<const uint2 *>(scales + (size_t)(k0 / G) * N + nq);
-        const uint32_t sbits[4] = {sraw.x & 0xffffu, sraw.x >> 16, sraw.y & 0xffffu, sraw.y >> 16};
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-            float v[8];
-            decode8<BITS>(w, c, v);
-            // (code - c_b) has 4 significant bits and the fp16 scale 11: the float product is
-            // exact, so this is the single rounding the reference performs
-            const float sc = __half2float(__ushort_as_half((unsigned short)sbits[c]));
-#pragma unroll
-            for (int i = 0; i < 8; i++) s_norm[4 * quad + c][8 * u + i] = __half_as_ushort(__float2half_rn(v[i] * sc));
-        }
-    }
     __syncthreads();
-    for (int e = t; e < kUnpackRows * (kUnpackCols / 8); e += 256) {
-        const int seg = e & 15, nl = e >> 4;
-        const int d = d0 + 8 * seg;
-        if (d >= d1 || n0 + nl >= N) continue;
-        unsigned short h[8];
+    // a thread writes the same 8-column segment of every row it handles: its sources are read once
+    static_assert(256 % (kUnpackCols / 8) == 0, "a thread keeps its segment across rows");
+    const int seg = t & 15;
+    const int dseg = d0 + 8 * seg;
+    int src[8];
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const int src = s_src[8 * seg + j];
-            h[j] = src >= 0 ? s_norm[nl][src] : s_ch[-1 - src][nl];
+    for (int j = 0; j < 8; j++) src[j] = s_src[8 * seg + j];
+
+    // The column range's geometry is found once; the workgroup then walks `blocks` blocks of
+    // kUnpackRows rows, with the packed codes of the next block requested before the current one
+    // is written out.  units * 16 items of (8 positions x 4 rows) per block: with the usual 17
+    // units that is 272 for 256 threads, so a thread may own two.
+    constexpr int kItems = (kUnpackUnits * 16 + 255) / 256;
+    uint32_t w[kItems][BITS];
+    uint2 sraw[kItems];
+    bool live[kItems];
+    auto request = [&](int n0) {
+#pragma unroll
+        for (int it = 0; it < kItems; it++) {
+            const int e = t + 256 * it;
+            const int u = e >> 4, quad = e & 15;
+            const int k0 = ku0 + 8 * u, nq = n0 + 4 * quad;
+            live[it] = e < units * 16 && k0 < Kn && nq < N;
+            if (live[it]) {
+#pragma unroll
+                for (int r = 0; r < BITS; r++)
+                    w[it][r] = *reinterpret_cast<const uint32_t *>(qweight + (size_t)(k0 / 8 * BITS + r) * N + nq);
+                sraw[it] = *reinterpret_cast<const uint2 *>(scales + (size_t)(k0 / G) * N + nq);
+            }
         }
-        uint4 out;
-        out.x = h[0] | (uint32_t)h[1] << 16;
-        out.y = h[2] | (uint32_t)h[3] << 16;
-        out.z = h[4] | (uint32_t)h[5] << 16;
-        out.w = h[6] | (uint32_t)h[7] << 16;
-        *reinterpret_cast<uint4 *>(dense + (size_t)(n0 + nl) * K + d) = out;
+    };
+    const int nb0 = blockIdx.y * blocks * kUnpackRows;
+    request(nb0);
+    for (int b = 0; b < blocks; b++) {
+        const int n0 = nb0 + b * kUnpackRows;
+        if (n0 >= N) break;  // uniform
+        for (int e = t; e < (c_hi - c_lo) * kUnpackRows; e += 256) {
+            const int c = e / kUnpackRows, nl = e % kUnpackRows;
+            s_ch[c][nl] = n0 + nl < N ? __half_as_ushort(cherry_weight[(size_t)(c_lo + c) * N + n0 + nl]) : 0;
+        }
+#pragma unroll
+        for (int it = 0; it < kItems; it++) {
+            if (!live[it]) continue;
+            const int e = t + 256 * it;
+            const int u = e >> 4, quad = e & 15;
+            const uint32_t sbits[4] = {sraw[it].x & 0xffffu, sraw[it].x >> 16, sraw[it].y & 0xffffu, sraw[it].y >> 16};
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                float v[8];
+                decode8<BITS>(w[it], c, v);
+                // (code - c_b) has 4 significant bits and the fp16 scale 11: the float product is
+                // exact, so this is the single rounding the reference performs
+                const float sc = __half2float(__ushort_as_half((unsigned short)sbits[c]));
+#pragma unroll
+                for (int i = 0; i < 8; i++)
+                    s_norm[4 * quad + c][8 * u + i] = __half_as_ushort(__float2half_rn(v[i] * sc));
+            }
+        }
+        __syncthreads();
+        if (b + 1 < blocks && n0 + kUnpackRows < N) request(n0 + kUnpackRows);
+        if (dseg < d1) {
+#pragma unroll
+            for (int i = 0; i < kUnpackRows * (kUnpackCols / 8) / 256; i++) {
+                const int nl = (t >> 4) + 16 * i;
+                if (n0 + nl >= N) continue;
+                unsigned short h[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) h[j] = src[j] >= 0 ? s_norm[nl][src[j]] : s_ch[-1 - src[j]][nl];
+                uint4 out;
+                out.x = h[0] | (uint32_t)h[1] << 16;
+                out.y = h[2] | (uint32_t)h[3] << 16;
+                out.z = h[4] | (uint32_t)h[5] << 16;
+                out.w = h[6] | (uint32_t)h[7] << 16;
+                *reinterpret_cast<uint4 *>(dense + (size_t)(n0 + nl) * K + dseg) = out;
+            }
+        }
+        __syncthreads();  // the next block's decode overwrites s_norm / s_ch
     }
 }
 
 hipError_t launch_unpack(int bits, const uint8_t *qweight, const __half *cherry_weight,
                          const int16_t *cherry_indices, const __half *scales, __half *dense, int K, int N,
                          int C, int G, hipStream_t stream) {
-    dim3 grid(ceil_div(K, kUnpackCols), ceil_div(N, kUnpackRows));
-    if (grid.x == 0 || grid.y == 0) return hipSuccess;
+    if (K <= 0 || N <= 0) return hipSuccess;
+    // more row blocks per workgroup hide the load latency better, as long as the launch still
+    // gives every CU several workgroups
+    auto workgroups = [&](int b) { return (long)ceil_div(K, kUnpackCols) * ceil_div(N, kUnpackRows * b); };
+    const int blocks = workgroups(kUnpackMaxBlocks) >= 4096 ? kUnpackMaxBlocks : workgroups(2) >= 512 ? 2 : 1;
+    dim3 grid(ceil_div(K, kUnpackCols), ceil_div(N, kUnpackRows * blocks));
     if (bits == 4)
         hipLaunchKernelGGL(unpack_kernel<4>, grid, dim3(256), 0, stream, qweight, cherry_weight, cherry_indices,
-                           scales, dense, K, N, C, G);
+                           scales, dense, K, N, C, G, blocks);
     else
         hipLaunchKernelGGL(unpack_kernel<3>, grid, dim3(256), 0, stream, qweight, cherry_weight, cherry_indices,
-                           scales, dense, K, N, C, G);
+                           scales, dense, K, N, C, G, blocks);
     return hipGetLastError();
 }
 
