@@ -216,6 +216,7 @@ int cherryq_unpack_f16(int w_bits, const uint8_t *qweight, const void *cherry_we
     if (w_bits != 3 && w_bits != 4) return CHERRYQ_E_BITS;
     int K = in_features, N = out_features, C = num_cherries;
     if (K <= 0 || N <= 0 || C < 0 || C > K || K % 8 || N % 8 || C % 8) return CHERRYQ_E_SHAPE;
+    if (C > 0 && K > 32768) return CHERRYQ_E_SHAPE;  // int16 channel indices cannot name the columns
     if (group_size <= 0 || group_size % 8) return CHERRYQ_E_GROUP;
     if (!dense) return CHERRYQ_E_NULL;
     if (K - C > 0 && (!qweight || !scales)) return CHERRYQ_E_NULL;
@@ -235,6 +236,7 @@ int cherryq_pack_f16(int w_bits, const void *weight, const int16_t *cherry_indic
     if (w_bits != 3 && w_bits != 4) return CHERRYQ_E_BITS;
     const int K = in_features, N = out_features, C = num_cherries;
     if (K <= 0 || N <= 0 || C < 0 || C > K || K % 8 || C % 8) return CHERRYQ_E_SHAPE;
+    if (C > 0 && K > 32768) return CHERRYQ_E_SHAPE;  // int16 channel indices cannot name the columns
     if (group_size <= 0) return CHERRYQ_E_GROUP;
     if (!weight) return CHERRYQ_E_NULL;
     if (K - C > 0 && (!qweight || !scales)) return CHERRYQ_E_NULL;
@@ -299,6 +301,7 @@ int cherryq_decode_matvec_group_f16(int w_bits, const void *vec, const void *vec
     if (!layers) return CHERRYQ_E_NULL;
     if (n_layers < 1 || n_layers > kMaxGroup) return CHERRYQ_E_SHAPE;
     const int K = in_features, C = num_cherries, G = group_size;
+    if (C > 0 && K > 32768) return CHERRYQ_E_SHAPE;  // int16 channel indices cannot name the columns
     int outs[kMaxGroup];
     for (int i = 0; i < n_layers; i++) outs[i] = layers[i].out_features;
     if (workspace_bytes < cherryq_group_workspace_bytes(n_layers, outs)) return CHERRYQ_E_WORKSPACE;

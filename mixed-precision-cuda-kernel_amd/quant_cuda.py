@@ -86,29 +86,33 @@ def _check(t: torch.Tensor, name: str, dtype, ndim: int, device=None):
 
 # Per (device, stream): a zero-initialised workspace (the kernels leave it all zero after every
 # call, so it is reusable as is) and an uninitialised scratch buffer for the batched path.  Both
-# grow on demand.
+# grow on demand, at least doubling.  An outgrown buffer is kept alive rather than freed: a HIP
+# graph captured earlier on that stream may still hold its address (doubling bounds what is kept
+# to the size of the live buffer).
 _workspaces: dict = {}
 _scratches: dict = {}
+_outgrown: list = []
+
+
+def _grown(table: dict, key, nbytes: int, floor: int, alloc, device) -> torch.Tensor:
+    buf = table.get(key)
+    if buf is None or buf.numel() < nbytes:
+        if buf is not None:
+            _outgrown.append(buf)
+            nbytes = max(nbytes, 2 * buf.numel())
+        buf = alloc(max(nbytes, floor), dtype=torch.uint8, device=device)
+        table[key] = buf
+    return buf
 
 
 def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
-    key = (device.index, stream)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(max(nbytes, 1 << 18), dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
-    return ws
+    return _grown(_workspaces, (device.index, stream), nbytes, 1 << 18, torch.zeros, device)
 
 
 def _scratch(device: torch.device, stream: int, nbytes: int):
     if nbytes == 0:
         return None
-    key = (device.index, stream)
-    sc = _scratches.get(key)
-    if sc is None or sc.numel() < nbytes:
-        sc = torch.empty(nbytes, dtype=torch.uint8, device=device)
-        _scratches[key] = sc
-    return sc
+    return _grown(_scratches, (device.index, stream), nbytes, 1, torch.empty, device)
 
 
 def _ptr(t: torch.Tensor):

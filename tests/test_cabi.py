@@ -110,6 +110,15 @@ def test_dequant_validation(lib):
     u.restype = ctypes.c_int
     assert u(5, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 4096, 4096, 16, 128, None) == -5
     assert u(4, 0x1000, 0x1000, 0x1000, 0x1000, None, 4096, 4096, 16, 128, None) == -1
+    assert u(4, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 32768 + 8, 4096, 16, 128, None) == -2  # int16 indices
+    assert u(4, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 4096, 4100, 16, 128, None) == -2
+    p = lib.cherryq_pack_f16
+    p.argtypes = [ctypes.c_int] + [ctypes.c_void_p] * 5 + [ctypes.c_int] * 4 + [ctypes.c_void_p]
+    p.restype = ctypes.c_int
+    assert p(2, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 4096, 4096, 16, 128, None) == -5
+    assert p(4, None, 0x1000, 0x1000, 0x1000, 0x1000, 4096, 4096, 16, 128, None) == -1
+    assert p(4, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 32768 + 8, 4096, 16, 128, None) == -2
+    assert p(4, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 4096, 4096, 16, 0, None) == -3
 
 
 def test_python_binding_fails_loudly_without_gpu_tensors():
