@@ -99,14 +99,27 @@ GemmPlan gemm_plan(int M, int K, int N, int C) {
 // One thread per (row, group of 8 positions): x[row][normal(8 g + ord[kk])] in the normal part,
 // x[row][idx[c]] in the cherry part, 0 in the padding (rows >= M, positions past the end).  The 16
 // bytes go where the matrix core wants them: block (row / 32, g / 2) of 1 KB, lane (g % 2) * 32 +
-// row % 32 -- the A fragment of v_mfma_f32_32x32x16_f16 for 32 rows x 16 positions.
+// row % 32 -- the A fragment of v_mfma_f32_32x32x16_f16 for 32 rows x 16 positions.  A wavefront
+// fills one such block (its 64 stores are 1 KB of contiguous memory; lines written piecewise by
+// workgroups on different XCDs reach HBM as partial writes), and the four wavefronts of a
+// workgroup take four adjacent blocks, so that together they read whole lines of the 32 rows.
 template <int BITS>
 __global__ __launch_bounds__(256) void gemm_prep_kernel(const __half *__restrict__ x,
-                                                        const int16_t *__restrict__ cherry_indices,
+                                                        const int16_t *cherry_indices,
                                                         uint4 *__restrict__ a, int M, int K, int C, int Kp,
                                                         int groups_normal) {
-    const int g = blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
-    if (g >= Kp / 8) return;
+    // the searches below are chains of dependent loads: from LDS when the index list fits
+    constexpr int kIdxCap = 1024;
+    __shared__ int16_t s_idx[kIdxCap];
+    if (C <= kIdxCap) {
+        for (int i = threadIdx.x; i < C; i += 256) s_idx[i] = cherry_indices[i];
+        __syncthreads();
+        cherry_indices = s_idx;
+    }
+    const int lane = threadIdx.x & 63;
+    const int pb = blockIdx.x * 4 + (threadIdx.x >> 6);  // block of 16 positions
+    if (pb >= Kp / 16) return;
+    const int g = 2 * pb + (lane >> 5), row = blockIdx.y * 32 + (lane & 31);
     const int Kn = K - C;
     unsigned short h[8];
 #pragma unroll
@@ -123,10 +136,29 @@ __global__ __launch_bounds__(256) void gemm_prep_kernel(const __half *__restrict
                 while (lo < C && (int)cherry_indices[lo] - lo <= kb + j) lo++;
                 lows[j] = lo;
             }
+            const int s0 = kb + lows[0];
+            if (lows[7] == lows[0] && kb + 8 <= Kn && (s0 & ~1) + 10 <= K) {
+                // no cherry channel inside the group: 8 adjacent source columns, fetched as five
+                // aligned dwords and shifted by one half when the first column is odd
+                const uint32_t *src = reinterpret_cast<const uint32_t *>(xr + (s0 & ~1));
+                uint32_t w[5];
 #pragma unroll
-            for (int kk = 0; kk < 8; kk++) {
-                const int j = gemm_ord<BITS>(kk);
-                if (kb + j < Kn) h[kk] = __half_as_ushort(xr[kb + j + lows[j]]);
+                for (int d = 0; d < 5; d++) w[d] = src[d];
+                unsigned short v[8];
+#pragma unroll
+                for (int d = 0; d < 4; d++) {
+                    const uint32_t pair = (s0 & 1) ? __builtin_amdgcn_alignbit(w[d + 1], w[d], 16) : w[d];
+                    v[2 * d] = (unsigned short)pair;
+                    v[2 * d + 1] = (unsigned short)(pair >> 16);
+                }
+#pragma unroll
+                for (int kk = 0; kk < 8; kk++) h[kk] = v[gemm_ord<BITS>(kk)];
+            } else {
+#pragma unroll
+                for (int kk = 0; kk < 8; kk++) {
+                    const int j = gemm_ord<BITS>(kk);
+                    if (kb + j < Kn) h[kk] = __half_as_ushort(xr[kb + j + lows[j]]);
+                }
             }
         } else {
             const int c0 = (g - groups_normal) * 8;
@@ -135,8 +167,8 @@ __global__ __launch_bounds__(256) void gemm_prep_kernel(const __half *__restrict
                 if (c0 + kk < C) h[kk] = __half_as_ushort(xr[(int)cherry_indices[c0 + kk]]);
         }
     }
-    const size_t block = (size_t)(row >> 5) * (Kp / 16) + (g >> 1);
-    a[block * 64 + (g & 1) * 32 + (row & 31)] =
+    const size_t block = (size_t)blockIdx.y * (Kp / 16) + pb;
+    a[block * 64 + lane] =
         make_uint4(h[0] | h[1] << 16, h[2] | h[3] << 16, h[4] | h[5] << 16, h[6] | h[7] << 16);
 }
 
@@ -444,7 +476,7 @@ static hipError_t launch_gemm_bits(const __half *vec, const uint8_t *qweight, co
     __half *a = reinterpret_cast<__half *>(scratch);
     float *partial = reinterpret_cast<float *>(reinterpret_cast<char *>(scratch) + plan.a_bytes);
     unsigned *tickets = reinterpret_cast<unsigned *>(workspace);
-    hipLaunchKernelGGL(gemm_prep_kernel<BITS>, dim3(ceil_div(plan.Kp / 8, 256), plan.Mp), dim3(256), 0, stream, vec,
+    hipLaunchKernelGGL(gemm_prep_kernel<BITS>, dim3(ceil_div(plan.Kp / 16, 4), plan.Mp / 32), dim3(256), 0, stream, vec,
                        cherry_indices, reinterpret_cast<uint4 *>(a), M, K, C, plan.Kp, plan.steps_normal * 8);
     hipLaunchKernelGGL(gemm_kernel<BITS>, dim3(plan.mtiles * plan.ntiles, plan.splits), dim3(256), 0, stream, qweight,
                        cherry_weight, scales, mul, a, partial, tickets, M, K, N, C, G, accumulate, plan);
