@@ -494,6 +494,22 @@ def test_unpack_kernel_bit_exact(qc, bits, k, n, gs):
     np.testing.assert_array_equal(dense.cpu().numpy(), c_oracle.unpack(p, bits, gs, k))
 
 
+@pytest.mark.parametrize("bits,k,n,frac", [(4, 8192, 28672, 1 / 256), (3, 8200, 16392, 1 / 32)])
+def test_unpack_kernel_bit_exact_large(qc, bits, k, n, frac):
+    """Launches big enough for a workgroup to walk several blocks of rows (the last one ragged),
+    random codes, checked in slices of rows so that the host side stays small."""
+    announce("unpack large", bits, k, n)
+    p = orc.synthetic_packed_fast(k, n, bits, 128, seed=n, cherry_fraction=frac)
+    t = dev(p)
+    dense = qc.unpack_cherryq(bits, t["qweight"], t["cherry_weight"], t["cherry_indices"], t["scales"], k, 128)
+    torch.cuda.synchronize()
+    for n0 in list(range(0, n, 4096)):
+        n1 = min(n0 + 4096, n)
+        part = {"cherry_indices": p["cherry_indices"], "cherry_weight": np.ascontiguousarray(p["cherry_weight"][:, n0:n1]),
+                "qweight": np.ascontiguousarray(p["qweight"][:, n0:n1]), "scales": np.ascontiguousarray(p["scales"][:, n0:n1])}
+        np.testing.assert_array_equal(dense[n0:n1].cpu().numpy(), c_oracle.unpack(part, bits, 128, k))
+
+
 @pytest.mark.parametrize("bits,k,n,gs", [(3, 4096, 1024, 128), (4, 4096, 1024, 128), (4, 11008, 264, 128)])
 def test_dequantize_normal_entry_points(qc, bits, k, n, gs):
     announce("DequantizeNormal", bits, k, n)
