@@ -130,8 +130,23 @@ def time_gpu(bits, k, n, group, steps, warmup, batch=1, use_graph=True):
                 step(warmup + i)
             e1.record(stream)
         stream.synchronize()
-    dev_us = e0.elapsed_time(e1) * 1e3 / steps
-    return dev_us, wall_us, base, x, out, copies
+        dev_us = e0.elapsed_time(e1) * 1e3 / steps
+        # the same launches on ONE copy: the packed layer then comes from the Infinity Cache
+        # (reported beside the HBM figure, labelled; it is never the headline value)
+        resident_us = None
+        if use_graph:
+            rgraph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(rgraph, stream=stream):
+                for i in range(steps):
+                    step(0)
+            rgraph.replay()
+            stream.synchronize()
+            e0.record(stream)
+            rgraph.replay()
+            e1.record(stream)
+            stream.synchronize()
+            resident_us = e0.elapsed_time(e1) * 1e3 / steps
+    return dev_us, wall_us, base, x, out, copies, resident_us
 
 
 def roofline_reference(copies, steps):
@@ -353,7 +368,7 @@ def main():
             torch.cuda.empty_cache()
 
     bits, k, n = WORKLOADS[args.workload]
-    us, wall_us, base, x, out, copies = time_gpu(bits, k, n, args.group, args.steps, args.warmup, batch=args.batch,
+    us, wall_us, base, x, out, copies, resident_us = time_gpu(bits, k, n, args.group, args.steps, args.warmup, batch=args.batch,
                                                 use_graph=not args.no_graph)
     ab = algorithmic_bytes(bits, k, n, args.batch, args.group)
     gbs = ab / us / 1e3
@@ -374,11 +389,13 @@ def main():
                      "traffic": MEASURED_TRAFFIC.get((args.workload, args.batch)),
                      "algorithmic_bytes_per_launch": ab,
                      "kernel": f"cq::matvec_kernel<{bits}>" if args.batch == 1 else
-                               f"cq::matvec_kernel<{bits}, rows {2 if args.batch == 2 else 4}>"
-                               if args.batch == 2 or (args.batch <= 4 and (k - k // 256 // 8 * 8) // 8 * bits * n <= 20 << 20) else
+                               f"cq::matvec_kernel<{bits}, rows {2 if args.batch == 2 else 4}>" if args.batch <= 4 else
                                f"cq::batch_prep_kernel<{bits}> + cq::batch_kernel<{bits}>" if args.batch <= 16 else
-                               f"cq::gemm_prep_kernel<{bits}> + cq::gemm_kernel<{bits}, 2>"},
+                               f"cq::gemm_prep_kernel<{bits}> + cq::gemm_kernel<{bits}>"},
     }
+    if resident_us is not None:
+        result["roofline"]["cache_resident"] = {"us": round(resident_us, 3), "gbs": round(ab / resident_us / 1e3, 1),
+                                                "note": "one weight copy replayed: served by the Infinity Cache, not HBM"}
     if args.batch == 1:
         result["roofline"]["reference"] = roofline_reference(copies, args.steps)
     if not args.no_decode:
