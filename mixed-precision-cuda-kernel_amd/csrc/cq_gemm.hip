@@ -45,11 +45,15 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kGemmTM = 128, kGemmTN = 128, kGemmTK = 64;
+constexpr int kGemmTN = 128, kGemmTK = 64;  // output rows per tile: 64 x GemmPlan::mi
 constexpr int kGemmPitch = kGemmTK * 2 + 16;               // bytes per LDS row
 constexpr int kGemmStageB = kGemmTN * kGemmPitch;          // dequantised weights, one stage
 constexpr int kGemmMaxSplits = 8;
-constexpr int kGemmResidentWgs = 512;  // 256 CUs x 2 workgroups (two waves per SIMD at this register count)
+constexpr int kGemmMaxSplitsSmall = 12;  // 64-row tiles
+constexpr int kGemmResidentWgs = 512;       // 256 CUs x 2 workgroups (two waves per SIMD at this register count)
+constexpr int kGemmResidentWgsSmall4 = 1024;  // 64-row tiles, 4-bit: four per CU
+constexpr int kGemmResidentWgsSmall3 = 768;   // 64-row tiles, 3-bit: three per CU (its decode needs more registers)
+constexpr int kGemmSmallRows = 64;           // up to here a call has one 64-row tile per column tile
 constexpr uint32_t kRsrcFlagsG = 0x00020000u;
 constexpr uint32_t kOobG = 0x80000000u;
 
@@ -66,31 +70,45 @@ __host__ __device__ constexpr int gemm_pos(int kk) {
     return BITS == 4 ? ((kk & 2) ? 4 : 0) : (int)((0x56274310u >> (4 * kk)) & 7u);
 }
 
-GemmPlan gemm_plan(int M, int K, int N, int C) {
+GemmPlan gemm_plan(int bits, int M, int K, int N, int C) {
     GemmPlan p;
-    p.mtiles = ceil_div(M, kGemmTM);
+    // Few rows: 64-row tiles halve the matrix-core work and the fragment loads of a step, and
+    // the smaller register set lets four workgroups share a CU, so K can be split further.
+    p.mi = M <= kGemmSmallRows ? 1 : 2;
+    const int tm = 64 * p.mi;
+    const int resident = p.mi == 2 ? kGemmResidentWgs : kGemmResidentWgsSmall3;
+    p.mtiles = ceil_div(M, tm);
     p.ntiles = ceil_div(N, kGemmTN);
     p.steps_normal = ceil_div(K - C, kGemmTK);
     p.steps_total = p.steps_normal + ceil_div(C, kGemmTK);
     p.Kp = p.steps_total * kGemmTK;
-    p.Mp = p.mtiles * kGemmTM;
+    p.Mp = p.mtiles * tm;
     // K splits: enough workgroups for two per CU, at least 8 steps each
     int splits = 1;
     const int tiles = p.mtiles * p.ntiles;
     // as many splits as still give ONE resident round of workgroups (two per CU; a few workgroups
     // more start a second round and double the time), at least 8 steps each
-    while (splits < kGemmMaxSplits && tiles * (splits + 1) <= kGemmResidentWgs && p.steps_total / (splits + 1) >= 8)
+    while (splits < kGemmMaxSplits && tiles * (splits + 1) <= resident && p.steps_total / (splits + 1) >= 8)
         splits++;
     // steps per split: 2 + 6 k, the trip structure of the kernel's branch-free loop (two steps of
     // lead-in, six per trip); only the last split may be ragged
     p.steps_per_split = ceil_div(p.steps_total, splits);
     if (splits > 1) p.steps_per_split = 2 + 6 * ceil_div(max(p.steps_per_split - 2, 1), 6);
+    if (p.mi == 1 && p.steps_total > 8) {
+        // 64-row tiles: the shortest split length of that form whose workgroups are resident at once
+        // (ends at one split at the latest: more tiles than resident workgroups are not split)
+        int sps = 8;
+        while (sps < p.steps_total &&
+               (ceil_div(p.steps_total, sps) > kGemmMaxSplitsSmall || tiles * ceil_div(p.steps_total, sps) > resident))
+            sps += 6;
+        p.steps_per_split = sps;
+    }
     p.splits = ceil_div(p.steps_total, p.steps_per_split);
     // zero-kept workspace: one ticket per output tile
     p.workspace_bytes = ((size_t)tiles * sizeof(unsigned) + 255) / 256 * 256;
     // scratch: compacted activations, then the partial tiles
     p.a_bytes = ((size_t)p.Mp * p.Kp * sizeof(__half) + 255) / 256 * 256;
-    p.partial_bytes = p.splits > 1 ? (size_t)p.splits * tiles * kGemmTM * kGemmTN * sizeof(float) : 0;
+    p.partial_bytes = p.splits > 1 ? (size_t)p.splits * tiles * tm * kGemmTN * sizeof(float) : 0;
     p.scratch_bytes = p.a_bytes + (p.partial_bytes + 255) / 256 * 256;
     return p;
 }
@@ -174,10 +192,11 @@ __global__ __launch_bounds__(256) void gemm_prep_kernel(const __half *__restrict
 
 // ---- main kernel ---------------------------------------------------------------------------------
 // What a thread holds of one K step between the global loads and their use.
+template <int MI>
 struct GemmStepRegs {
     uint32_t w[4];      // 4 (3) byte rows x 4 columns of packed codes
     uint32_t sc0, sc1;  // the 4 columns' group scales
-    u32x4 a[2][4];      // A fragments: 2 row tiles of 32 x 4 sub-steps of 16 positions
+    u32x4 a[MI][4];     // A fragments: MI row tiles of 32 x 4 sub-steps of 16 positions
 };
 
 // Packed fp16 constants per output dword d (low half: kk = 2 d, high half: kk = 2 d + 1).  With
@@ -201,8 +220,9 @@ struct GemmConst {
     }
 };
 
-template <int BITS>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_kernel(
+template <int BITS, int MI>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
+    MI == 2 ? 2 : 3, MI == 2 ? 2 : 3))) void gemm_kernel(
     const uint8_t *__restrict__ qweight, const __half *__restrict__ cherry_weight,
     const __half *__restrict__ scales, __half *__restrict__ out, const __half *__restrict__ a_frag,
     float *__restrict__ partial, unsigned *__restrict__ tickets, int M, int K, int N, int C, int G,
@@ -213,7 +233,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int ntile = blockIdx.x % plan.ntiles, mtile = blockIdx.x / plan.ntiles, split = blockIdx.y;
-    const int m0 = mtile * kGemmTM, n0 = ntile * kGemmTN;
+    constexpr int kTM = 64 * MI;
+    const int m0 = mtile * kTM, n0 = ntile * kGemmTN;
     const int Kn = K - C;
     // B staging roles: column quad cq, position group kg.  16 consecutive lanes = 4 column quads x 4
     // position groups: their 16-byte LDS writes, 144 bytes apart per row, then fall into 16
@@ -227,18 +248,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         __builtin_amdgcn_make_buffer_rsrc((void *)scales, 0, ceil_div(Kn, G) * N * 2, kRsrcFlagsG);
     const __amdgpu_buffer_rsrc_t rc =
         __builtin_amdgcn_make_buffer_rsrc((void *)cherry_weight, 0, C * N * 2, kRsrcFlagsG);
-    // this wave's A fragments: row tiles (m0 / 32 + 2 wm + i), blocks of 64 lanes x 16 bytes
+    // this wave's A fragments: row tiles (m0 / 32 + MI wm + i), blocks of 64 lanes x 16 bytes
     const u32x4 *afrag = reinterpret_cast<const u32x4 *>(a_frag) +
-                         ((size_t)(m0 / 32 + 2 * wm) * (plan.Kp / 16)) * 64 + lane;
+                         ((size_t)(m0 / 32 + MI * wm) * (plan.Kp / 16)) * 64 + lane;
     const size_t afrag_tile = (size_t)(plan.Kp / 16) * 64;
 
-    auto load_a = [=](u32x4 (&av)[2][4], int st) {
+    auto load_a = [=](u32x4 (&av)[MI][4], int st) {
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < MI; i++)
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) av[i][ks] = afrag[i * afrag_tile + (size_t)(st * 4 + ks) * 64];
     };
-    auto load_step = [=](GemmStepRegs &r, int st) {
+    auto load_step = [=](GemmStepRegs<MI> &r, int st) {
         const uint32_t woff = col_ok ? (uint32_t)((st * 8 + kg) * R * N + n0 + 4 * cq) : kOobG;
 #pragma unroll
         for (int i = 0; i < R; i++) r.w[i] = __builtin_amdgcn_raw_buffer_load_b32(rw, woff + (uint32_t)(i * N), 0, 0);
@@ -250,7 +271,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         load_a(r.a, st);
     };
     // packed codes -> fp16 weights -> LDS stage `buf`
-    auto store_step = [=](const GemmStepRegs &r, int buf) {
+    auto store_step = [=](const GemmStepRegs<MI> &r, int buf) {
         unsigned char *sb = s_b + buf * kGemmStageB;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -289,9 +310,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
     };
 
-    float16_t acc[2][2];
+    float16_t acc[MI][2];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -300,7 +321,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int st_begin = split * plan.steps_per_split;
     const int st_end = min(st_begin + plan.steps_per_split, plan.steps_total);
     const unsigned char *sb0 = s_b + (wn * 64 + (lane & 31)) * kGemmPitch + (lane >> 5) * 16;
-    auto compute = [&](const u32x4 (&av)[2][4], int buf) {
+    auto compute = [&](const u32x4 (&av)[MI][4], int buf) {
         const unsigned char *sb = sb0 + buf * kGemmStageB;
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
@@ -308,7 +329,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
             for (int j = 0; j < 2; j++) bf[j] = *reinterpret_cast<const half8_t *>(sb + j * 32 * kGemmPitch + ks * 32);
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < MI; i++)
 #pragma unroll
                 for (int j = 0; j < 2; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, av[i][ks]), bf[j],
@@ -322,7 +343,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     {
         constexpr int kRing = 3;
         const int n_end = min(st_end, plan.steps_normal);
-        GemmStepRegs regs[kRing];
+        GemmStepRegs<MI> regs[kRing];
 #pragma unroll
         for (int i = 0; i < kRing - 1; i++)
             if (st_begin + i < n_end) load_step(regs[i], st_begin + i);
@@ -361,7 +382,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
     // Cherry steps (one or two per call): plain load, stage, compute.
     for (int st = max(st_begin, plan.steps_normal); st < st_end; st++) {
-        u32x4 av[2][4];
+        u32x4 av[MI][4];
         u32x2 cw[8];  // 8 cherry rows x 4 columns of fp16
         load_a(av, st);
         const int c0 = (st - plan.steps_normal) * kGemmTK + 8 * kg;
@@ -386,11 +407,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (plan.splits > 1) {
         // partial tiles in the accumulators' own order: element q of a lane at [q][lane], so that
         // every store and load instruction covers 256 contiguous bytes
-        const size_t tile_elems = (size_t)kGemmTM * kGemmTN;
+        const size_t tile_elems = (size_t)kTM * kGemmTN;
         const size_t tiles = (size_t)plan.mtiles * plan.ntiles;
-        float *mine = partial + ((size_t)split * tiles + blockIdx.x) * tile_elems + wave * 4096 + lane;
+        float *mine = partial + ((size_t)split * tiles + blockIdx.x) * tile_elems + wave * (2048 * MI) + lane;
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < MI; i++)
 #pragma unroll
             for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -409,27 +430,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if (!*s_last) return;
         if (tid == 0) __hip_atomic_store(&tickets[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < MI; i++)
 #pragma unroll
             for (int j = 0; j < 2; j++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
-        // two splits (128 loads) in flight at a time, added in split order: independent of arrival order
+        // two splits (64 MI loads) in flight at a time, added in split order: independent of arrival order
         for (int s0 = 0; s0 < plan.splits; s0 += 2) {
-            float v[2][64];
+            float v[2][32 * MI];
 #pragma unroll
             for (int ds = 0; ds < 2; ds++) {
                 const int sx = min(s0 + ds, plan.splits - 1);
-                const float *theirs = partial + ((size_t)sx * tiles + blockIdx.x) * tile_elems + wave * 4096 + lane;
+                const float *theirs = partial + ((size_t)sx * tiles + blockIdx.x) * tile_elems + wave * (2048 * MI) + lane;
 #pragma unroll
-                for (int q = 0; q < 64; q++)
+                for (int q = 0; q < 32 * MI; q++)
                     v[ds][q] = __hip_atomic_load(theirs + q * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
 #pragma unroll
             for (int ds = 0; ds < 2; ds++)
                 if (s0 + ds < plan.splits) {
 #pragma unroll
-                    for (int i = 0; i < 2; i++)
+                    for (int i = 0; i < MI; i++)
 #pragma unroll
                         for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -438,13 +459,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
     }
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int n = n0 + wn * 64 + j * 32 + col_l;
 #pragma unroll
             for (int e = 0; e < 16; e++) {
-                const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + row_l + (e & 3);
+                const int m = m0 + wm * (32 * MI) + i * 32 + 8 * (e >> 2) + row_l + (e & 3);
                 if (n < N && m < M) {
                     __half *o = out + (size_t)m * N + n;
                     float v = acc[i][j][e];
@@ -472,14 +493,20 @@ static hipError_t launch_gemm_bits(const __half *vec, const uint8_t *qweight, co
                                    const int16_t *cherry_indices, const __half *scales, __half *mul, int M, int K,
                                    int N, int C, int G, int accumulate, void *workspace, void *scratch,
                                    hipStream_t stream) {
-    const GemmPlan plan = gemm_plan(M, K, N, C);
+    const GemmPlan plan = gemm_plan(BITS, M, K, N, C);
+    if (plan.splits < 1 || plan.splits > 65535 || plan.steps_per_split < 1 || plan.mtiles < 1 || plan.ntiles < 1)
+        return hipErrorInvalidConfiguration;  // never expected: the grid below is built from these
     __half *a = reinterpret_cast<__half *>(scratch);
     float *partial = reinterpret_cast<float *>(reinterpret_cast<char *>(scratch) + plan.a_bytes);
     unsigned *tickets = reinterpret_cast<unsigned *>(workspace);
     hipLaunchKernelGGL(gemm_prep_kernel<BITS>, dim3(ceil_div(plan.Kp / 16, 4), plan.Mp / 32), dim3(256), 0, stream, vec,
                        cherry_indices, reinterpret_cast<uint4 *>(a), M, K, C, plan.Kp, plan.steps_normal * 8);
-    hipLaunchKernelGGL(gemm_kernel<BITS>, dim3(plan.mtiles * plan.ntiles, plan.splits), dim3(256), 0, stream, qweight,
-                       cherry_weight, scales, mul, a, partial, tickets, M, K, N, C, G, accumulate, plan);
+    if (plan.mi == 1)
+        hipLaunchKernelGGL((gemm_kernel<BITS, 1>), dim3(plan.mtiles * plan.ntiles, plan.splits), dim3(256), 0, stream,
+                           qweight, cherry_weight, scales, mul, a, partial, tickets, M, K, N, C, G, accumulate, plan);
+    else
+        hipLaunchKernelGGL((gemm_kernel<BITS, 2>), dim3(plan.mtiles * plan.ntiles, plan.splits), dim3(256), 0, stream,
+                           qweight, cherry_weight, scales, mul, a, partial, tickets, M, K, N, C, G, accumulate, plan);
     return hipGetLastError();
 }
 

@@ -77,7 +77,8 @@ size_t scratch_bytes(int B, int K, int N, int C);
 
 // cq_gemm.hip: more than 16 rows (prompt processing) -- dequantise into LDS, fp16 MFMA tiles.
 struct GemmPlan {
-    int mtiles, ntiles;               // 128 x 128 output tiles
+    int mi;                           // 32-row tiles per wavefront: 2 (128-row output tiles) or 1 (64-row)
+    int mtiles, ntiles;               // (64 mi) x 128 output tiles
     int steps_normal, steps_total;    // K steps of 64 positions: packed part, then the cherry rows
     int Kp, Mp;                       // padded sizes of the compacted activation copy
     int splits, steps_per_split;      // K splits (grid.y)
@@ -86,7 +87,7 @@ struct GemmPlan {
     size_t scratch_bytes;
 };
 constexpr int kGemmMinRows = 17;  // fewer rows go through the 16-row kernel
-GemmPlan gemm_plan(int M, int K, int N, int C);
+GemmPlan gemm_plan(int bits, int M, int K, int N, int C);  // the split count depends on the code width
 bool gemm_supported(int bits, int M, int K, int N, int C, int G);
 hipError_t launch_gemm(int bits, const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
                        const int16_t *cherry_indices, const __half *scales, __half *mul, int M, int K, int N, int C,

@@ -72,6 +72,20 @@ def _call(fn, *, vec=0x1000, qw=0x1000, cw=0x1000, idx=0x1000, sc=0x1000, mul=0x
     return fn(vec, qw, cw, idx, sc, mul, b, k, n, c, g, acc, ws, wsb, scr, scrb, stream)
 
 
+def test_scratch_sizes_stay_bounded_for_every_row_count_and_width(lib):
+    """The prompt-sized path plans its K splits on the host; whatever the shape, the scratch it
+    asks for lies between the compacted activations alone and that plus a dozen partial outputs
+    (a plan that ran away would show up here as a nonsensical size)."""
+    for rows in (17, 40, 64, 65, 128, 256, 1000):
+        for k in (256, 4096, 8192, 11008):
+            for n in (8, 4096, 28672, 98312, 128256):
+                c = -(-k // 256) // 8 * 8
+                got = lib.cherryq_scratch_bytes(rows, k, n, c)
+                assert got >= rows * (k - c) * 2, (rows, k, n, got)
+                assert got <= (rows + 128) * (k + 192) * 2 + 13 * (rows + 128) * (n + 128) * 4 + 4096, (rows, k, n, got)
+                assert lib.cherryq_workspace_bytes(rows, k, n, c) <= 64 * (n + 256) * 8 + (rows + 128) * (n + 128) // 64, (rows, k, n)
+
+
 def test_argument_validation_rejects_before_launch(lib):
     f4, f3, f3f = lib.cherryq_vecquant4matmul_f16, lib.cherryq_vecquant3matmul_f16, lib.cherryq_vecquant3matmul_f32
     assert _call(f4, g=64) == -3          # reference: AT_ERROR for group_size < 128

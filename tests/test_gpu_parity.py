@@ -650,6 +650,10 @@ def column_sample(p, rng, count):
     (4, 128, 28672, 512, 20),      # 112 cherry rows: two cherry steps
     (4, 128, 2048, 4096, 1100),    # nine row tiles, no K split
     (3, 128, 4096, 11008, 200),    # 7B gate/up, two row tiles
+    (4, 128, 4096, 11008, 64),     # 64-row tiles: the whole call is one row tile
+    (3, 128, 4096, 4096, 33),      # 64-row tiles, 3-bit
+    (4, 128, 512, 98312, 40),      # 64-row tiles, more column tiles than resident workgroups: no K split
+    (4, 128, 11008, 4096, 65),     # first row count on 128-row tiles again
 ])
 def test_gemm_rows_against_oracle(qc, bits, gs, k, n, rows):
     """More than 16 rows: the tiled dequantise + MFMA kernel against the C oracle (a column sample
