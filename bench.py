@@ -263,6 +263,33 @@ def decode_benchmark(prompt_len=128, new_tokens=128, w_bits=4, seed=0):
     return res
 
 
+def unpack_table(group):
+    """Dense dequantisation (QuantLinear.unpack on the GPU) of whole layers: device time per call
+    and the bytes it moves (packed buffers read once, dense fp16 weight written once)."""
+    import torch
+    import quant_cuda
+    for bits in (4, 3):
+        for k, n in ((4096, 11008), (11008, 4096), (4096, 4096), (8192, 28672)):
+            _, (t, _) = make_copies(bits, k, n, group, 0, seed=k + bits)
+            fn = lambda: quant_cuda.unpack_cherryq(bits, t["qweight"], t["cherry_weight"], t["cherry_indices"],
+                                                   t["scales"], k, group)
+            for _ in range(3):
+                fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(20):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) / 20 * 1e3
+            ab = sum(v.numel() * v.element_size() for v in t.values()) + 2.0 * k * n
+            print(f"unpack {bits}-bit {k:5d}->{n:5d}: {us:7.2f} us  {ab / us / 1e3:7.1f} GB/s "
+                  f"({ab / us / 1e3 / HBM_PEAK_GBS * 100:4.1f}% of 8 TB/s; packed read + dense fp16 write)",
+                  file=sys.stderr, flush=True)
+            del t
+            torch.cuda.empty_cache()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -272,6 +299,8 @@ def main():
     ap.add_argument("--group", type=int, default=128)
     ap.add_argument("--batch", type=int, default=1, help="activation rows per call (2..4: streaming kernel with several rows or, like 5..16, the small-batch matrix-core kernel; more: tiled GEMM kernel)")
     ap.add_argument("--all", action="store_true", help="also print a table of every workload to stderr")
+    ap.add_argument("--unpack-only", action="store_true",
+                    help="print the dense-dequantisation table to stderr and exit (for profiling that kernel)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the 7B-shape decode measurement")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a graph replay")
@@ -298,6 +327,9 @@ def main():
         del src, dst
         torch.cuda.empty_cache()
 
+    if args.unpack_only:
+        unpack_table(args.group)
+        return
     if args.all:
         # the small-batch path (matrix cores) on the 13B and 70B layer shapes
         for name, b in (("llama7b_gate_up_w4", 2), ("llama7b_attn_w4", 2), ("llama7b_attn_w4", 4),
@@ -358,6 +390,7 @@ def main():
                       f"torch operations {us_torch:8.1f} us", file=sys.stderr, flush=True)
                 del lin, dst, wsrc
                 torch.cuda.empty_cache()
+        unpack_table(args.group)
         for name, (bits, k, n) in WORKLOADS.items():
             us, wall_us, *_ = time_gpu(bits, k, n, args.group, max(200, args.steps // 4), args.warmup,
                                       use_graph=not args.no_graph)
