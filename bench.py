@@ -424,7 +424,7 @@ def main():
                      "kernel": f"cq::matvec_kernel<{bits}>" if args.batch == 1 else
                                f"cq::matvec_kernel<{bits}, rows {2 if args.batch == 2 else 4}>" if args.batch <= 4 else
                                f"cq::batch_prep_kernel<{bits}> + cq::batch_kernel<{bits}>" if args.batch <= 16 else
-                               f"cq::gemm_prep_kernel<{bits}> + cq::gemm_kernel<{bits}, {1 if args.batch <= 64 else 2}>"},
+                               f"cq::gemm_prep_kernel<{bits}> + cq::gemm_kernel<{bits}, {32 if args.batch <= 32 else 64 if args.batch <= 64 else 128}>"},
     }
     if resident_us is not None:
         result["roofline"]["cache_resident"] = {"us": round(resident_us, 3), "gbs": round(ab / resident_us / 1e3, 1),

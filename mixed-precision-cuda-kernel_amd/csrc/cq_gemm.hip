@@ -45,15 +45,15 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kGemmTN = 128, kGemmTK = 64;  // output rows per tile: 64 x GemmPlan::mi
+constexpr int kGemmTN = 128, kGemmTK = 64;  // output rows per tile: GemmPlan::tm
 constexpr int kGemmPitch = kGemmTK * 2 + 16;               // bytes per LDS row
 constexpr int kGemmStageB = kGemmTN * kGemmPitch;          // dequantised weights, one stage
 constexpr int kGemmMaxSplits = 8;
 constexpr int kGemmMaxSplitsSmall = 12;  // 64-row tiles
 constexpr int kGemmResidentWgs = 512;       // 256 CUs x 2 workgroups (two waves per SIMD at this register count)
-constexpr int kGemmResidentWgsSmall4 = 1024;  // 64-row tiles, 4-bit: four per CU
-constexpr int kGemmResidentWgsSmall3 = 768;   // 64-row tiles, 3-bit: three per CU (its decode needs more registers)
-constexpr int kGemmSmallRows = 64;           // up to here a call has one 64-row tile per column tile
+constexpr int kGemmResidentWgs64 = 768;      // 64-row tiles: three workgroups per CU
+constexpr int kGemmResidentWgs32 = 1024;     // 32-row tiles: four per CU
+constexpr int kGemmSmallRows = 64;           // up to here a call has one 64-row (or 32-row) tile per column tile
 constexpr uint32_t kRsrcFlagsG = 0x00020000u;
 constexpr uint32_t kOobG = 0x80000000u;
 
@@ -74,9 +74,10 @@ GemmPlan gemm_plan(int bits, int M, int K, int N, int C) {
     GemmPlan p;
     // Few rows: 64-row tiles halve the matrix-core work and the fragment loads of a step, and
     // the smaller register set lets four workgroups share a CU, so K can be split further.
-    p.mi = M <= kGemmSmallRows ? 1 : 2;
-    const int tm = 64 * p.mi;
-    const int resident = p.mi == 2 ? kGemmResidentWgs : kGemmResidentWgsSmall3;
+    (void)bits;
+    p.tm = M <= 32 ? 32 : M <= kGemmSmallRows ? 64 : 128;
+    const int tm = p.tm;
+    const int resident = tm == 128 ? kGemmResidentWgs : tm == 64 ? kGemmResidentWgs64 : kGemmResidentWgs32;
     p.mtiles = ceil_div(M, tm);
     p.ntiles = ceil_div(N, kGemmTN);
     p.steps_normal = ceil_div(K - C, kGemmTK);
@@ -94,8 +95,8 @@ GemmPlan gemm_plan(int bits, int M, int K, int N, int C) {
     // lead-in, six per trip); only the last split may be ragged
     p.steps_per_split = ceil_div(p.steps_total, splits);
     if (splits > 1) p.steps_per_split = 2 + 6 * ceil_div(max(p.steps_per_split - 2, 1), 6);
-    if (p.mi == 1 && p.steps_total > 8) {
-        // 64-row tiles: the shortest split length of that form whose workgroups are resident at once
+    if (tm < 128 && p.steps_total > 8) {
+        // small tiles: the shortest split length of that form whose workgroups are resident at once
         // (ends at one split at the latest: more tiles than resident workgroups are not split)
         int sps = 8;
         while (sps < p.steps_total &&
@@ -220,9 +221,9 @@ struct GemmConst {
     }
 };
 
-template <int BITS, int MI>
+template <int BITS, int TM>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
-    MI == 2 ? 2 : 3, MI == 2 ? 2 : 3))) void gemm_kernel(
+    TM == 128 ? 2 : TM == 64 ? 3 : 4, TM == 128 ? 2 : TM == 64 ? 3 : 4))) void gemm_kernel(
     const uint8_t *__restrict__ qweight, const __half *__restrict__ cherry_weight,
     const __half *__restrict__ scales, __half *__restrict__ out, const __half *__restrict__ a_frag,
     float *__restrict__ partial, unsigned *__restrict__ tickets, int M, int K, int N, int C, int G,
@@ -230,16 +231,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
     __shared__ __attribute__((aligned(16))) unsigned char s_b[2 * kGemmStageB];  // [2][128 columns][pitch]
 
     constexpr int R = BITS == 4 ? 4 : 3;  // byte rows per 8 positions
+    // A wavefront owns MI x NJ tiles of 32 x 32: the four wavefronts sit 2 x 2 on a 128- or 64-row
+    // tile and side by side on a 32-row one.
+    constexpr int MI = TM == 128 ? 2 : 1, NJ = TM == 32 ? 1 : 2;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = TM == 32 ? 0 : wave >> 1, wn = TM == 32 ? wave : wave & 1;
+    const int sm = wave >> 1, sn = wave & 1;  // the wavefront's share of the B staging work
     const int ntile = blockIdx.x % plan.ntiles, mtile = blockIdx.x / plan.ntiles, split = blockIdx.y;
-    constexpr int kTM = 64 * MI;
+    constexpr int kTM = TM;
     const int m0 = mtile * kTM, n0 = ntile * kGemmTN;
     const int Kn = K - C;
     // B staging roles: column quad cq, position group kg.  16 consecutive lanes = 4 column quads x 4
     // position groups: their 16-byte LDS writes, 144 bytes apart per row, then fall into 16
     // different bank groups.
-    const int cq = wn * 16 + (lane >> 4) * 4 + (lane & 3), kg = wm * 4 + ((lane >> 2) & 3);
+    const int cq = sn * 16 + (lane >> 4) * 4 + (lane & 3), kg = sm * 4 + ((lane >> 2) & 3);
     const bool col_ok = n0 + 4 * cq < N;
 
     const __amdgpu_buffer_rsrc_t rw =
@@ -310,28 +315,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
         }
     };
 
-    float16_t acc[MI][2];
+    float16_t acc[MI][NJ];
 #pragma unroll
     for (int i = 0; i < MI; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < NJ; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
     const int st_begin = split * plan.steps_per_split;
     const int st_end = min(st_begin + plan.steps_per_split, plan.steps_total);
-    const unsigned char *sb0 = s_b + (wn * 64 + (lane & 31)) * kGemmPitch + (lane >> 5) * 16;
+    const unsigned char *sb0 = s_b + (wn * (32 * NJ) + (lane & 31)) * kGemmPitch + (lane >> 5) * 16;
     auto compute = [&](const u32x4 (&av)[MI][4], int buf) {
         const unsigned char *sb = sb0 + buf * kGemmStageB;
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
-            half8_t bf[2];
+            half8_t bf[NJ];
 #pragma unroll
-            for (int j = 0; j < 2; j++) bf[j] = *reinterpret_cast<const half8_t *>(sb + j * 32 * kGemmPitch + ks * 32);
+            for (int j = 0; j < NJ; j++) bf[j] = *reinterpret_cast<const half8_t *>(sb + j * 32 * kGemmPitch + ks * 32);
 #pragma unroll
             for (int i = 0; i < MI; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++)
+                for (int j = 0; j < NJ; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, av[i][ks]), bf[j],
                                                                       acc[i][j], 0, 0, 0);
         }
@@ -409,14 +414,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
         // every store and load instruction covers 256 contiguous bytes
         const size_t tile_elems = (size_t)kTM * kGemmTN;
         const size_t tiles = (size_t)plan.mtiles * plan.ntiles;
-        float *mine = partial + ((size_t)split * tiles + blockIdx.x) * tile_elems + wave * (2048 * MI) + lane;
+        constexpr int kQ = MI * NJ * 16;  // accumulator words per lane
+        float *mine = partial + ((size_t)split * tiles + blockIdx.x) * tile_elems + wave * (kQ * 64) + lane;
 #pragma unroll
         for (int i = 0; i < MI; i++)
 #pragma unroll
-            for (int j = 0; j < 2; j++)
+            for (int j = 0; j < NJ; j++)
 #pragma unroll
                 for (int e = 0; e < 16; e++)
-                    __hip_atomic_store(mine + ((i * 2 + j) * 16 + e) * 64, acc[i][j][e], __ATOMIC_RELAXED,
+                    __hip_atomic_store(mine + ((i * NJ + j) * 16 + e) * 64, acc[i][j][e], __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
         int *s_last = reinterpret_cast<int *>(s_b);  // the stages have been consumed
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
@@ -432,18 +438,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
 #pragma unroll
         for (int i = 0; i < MI; i++)
 #pragma unroll
-            for (int j = 0; j < 2; j++)
+            for (int j = 0; j < NJ; j++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
-        // two splits (64 MI loads) in flight at a time, added in split order: independent of arrival order
+        // two splits (2 kQ loads) in flight at a time, added in split order: independent of arrival order
         for (int s0 = 0; s0 < plan.splits; s0 += 2) {
-            float v[2][32 * MI];
+            float v[2][kQ];
 #pragma unroll
             for (int ds = 0; ds < 2; ds++) {
                 const int sx = min(s0 + ds, plan.splits - 1);
-                const float *theirs = partial + ((size_t)sx * tiles + blockIdx.x) * tile_elems + wave * (2048 * MI) + lane;
+                const float *theirs = partial + ((size_t)sx * tiles + blockIdx.x) * tile_elems + wave * (kQ * 64) + lane;
 #pragma unroll
-                for (int q = 0; q < 32 * MI; q++)
+                for (int q = 0; q < kQ; q++)
                     v[ds][q] = __hip_atomic_load(theirs + q * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
 #pragma unroll
@@ -452,17 +458,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
 #pragma unroll
                     for (int i = 0; i < MI; i++)
 #pragma unroll
-                        for (int j = 0; j < 2; j++)
+                        for (int j = 0; j < NJ; j++)
 #pragma unroll
-                            for (int e = 0; e < 16; e++) acc[i][j][e] += v[ds][(i * 2 + j) * 16 + e];
+                            for (int e = 0; e < 16; e++) acc[i][j][e] += v[ds][(i * NJ + j) * 16 + e];
                 }
         }
     }
 #pragma unroll
     for (int i = 0; i < MI; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int n = n0 + wn * 64 + j * 32 + col_l;
+        for (int j = 0; j < NJ; j++) {
+            const int n = n0 + wn * (32 * NJ) + j * 32 + col_l;
 #pragma unroll
             for (int e = 0; e < 16; e++) {
                 const int m = m0 + wm * (32 * MI) + i * 32 + 8 * (e >> 2) + row_l + (e & 3);
@@ -501,12 +507,16 @@ static hipError_t launch_gemm_bits(const __half *vec, const uint8_t *qweight, co
     unsigned *tickets = reinterpret_cast<unsigned *>(workspace);
     hipLaunchKernelGGL(gemm_prep_kernel<BITS>, dim3(ceil_div(plan.Kp / 16, 4), plan.Mp / 32), dim3(256), 0, stream, vec,
                        cherry_indices, reinterpret_cast<uint4 *>(a), M, K, C, plan.Kp, plan.steps_normal * 8);
-    if (plan.mi == 1)
-        hipLaunchKernelGGL((gemm_kernel<BITS, 1>), dim3(plan.mtiles * plan.ntiles, plan.splits), dim3(256), 0, stream,
-                           qweight, cherry_weight, scales, mul, a, partial, tickets, M, K, N, C, G, accumulate, plan);
+    const dim3 grid(plan.mtiles * plan.ntiles, plan.splits);
+    if (plan.tm == 32)
+        hipLaunchKernelGGL((gemm_kernel<BITS, 32>), grid, dim3(256), 0, stream, qweight, cherry_weight, scales, mul, a,
+                           partial, tickets, M, K, N, C, G, accumulate, plan);
+    else if (plan.tm == 64)
+        hipLaunchKernelGGL((gemm_kernel<BITS, 64>), grid, dim3(256), 0, stream, qweight, cherry_weight, scales, mul, a,
+                           partial, tickets, M, K, N, C, G, accumulate, plan);
     else
-        hipLaunchKernelGGL((gemm_kernel<BITS, 2>), dim3(plan.mtiles * plan.ntiles, plan.splits), dim3(256), 0, stream,
-                           qweight, cherry_weight, scales, mul, a, partial, tickets, M, K, N, C, G, accumulate, plan);
+        hipLaunchKernelGGL((gemm_kernel<BITS, 128>), grid, dim3(256), 0, stream, qweight, cherry_weight, scales, mul, a,
+                           partial, tickets, M, K, N, C, G, accumulate, plan);
     return hipGetLastError();
 }
 

@@ -77,8 +77,8 @@ size_t scratch_bytes(int B, int K, int N, int C);
 
 // cq_gemm.hip: more than 16 rows (prompt processing) -- dequantise into LDS, fp16 MFMA tiles.
 struct GemmPlan {
-    int mi;                           // 32-row tiles per wavefront: 2 (128-row output tiles) or 1 (64-row)
-    int mtiles, ntiles;               // (64 mi) x 128 output tiles
+    int tm;                           // rows of an output tile: 128, 64 (calls of up to 64 rows) or 32 (up to 32)
+    int mtiles, ntiles;               // tm x 128 output tiles
     int steps_normal, steps_total;    // K steps of 64 positions: packed part, then the cherry rows
     int Kp, Mp;                       // padded sizes of the compacted activation copy
     int splits, steps_per_split;      // K splits (grid.y)

@@ -24,10 +24,10 @@ int main() {
                         if (K - C <= 0) continue;
                         const cq::GemmPlan p = cq::gemm_plan(bits, M, K, N, C);
                         count++;
-                        const int tm = 64 * p.mi;
+                        const int tm = p.tm;
                         const long wgs = (long)p.mtiles * p.ntiles * p.splits;
                         const bool ok =
-                            (p.mi == 1 || p.mi == 2) && p.splits >= 1 && p.splits <= 16 && p.steps_per_split >= 1 &&
+                            (tm == 32 || tm == 64 || tm == 128) && p.splits >= 1 && p.splits <= 16 && p.steps_per_split >= 1 &&
                             (long)p.splits * p.steps_per_split >= p.steps_total &&
                             (long)(p.splits - 1) * p.steps_per_split < p.steps_total &&
                             (p.splits == 1 || (p.steps_per_split - 2) % 6 == 0) && p.mtiles * tm >= M &&
@@ -39,8 +39,8 @@ int main() {
                             (p.splits == 1 || wgs <= 1024);
                         if (!ok) {
                             bad++;
-                            std::printf("bad plan: bits %d M %d K %d N %d C %d -> mi %d tiles %d x %d steps %d splits %d x %d\n",
-                                        bits, M, K, N, C, p.mi, p.mtiles, p.ntiles, p.steps_total, p.splits,
+                            std::printf("bad plan: bits %d M %d K %d N %d C %d -> tile rows %d tiles %d x %d steps %d splits %d x %d\n",
+                                        bits, M, K, N, C, p.tm, p.mtiles, p.ntiles, p.steps_total, p.splits,
                                         p.steps_per_split);
                         }
                     }

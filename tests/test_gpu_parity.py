@@ -651,6 +651,8 @@ def column_sample(p, rng, count):
     (4, 128, 2048, 4096, 1100),    # nine row tiles, no K split
     (3, 128, 4096, 11008, 200),    # 7B gate/up, two row tiles
     (4, 128, 4096, 11008, 64),     # 64-row tiles: the whole call is one row tile
+    (4, 128, 4096, 11008, 32),     # 32-row tiles: four wavefronts side by side, nine K splits
+    (3, 64, 2048, 264, 24),        # 32-row tiles, 3-bit, 64-wide groups, ragged N
     (3, 128, 4096, 4096, 33),      # 64-row tiles, 3-bit
     (4, 128, 512, 98312, 40),      # 64-row tiles, more column tiles than resident workgroups: no K split
     (4, 128, 11008, 4096, 65),     # first row count on 128-row tiles again
