@@ -27,6 +27,11 @@
 // kernel was bound by LDS bandwidth (about 64 bytes per clock and CU for 16-byte accesses);
 // keeping A out of it halves that traffic.
 //
+// Calls of few rows use smaller output tiles (template parameter TM): 64 rows (one 32-row tile per
+// wavefront, three workgroups per CU) up to 64 rows, 32 rows (the four wavefronts side by side,
+// four workgroups per CU) up to 32 -- less matrix-core work on padding rows, and the smaller
+// register sets leave room for more K splits.
+//
 // K splits (when the tiles alone would leave CUs idle) meet in per-split fp32 partial tiles and
 // one ticket per output tile; the last workgroup adds the partials in split order, so the result
 // does not depend on arrival order.
