@@ -35,10 +35,8 @@ size_t workspace_bytes(int B, int K, int N, int C) {
         if (b2 > bytes) bytes = b2;
     }
     if (B >= kGemmMinRows) {
-        for (int bits = 3; bits <= 4; bits++) {  // the query does not know the code width
-            size_t b3 = gemm_plan(bits, B, K, N, C).workspace_bytes;
-            if (b3 > bytes) bytes = b3;
-        }
+        size_t b3 = gemm_plan(B, K, N, C).workspace_bytes;
+        if (b3 > bytes) bytes = b3;
     }
     return bytes;
 }
@@ -49,10 +47,8 @@ size_t scratch_bytes(int B, int K, int N, int C) {
     size_t bytes = B >= 2 ? batch_workspace(K, N, C).scratch_total : 0;
     if (B >= 2 && f32_scratch_bytes(K, C) > bytes) bytes = f32_scratch_bytes(K, C);  // fp32-tensor variant
     if (B >= kGemmMinRows) {
-        for (int bits = 3; bits <= 4; bits++) {
-            size_t b3 = gemm_plan(bits, B, K, N, C).scratch_bytes;
-            if (b3 > bytes) bytes = b3;
-        }
+        size_t b3 = gemm_plan(B, K, N, C).scratch_bytes;
+        if (b3 > bytes) bytes = b3;
     }
     return bytes;
 }

@@ -75,11 +75,10 @@ __host__ __device__ constexpr int gemm_pos(int kk) {
     return BITS == 4 ? ((kk & 2) ? 4 : 0) : (int)((0x56274310u >> (4 * kk)) & 7u);
 }
 
-GemmPlan gemm_plan(int bits, int M, int K, int N, int C) {
+GemmPlan gemm_plan(int M, int K, int N, int C) {
     GemmPlan p;
     // Few rows: 64-row tiles halve the matrix-core work and the fragment loads of a step, and
     // the smaller register set lets four workgroups share a CU, so K can be split further.
-    (void)bits;
     p.tm = M <= 32 ? 32 : M <= kGemmSmallRows ? 64 : 128;
     const int tm = p.tm;
     const int resident = tm == 128 ? kGemmResidentWgs : tm == 64 ? kGemmResidentWgs64 : kGemmResidentWgs32;
@@ -488,7 +487,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
 }
 
 bool gemm_supported(int bits, int M, int K, int N, int C, int G) {
-    (void)bits;
     if (M < 2) return false;
     if (G % kGemmTK) return false;  // a step must not straddle a group
     if (K - C <= 0) return false;
@@ -504,7 +502,7 @@ static hipError_t launch_gemm_bits(const __half *vec, const uint8_t *qweight, co
                                    const int16_t *cherry_indices, const __half *scales, __half *mul, int M, int K,
                                    int N, int C, int G, int accumulate, void *workspace, void *scratch,
                                    hipStream_t stream) {
-    const GemmPlan plan = gemm_plan(BITS, M, K, N, C);
+    const GemmPlan plan = gemm_plan(M, K, N, C);
     if (plan.splits < 1 || plan.splits > 65535 || plan.steps_per_split < 1 || plan.mtiles < 1 || plan.ntiles < 1)
         return hipErrorInvalidConfiguration;  // never expected: the grid below is built from these
     __half *a = reinterpret_cast<__half *>(scratch);

@@ -87,7 +87,7 @@ struct GemmPlan {
     size_t scratch_bytes;
 };
 constexpr int kGemmMinRows = 17;  // fewer rows go through the 16-row kernel
-GemmPlan gemm_plan(int bits, int M, int K, int N, int C);  // the split count depends on the code width
+GemmPlan gemm_plan(int M, int K, int N, int C);
 bool gemm_supported(int bits, int M, int K, int N, int C, int G);
 hipError_t launch_gemm(int bits, const __half *vec, const uint8_t *qweight, const __half *cherry_weight,
                        const int16_t *cherry_indices, const __half *scales, __half *mul, int M, int K, int N, int C,

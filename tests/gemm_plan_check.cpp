@@ -18,32 +18,31 @@ int main() {
     for (int M : Ms)
         for (int K : Ks)
             for (int N : Ns)
-                for (int bits = 3; bits <= 4; bits++)
-                    for (int cf = 0; cf < 3; cf++) {
-                        const int C = cf == 0 ? 0 : cf == 1 ? (K + 255) / 256 / 8 * 8 : K / 8 / 8 * 8;
-                        if (K - C <= 0) continue;
-                        const cq::GemmPlan p = cq::gemm_plan(bits, M, K, N, C);
-                        count++;
-                        const int tm = p.tm;
-                        const long wgs = (long)p.mtiles * p.ntiles * p.splits;
-                        const bool ok =
-                            (tm == 32 || tm == 64 || tm == 128) && p.splits >= 1 && p.splits <= 16 && p.steps_per_split >= 1 &&
-                            (long)p.splits * p.steps_per_split >= p.steps_total &&
-                            (long)(p.splits - 1) * p.steps_per_split < p.steps_total &&
-                            (p.splits == 1 || (p.steps_per_split - 2) % 6 == 0) && p.mtiles * tm >= M &&
-                            (p.mtiles - 1) * tm < M && p.Mp == p.mtiles * tm && p.Kp == p.steps_total * 64 &&
-                            p.steps_total * 64 >= K && p.ntiles * 128 >= N && (p.ntiles - 1) * 128 < N &&
-                            p.partial_bytes ==
-                                (p.splits > 1 ? (size_t)p.splits * p.mtiles * p.ntiles * tm * 128 * sizeof(float) : 0) &&
-                            p.a_bytes >= (size_t)p.Mp * p.Kp * 2 && p.scratch_bytes >= p.a_bytes + p.partial_bytes &&
-                            (p.splits == 1 || wgs <= 1024);
-                        if (!ok) {
-                            bad++;
-                            std::printf("bad plan: bits %d M %d K %d N %d C %d -> tile rows %d tiles %d x %d steps %d splits %d x %d\n",
-                                        bits, M, K, N, C, p.tm, p.mtiles, p.ntiles, p.steps_total, p.splits,
-                                        p.steps_per_split);
-                        }
+                for (int cf = 0; cf < 3; cf++) {
+                    const int C = cf == 0 ? 0 : cf == 1 ? (K + 255) / 256 / 8 * 8 : K / 8 / 8 * 8;
+                    if (K - C <= 0) continue;
+                    const cq::GemmPlan p = cq::gemm_plan(M, K, N, C);
+                    count++;
+                    const int tm = p.tm;
+                    const long wgs = (long)p.mtiles * p.ntiles * p.splits;
+                    const bool ok =
+                        (tm == 32 || tm == 64 || tm == 128) && p.splits >= 1 && p.splits <= 16 && p.steps_per_split >= 1 &&
+                        (long)p.splits * p.steps_per_split >= p.steps_total &&
+                        (long)(p.splits - 1) * p.steps_per_split < p.steps_total &&
+                        (p.splits == 1 || (p.steps_per_split - 2) % 6 == 0) && p.mtiles * tm >= M &&
+                        (p.mtiles - 1) * tm < M && p.Mp == p.mtiles * tm && p.Kp == p.steps_total * 64 &&
+                        p.steps_total * 64 >= K && p.ntiles * 128 >= N && (p.ntiles - 1) * 128 < N &&
+                        p.partial_bytes ==
+                            (p.splits > 1 ? (size_t)p.splits * p.mtiles * p.ntiles * tm * 128 * sizeof(float) : 0) &&
+                        p.a_bytes >= (size_t)p.Mp * p.Kp * 2 && p.scratch_bytes >= p.a_bytes + p.partial_bytes &&
+                        (p.splits == 1 || wgs <= 1024);
+                    if (!ok) {
+                        bad++;
+                        std::printf("bad plan: M %d K %d N %d C %d -> tile rows %d tiles %d x %d steps %d splits %d x %d\n",
+                                    M, K, N, C, p.tm, p.mtiles, p.ntiles, p.steps_total, p.splits,
+                                    p.steps_per_split);
                     }
+                }
     std::printf("%ld plans checked, %ld bad\n", count, bad);
     return bad ? 1 : 0;
 }
