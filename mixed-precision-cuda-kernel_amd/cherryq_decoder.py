@@ -98,7 +98,7 @@ def _ok(rc, what):
 
 
 def _stream():
-    return torch.cuda.current_stream().cuda_stream
+    return quant_cuda._current_stream(torch.cuda.current_device())
 
 
 @dataclass

@@ -242,7 +242,7 @@ def _dequantize_normal(fn, what, w_bits, qweight, scaling_factors, out, height, 
         raise RuntimeError(f"out shape {tuple(out.shape)} cannot hold ({kn}, {n})")
     with torch.cuda.device(dev):
         rc = fn(_ptr(qweight), _ptr(scaling_factors), _ptr(out), height, n, cherry_size, group_size,
-                torch.cuda.current_stream(dev).cuda_stream)
+                _current_stream(dev.index))
     if rc != 0:
         _fail(rc, what)
 
@@ -281,7 +281,7 @@ def unpack_cherryq(w_bits, qweight, cherry_weight, cherry_indices, scaling_facto
     with torch.cuda.device(dev):
         rc = _lib.cherryq_unpack_f16(w_bits, _ptr(qweight), _ptr(cherry_weight), _ptr(cherry_indices),
                                      _ptr(scaling_factors), dense.data_ptr(), int(in_features), n, c,
-                                     int(group_size), torch.cuda.current_stream(dev).cuda_stream)
+                                     int(group_size), _current_stream(dev.index))
     if rc != 0:
         _fail(rc, "unpack_cherryq")
     return dense
@@ -311,7 +311,7 @@ def pack_cherryq(w_bits, weight, cherry_indices, group_size):
     cherry_weight = torch.empty((c, n), dtype=torch.float16, device=dev)
     with torch.cuda.device(dev):
         rc = _lib.cherryq_pack_f16(w_bits, weight.data_ptr(), _ptr(idx), _ptr(qweight), _ptr(scales),
-                                   _ptr(cherry_weight), k, n, c, group_size, torch.cuda.current_stream(dev).cuda_stream)
+                                   _ptr(cherry_weight), k, n, c, group_size, _current_stream(dev.index))
     if rc != 0:
         _fail(rc, "pack_cherryq")
     return idx, cherry_weight, qweight, scales
@@ -359,7 +359,7 @@ def fake_quant_cherryq(w_bits, weight, cherry_indices, group_size, ste=False, ou
     fn = _lib.cherryq_fake_quant_f16 if weight.dtype == torch.float16 else _lib.cherryq_fake_quant_f32
     with torch.cuda.device(dev):
         rc = fn(int(w_bits), weight.data_ptr(), _ptr(idx), out.data_ptr(), k, n, idx.numel(), g, int(bool(ste)),
-                torch.cuda.current_stream(dev).cuda_stream)
+                _current_stream(dev.index))
     if rc != 0:
         _fail(rc, "fake_quant_cherryq")
     return out
