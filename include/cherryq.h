@@ -189,6 +189,36 @@ int cherryq_fake_quant_f32(int w_bits, const void *weight, const int32_t *cherry
                            void *stream);
 
 /*
+ * Load-time repack of a packed layer into a weight stream laid out for this GPU, and the batch-1
+ * matvec over it.  The reference has no counterpart: its kernels read the checkpoint layout
+ * directly (csrc/quant_cuda_kernel.cu:811-831 4-bit, :649-667 3-bit) and so does every entry point
+ * above.  The stream holds the same information -- every code, scale, cherry row and cherry index,
+ * bit for bit; cherryq_unprepack_f16 is the exact inverse -- rearranged so that 16 output columns'
+ * whole input range is one contiguous record of 1 KB (768 B for 3 bits) pieces that a wavefront
+ * loads with one instruction and masks straight into matrix-core operands.  A workgroup then owns
+ * whole output columns: no partial sums leave it, so the call needs no workspace, uses no atomics
+ * and rounds once from fp32, like the entry points above.  Arithmetic contract and result are
+ * those of cherryq_vecquant{3,4}matmul_f16 at batch 1 (mul = or += vec W^T).
+ *
+ * stream: cherryq_prepack_bytes() bytes, 256-byte aligned, written by cherryq_prepack_f16 once
+ * per layer.  group_size must be a multiple of 128 (the stream stores one scale row per 128
+ * positions); cherryq_prepack_supported() says whether a shape is taken at all (at most 128
+ * cherry channels, at most 16384 + 128 input channels, batch 1).  vec must be 16-byte aligned.
+ */
+size_t cherryq_prepack_bytes(int w_bits, int in_features, int out_features, int num_cherries);
+int cherryq_prepack_supported(int w_bits, int batch, int in_features, int out_features, int num_cherries,
+                              int group_size);
+int cherryq_prepack_f16(int w_bits, const uint8_t *qweight, const void *cherry_weight, const int16_t *cherry_indices,
+                        const void *scales, void *stream, size_t stream_bytes, int in_features, int out_features,
+                        int num_cherries, int group_size, void *hip_stream);
+int cherryq_unprepack_f16(int w_bits, const void *stream, size_t stream_bytes, uint8_t *qweight, void *cherry_weight,
+                          int16_t *cherry_indices, void *scales, int in_features, int out_features, int num_cherries,
+                          int group_size, void *hip_stream);
+int cherryq_matvec_prepacked_f16(int w_bits, const void *vec, const void *stream, size_t stream_bytes, void *mul,
+                                 int batch, int in_features, int out_features, int num_cherries, int accumulate,
+                                 void *hip_stream);
+
+/*
  * One batch-1 launch over 1..4 packed layers that read the SAME activation vector and share
  * in_features, num_cherries, group_size and w_bits: q/k/v_proj (llama/modeling_llama_quant.py
  * :346-348 of the reference) or gate/up_proj (:251).  Arithmetic per layer is that of

@@ -17,7 +17,7 @@ HERE = Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
 OBJ = HERE / "build"
 LIB = HERE / "libcherryq.so"
-SOURCES = ["cq_api.hip", "cq_generic.hip", "cq_matvec.hip", "cq_batch.hip", "cq_gemm.hip", "cq_f32.hip", "cq_decode.hip", "cq_pack.hip", "cq_fakequant.hip", "cq_probe.hip"]
+SOURCES = ["cq_api.hip", "cq_generic.hip", "cq_matvec.hip", "cq_stream.hip", "cq_batch.hip", "cq_gemm.hip", "cq_f32.hip", "cq_decode.hip", "cq_pack.hip", "cq_fakequant.hip", "cq_probe.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",

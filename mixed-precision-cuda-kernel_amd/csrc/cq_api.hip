@@ -281,6 +281,71 @@ int cherryq_probe_stream_read(const void *buf, size_t bytes, void *sink, void *s
 
 int cherryq_probe_empty_launch(void *stream) { return (int)cq::launch_probe_empty(reinterpret_cast<hipStream_t>(stream)); }
 
+// ---- load-time repacked weight stream (see include/cherryq.h) -----------------------------------
+
+size_t cherryq_prepack_bytes(int w_bits, int in_features, int out_features, int num_cherries) {
+    if ((w_bits != 3 && w_bits != 4) || in_features <= 0 || out_features <= 0 || num_cherries < 0 ||
+        num_cherries >= in_features)
+        return 0;
+    return cq::stream_bytes(w_bits, in_features, out_features, num_cherries);
+}
+
+int cherryq_prepack_supported(int w_bits, int batch, int in_features, int out_features, int num_cherries,
+                              int group_size) {
+    return cq::stream_supported(w_bits, batch, in_features, out_features, num_cherries, group_size) ? 1 : 0;
+}
+
+static int prepack_check(int w_bits, int K, int N, int C, int G, size_t stream_bytes_given) {
+    if (w_bits != 3 && w_bits != 4) return CHERRYQ_E_BITS;
+    if (K <= 0 || N <= 0 || C < 0 || C >= K || K % 8 || N % 8 || C % 8) return CHERRYQ_E_SHAPE;
+    if (C > 0 && K > 32768) return CHERRYQ_E_SHAPE;  // int16 channel indices cannot name the columns
+    if (G <= 0 || G % cq::kStreamUnitK) return CHERRYQ_E_GROUP;
+    if (!cq::stream_supported(w_bits, 1, K, N, C, G)) return CHERRYQ_E_UNSUPPORTED;
+    if (stream_bytes_given < cq::stream_bytes(w_bits, K, N, C)) return CHERRYQ_E_WORKSPACE;
+    return CHERRYQ_OK;
+}
+
+int cherryq_prepack_f16(int w_bits, const uint8_t *qweight, const void *cherry_weight, const int16_t *cherry_indices,
+                        const void *scales, void *stream, size_t stream_bytes, int in_features, int out_features,
+                        int num_cherries, int group_size, void *hip_stream) {
+    int rc = prepack_check(w_bits, in_features, out_features, num_cherries, group_size, stream_bytes);
+    if (rc) return rc;
+    if (!qweight || !scales || !stream || (num_cherries > 0 && (!cherry_weight || !cherry_indices))) return CHERRYQ_E_NULL;
+    if (!cq::aligned(stream, 256)) return CHERRYQ_E_ALIGN;
+    return (int)cq::launch_stream_pack(w_bits, qweight, reinterpret_cast<const __half *>(cherry_weight), cherry_indices,
+                                       reinterpret_cast<const __half *>(scales), reinterpret_cast<uint8_t *>(stream),
+                                       in_features, out_features, num_cherries, group_size,
+                                       reinterpret_cast<hipStream_t>(hip_stream));
+}
+
+int cherryq_unprepack_f16(int w_bits, const void *stream, size_t stream_bytes, uint8_t *qweight, void *cherry_weight,
+                          int16_t *cherry_indices, void *scales, int in_features, int out_features, int num_cherries,
+                          int group_size, void *hip_stream) {
+    int rc = prepack_check(w_bits, in_features, out_features, num_cherries, group_size, stream_bytes);
+    if (rc) return rc;
+    if (!qweight || !scales || !stream || (num_cherries > 0 && (!cherry_weight || !cherry_indices))) return CHERRYQ_E_NULL;
+    if (!cq::aligned(stream, 256)) return CHERRYQ_E_ALIGN;
+    return (int)cq::launch_stream_unpack(w_bits, reinterpret_cast<const uint8_t *>(stream), qweight,
+                                         reinterpret_cast<__half *>(cherry_weight), cherry_indices,
+                                         reinterpret_cast<__half *>(scales), in_features, out_features, num_cherries,
+                                         group_size, reinterpret_cast<hipStream_t>(hip_stream));
+}
+
+int cherryq_matvec_prepacked_f16(int w_bits, const void *vec, const void *stream, size_t stream_bytes, void *mul,
+                                 int batch, int in_features, int out_features, int num_cherries, int accumulate,
+                                 void *hip_stream) {
+    int rc = prepack_check(w_bits, in_features, out_features, num_cherries, cq::kStreamUnitK, stream_bytes);
+    if (rc) return rc;
+    if (batch < 0) return CHERRYQ_E_SHAPE;
+    if (batch == 0) return CHERRYQ_OK;
+    if (batch != 1) return CHERRYQ_E_UNSUPPORTED;
+    if (!vec || !stream || !mul) return CHERRYQ_E_NULL;
+    if (!cq::aligned(stream, 256) || !cq::aligned(vec, 16) || !cq::aligned(mul, 2)) return CHERRYQ_E_ALIGN;
+    return (int)cq::launch_stream(w_bits, reinterpret_cast<const __half *>(vec), reinterpret_cast<const uint8_t *>(stream),
+                                  reinterpret_cast<__half *>(mul), in_features, out_features, num_cherries, accumulate,
+                                  reinterpret_cast<hipStream_t>(hip_stream));
+}
+
 // ---- decode-step entry points (see include/cherryq.h) ------------------------------------------
 
 size_t cherryq_group_workspace_bytes(int n_layers, const int *out_features) {

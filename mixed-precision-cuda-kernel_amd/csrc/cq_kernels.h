@@ -93,6 +93,26 @@ hipError_t launch_gemm(int bits, const __half *vec, const uint8_t *qweight, cons
                        const int16_t *cherry_indices, const __half *scales, __half *mul, int M, int K, int N, int C,
                        int G, int accumulate, void *workspace, void *scratch, hipStream_t stream);
 
+// cq_stream.hip: batch-1 matvec over a load-time repacked weight stream (tiles of 16 columns, each
+// tile's whole K range contiguous; no split-K, no workspace).
+constexpr int kStreamTileCols = 16;
+constexpr int kStreamUnitK = 128;
+struct StreamGeo {
+    int bits, K, N, C, Kn, ng, ntiles;
+    uint32_t off_cherry, off_units, record_bytes;  // byte offsets inside a tile record, record size
+    uint32_t hdr_bytes;                             // gather table + cherry columns in front of the tiles
+};
+StreamGeo stream_geo(int bits, int K, int N, int C);
+size_t stream_bytes(int bits, int K, int N, int C);
+bool stream_supported(int bits, int B, int K, int N, int C, int G);
+hipError_t launch_stream(int bits, const __half *vec, const uint8_t *stream, __half *mul, int K, int N, int C,
+                         int accumulate, hipStream_t s);
+hipError_t launch_stream_pack(int bits, const uint8_t *qweight, const __half *cherry_weight,
+                              const int16_t *cherry_indices, const __half *scales, uint8_t *stream, int K, int N,
+                              int C, int G, hipStream_t s);
+hipError_t launch_stream_unpack(int bits, const uint8_t *stream, uint8_t *qweight, __half *cherry_weight,
+                                int16_t *cherry_indices, __half *scales, int K, int N, int C, int G, hipStream_t s);
+
 // cq_pack.hip: dense fp16 weight -> packed buffers on the device.
 hipError_t launch_pack(int bits, const __half *w, const int16_t *idx, uint8_t *qweight, __half *scales,
                        __half *cherry_weight, int K, int N, int C, int G, hipStream_t stream);

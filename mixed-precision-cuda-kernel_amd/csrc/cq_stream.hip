@@ -1,0 +1,575 @@
+// Fused dequant + matvec over a load-time repacked weight stream (gfx950).
+//
+// The reference layout (qweight (Kn/8*b, N), N contiguous) forces a kernel to split K across
+// workgroups: a byte row holds one or two positions of every column, so a wavefront that wants
+// wide loads owns many columns and few positions, and the partial sums of many workgroups have to
+// meet in memory.  The stream layout below is the same information rearranged once, at load time,
+// for the way CDNA4 wants to consume it:
+//
+//   * 16 output columns form a tile; a tile's whole K range is one contiguous record
+//         [scales: ng x 16 fp16][cherry rows: C x 16 fp16][units: ng x 1 KB (4-bit) / 768 B (3-bit)]
+//     (sections padded to 256 bytes).  A workgroup owns whole tiles, so no partial sum ever leaves
+//     the workgroup: no atomics, no workspace, one fp16 store per output.
+//   * a unit is 128 compacted positions (one scale group when G = 128) x 16 columns.  Lane
+//     (kq = lane / 16, n = lane % 16) holds the 32 codes of column n at positions
+//     128 g + 32 kq + 0..31 in 4 (3) consecutive dwords, so a wavefront reads a unit as ONE
+//     dwordx4 (dwordx3) load of 1 KB (768 B) contiguous bytes.
+//   * inside a lane's dwords the codes sit where a single v_and_b32 turns them into an MFMA
+//     operand: a field masked in place at bit p <= 8 of a 16-bit half IS the fp16 subnormal
+//     code * 2^(p-24).  4-bit: fields at bit 0 and 4 of each half directly, the other two after
+//     one shift by 8 (5 VALU instructions per 8 codes, no v_perm).  3-bit: fields at bit 0, 3, 6
+//     directly, two more after one shift by 9, and the 6 left-over bits of the three dwords form
+//     the last two codes (23 instructions per 32 codes) -- here the values truly straddle dwords.
+//   * v_mfma_f32_16x16x32_f16 (and 16x16x16 for the 3-bit remainders) multiplies: B = the lane's
+//     masked fields, A = the activations of the same positions from LDS, and the MFMA's K
+//     dimension runs across the four lane groups, so the reduction over a unit's 128 positions
+//     costs nothing.  Fields of different bit positions go to different accumulators (scaled by
+//     2^(24-p) afterwards), so the activations enter unscaled and every product is exact.
+//   * the activation vector is compacted around the cherry channels ONCE per workgroup into LDS
+//     (raw copy -> gather), together with the per-group sums for the grid offset -c_b * sum(x).
+//
+// Arithmetic contract: csrc/quant_cuda_kernel.cu:718-835 (4-bit) and 558-672 (3-bit) of the
+// reference; fp32 accumulation, one rounding to fp16.  Replaces the per-thread decode loops at
+// :811-831 / :649-667 and the serial batch loop :797-834.
+#include "cq_common.cuh"
+#include "cq_kernels.h"
+
+namespace cq {
+
+typedef _Float16 sh8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 sh4_t __attribute__((ext_vector_type(4)));
+typedef float sf4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t su4 __attribute__((ext_vector_type(4)));
+typedef uint32_t su3 __attribute__((ext_vector_type(3)));
+typedef uint32_t su2 __attribute__((ext_vector_type(2)));
+typedef _Float16 sh2_t __attribute__((ext_vector_type(2)));
+
+constexpr uint32_t kSFlags = 0x00020000u;
+constexpr uint32_t kSOob = 0x80000000u;
+constexpr int kStreamMaxXLoads = 4;  // 16-byte loads of raw activations per thread
+constexpr int kStreamRawPad = 512 + 128 + 8;  // zero halves kept behind the raw activations in LDS
+
+static inline uint32_t align256(uint32_t v) { return (v + 255u) & ~255u; }
+
+StreamGeo stream_geo(int bits, int K, int N, int C) {
+    StreamGeo g;
+    g.bits = bits;
+    g.K = K;
+    g.N = N;
+    g.C = C;
+    g.Kn = K - C;
+    g.ng = ceil_div(K - C, kStreamUnitK);
+    g.ntiles = ceil_div(N, kStreamTileCols);
+    g.off_cherry = align256((uint32_t)g.ng * 32u);
+    g.off_units = g.off_cherry + align256((uint32_t)C * 32u);
+    g.record_bytes = g.off_units + (uint32_t)g.ng * (bits == 4 ? 1024u : 768u);
+    g.hdr_bytes = align256((uint32_t)(((g.ng * kStreamUnitK + 511) & ~511) + 2 * ((C + 31) & ~31)));
+    return g;
+}
+
+size_t stream_bytes(int bits, int K, int N, int C) {
+    const StreamGeo g = stream_geo(bits, K, N, C);
+    return g.hdr_bytes + (size_t)g.ntiles * g.record_bytes;
+}
+
+// ---- where code q (0..31) of a lane lives ----------------------------------------------------
+// 4-bit: MFMA j = q / 8 takes slot r = q % 8 from dword 2 (j & 1) + r / 4, nibble {0, 4, 2, 6}[r % 4]
+// (+ 1 for j >= 2, the fields that sit at bit 4 of their half).
+__host__ __device__ constexpr int s4_dword(int q) { return 2 * ((q >> 3) & 1) + ((q & 7) >> 2); }
+__host__ __device__ constexpr int s4_bit(int q) { return 4 * ((int)((0x6240u >> (4 * (q & 3))) & 15u) + (q >> 4)); }
+// 3-bit: returns dword (0..2) and bit, or dword 3 for the two codes assembled from the left-over
+// bits (bit 15 + 16 h of dwords 0, 1, 2 = code bits 0, 1, 2), with `bit` = 16 h.
+__host__ __device__ constexpr int s3_dword(int q) {
+    return q < 24 ? (((q & 7) < 6) ? ((q & 7) >> 1) : (q < 16 ? 0 : 3)) : 1 + ((q & 3) >> 1);
+}
+__host__ __device__ constexpr int s3_bit(int q) {
+    const int h = q & 1;
+    if (q < 24) {
+        const int f = ((q & 7) < 6) ? (q >> 3) : (q >> 3) + 3;  // q < 16 only for the second form
+        return ((q & 7) < 6 || q < 16) ? 16 * h + 3 * f : 16 * h;
+    }
+    return 16 * h + 3 * (q < 28 ? 3 : 4);
+}
+
+// ---- prepack: reference buffers -> stream ------------------------------------------------------
+template <int BITS>
+__device__ inline uint32_t ref_code(const uint8_t *__restrict__ qweight, int k, int n, int N) {
+    if (BITS == 4) return (qweight[(size_t)(k >> 1) * N + n] >> (4 * (k & 1))) & 15u;
+    const size_t r = (size_t)(k >> 3) * 3;
+    const uint32_t w24 = qweight[r * N + n] | (qweight[(r + 1) * N + n] << 8) | (qweight[(r + 2) * N + n] << 16);
+    return (w24 >> (3 * (k & 7))) & 7u;
+}
+
+template <int BITS>
+__global__ __launch_bounds__(256) void stream_pack_kernel(const uint8_t *__restrict__ qweight,
+                                                          const __half *__restrict__ cherry_weight,
+                                                          const __half *__restrict__ scales,
+                                                          uint8_t *__restrict__ stream, int G, StreamGeo geo) {
+    const int tile = blockIdx.x;
+    uint8_t *rec = stream + geo.hdr_bytes + (size_t)tile * geo.record_bytes;
+    const int N = geo.N, Kn = geo.Kn;
+    // sections the kernel never writes codes into start out zero (padding)
+    for (uint32_t i = threadIdx.x; i < geo.off_units / 4; i += 256) reinterpret_cast<uint32_t *>(rec)[i] = 0u;
+    __syncthreads();
+    for (int i = threadIdx.x; i < geo.ng * 16; i += 256) {
+        const int g = i >> 4, n = tile * 16 + (i & 15);
+        reinterpret_cast<__half *>(rec)[i] = n < N ? scales[(size_t)(g * kStreamUnitK / G) * N + n] : __float2half(0.f);
+    }
+    for (int i = threadIdx.x; i < geo.C * 16; i += 256) {
+        // piece (lg, nn): 8 halves = cherry rows 8 lg .. 8 lg + 7 of column nn
+        const int piece = i >> 3, e = i & 7, lg = piece >> 4, n = tile * 16 + (piece & 15);
+        reinterpret_cast<__half *>(rec + geo.off_cherry)[i] =
+            n < N ? cherry_weight[(size_t)(8 * lg + e) * N + n] : __float2half(0.f);
+    }
+    constexpr int DW = BITS;  // dwords per lane and unit
+    for (int i = threadIdx.x; i < geo.ng * 64; i += 256) {
+        const int g = i >> 6, lane = i & 63, kq = lane >> 4, n = tile * 16 + (lane & 15);
+        uint32_t d[4] = {0u, 0u, 0u, 0u};
+        for (int q = 0; q < 32; q++) {
+            const int k = g * kStreamUnitK + 32 * kq + q;
+            const uint32_t code = (k < Kn && n < N) ? ref_code<BITS>(qweight, k, n, N) : 0u;
+            if (BITS == 4) {
+                d[s4_dword(q)] |= code << s4_bit(q);
+            } else if (s3_dword(q) < 3) {
+                d[s3_dword(q)] |= code << s3_bit(q);
+            } else {
+                const int b = s3_bit(q) + 15;
+                d[0] |= (code & 1u) << b;
+                d[1] |= ((code >> 1) & 1u) << b;
+                d[2] |= ((code >> 2) & 1u) << b;
+            }
+        }
+        uint32_t *o = reinterpret_cast<uint32_t *>(rec + geo.off_units + (size_t)g * (64 * DW * 4)) + lane * DW;
+        for (int j = 0; j < DW; j++) o[j] = d[j];
+    }
+}
+
+// stream -> reference buffers (the inverse; restores a state dict from a prepacked module)
+template <int BITS>
+__global__ __launch_bounds__(256) void stream_unpack_kernel(const uint8_t *__restrict__ stream,
+                                                            uint8_t *__restrict__ qweight,
+                                                            __half *__restrict__ cherry_weight,
+                                                            __half *__restrict__ scales, int G, StreamGeo geo) {
+    const int tile = blockIdx.x;
+    const uint8_t *rec = stream + geo.hdr_bytes + (size_t)tile * geo.record_bytes;
+    const int N = geo.N, Kn = geo.Kn;
+    const int ngr = ceil_div(Kn, G);
+    for (int i = threadIdx.x; i < ngr * 16; i += 256) {
+        const int gr = i >> 4, n = tile * 16 + (i & 15);
+        if (n < N) scales[(size_t)gr * N + n] = reinterpret_cast<const __half *>(rec)[(gr * (G / kStreamUnitK)) * 16 + (i & 15)];
+    }
+    for (int i = threadIdx.x; i < geo.C * 16; i += 256) {
+        const int piece = i >> 3, e = i & 7, lg = piece >> 4, n = tile * 16 + (piece & 15);
+        if (n < N) cherry_weight[(size_t)(8 * lg + e) * N + n] = reinterpret_cast<const __half *>(rec + geo.off_cherry)[i];
+    }
+    constexpr int DW = BITS;
+    for (int i = threadIdx.x; i < geo.ng * 64; i += 256) {
+        const int g = i >> 6, lane = i & 63, kq = lane >> 4, n = tile * 16 + (lane & 15);
+        if (n >= N) continue;
+        const uint32_t *o = reinterpret_cast<const uint32_t *>(rec + geo.off_units + (size_t)g * (64 * DW * 4)) + lane * DW;
+        uint32_t d[4] = {0u, 0u, 0u, 0u};
+        for (int j = 0; j < DW; j++) d[j] = o[j];
+        uint32_t code[32];
+        for (int q = 0; q < 32; q++) {
+            if (BITS == 4) {
+                code[q] = (d[s4_dword(q)] >> s4_bit(q)) & 15u;
+            } else if (s3_dword(q) < 3) {
+                code[q] = (d[s3_dword(q)] >> s3_bit(q)) & 7u;
+            } else {
+                const int b = s3_bit(q) + 15;
+                code[q] = ((d[0] >> b) & 1u) | (((d[1] >> b) & 1u) << 1) | (((d[2] >> b) & 1u) << 2);
+            }
+        }
+        const int k0 = g * kStreamUnitK + 32 * kq;
+        if (BITS == 4) {
+            for (int q = 0; q < 32; q += 2)
+                if (k0 + q < Kn) qweight[(size_t)((k0 + q) >> 1) * N + n] = (uint8_t)(code[q] | (code[q + 1] << 4));
+        } else {
+            for (int q = 0; q < 32; q += 8) {
+                if (k0 + q >= Kn) continue;
+                uint32_t w24 = 0;
+                for (int e = 0; e < 8; e++) w24 |= code[q + e] << (3 * e);
+                const size_t r = (size_t)((k0 + q) >> 3) * 3;
+                qweight[r * N + n] = (uint8_t)w24;
+                qweight[(r + 1) * N + n] = (uint8_t)(w24 >> 8);
+                qweight[(r + 2) * N + n] = (uint8_t)(w24 >> 16);
+            }
+        }
+    }
+}
+
+// header: for every compacted position k the number of cherry columns in front of it, low(k) (the
+// position reads activation column k + low(k); padding positions hold C and so read beyond the last
+// column, where the kernel keeps zeros), one byte
+// each, stored per block of 512 positions so that lane l of a wavefront finds the entries of
+// positions l, l + 64, ..., l + 448 in 8 consecutive bytes; then the cherry columns (uint16,
+// padded with K, the column the kernel keeps zero)
+__global__ __launch_bounds__(256) void stream_header_kernel(const int16_t *__restrict__ cherry_indices,
+                                                            uint8_t *__restrict__ hdr, StreamGeo geo) {
+    const int Knp512 = (geo.ng * kStreamUnitK + 511) & ~511, Cp = (geo.C + 31) & ~31;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < Knp512) {
+        const int blk = i >> 9, l = (i >> 3) & 63, j = i & 7;
+        const int k = blk * 512 + 64 * j + l;
+        hdr[i] = (uint8_t)(k < geo.Kn ? gather_offset(cherry_indices, geo.C, k) : geo.C);
+    } else if (i < Knp512 + Cp) {
+        const int m = i - Knp512;
+        reinterpret_cast<uint16_t *>(hdr + Knp512)[m] = (uint16_t)(m < geo.C ? (int)cherry_indices[m] : geo.K);
+    }
+    if (i >= Knp512 + 2 * Cp && i < (int)geo.hdr_bytes) hdr[i] = 0;  // padding of the header
+}
+
+__global__ __launch_bounds__(256) void stream_header_unpack_kernel(const uint8_t *__restrict__ hdr,
+                                                                   int16_t *__restrict__ cherry_indices, StreamGeo geo) {
+    const int Knp512 = (geo.ng * kStreamUnitK + 511) & ~511;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < geo.C) cherry_indices[i] = (int16_t)reinterpret_cast<const uint16_t *>(hdr + Knp512)[i];
+}
+
+// ---- the matvec --------------------------------------------------------------------------------
+__device__ inline sh8_t as_h8(su4 v) { return __builtin_bit_cast(sh8_t, v); }
+__device__ inline sh4_t as_h4(su2 v) { return __builtin_bit_cast(sh4_t, v); }
+
+// One unit (128 positions x 16 columns) against the activations of the same positions: the
+// sum over the unit of x * code for the lane's column (row 0 of the MFMA tile, which every lane
+// group receives because every row of A holds the same activations).
+template <int BITS>
+__device__ inline float unit_dot(const su4 w, const unsigned short *xa) {
+    const sf4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (BITS == 4) {
+        const su4 y = {w[0] >> 8, w[1] >> 8, w[2] >> 8, w[3] >> 8};
+        const sh8_t a0 = *reinterpret_cast<const sh8_t *>(xa);
+        const sh8_t a1 = *reinterpret_cast<const sh8_t *>(xa + 8);
+        const sh8_t a2 = *reinterpret_cast<const sh8_t *>(xa + 16);
+        const sh8_t a3 = *reinterpret_cast<const sh8_t *>(xa + 24);
+        const su4 b0 = {w[0] & 0x000f000fu, y[0] & 0x000f000fu, w[1] & 0x000f000fu, y[1] & 0x000f000fu};
+        const su4 b1 = {w[2] & 0x000f000fu, y[2] & 0x000f000fu, w[3] & 0x000f000fu, y[3] & 0x000f000fu};
+        const su4 b2 = {w[0] & 0x00f000f0u, y[0] & 0x00f000f0u, w[1] & 0x00f000f0u, y[1] & 0x00f000f0u};
+        const su4 b3 = {w[2] & 0x00f000f0u, y[2] & 0x00f000f0u, w[3] & 0x00f000f0u, y[3] & 0x00f000f0u};
+        sf4_t dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, as_h8(b0), zero4, 0, 0, 0);
+        sf4_t dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, as_h8(b2), zero4, 0, 0, 0);
+        dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, as_h8(b1), dl, 0, 0, 0);
+        dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(a3, as_h8(b3), dh, 0, 0, 0);
+        return dl[0] * 16777216.0f + dh[0] * 1048576.0f;
+    } else {
+        const su3 y = {w[0] >> 9, w[1] >> 9, w[2] >> 9};
+        const sh8_t a0 = *reinterpret_cast<const sh8_t *>(xa);        // positions 0..7: fields at bit 0
+        const sh8_t a2 = *reinterpret_cast<const sh8_t *>(xa + 8);    // 8..15: bit 3
+        const sh8_t a4 = *reinterpret_cast<const sh8_t *>(xa + 16);   // 16..23: bit 6
+        const sh4_t a1 = *reinterpret_cast<const sh4_t *>(xa + 24);   // 24..27: bit 0
+        const sh4_t a3 = *reinterpret_cast<const sh4_t *>(xa + 28);   // 28..31: bit 3
+        const uint32_t z = (y[0] & 0x00400040u) | ((y[1] & 0x00400040u) << 1) | ((y[2] & 0x00400040u) << 2);
+        const su4 b0 = {w[0] & 0x00070007u, w[1] & 0x00070007u, w[2] & 0x00070007u, y[0] & 0x00070007u};
+        const su4 b2 = {w[0] & 0x00380038u, w[1] & 0x00380038u, w[2] & 0x00380038u, y[0] & 0x00380038u};
+        const su4 b4 = {w[0] & 0x01c001c0u, w[1] & 0x01c001c0u, w[2] & 0x01c001c0u, z};
+        const su2 b1 = {y[1] & 0x00070007u, y[2] & 0x00070007u};
+        const su2 b3 = {y[1] & 0x00380038u, y[2] & 0x00380038u};
+        sf4_t d0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, as_h8(b0), zero4, 0, 0, 0);
+        sf4_t d3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, as_h8(b2), zero4, 0, 0, 0);
+        const sf4_t d6 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a4, as_h8(b4), zero4, 0, 0, 0);
+        d0 = __builtin_amdgcn_mfma_f32_16x16x16f16(a1, as_h4(b1), d0, 0, 0, 0);
+        d3 = __builtin_amdgcn_mfma_f32_16x16x16f16(a3, as_h4(b3), d3, 0, 0, 0);
+        return d0[0] * 16777216.0f + d3[0] * 2097152.0f + d6[0] * 262144.0f;
+    }
+}
+
+// A workgroup is W computing wavefronts plus S staging wavefronts and owns T tiles (W % T == 0):
+// computing wavefront w works on tile w % T and takes the units g = w / T, w / T + W / T, ... of it
+// (at most L), D loads in flight.  Staging wavefront j prepares NB consecutive blocks of 512
+// compacted positions (S * NB blocks cover K).
+//
+// Order of events.  A CU admits vector loads only as fast as earlier ones return, so whatever a
+// wavefront does after queueing weight loads waits in that queue with them.  Therefore: (1) every
+// wavefront requests its 16 bytes per thread of the activation vector alone (the staging
+// wavefronts also the gather table and the cherry columns from the stream header), copies them
+// to LDS and meets the others -- under a microsecond after the start, nothing else being in the
+// queues; (2) the computing wavefronts queue their cherry rows, scales and first D units, while
+// the staging wavefronts, which never touch the weight stream, gather the activations into MFMA
+// operand order (conflict-free: lane l takes positions l, l + 64, ...), add up every unit's
+// activations for the grid offset, and raise a counter in LDS; (3) a computing wavefront looks
+// at the counter when its loads are queued, then consumes its units in order, refilling every
+// slot it frees.
+template <int BITS, int W, int T, int D, int L, int S, int NB>
+__global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__restrict__ x,
+                                                              const uint8_t *__restrict__ stream,
+                                                              __half *__restrict__ mul, int accumulate,
+                                                              StreamGeo geo) {
+    static_assert(L % 4 == 0 && W % T == 0 && D <= L, "");
+    constexpr int WT = W / T;
+    constexpr int NT = 64 * (W + S);
+    constexpr int UB = BITS == 4 ? 1024 : 768;
+    constexpr float kGrid = BITS == 4 ? -7.5f : -3.5f;
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kq = lane >> 4, nn = lane & 15;
+    const bool stager = wave >= W;
+    const int K = geo.K, C = geo.C, ng = geo.ng, N = geo.N;
+    const int Knp = ng * kStreamUnitK;
+    const int Cp = (C + 31) & ~31;
+    const int Knp512 = (Knp + 511) & ~511;
+    const int nblk = Knp512 >> 9;  // blocks of 512 positions
+    // LDS: counter | raw activations (+ zeros) | compacted activations | cherry activations | unit sums | partial outputs
+    int *s_flag = reinterpret_cast<int *>(smem);
+    unsigned short *s_raw = reinterpret_cast<unsigned short *>(smem + 16);
+    unsigned short *s_xs = s_raw + K + kStreamRawPad;
+    unsigned short *s_xc = s_xs + Knp512;
+    float *s_xsum = reinterpret_cast<float *>(s_xc + Cp);
+    float *s_red = s_xsum + 4 * nblk;
+
+    // ---- (1) raw activations, everyone; gather table and cherry columns, staging wavefronts
+    su4 xr[kStreamMaxXLoads];
+    su2 tb[NB];
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, K * 2, kSFlags);
+    const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc((void *)stream, 0, (int)geo.hdr_bytes, kSFlags);
+#pragma unroll
+    for (int i = 0; i < kStreamMaxXLoads; i++)
+        if (i * NT * 8 < K) xr[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, (uint32_t)(tid + i * NT) * 16u, 0, 0);
+    const int ws = wave - W;  // index among the staging wavefronts
+    const int b0 = ws * NB, b1 = min(nblk, b0 + NB);
+    uint32_t ci0 = 0, ci1 = 0;
+    if (stager) {
+#pragma unroll
+        for (int i = 0; i < NB; i++)
+            tb[i] = __builtin_amdgcn_raw_buffer_load_b64(rh, b0 + i < b1 ? (uint32_t)((b0 + i) * 512 + lane * 8) : kSOob, 0, 0);
+        if (ws == 0) {
+            ci0 = __builtin_amdgcn_raw_buffer_load_b16(rh, lane < Cp ? (uint32_t)(Knp512 + lane * 2) : kSOob, 0, 0);
+            ci1 = __builtin_amdgcn_raw_buffer_load_b16(rh, lane + 64 < Cp ? (uint32_t)(Knp512 + (lane + 64) * 2) : kSOob, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < kStreamMaxXLoads; i++)
+        if (i * NT * 8 < K && (tid + i * NT) * 8 < K) reinterpret_cast<su4 *>(s_raw)[tid + i * NT] = xr[i];
+    // zeros behind the activations: what padding positions (and padded cherry columns) read
+    if (tid < kStreamRawPad / 8) reinterpret_cast<su4 *>(s_raw)[(K >> 3) + tid] = (su4){0u, 0u, 0u, 0u};
+    if (tid == 0) *s_flag = 0;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+
+    float tot = 0.f;
+    if (stager) {
+        // ---- (2b) xs[k] = x[k + low(k)] for the positions of blocks [b0, b1), and the sum of every unit
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            const int blk = b0 + i;
+            if (blk < b1) {
+                const su2 t = tb[i];
+                unsigned short h[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    h[j] = s_raw[blk * 512 + 64 * j + lane + (int)((t[j >> 2] >> (8 * (j & 3))) & 0xffu)];
+                float f[4];
+#pragma unroll
+                for (int j = 0; j < 8; j++) s_xs[blk * 512 + 64 * j + lane] = h[j];
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+                    f[u] = __half2float(__ushort_as_half(h[2 * u])) + __half2float(__ushort_as_half(h[2 * u + 1]));
+                // the block's four unit sums in one pass: the two swaps leave unit 0 | 2 | 1 | 3 in
+                // the four 16-lane rows, the rotations finish each row
+                const float s01 = swap32_add(f[0], f[1]);
+                const float s23 = swap32_add(f[2], f[3]);
+                const float r = row_sum(swap16_add(s01, s23));
+                if (nn == 0) s_xsum[blk * 4 + ((kq >> 1) | ((kq & 1) << 1))] = r;
+            }
+        }
+        if (ws == 0) {
+            if (lane < Cp) s_xc[lane] = s_raw[ci0 & 0xffffu];
+            if (lane + 64 < Cp) s_xc[lane + 64] = s_raw[ci1 & 0xffffu];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        if (lane == 0) __hip_atomic_fetch_add(s_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    } else {
+        // ---- (2a) computing wavefront.  Lane group kq keeps the scales of the units i with
+        // i % 4 == kq (every lane group ends up with the same MFMA results, so each finishes a
+        // quarter of the units; the quarters are added at the end).  Every unit of a tile past the
+        // last reads zeros through an empty descriptor.
+        const int tl = wave % T, cls = wave / T;
+        const int tile = blockIdx.x * T + tl;
+        const bool tile_ok = tile < geo.ntiles;
+        const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(stream + geo.hdr_bytes + (size_t)(tile_ok ? tile : 0) * geo.record_bytes), 0,
+            tile_ok ? (int)geo.record_bytes : 0, kSFlags);
+        uint32_t sc[L / 4];
+        su4 wbuf[D];
+        su4 cw[4];
+        const bool cherry_wave = cls == WT - 1;
+        // cherry rows first: they are consumed first, which frees their registers for the units
+        if (cherry_wave) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int lg = 4 * j + kq;
+                cw[j] = __builtin_amdgcn_raw_buffer_load_b128(
+                    rt, 8 * lg < C ? geo.off_cherry + (uint32_t)(lg * 16 + nn) * 16u : kSOob, 0, 2);
+            }
+        }
+        const uint32_t sc_off = (uint32_t)((cls + kq * WT) * 32 + nn * 2);
+#pragma unroll
+        for (int i = 0; i < L / 4; i++)
+            sc[i] = __builtin_amdgcn_raw_buffer_load_b16(rt, cls + (4 * i + kq) * WT < ng ? sc_off : kSOob, 4 * i * WT * 32, 0);
+        const uint32_t w_off = geo.off_units + (uint32_t)(cls * UB + lane * (BITS * 4));
+        auto load_unit = [&](int i) -> su4 {
+            // a unit past the last reads zeros: the vector offset alone lies outside the descriptor
+            const uint32_t off = cls + i * WT < ng ? w_off : kSOob;
+            if constexpr (BITS == 4) {
+                return __builtin_amdgcn_raw_buffer_load_b128(rt, off, i * WT * UB, 2);
+            } else {
+                const su3 v = __builtin_amdgcn_raw_buffer_load_b96(rt, off, i * WT * UB, 2);
+                return (su4){v[0], v[1], v[2], 0u};
+            }
+        };
+#pragma unroll
+        for (int i = 0; i < D; i++) wbuf[i] = load_unit(i);
+        // ---- (3) the staged activations are needed from here on
+        while (__hip_atomic_load(s_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < S) __builtin_amdgcn_s_sleep(1);
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+        float totc = 0.f;
+        if (cherry_wave) {
+            sf4_t dc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (32 * j < C) {
+                    const sh8_t a = *reinterpret_cast<const sh8_t *>(s_xc + 32 * j + 8 * kq);
+                    dc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, as_h8(cw[j]), dc, 0, 0, 0);
+                }
+            totc = dc[0];
+        }
+        // units, in order; every consumed slot is refilled with the unit D further on
+        const unsigned short *xa0 = s_xs + cls * kStreamUnitK + 32 * kq;
+        const float *xsum0 = s_xsum + cls;
+#pragma unroll
+        for (int i = 0; i < L; i++) {
+            if (cls + i * WT >= ng) break;
+            const float sf = (i & 3) == kq ? __half2float(__ushort_as_half((unsigned short)sc[i >> 2])) : 0.f;
+            const su4 w = wbuf[i % D];
+            const float v = unit_dot<BITS>(w, xa0 + i * WT * kStreamUnitK);
+            if (i + D < L) wbuf[i % D] = load_unit(i + D);
+            tot += (v + kGrid * xsum0[i * WT]) * sf;
+        }
+        // the four lane groups' quarters
+        tot = swap32_add(tot, tot);
+        tot = swap16_add(tot, tot) + totc;
+        if (kq == 0) s_red[wave * 16 + nn] = tot;
+    }
+
+    // ---- across the tile's wavefronts, then one store per output
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    if (tid < 16 * T) {
+        const int otl = tid >> 4, n = (blockIdx.x * T + otl) * 16 + (tid & 15);
+        if (n < N) {
+            float v = 0.f;
+#pragma unroll
+            for (int c = 0; c < WT; c++) v += s_red[(c * T + otl) * 16 + (tid & 15)];
+            if (accumulate) v += __half2float(mul[n]);
+            mul[n] = __float2half_rn(v);
+        }
+    }
+}
+
+static size_t stream_lds_bytes(const StreamGeo &g, int W) {
+    const int Knp512 = (g.ng * kStreamUnitK + 511) & ~511, Cp = (g.C + 31) & ~31;
+    return 16 + (size_t)(g.K + kStreamRawPad + Knp512 + Cp) * 2 + (size_t)(Knp512 / 128) * 4 + (size_t)W * 16 * 4;
+}
+
+// Launch geometries (W computing wavefronts, T tiles, D loads in flight, L units per wavefront at
+// most, S staging wavefronts of NB blocks each), by the number of 128-position units of a column.
+// One tile per workgroup throughout: whole tiles are the grain in which the work spreads over the
+// CUs, and two tiles per workgroup measured 20-30 % slower on the 4096 -> 11008 layer for that
+// reason.  All of a wavefront's loads are queued at once where the registers allow (D = L).
+struct StreamCfg {
+    int W, T, D, L, S, NB, max_units;
+};
+static constexpr StreamCfg kStreamCfgs[] = {
+    {4, 1, 8, 8, 1, 8, 32}, {4, 1, 8, 12, 2, 8, 48}, {8, 1, 8, 8, 2, 8, 64}, {8, 1, 8, 12, 3, 8, 96}, {8, 1, 8, 16, 4, 8, 128},
+};
+constexpr int kStreamCfgCount = sizeof(kStreamCfgs) / sizeof(kStreamCfgs[0]);
+
+static int stream_pick(const StreamGeo &geo) {
+    for (int i = 0; i < kStreamCfgCount; i++)
+        if (geo.ng <= kStreamCfgs[i].max_units) return i;
+    return -1;
+}
+
+bool stream_supported(int bits, int B, int K, int N, int C, int G) {
+    if (bits != 3 && bits != 4) return false;
+    if (B != 1) return false;
+    if (G <= 0 || G % kStreamUnitK) return false;
+    if (K - C <= 0 || C > 128 || K > 32768) return false;
+    if (K % 8 || N % 8 || C % 8) return false;
+    const StreamGeo geo = stream_geo(bits, K, N, C);
+    const int i = stream_pick(geo);
+    if (i < 0) return false;
+    return stream_lds_bytes(geo, kStreamCfgs[i].W) <= 160 * 1024;
+}
+
+template <int BITS, int I>
+static hipError_t launch_stream_cfg(const __half *vec, const uint8_t *stream, __half *mul, int accumulate,
+                                    const StreamGeo &geo, hipStream_t s) {
+    constexpr StreamCfg c = kStreamCfgs[I];
+    // what the kernel's fixed-size register arrays assume
+    if (geo.ng * kStreamUnitK > c.NB * 512 * c.S || geo.K > kStreamMaxXLoads * 8 * 64 * (c.W + c.S) ||
+        ceil_div(geo.ng, c.W / c.T) > c.L)
+        return hipErrorInvalidValue;
+    const size_t lds = stream_lds_bytes(geo, c.W);
+    if (lds > 160 * 1024) return hipErrorInvalidValue;
+    auto kern = stream_kernel<BITS, c.W, c.T, c.D, c.L, c.S, c.NB>;
+    static bool big_lds_enabled = false;  // (per instantiation; the attribute is idempotent, a race only repeats the call)
+    if (lds > 48 * 1024 && !big_lds_enabled) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        big_lds_enabled = true;
+    }
+    const dim3 grid(ceil_div(geo.ntiles, c.T)), block(64 * (c.W + c.S));
+    hipLaunchKernelGGL(kern, grid, block, lds, s, vec, stream, mul, accumulate, geo);
+    return hipGetLastError();
+}
+
+template <int BITS>
+static hipError_t launch_stream_bits(const __half *vec, const uint8_t *stream, __half *mul, int accumulate,
+                                     const StreamGeo &geo, hipStream_t s) {
+    switch (stream_pick(geo)) {
+        case 0: return launch_stream_cfg<BITS, 0>(vec, stream, mul, accumulate, geo, s);
+        case 1: return launch_stream_cfg<BITS, 1>(vec, stream, mul, accumulate, geo, s);
+        case 2: return launch_stream_cfg<BITS, 2>(vec, stream, mul, accumulate, geo, s);
+        case 3: return launch_stream_cfg<BITS, 3>(vec, stream, mul, accumulate, geo, s);
+        case 4: return launch_stream_cfg<BITS, 4>(vec, stream, mul, accumulate, geo, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_stream(int bits, const __half *vec, const uint8_t *stream, __half *mul, int K, int N, int C,
+                         int accumulate, hipStream_t s) {
+    const StreamGeo geo = stream_geo(bits, K, N, C);
+    if (bits == 4) return launch_stream_bits<4>(vec, stream, mul, accumulate, geo, s);
+    return launch_stream_bits<3>(vec, stream, mul, accumulate, geo, s);
+}
+
+hipError_t launch_stream_pack(int bits, const uint8_t *qweight, const __half *cherry_weight,
+                              const int16_t *cherry_indices, const __half *scales, uint8_t *stream, int K, int N,
+                              int C, int G, hipStream_t s) {
+    const StreamGeo geo = stream_geo(bits, K, N, C);
+    hipLaunchKernelGGL(stream_header_kernel, dim3(ceil_div((int)geo.hdr_bytes, 256)), dim3(256), 0, s, cherry_indices, stream,
+                       geo);
+    if (bits == 4)
+        hipLaunchKernelGGL(stream_pack_kernel<4>, dim3(geo.ntiles), dim3(256), 0, s, qweight, cherry_weight, scales, stream, G, geo);
+    else
+        hipLaunchKernelGGL(stream_pack_kernel<3>, dim3(geo.ntiles), dim3(256), 0, s, qweight, cherry_weight, scales, stream, G, geo);
+    return hipGetLastError();
+}
+
+hipError_t launch_stream_unpack(int bits, const uint8_t *stream, uint8_t *qweight, __half *cherry_weight,
+                                int16_t *cherry_indices, __half *scales, int K, int N, int C, int G, hipStream_t s) {
+    const StreamGeo geo = stream_geo(bits, K, N, C);
+    if (C > 0)
+        hipLaunchKernelGGL(stream_header_unpack_kernel, dim3(ceil_div(C, 256)), dim3(256), 0, s,
+                           stream, cherry_indices, geo);
+    if (bits == 4)
+        hipLaunchKernelGGL(stream_unpack_kernel<4>, dim3(geo.ntiles), dim3(256), 0, s, stream, qweight, cherry_weight, scales, G, geo);
+    else
+        hipLaunchKernelGGL(stream_unpack_kernel<3>, dim3(geo.ntiles), dim3(256), 0, s, stream, qweight, cherry_weight, scales, G, geo);
+    return hipGetLastError();
+}
+
+}  // namespace cq

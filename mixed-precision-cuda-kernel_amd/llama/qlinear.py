@@ -166,6 +166,43 @@ class QuantLinear(nn.Module):
         weight[..., self.cherry_indices.long()] = self.cherry_weight.t()
         return weight
 
+    # ---- load-time repack (no counterpart in the reference) -----------------------------------
+    @torch.inference_mode()
+    def prepack(self, release_reference: bool = False):
+        """Rearrange the packed buffers, once, into the weight stream the batch-1 kernel of this
+        GPU reads fastest (quant_cuda.prepack_cherryq).  The state-dict buffers stay as they are
+        unless `release_reference` frees them (unprepack() brings them back, bit for bit).
+        Returns True if the layer's shape is taken; otherwise the module is left unchanged and
+        keeps using the kernels that read the checkpoint layout."""
+        if self.w_bits not in (3, 4) or not self.qweight.is_cuda or self.dequantized:
+            return False
+        if not quant_cuda.prepack_supported(self.w_bits, 1, self.in_features, self.out_features,
+                                            self.num_cherries, self.group_size):
+            return False
+        self._stream = quant_cuda.prepack_cherryq(self.w_bits, self.qweight, self.cherry_weight, self.cherry_indices,
+                                                  self.scales, self.in_features, self.group_size)
+        if release_reference:
+            dev = self.qweight.device
+            self.qweight = torch.empty((0, self.out_features), dtype=torch.uint8, device=dev)
+            self.scales = torch.empty((0, self.out_features), dtype=torch.float16, device=dev)
+            self.cherry_weight = torch.empty((0, self.out_features), dtype=torch.float16, device=dev)
+            self._released = True
+        return True
+
+    @torch.inference_mode()
+    def unprepack(self):
+        """Drop the weight stream; if prepack() released the checkpoint-layout buffers, rebuild
+        them from it first."""
+        stream = getattr(self, "_stream", None)
+        if stream is None:
+            return
+        if getattr(self, "_released", False):
+            (self.cherry_indices, self.cherry_weight, self.qweight,
+             self.scales) = quant_cuda.unprepack_cherryq(self.w_bits, stream, self.in_features, self.out_features,
+                                                         self.num_cherries, self.group_size)
+            self._released = False
+        self._stream = None
+
     # ---- forward ------------------------------------------------------------------------------
     @torch.inference_mode()
     def forward(self, x: torch.Tensor):
@@ -179,7 +216,14 @@ class QuantLinear(nn.Module):
             if x2.dtype != torch.float16:
                 x2 = x2.to(torch.float16)
             x2 = x2.contiguous()
-            if x2.shape[0] >= self.prefill_rows:
+            stream = getattr(self, "_stream", None)
+            if stream is not None and x2.shape[0] == 1:
+                out = torch.empty(1, self.out_features, dtype=torch.float16, device=stream.device)
+                quant_cuda.matvec_prepacked_cherryq(self.w_bits, x2, stream, out, self.in_features, self.num_cherries)
+            elif getattr(self, "_released", False):
+                raise RuntimeError("prepack(release_reference=True) left only the batch-1 weight stream; "
+                                   "call unprepack() before using other batch sizes")
+            elif x2.shape[0] >= self.prefill_rows:
                 # prompt-sized batches: one bit-exact dequantisation pass on the GPU into a transient
                 # dense weight, then a library fp16 GEMM -- the arithmetic of the dequantised branch
                 # below (llama/qlinear.py:183-195) without keeping the dense weight

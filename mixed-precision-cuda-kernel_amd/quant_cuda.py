@@ -52,6 +52,16 @@ _lib.cherryq_pack_f16.restype = _int
 for _name in ("cherryq_fake_quant_f16", "cherryq_fake_quant_f32"):
     getattr(_lib, _name).argtypes = [_int, _vp, _vp, _vp, _int, _int, _int, _int, _int, _vp]
     getattr(_lib, _name).restype = _int
+_lib.cherryq_prepack_bytes.argtypes = [_int, _int, _int, _int]
+_lib.cherryq_prepack_bytes.restype = _sz
+_lib.cherryq_prepack_supported.argtypes = [_int, _int, _int, _int, _int, _int]
+_lib.cherryq_prepack_supported.restype = _int
+_lib.cherryq_prepack_f16.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _sz, _int, _int, _int, _int, _vp]
+_lib.cherryq_prepack_f16.restype = _int
+_lib.cherryq_unprepack_f16.argtypes = [_int, _vp, _sz, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp]
+_lib.cherryq_unprepack_f16.restype = _int
+_lib.cherryq_matvec_prepacked_f16.argtypes = [_int, _vp, _vp, _sz, _vp, _int, _int, _int, _int, _int, _vp]
+_lib.cherryq_matvec_prepacked_f16.restype = _int
 _lib.cherryq_workspace_bytes.argtypes = [_int, _int, _int, _int]
 _lib.cherryq_workspace_bytes.restype = _sz
 _lib.cherryq_scratch_bytes.argtypes = [_int, _int, _int, _int]
@@ -315,6 +325,82 @@ def pack_cherryq(w_bits, weight, cherry_indices, group_size):
     if rc != 0:
         _fail(rc, "pack_cherryq")
     return idx, cherry_weight, qweight, scales
+
+
+def prepack_supported(w_bits, batch, in_features, out_features, num_cherries, group_size) -> bool:
+    """Whether the load-time repacked path takes this call shape (batch 1, group size a multiple
+    of 128, at most 128 cherry channels and 16384 quantised input channels)."""
+    return bool(_lib.cherryq_prepack_supported(int(w_bits), int(batch), int(in_features), int(out_features),
+                                               int(num_cherries), int(group_size)))
+
+
+def prepack_cherryq(w_bits, qweight, cherry_weight, cherry_indices, scaling_factors, in_features, group_size):
+    """The packed buffers of one layer rearranged, once, into the weight stream the batch-1 matvec
+    of this GPU reads fastest (16 output columns' whole input range contiguous, codes placed
+    where one mask makes them matrix-core operands).  Same information bit for bit;
+    unprepack_cherryq is the exact inverse.  No counterpart in the reference extension."""
+    _check(qweight, "qweight", torch.uint8, 2)
+    dev = qweight.device
+    _check(cherry_weight, "cherry_weight", torch.float16, 2, dev)
+    _check(cherry_indices, "cherry_indices", torch.int16, 1, dev)
+    _check(scaling_factors, "scaling_factors", torch.float16, 2, dev)
+    k, n, c, g = int(in_features), qweight.shape[1], cherry_indices.shape[0], int(group_size)
+    kn = k - c
+    if qweight.shape[0] * 8 != kn * w_bits or tuple(cherry_weight.shape) != (c, n):
+        raise RuntimeError("prepack_cherryq: buffer shapes do not match in_features / w_bits")
+    if g <= 0 or tuple(scaling_factors.shape) != (-(-kn // g), n):
+        raise RuntimeError(f"scaling_factors shape {tuple(scaling_factors.shape)} does not match group_size={g}")
+    if not prepack_supported(w_bits, 1, k, n, c, g):
+        raise RuntimeError(f"prepack_cherryq: shape not taken (w_bits={w_bits}, in={k}, out={n}, cherries={c}, group={g})")
+    nbytes = _lib.cherryq_prepack_bytes(w_bits, k, n, c)
+    stream = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.cherryq_prepack_f16(w_bits, _ptr(qweight), _ptr(cherry_weight), _ptr(cherry_indices),
+                                      _ptr(scaling_factors), stream.data_ptr(), nbytes, k, n, c, g,
+                                      _current_stream(dev.index))
+    if rc != 0:
+        _fail(rc, "prepack_cherryq")
+    return stream
+
+
+def unprepack_cherryq(w_bits, stream, in_features, out_features, num_cherries, group_size):
+    """Inverse of prepack_cherryq: (cherry_indices, cherry_weight, qweight, scales), bit for bit
+    the buffers the stream was made from."""
+    _check(stream, "stream", torch.uint8, 1)
+    dev = stream.device
+    k, n, c, g = int(in_features), int(out_features), int(num_cherries), int(group_size)
+    kn = k - c
+    idx = torch.empty(c, dtype=torch.int16, device=dev)
+    cw = torch.empty((c, n), dtype=torch.float16, device=dev)
+    qweight = torch.empty((kn // 8 * w_bits, n), dtype=torch.uint8, device=dev)
+    scales = torch.empty((-(-kn // g), n), dtype=torch.float16, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.cherryq_unprepack_f16(w_bits, stream.data_ptr(), stream.numel(), _ptr(qweight), _ptr(cw), _ptr(idx),
+                                        _ptr(scales), k, n, c, g, _current_stream(dev.index))
+    if rc != 0:
+        _fail(rc, "unprepack_cherryq")
+    return idx, cw, qweight, scales
+
+
+def matvec_prepacked_cherryq(w_bits, vec, stream, out, in_features, num_cherries, accumulate=False):
+    """out (1, N) = (or +=) vec (1, K) @ W^T over a stream made by prepack_cherryq.  Result and
+    arithmetic contract are those of vecquant{3,4}matmul_cherryq at batch 1; no workspace, no
+    atomics."""
+    _check(vec, "vec", torch.float16, 2)
+    dev = vec.device
+    _check(stream, "stream", torch.uint8, 1, dev)
+    _check(out, "out", torch.float16, 2, dev)
+    batch, k = vec.shape
+    if k != int(in_features) or out.shape[0] != batch:
+        raise RuntimeError(f"matvec_prepacked_cherryq: vec {tuple(vec.shape)} / out {tuple(out.shape)} do not match")
+    if batch == 0:
+        return
+    with torch.cuda.device(dev):
+        rc = _lib.cherryq_matvec_prepacked_f16(w_bits, vec.data_ptr(), stream.data_ptr(), stream.numel(),
+                                               out.data_ptr(), batch, k, out.shape[1], int(num_cherries),
+                                               1 if accumulate else 0, _current_stream(dev.index))
+    if rc != 0:
+        _fail(rc, "matvec_prepacked_cherryq")
 
 
 FAKE_QUANT_MAX_IN_FEATURES = 65536

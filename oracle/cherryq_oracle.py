@@ -422,6 +422,126 @@ def synthetic_packed_fast(in_features, out_features, w_bits, group_size=128, see
     return {"cherry_indices": idx, "cherry_weight": cw, "qweight": qweight, "scales": scales}
 
 
+# --------------------------------------------------------------------------- weight stream
+# The load-time repack of include/cherryq.h (cherryq_prepack_f16) has no counterpart in the
+# reference: it is this build's own rearrangement of the reference buffers.  What pins it is
+# that it is a bijection of them: stream_unpack(stream_pack(p)) == p for every buffer, and the
+# device kernels must produce these very bytes.  Codes are read from `qweight` with unpack_codes
+# (llama/qlinear.py:120-150), positions are the compacted normal positions of
+# csrc/quant_cuda_kernel.cu:785-795.
+
+def _align256(v):
+    return (v + 255) & ~255
+
+
+def stream_geometry(w_bits, in_features, out_features, num_cherries):
+    kn = in_features - num_cherries
+    ng = -(-kn // 128)
+    cp = (num_cherries + 31) & ~31
+    off_cherry = _align256(ng * 32)
+    off_units = off_cherry + _align256(num_cherries * 32)
+    unit_bytes = 1024 if w_bits == 4 else 768
+    return dict(kn=kn, ng=ng, cp=cp, ntiles=-(-out_features // 16), off_cherry=off_cherry, off_units=off_units,
+                unit_bytes=unit_bytes, record_bytes=off_units + ng * unit_bytes,
+                knp512=(ng * 128 + 511) & ~511, hdr_bytes=_align256(((ng * 128 + 511) & ~511) + 2 * cp))
+
+
+def _stream_slot(w_bits):
+    """For code q (0..31) of a lane: (dword, bit) of its field, dword 3 = the two 3-bit codes
+    spread over bit 15 + 16 h of dwords 0..2."""
+    slots = []
+    for q in range(32):
+        if w_bits == 4:
+            j, r = q >> 3, q & 7
+            slots.append((2 * (j & 1) + (r >> 2), 4 * ([0, 4, 2, 6][r & 3] + (j >> 1))))
+        else:
+            h = q & 1
+            if q < 24:
+                r, m = q & 7, q >> 3
+                if r < 6:
+                    slots.append((r >> 1, 16 * h + 3 * m))
+                elif q < 16:
+                    slots.append((0, 16 * h + 3 * (m + 3)))
+                else:
+                    slots.append((3, 16 * h))
+            else:
+                slots.append((1 + ((q & 3) >> 1), 16 * h + 3 * (3 if q < 28 else 4)))
+    return slots
+
+
+def stream_pack(packed, w_bits, group_size, in_features):
+    """Reference buffers -> weight stream (uint8 array), as cherryq_prepack_f16 lays it out."""
+    qweight, scales = packed["qweight"], packed["scales"]
+    cw, idx = packed["cherry_weight"], packed["cherry_indices"].astype(np.int64)
+    n = qweight.shape[1]
+    c = idx.shape[0]
+    g = stream_geometry(w_bits, in_features, n, c)
+    kn, ng = g["kn"], g["ng"]
+    assert group_size % 128 == 0
+    out = np.zeros(g["hdr_bytes"] + g["ntiles"] * g["record_bytes"], dtype=np.uint8)
+    # header: low(k) per compacted position, lane-transposed per block of 512; then cherry columns
+    k = np.arange(g["knp512"])
+    low = np.where(k < kn, gather_offset(np.minimum(k, max(kn - 1, 0)), idx), c).astype(np.uint8)
+    blk, l, j = k >> 9, (k >> 3) & 63, k & 7           # stored index -> position blk*512 + 64 j + l
+    out[:g["knp512"]] = low[blk * 512 + 64 * j + l]
+    cidx = np.full(g["cp"], in_features, dtype=np.uint16)
+    cidx[:c] = idx
+    out[g["knp512"]:g["knp512"] + 2 * g["cp"]] = cidx.view(np.uint8)
+    codes = np.zeros((ng * 128, g["ntiles"] * 16), dtype=np.uint32)
+    codes[:kn, :n] = unpack_codes(qweight, w_bits)
+    sc = np.zeros((ng, g["ntiles"] * 16), dtype=np.float16)
+    sc[:, :n] = scales[(np.arange(ng) * 128) // group_size]
+    cwp = np.zeros((c, g["ntiles"] * 16), dtype=np.float16)
+    cwp[:, :n] = cw
+    slots = _stream_slot(w_bits)
+    dw = w_bits
+    # units: [tile][g][lane = kq*16 + nn][dword]
+    cu = codes.reshape(ng, 4, 32, g["ntiles"], 16)       # g, kq, q, tile, nn
+    words = np.zeros((g["ntiles"], ng, 4, 16, 4), dtype=np.uint32)
+    for q, (d, bit) in enumerate(slots):
+        v = cu[:, :, q].transpose(2, 0, 1, 3)             # tile, g, kq, nn
+        if d < 3 or w_bits == 4:
+            words[..., d] |= v << bit
+        else:
+            for b in range(3):
+                words[..., b] |= ((v >> b) & 1) << (bit + 15)
+    rec = out[g["hdr_bytes"]:].reshape(g["ntiles"], g["record_bytes"])
+    rec[:, :ng * 32] = sc.reshape(ng, g["ntiles"], 16).transpose(1, 0, 2).reshape(g["ntiles"], -1).view(np.uint8)
+    if c:
+        # piece (lg, nn): cherry rows 8 lg .. 8 lg + 7 of column nn
+        cp_ = cwp.reshape(c // 8, 8, g["ntiles"], 16).transpose(2, 0, 3, 1)   # tile, lg, nn, e
+        rec[:, g["off_cherry"]:g["off_cherry"] + c * 32] = np.ascontiguousarray(cp_).reshape(g["ntiles"], -1).view(np.uint8)
+    rec[:, g["off_units"]:] = np.ascontiguousarray(words[..., :dw]).reshape(g["ntiles"], -1).view(np.uint8)
+    return out
+
+
+def stream_unpack(stream, w_bits, group_size, in_features, out_features, num_cherries):
+    """Inverse of stream_pack: the reference buffers back, bit for bit."""
+    g = stream_geometry(w_bits, in_features, out_features, num_cherries)
+    kn, ng, n, c = g["kn"], g["ng"], out_features, num_cherries
+    cidx = stream[g["knp512"]:g["knp512"] + 2 * g["cp"]].view(np.uint16)[:c].astype(np.int16)
+    rec = stream[g["hdr_bytes"]:].reshape(g["ntiles"], g["record_bytes"])
+    sc = rec[:, :ng * 32].copy().view(np.float16).reshape(g["ntiles"], ng, 16).transpose(1, 0, 2).reshape(ng, -1)[:, :n]
+    ngr = -(-kn // group_size)
+    scales = sc[(np.arange(ngr) * group_size) // 128]
+    cw = np.zeros((c, n), dtype=np.float16)
+    if c:
+        cp_ = rec[:, g["off_cherry"]:g["off_cherry"] + c * 32].copy().view(np.float16).reshape(g["ntiles"], c // 8, 16, 8)
+        cw = cp_.transpose(1, 3, 0, 2).reshape(c, -1)[:, :n]
+    dw = w_bits
+    words = rec[:, g["off_units"]:].copy().view(np.uint32).reshape(g["ntiles"], ng, 4, 16, dw)
+    codes = np.zeros((ng, 4, 32, g["ntiles"], 16), dtype=np.uint8)
+    for q, (d, bit) in enumerate(_stream_slot(w_bits)):
+        if d < 3 or w_bits == 4:
+            v = (words[..., d] >> bit) & (2 ** w_bits - 1)
+        else:
+            v = sum((((words[..., b] >> (bit + 15)) & 1) << b) for b in range(3))
+        codes[:, :, q] = v.transpose(1, 2, 0, 3)
+    codes = codes.reshape(ng * 128, -1)[:kn, :n]
+    return {"cherry_indices": cidx, "cherry_weight": np.ascontiguousarray(cw), "qweight": pack_codes(codes, w_bits),
+            "scales": np.ascontiguousarray(scales)}
+
+
 def rel_l2(a, b) -> float:
     a = np.asarray(a, dtype=np.float64)
     b = np.asarray(b, dtype=np.float64)

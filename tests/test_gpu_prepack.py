@@ -1,0 +1,222 @@
+"""The load-time repacked weight stream (cherryq_prepack_f16 / cherryq_matvec_prepacked_f16) against
+the CPU oracle on identical REFERENCE-layout inputs (MI355X only).
+
+The repack is a bijection of the reference buffers: the device stream must equal the oracle's
+numpy statement of the layout byte for byte, and unprepack must give the buffers back.  The
+matvec over it meets the same bars as the kernels that read the checkpoint layout: rel-L2 <= 1e-3
+against the oracle's dequantise-and-matmul, one-hot activations read the dequantised weights
+back bit for bit.
+"""
+import ctypes
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cherryq_oracle as orc
+from oracle import c_oracle
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3
+NAMES = ("cherry_indices", "cherry_weight", "qweight", "scales")
+
+
+@pytest.fixture(scope="module")
+def qc():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    import quant_cuda
+    return quant_cuda
+
+
+def announce(*a):
+    print("[case]", *a, flush=True)
+    sys.stdout.flush()
+
+
+def dev(p):
+    return {k: torch.from_numpy(np.ascontiguousarray(v)).cuda() for k, v in p.items() if k in NAMES}
+
+
+def prepack(qc, bits, p, k, gs=128):
+    d = dev(p)
+    return qc.prepack_cherryq(bits, d["qweight"], d["cherry_weight"], d["cherry_indices"], d["scales"], k, gs)
+
+
+def run(qc, bits, stream, x, n, c, out=None, accumulate=False):
+    xt = torch.from_numpy(x).cuda()
+    o = torch.full((1, n), float("nan"), dtype=torch.float16, device="cuda") if out is None else torch.from_numpy(out).cuda()
+    qc.matvec_prepacked_cherryq(bits, xt, stream, o, x.shape[1], c, accumulate=accumulate)
+    torch.cuda.synchronize()
+    return o.cpu().numpy()
+
+
+# shapes: the headline layers, every launch geometry (units per column 32 / 40 / 64 / 86 / 108), ragged
+# last unit, N not a multiple of 16, no cherries at all, two cherry MFMA steps (C = 48)
+SHAPES = [(4, 4096, 11008), (3, 4096, 11008), (4, 11008, 4096), (3, 11008, 4096), (4, 4096, 4096), (3, 4096, 4096),
+          (3, 5120, 5120), (3, 5120, 13824), (3, 13824, 5120), (4, 8192, 8192), (4, 8192, 1024),
+          (4, 1024, 264), (3, 1024, 264), (4, 2304, 40), (3, 768, 24)]
+
+
+@pytest.mark.parametrize("bits,k,n", SHAPES)
+def test_stream_is_the_oracle_layout_and_unprepack_inverts_it(qc, bits, k, n):
+    announce("prepack", bits, k, n)
+    p = orc.synthetic_packed_fast(k, n, bits, 128, seed=k + n + bits)
+    c = p["cherry_indices"].shape[0]
+    stream = prepack(qc, bits, p, k)
+    torch.cuda.synchronize()
+    want = orc.stream_pack(p, bits, 128, k)
+    np.testing.assert_array_equal(stream.cpu().numpy(), want)
+    back = qc.unprepack_cherryq(bits, stream, k, n, c, 128)
+    torch.cuda.synchronize()
+    for name, t in zip(NAMES, back):
+        np.testing.assert_array_equal(t.cpu().numpy(), p[name], err_msg=name)
+
+
+@pytest.mark.parametrize("bits,k,n", SHAPES)
+def test_prepacked_matvec_against_oracle(qc, bits, k, n):
+    announce("prepacked matvec", bits, k, n)
+    small = k * n <= 4096 * 4096
+    if small:
+        _, p = orc.synthetic_layer(k, n, bits, 128, seed=k + n + bits)
+    else:
+        p = orc.synthetic_packed_fast(k, n, bits, 128, seed=k + n + bits)
+    c = p["cherry_indices"].shape[0]
+    x = np.random.default_rng(7).standard_normal((1, k)).astype(np.float16)
+    y = run(qc, bits, prepack(qc, bits, p, k), x, n, c)
+    assert np.isfinite(y).all()
+    y_fused = c_oracle.fused(x, p, bits, 128)
+    e = orc.rel_l2(y, y_fused)
+    print(f"  rel-L2 vs the un-rounded contract {e:.2e}")
+    assert e <= TOL
+    if small:
+        dense = c_oracle.unpack(p, bits, 128, k)
+        assert orc.rel_l2(y, c_oracle.linear(x, dense, want_f64=True)[1]) <= TOL
+    ulp_ok = np.abs(y.astype(np.float64) - y_fused) <= np.abs(y_fused) * 2 ** -10 + 1e-3
+    assert ulp_ok.mean() > 0.999
+
+
+@pytest.mark.parametrize("bits,k,n", [(4, 4096, 4096), (3, 4096, 4096), (4, 11008, 512), (3, 11008, 512),
+                                      (3, 5120, 520), (4, 8192, 264), (3, 13824, 264)])
+def test_prepacked_one_hot_reads_back_dequantised_weights(qc, bits, k, n):
+    """x = e_j returns column j of the dense weight: decode, gather around the cherry channels and
+    the per-unit grid offset are exact.  Positions probe every code slot of a lane's 32 and both
+    ends of units, blocks of 512 and the ragged last unit."""
+    announce("prepacked one-hot", bits, k, n)
+    _, p = orc.synthetic_layer(k, n, bits, 128, seed=5)
+    c = p["cherry_indices"].shape[0]
+    stream = prepack(qc, bits, p, k)
+    dense = c_oracle.unpack(p, bits, 128, k)
+    idx = p["cherry_indices"].astype(np.int64)
+    nidx = orc.normal_indices(k, idx)
+    kn = len(nidx)
+    probes = sorted(set([int(nidx[q]) for q in list(range(0, 34)) + [63, 64, 127, 128, 511, 512, 513, kn - 1, kn - 2,
+                                                                     kn - 113, kn // 2 + 3, (kn // 128) * 128 - 1,
+                                                                     min(kn - 1, (kn // 128) * 128)]]
+                        + [int(idx[0]), int(idx[-1]), int(idx[len(idx) // 2])]))
+    for j in probes:
+        x = np.zeros((1, k), dtype=np.float16)
+        x[0, j] = 1
+        y = run(qc, bits, stream, x, n, c)
+        np.testing.assert_array_equal(y[0], dense[:, j], err_msg=f"column {j}")
+    # a single small activation: the exact product rounded once (into the subnormal range)
+    x = np.zeros((1, k), dtype=np.float16)
+    x[0, probes[5]] = np.float16(2 ** -9)
+    y = run(qc, bits, stream, x, n, c)
+    np.testing.assert_array_equal(y[0], c_oracle.fused(x, p, bits, 128)[0].astype(np.float16))
+
+
+def test_prepacked_matches_reference_layout_kernel_accumulate_and_group_256(qc):
+    """Same inputs through both paths agree to the last fp16 bit almost everywhere (both round one
+    fp32 sum); accumulate adds into `out`; a group size of 256 is two units per scale row."""
+    bits, k, n = 4, 4096, 1024
+    _, p = orc.synthetic_layer(k, n, bits, 256, seed=9)
+    c = p["cherry_indices"].shape[0]
+    d = dev(p)
+    x = np.random.default_rng(3).standard_normal((1, k)).astype(np.float16)
+    stream = qc.prepack_cherryq(bits, d["qweight"], d["cherry_weight"], d["cherry_indices"], d["scales"], k, 256)
+    back = qc.unprepack_cherryq(bits, stream, k, n, c, 256)
+    np.testing.assert_array_equal(back[3].cpu().numpy(), p["scales"])
+    y = run(qc, bits, stream, x, n, c)
+    ref = torch.zeros(1, n, dtype=torch.float16, device="cuda")
+    qc.matmul_cherryq(bits, torch.from_numpy(x).cuda(), d["qweight"], d["cherry_weight"], d["cherry_indices"],
+                      d["scales"], ref, 256, accumulate=False)
+    torch.cuda.synchronize()
+    r = ref.cpu().numpy()
+    assert (y == r).mean() > 0.9 and orc.rel_l2(y, r) < 3e-4  # different summation orders: the last bit may differ
+    assert orc.rel_l2(y, c_oracle.fused(x, p, bits, 256)) <= TOL
+    base = np.random.default_rng(4).standard_normal((1, n)).astype(np.float16)
+    y2 = run(qc, bits, stream, x, n, c, out=base.copy(), accumulate=True)
+    want = (c_oracle.fused(x, p, bits, 256) + base.astype(np.float64)).astype(np.float16)
+    assert orc.rel_l2(y2, want) <= TOL
+    # run-to-run identical (no atomics anywhere in this path)
+    np.testing.assert_array_equal(run(qc, bits, stream, x, n, c), y)
+
+
+def test_prepacked_linearity_at_full_size(qc):
+    """4096 -> 11008, both bit widths: f(2 x) == 2 f(x) exactly (powers of two commute with every
+    rounding involved) and a column sample against the C oracle."""
+    for bits in (4, 3):
+        k, n = 4096, 11008
+        p = orc.synthetic_packed_fast(k, n, bits, 128, seed=3)
+        c = p["cherry_indices"].shape[0]
+        stream = prepack(qc, bits, p, k)
+        rng = np.random.default_rng(11)
+        x1 = rng.standard_normal((1, k)).astype(np.float16)
+        y1 = run(qc, bits, stream, x1, n, c)
+        y2 = run(qc, bits, stream, (x1 * np.float16(2)).astype(np.float16), n, c)
+        np.testing.assert_array_equal(y2, (y1.astype(np.float32) * 2).astype(np.float16))
+
+
+def test_quantlinear_prepack_forward_and_release(qc):
+    from llama.qlinear import QuantLinear
+    from llama.quantizer import FullSymQuantizer
+    for bits in (4, 3):
+        k, n = 4096, 1024
+        _, p = orc.synthetic_layer(k, n, bits, 128, seed=21 + bits)
+        m = QuantLinear(bits, 128, FullSymQuantizer, 1 / 256, k, n, bias=False)
+        for name in NAMES:
+            setattr(m, name, torch.from_numpy(p[name]))
+        m = m.cuda()
+        x = torch.from_numpy(np.random.default_rng(5).standard_normal((1, 1, k)).astype(np.float16)).cuda()
+        y0 = m(x)
+        assert m.prepack()
+        y1 = m(x)
+        want = c_oracle.fused(x.reshape(1, k).cpu().numpy(), p, bits, 128)
+        assert orc.rel_l2(y1.reshape(1, n).cpu().numpy(), want) <= TOL
+        assert orc.rel_l2(y1.cpu().numpy(), y0.cpu().numpy()) < 3e-4
+        # other batch sizes keep using the checkpoint-layout kernels
+        xb = torch.from_numpy(np.random.default_rng(6).standard_normal((3, k)).astype(np.float16)).cuda()
+        assert m(xb).shape == (3, n)
+        # release the checkpoint-layout buffers, then bring them back bit for bit
+        assert m.prepack(release_reference=True)
+        assert m.qweight.numel() == 0
+        y2 = m(x)
+        assert torch.equal(y1, y2)
+        with pytest.raises(RuntimeError):
+            m(xb)
+        m.unprepack()
+        for name in NAMES:
+            np.testing.assert_array_equal(getattr(m, name).cpu().numpy(), p[name], err_msg=name)
+        assert m(xb).shape == (3, n)
+
+
+def test_prepacked_c_abi_rejections(qc):
+    lib = qc._lib
+    assert lib.cherryq_prepack_bytes(5, 4096, 4096, 16) == 0
+    assert lib.cherryq_prepack_supported(4, 2, 4096, 4096, 16, 128) == 0      # batch 1 only
+    assert lib.cherryq_prepack_supported(4, 1, 4096, 4096, 16, 64) == 0       # group size a multiple of 128
+    assert lib.cherryq_prepack_supported(4, 1, 28672, 8192, 112, 128) == 0    # more than 16384 quantised channels
+    assert lib.cherryq_prepack_supported(3, 1, 13824, 5120, 48, 128) == 1
+    nbytes = lib.cherryq_prepack_bytes(4, 4096, 1024, 16)
+    buf = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    x = torch.zeros(1, 4096, dtype=torch.float16, device="cuda")
+    y = torch.zeros(1, 1024, dtype=torch.float16, device="cuda")
+    f = lib.cherryq_matvec_prepacked_f16
+    assert f(4, x.data_ptr(), buf.data_ptr(), nbytes - 1, y.data_ptr(), 1, 4096, 1024, 16, 0, None) == -4
+    assert f(4, x.data_ptr(), buf.data_ptr(), nbytes, y.data_ptr(), 2, 4096, 1024, 16, 0, None) == -7
+    assert f(4, x.data_ptr(), buf.data_ptr(), nbytes, y.data_ptr(), 0, 4096, 1024, 16, 0, None) == 0
+    assert f(4, None, buf.data_ptr(), nbytes, y.data_ptr(), 1, 4096, 1024, 16, 0, None) == -1
+    assert f(4, x.data_ptr() + 2, buf.data_ptr(), nbytes, y.data_ptr(), 1, 4096, 1024, 16, 0, None) == -6
+    assert f(2, x.data_ptr(), buf.data_ptr(), nbytes, y.data_ptr(), 1, 4096, 1024, 16, 0, None) == -5
