@@ -47,7 +47,8 @@ WORKLOADS = {
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, each
 # counter scaled by its reading for a 256 MiB device copy (x2.000 and x1.000); the counters
 # cannot be read while timing, so the figure is recorded here for the workloads measured.
-MEASURED_TRAFFIC = {("llama7b_gate_up_w4", 1): 25320960}
+MEASURED_TRAFFIC = {("llama7b_gate_up_w4", 1, "reference"): 25320960,
+                    ("llama7b_gate_up_w4", 1, "prepacked"): 23887460}
 
 
 def algorithmic_bytes(bits, k, n, batch=1, group=128):
@@ -85,24 +86,73 @@ def make_copies(bits, k, n, group, min_bytes, seed=0):
     return base, copies
 
 
-def time_gpu(bits, k, n, group, steps, warmup, batch=1, use_graph=True):
+def _replays(steps):
+    """How many times the K-step sequence is repeated INSIDE the captured graph: enough that a short
+    run (the driver's --steps 20) is timed over about 2000 back-to-back launches, like a long one.
+    (Replaying a 20-launch graph 100 times instead read 0.5 us per launch higher: every replay
+    boundary costs about 10 us of launch latency that a serving loop's long graph does not pay.)"""
+    return max(1, -(-2000 // max(1, steps)))
+
+
+TIMED_REPLAYS = 5
+
+
+def _time_graph(stream, build, steps):
+    """Capture steps * _replays(steps) launches (build(i) enqueues launch i) into ONE HIP graph,
+    replay it TIMED_REPLAYS times with a HIP event before and after each replay (recorded on the
+    launch stream) and return the MEDIAN replay's microseconds per launch.  One untimed replay first."""
+    import torch
+    total = steps * _replays(steps)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        for i in range(total):
+            build(i)
+    graph.replay()
+    stream.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(TIMED_REPLAYS + 1)]
+    ev[0].record(stream)
+    for j in range(TIMED_REPLAYS):
+        graph.replay()
+        ev[j + 1].record(stream)
+    stream.synchronize()
+    per = sorted(ev[j].elapsed_time(ev[j + 1]) * 1e3 / total for j in range(TIMED_REPLAYS))
+    return per[len(per) // 2]
+
+
+def time_gpu(bits, k, n, group, steps, warmup, batch=1, use_graph=True, path="auto"):
     """Device time per fused call.  The `steps` launches (each on a different copy of the packed
     layer) are captured once into a HIP graph and replayed, so the figure is the GPU's launch-to-
-    launch time and not the Python binding's; HIP events bracket the replay on the launch stream.
-    Returns (device us per call, eager host wall us per call, ...)."""
+    launch time and not the Python binding's; HIP events bracket every replay on the launch stream.
+    path: "reference" = the kernels that read the checkpoint layout, "prepacked" = the load-time
+    repacked weight stream (batch 1), "auto" = what a loader gets: prepacked where the library
+    recommends it for the shape (quant_cuda.prepack_recommended).
+    Returns a dict (us, path, eager host wall us, cache-resident us, first copy as numpy, ...)."""
     import numpy as np
     import torch
     import quant_cuda
     base, copies = make_copies(bits, k, n, group, 640 << 20)
+    c = copies[0]["cherry_indices"].numel()
+    if path == "auto":
+        path = "prepacked" if batch == 1 and quant_cuda.prepack_recommended(bits, k, n, c, group) else "reference"
     x = torch.from_numpy(np.random.default_rng(1).standard_normal((batch, k)).astype(np.float16)).cuda()
     out = torch.zeros(batch, n, dtype=torch.float16, device="cuda")
+    if path == "prepacked":
+        for t in copies:
+            t["stream"] = quant_cuda.prepack_cherryq(bits, t["qweight"], t["cherry_weight"], t["cherry_indices"],
+                                                     t["scales"], k, group)
+            del t["qweight"]  # the 29 reference-layout copies are not needed any more
+        torch.cuda.empty_cache()
 
     def step(i):
         t = copies[i % len(copies)]
-        quant_cuda.matmul_cherryq(bits, x, t["qweight"], t["cherry_weight"], t["cherry_indices"], t["scales"], out,
-                                  group, accumulate=False)
+        if path == "prepacked":
+            quant_cuda.matvec_prepacked_cherryq(bits, x, t["stream"], out, k, c)
+        else:
+            quant_cuda.matmul_cherryq(bits, x, t["qweight"], t["cherry_weight"], t["cherry_indices"], t["scales"], out,
+                                      group, accumulate=False)
 
     stream = torch.cuda.Stream()
+    res = {"path": path, "base": base, "x": x, "out": out, "copies": copies, "resident_us": None}
     with torch.cuda.stream(stream):
         # eager: untimed warm-up, then the host-inclusive rate
         for i in range(warmup):
@@ -112,87 +162,67 @@ def time_gpu(bits, k, n, group, steps, warmup, batch=1, use_graph=True):
         for i in range(min(steps, 500)):
             step(warmup + i)
         stream.synchronize()
-        wall_us = (time.perf_counter() - t0) * 1e6 / min(steps, 500)
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        res["wall_us"] = (time.perf_counter() - t0) * 1e6 / min(steps, 500)
         if use_graph:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=stream):
-                for i in range(steps):
-                    step(warmup + i)
-            graph.replay()  # untimed replay: graph upload, first-touch effects
-            stream.synchronize()
-            e0.record(stream)
-            graph.replay()
-            e1.record(stream)
+            res["us"] = _time_graph(stream, lambda i: step(warmup + i), steps)
+            # the same launches on ONE copy: the packed layer then comes from the Infinity Cache
+            # (reported beside the HBM figure, labelled; it is never the headline value)
+            res["resident_us"] = _time_graph(stream, lambda i: step(0), steps)
         else:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(stream)
             for i in range(steps):
                 step(warmup + i)
             e1.record(stream)
-        stream.synchronize()
-        dev_us = e0.elapsed_time(e1) * 1e3 / steps
-        # the same launches on ONE copy: the packed layer then comes from the Infinity Cache
-        # (reported beside the HBM figure, labelled; it is never the headline value)
-        resident_us = None
-        if use_graph:
-            rgraph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(rgraph, stream=stream):
-                for i in range(steps):
-                    step(0)
-            rgraph.replay()
             stream.synchronize()
-            e0.record(stream)
-            rgraph.replay()
-            e1.record(stream)
-            stream.synchronize()
-            resident_us = e0.elapsed_time(e1) * 1e3 / steps
-    return dev_us, wall_us, base, x, out, copies, resident_us
+            res["us"] = e0.elapsed_time(e1) * 1e3 / steps
+    return res
 
 
-def roofline_reference(copies, steps):
-    """What the GPU does with the same packed bytes when a kernel only reads them (the library's
-    stream-read probe over each copy's qweight, same rotation, same graph replay), and the cost
-    of an empty launch.  Puts the fused kernel's time in proportion."""
+def roofline_reference(nbytes, steps):
+    """What the GPU does with the same number of bytes when a kernel only reads them, and what an
+    empty launch costs (libcherryq_probe.so, a bench-only library): the plain read is swept over
+    8 / 16 / 32 / 64 KB per workgroup and the read-once / default cache policy, same rotation over
+    > 512 MB, same graph replays; the fastest is reported.  Puts the fused kernel's time in proportion."""
     import ctypes
     import torch
-    import quant_cuda
-    lib = quant_cuda._lib
-    lib.cherryq_probe_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p]
+    lib = ctypes.CDLL(str(ROOT / "mixed-precision-cuda-kernel_amd" / "libcherryq_probe.so"))
+    lib.cherryq_probe_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int,
+                                              ctypes.c_int, ctypes.c_void_p]
     lib.cherryq_probe_empty_launch.argtypes = [ctypes.c_void_p]
     sink = torch.zeros(4, dtype=torch.int32, device="cuda")
-    nbytes = copies[0]["qweight"].numel()
+    per = (nbytes + 4095) // 4096 * 4096
+    ncopies = max(2, -(-(640 << 20) // per))
+    buf = torch.randint(0, 256, (per * ncopies,), dtype=torch.uint8, device="cuda")
     stream = torch.cuda.Stream()
-    out = {}
+    sweep = {}
     with torch.cuda.stream(stream):
-        for name in ("plain_read", "empty_launch"):
-            def step(i):
-                if name == "plain_read":
-                    rc = lib.cherryq_probe_stream_read(copies[i % len(copies)]["qweight"].data_ptr(), nbytes,
-                                                       sink.data_ptr(), stream.cuda_stream)
-                else:
-                    rc = lib.cherryq_probe_empty_launch(stream.cuda_stream)
-                assert rc == 0, rc
+        def timed(fn):
             for i in range(20):
-                step(i)
+                fn(i)
             stream.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=stream):
-                for i in range(steps):
-                    step(i)
-            graph.replay()
-            stream.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            graph.replay()
-            e1.record(stream)
-            stream.synchronize()
-            out[name] = e0.elapsed_time(e1) * 1e3 / steps
-    return {"plain_read_us": round(out["plain_read"], 3), "plain_read_bytes": nbytes,
-            "plain_read_gbs": round(nbytes / out["plain_read"] / 1e3, 1),
-            "empty_launch_us": round(out["empty_launch"], 3)}
+            return _time_graph(stream, fn, steps)
+
+        for kb in (8, 16, 32, 64):
+            for nt in (1, 0):
+                def read(i, kb=kb, nt=nt):
+                    rc = lib.cherryq_probe_stream_read(buf.data_ptr() + (i % ncopies) * per, nbytes, sink.data_ptr(), kb, nt,
+                                                       stream.cuda_stream)
+                    assert rc == 0, rc
+                sweep[f"{kb}KB{'_nt' if nt else ''}"] = round(timed(read), 3)
+
+        def empty(i):
+            assert lib.cherryq_probe_empty_launch(stream.cuda_stream) == 0
+        empty_us = timed(empty)
+    best = min(sweep, key=sweep.get)
+    del buf
+    torch.cuda.empty_cache()
+    return {"plain_read_us": sweep[best], "plain_read_shape": best, "plain_read_bytes": nbytes,
+            "plain_read_gbs": round(nbytes / sweep[best] / 1e3, 1), "plain_read_sweep_us": sweep,
+            "empty_launch_us": round(empty_us, 3)}
 
 
-def cpu_baseline(bits, k, n, group, base, x_np):
+def cpu_baseline(bits, k, n, group, base, x_np, seconds=8.0):
     """The reference CPU path -- QuantLinear.unpack() then linear -- restated in C (oracle),
     timed on this host: cold = unpack + matvec, cached = matvec on the dense fp16 weight."""
     import numpy as np
@@ -201,8 +231,8 @@ def cpu_baseline(bits, k, n, group, base, x_np):
     dense = np.zeros((n, k), dtype=np.float16)
     c_oracle.dequant_matmul(x_np, base, bits, group, dense)  # warm-up
     reps, cold = 0, []
-    t_end = time.perf_counter() + 8.0
-    while reps < 3 or time.perf_counter() < t_end:  # about 8 s of wall time on all host threads
+    t_end = time.perf_counter() + seconds
+    while reps < 3 or time.perf_counter() < t_end:  # a bounded sample: `seconds` of wall time on all host threads
         t0 = time.perf_counter()
         c_oracle.dequant_matmul(x_np, base, bits, group, dense)
         cold.append(time.perf_counter() - t0)
@@ -337,8 +367,8 @@ def main():
                         ("llama13b_down_w3", 8), ("llama70b_attn_w4", 16), ("llama70b_kv_w4", 16),
                         ("llama70b_gate_up_w4", 16), ("llama70b_down_w4", 16), ("llama7b_gate_up_w4", 16)):
             bits, k, n = WORKLOADS[name]
-            us, wall_us, *_ = time_gpu(bits, k, n, args.group, max(200, args.steps // 4), args.warmup, batch=b,
-                                      use_graph=not args.no_graph)
+            us = time_gpu(bits, k, n, args.group, max(200, args.steps // 4), args.warmup, batch=b,
+                          use_graph=not args.no_graph)["us"]
             ab = algorithmic_bytes(bits, k, n, b, args.group)
             fl = 2.0 * b * k * n
             print(f"{name:24s} {bits}-bit {k:5d}->{n:5d} batch {b:2d}: {us:7.2f} us  {ab / us / 1e3:7.1f} GB/s "
@@ -351,7 +381,7 @@ def main():
                         ("llama7b_gate_up_w3", 128), ("llama7b_down_w4", 128), ("llama7b_gate_up_w4", 512),
                         ("llama7b_gate_up_w4", 2048), ("llama70b_gate_up_w4", 128), ("llama70b_down_w4", 128)):
             bits, k, n = WORKLOADS[name]
-            us, wall_us, *_ = time_gpu(bits, k, n, args.group, 100, 10, batch=b, use_graph=not args.no_graph)
+            us = time_gpu(bits, k, n, args.group, 100, 10, batch=b, use_graph=not args.no_graph)["us"]
             ab = algorithmic_bytes(bits, k, n, b, args.group)
             fl = 2.0 * b * k * n
             print(f"{name:24s} {bits}-bit {k:5d}->{n:5d} rows {b:4d}: {us:7.2f} us  {fl / us / 1e6:6.1f} TFLOP/s "
@@ -392,21 +422,62 @@ def main():
                 torch.cuda.empty_cache()
         unpack_table(args.group)
         for name, (bits, k, n) in WORKLOADS.items():
-            us, wall_us, *_ = time_gpu(bits, k, n, args.group, max(200, args.steps // 4), args.warmup,
-                                      use_graph=not args.no_graph)
             ab = algorithmic_bytes(bits, k, n, 1, args.group)
-            print(f"{name:24s} {bits}-bit {k:5d}->{n:5d}: {us:7.2f} us/matvec  {ab / us / 1e3:7.1f} GB/s  "
-                  f"{ab / us / 1e3 / HBM_PEAK_GBS * 100:5.1f}% of 8 TB/s  (eager host wall {wall_us:.2f} us)",
-                  file=sys.stderr, flush=True)
+            line = f"{name:24s} {bits}-bit {k:5d}->{n:5d}:"
+            for path in ("reference", "prepacked"):
+                if path == "prepacked" and not quant_cuda.prepack_supported(bits, 1, k, n, -(-k // 256) // 8 * 8, args.group):
+                    line += "  prepacked: shape not taken"
+                    continue
+                r = time_gpu(bits, k, n, args.group, max(200, args.steps // 4), args.warmup, use_graph=not args.no_graph,
+                             path=path)
+                line += (f"  {path} {r['us']:6.2f} us {ab / r['us'] / 1e3:6.0f} GB/s "
+                         f"{ab / r['us'] / 1e3 / HBM_PEAK_GBS * 100:4.1f}%")
+                del r
+                torch.cuda.empty_cache()
+            print(line, file=sys.stderr, flush=True)
+
+    def kernel_name(bits, batch, path):
+        if path == "prepacked":
+            return f"cq::stream_kernel<{bits}>"
+        if batch == 1:
+            return f"cq::matvec_kernel<{bits}>"
+        if batch <= 4:
+            return f"cq::matvec_kernel<{bits}, rows {2 if batch == 2 else 4}>"
+        if batch <= 16:
+            return f"cq::batch_prep_kernel<{bits}> + cq::batch_kernel<{bits}>"
+        return f"cq::gemm_prep_kernel<{bits}> + cq::gemm_kernel<{bits}, {32 if batch <= 32 else 64 if batch <= 64 else 128}>"
+
+    def side_record(name, with_cpu=False):
+        """One more layer in the same JSON line: both paths' device time, achieved bandwidth of the faster."""
+        b_, k_, n_ = WORKLOADS[name]
+        ab_ = algorithmic_bytes(b_, k_, n_, 1, args.group)
+        rec = {"workload": name, "w_bits": b_, "in_features": k_, "out_features": n_, "algorithmic_bytes_per_launch": ab_}
+        best = None
+        for path in ("reference", "prepacked"):
+            import quant_cuda
+            if path == "prepacked" and not quant_cuda.prepack_supported(b_, 1, k_, n_, -(-k_ // 256) // 8 * 8, args.group):
+                continue
+            r = time_gpu(b_, k_, n_, args.group, args.steps, args.warmup, use_graph=not args.no_graph, path=path)
+            rec[f"{path}_us"] = round(r["us"], 3)
+            if best is None or r["us"] < best[0]:
+                best = (r["us"], path)
+            if with_cpu and path == "reference" and not args.no_cpu:
+                rec["cpu_baseline"] = cpu_baseline(b_, k_, n_, args.group, r["base"], r["x"].cpu().numpy(), seconds=4.0)
+            del r
             torch.cuda.empty_cache()
+        rec.update({"us": round(best[0], 3), "path": best[1], "kernel": kernel_name(b_, 1, best[1]),
+                    "achieved": round(ab_ / best[0] / 1e3, 1), "unit": "GB/s", "peak": HBM_PEAK_GBS,
+                    "frac": round(ab_ / best[0] / 1e3 / HBM_PEAK_GBS, 4)})
+        return rec
 
     bits, k, n = WORKLOADS[args.workload]
-    us, wall_us, base, x, out, copies, resident_us = time_gpu(bits, k, n, args.group, args.steps, args.warmup, batch=args.batch,
-                                                use_graph=not args.no_graph)
+    main_run = time_gpu(bits, k, n, args.group, args.steps, args.warmup, batch=args.batch, use_graph=not args.no_graph)
+    us, path = main_run["us"], main_run["path"]
     ab = algorithmic_bytes(bits, k, n, args.batch, args.group)
     gbs = ab / us / 1e3
-    x_host = x.cpu().numpy()
-    n_copies = len(copies)
+    x_host = main_run["x"].cpu().numpy()
+    base = main_run["base"]
+    traffic = MEASURED_TRAFFIC.get((args.workload, args.batch, path))
     result = {
         "metric": "us_per_matvec", "value": round(us, 3), "unit": "us", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us / 1e3, 6),
@@ -414,26 +485,43 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "w_bits": bits, "in_features": k, "out_features": n,
                    "group_size": args.group, "batch": args.batch, "cherries": -(-k // 256) // 8 * 8,
-                   "weight_copies_rotated": n_copies,
+                   "weight_copies_rotated": len(main_run["copies"]),
+                   "path": path + (" (weight stream repacked once at load time from the reference buffers)"
+                                   if path == "prepacked" else " (kernels that read the checkpoint layout)"),
                    "launch": "eager" if args.no_graph else "hip_graph_replay",
-                   "eager_host_wall_us_per_call": round(wall_us, 2)},
+                   "replays": None if args.no_graph else _replays(args.steps),
+                   "timing": ("one HIP graph of steps x replays launches; median over %d timed graph launches of "
+                              "(HIP-event time / launches)" % TIMED_REPLAYS),
+                   "eager_host_wall_us_per_call": round(main_run["wall_us"], 2)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC.get((args.workload, args.batch)),
+                     "traffic": traffic,
+                     "traffic_source": ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this workload and kernel, recorded in "
+                                        "bench.py (profiles/); not re-measured in this run") if traffic else
+                                       "not measured for this workload / kernel",
                      "algorithmic_bytes_per_launch": ab,
-                     "kernel": f"cq::matvec_kernel<{bits}>" if args.batch == 1 else
-                               f"cq::matvec_kernel<{bits}, rows {2 if args.batch == 2 else 4}>" if args.batch <= 4 else
-                               f"cq::batch_prep_kernel<{bits}> + cq::batch_kernel<{bits}>" if args.batch <= 16 else
-                               f"cq::gemm_prep_kernel<{bits}> + cq::gemm_kernel<{bits}, {32 if args.batch <= 32 else 64 if args.batch <= 64 else 128}>"},
+                     "kernel": kernel_name(bits, args.batch, path)},
     }
-    if resident_us is not None:
-        result["roofline"]["cache_resident"] = {"us": round(resident_us, 3), "gbs": round(ab / resident_us / 1e3, 1),
+    if main_run["resident_us"] is not None:
+        ru = main_run["resident_us"]
+        result["roofline"]["cache_resident"] = {"us": round(ru, 3), "gbs": round(ab / ru / 1e3, 1),
                                                 "note": "one weight copy replayed: served by the Infinity Cache, not HBM"}
-    if args.batch == 1:
-        result["roofline"]["reference"] = roofline_reference(copies, args.steps)
+    del main_run
+    torch.cuda.empty_cache()
+    if args.batch == 1 and not args.no_graph:
+        if path == "prepacked":
+            other = time_gpu(bits, k, n, args.group, args.steps, args.warmup, use_graph=True, path="reference")
+            result["config"]["reference_layout_us"] = round(other["us"], 3)
+            result["config"]["reference_layout_kernel"] = kernel_name(bits, 1, "reference")
+            del other
+            torch.cuda.empty_cache()
+        result["roofline"]["reference"] = roofline_reference(ab, args.steps)
+        if args.workload == "llama7b_gate_up_w4":
+            # the other half of the headline metric (3-bit, same layer) and config 0 (4096 -> 4096,
+            # 4-bit, with the reference's CPU path on that layer)
+            result["roofline_w3"] = side_record("llama7b_gate_up_w3")
+            result["config0"] = side_record("llama7b_attn_w4", with_cpu=True)
     if not args.no_decode:
-        del copies, x, out
-        torch.cuda.empty_cache()
         result["decode"] = decode_benchmark()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(bits, k, n, args.group, base, x_host)

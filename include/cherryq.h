@@ -138,24 +138,6 @@ int cherryq_unpack_f16(int w_bits, const uint8_t *qweight, const void *cherry_we
                        void *stream);
 
 /*
- * Decode-step glue for a LLaMA-shaped decoder, batch 1, fp16: what sits between two fused
- * matvecs in the caller's token step (llama/modeling_llama_quant.py of the reference: RMSNorm
- * :75-89, rotary embedding :179-210, attention over the KV cache :391-402 and :671-696, gated
- * MLP :251), one launch each, so that the step can be captured as a short HIP graph.  They have
- * no counterpart in the reference's extension, which leaves these operations to PyTorch.
- * `position` is a device pointer to the current token position (so a captured graph can be
- * replayed while the caller increments it); caches are [kv_head][max_len][head_dim].
- */
-/*
- * Roofline reference launches for measurement scripts; no counterpart in the reference and no
- * part in the product path.  cherryq_probe_stream_read reads `bytes` (< 2 GiB) of `buf` once with
- * the access shape of the weight stream and nothing else (sink: 4 writable bytes, never written
- * in practice); cherryq_probe_empty_launch launches an empty kernel.
- */
-int cherryq_probe_stream_read(const void *buf, size_t bytes, void *sink, void *stream);
-int cherryq_probe_empty_launch(void *stream);
-
-/*
  * pack() on the device: dense fp16 `weight` (out_features, in_features), row-major, and the
  * ASCENDING cherry channels -> qweight, scales (ceil(Kn/group_size), out_features) and
  * cherry_weight (num_cherries, out_features), bit for bit what QuantLinear.pack() computes on
@@ -208,6 +190,10 @@ int cherryq_fake_quant_f32(int w_bits, const void *weight, const int32_t *cherry
 size_t cherryq_prepack_bytes(int w_bits, int in_features, int out_features, int num_cherries);
 int cherryq_prepack_supported(int w_bits, int batch, int in_features, int out_features, int num_cherries,
                               int group_size);
+/* 1 where the matvec over the stream measured faster on MI355X than the one over the checkpoint
+ * layout (today: layers of at most 4096 non-cherry input channels), 0 elsewhere or if unsupported:
+ * what a loader asks before spending the extra copy of the weights. */
+int cherryq_prepack_recommended(int w_bits, int in_features, int out_features, int num_cherries, int group_size);
 int cherryq_prepack_f16(int w_bits, const uint8_t *qweight, const void *cherry_weight, const int16_t *cherry_indices,
                         const void *scales, void *stream, size_t stream_bytes, int in_features, int out_features,
                         int num_cherries, int group_size, void *hip_stream);
@@ -248,6 +234,15 @@ int cherryq_decode_matvec_group_f16(int w_bits, const void *vec, const void *vec
                                     int num_cherries, int group_size, int accumulate, void *workspace,
                                     size_t workspace_bytes, void *stream);
 
+/*
+ * Decode-step glue for a LLaMA-shaped decoder, batch 1, fp16: what sits between two fused
+ * matvecs in the caller's token step (llama/modeling_llama_quant.py of the reference: RMSNorm
+ * :75-89, rotary embedding :179-210, attention over the KV cache :391-402 and :671-696, gated
+ * MLP :251), one launch each, so that the step can be captured as a short HIP graph.  They have
+ * no counterpart in the reference's extension, which leaves these operations to PyTorch.
+ * `position` is a device pointer to the current token position (so a captured graph can be
+ * replayed while the caller increments it); caches are [kv_head][max_len][head_dim].
+ */
 int cherryq_decode_add_rmsnorm_f16(void *hidden, const void *delta /* may be NULL */, const void *weight,
                                    void *normed, int hidden_size, float eps, void *stream);
 int cherryq_decode_rope_cache_f16(void *q, const void *k, const void *v, void *k_cache, void *v_cache,

@@ -17,7 +17,8 @@ HERE = Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
 OBJ = HERE / "build"
 LIB = HERE / "libcherryq.so"
-SOURCES = ["cq_api.hip", "cq_generic.hip", "cq_matvec.hip", "cq_stream.hip", "cq_batch.hip", "cq_gemm.hip", "cq_f32.hip", "cq_decode.hip", "cq_pack.hip", "cq_fakequant.hip", "cq_probe.hip"]
+PROBE_LIB = HERE / "libcherryq_probe.so"  # bench-only roofline reference kernels, not part of the product library
+SOURCES = ["cq_api.hip", "cq_generic.hip", "cq_matvec.hip", "cq_stream.hip", "cq_batch.hip", "cq_gemm.hip", "cq_f32.hip", "cq_decode.hip", "cq_pack.hip", "cq_fakequant.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
@@ -62,6 +63,10 @@ def build(force: bool = False, verbose: bool = False) -> Path:
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stdout + r.stderr)
+    cmd = [HIPCC, *FLAGS, "-shared", "-o", str(PROBE_LIB), str(CSRC / "cq_probe.hip")]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("probe library failed:\n" + r.stdout + r.stderr)
     return LIB
 
 

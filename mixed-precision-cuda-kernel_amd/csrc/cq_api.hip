@@ -228,7 +228,7 @@ int cherryq_unpack_f16(int w_bits, const uint8_t *qweight, const void *cherry_we
                                   reinterpret_cast<hipStream_t>(stream));
 }
 
-// ---- device-side pack, measurement probes ----------------------------------------------------
+// ---- device-side pack, fake quantisation ----------------------------------------------------
 
 int cherryq_pack_f16(int w_bits, const void *weight, const int16_t *cherry_indices, uint8_t *qweight, void *scales,
                      void *cherry_weight, int in_features, int out_features, int num_cherries, int group_size,
@@ -272,15 +272,6 @@ int cherryq_fake_quant_f32(int w_bits, const void *weight, const int32_t *cherry
                             group_size, ste, stream);
 }
 
-int cherryq_probe_stream_read(const void *buf, size_t bytes, void *sink, void *stream) {
-    if (!buf || !sink) return CHERRYQ_E_NULL;
-    if (bytes >= 0x7fff0000ull) return CHERRYQ_E_SHAPE;
-    if (!cq::aligned(buf, 16) || !cq::aligned(sink, 4)) return CHERRYQ_E_ALIGN;
-    return (int)cq::launch_probe_read(buf, bytes, sink, reinterpret_cast<hipStream_t>(stream));
-}
-
-int cherryq_probe_empty_launch(void *stream) { return (int)cq::launch_probe_empty(reinterpret_cast<hipStream_t>(stream)); }
-
 // ---- load-time repacked weight stream (see include/cherryq.h) -----------------------------------
 
 size_t cherryq_prepack_bytes(int w_bits, int in_features, int out_features, int num_cherries) {
@@ -293,6 +284,11 @@ size_t cherryq_prepack_bytes(int w_bits, int in_features, int out_features, int 
 int cherryq_prepack_supported(int w_bits, int batch, int in_features, int out_features, int num_cherries,
                               int group_size) {
     return cq::stream_supported(w_bits, batch, in_features, out_features, num_cherries, group_size) ? 1 : 0;
+}
+
+int cherryq_prepack_recommended(int w_bits, int in_features, int out_features, int num_cherries, int group_size) {
+    if (!cq::stream_supported(w_bits, 1, in_features, out_features, num_cherries, group_size)) return 0;
+    return cq::stream_faster(w_bits, in_features, out_features, num_cherries) ? 1 : 0;
 }
 
 static int prepack_check(int w_bits, int K, int N, int C, int G, size_t stream_bytes_given) {

@@ -104,6 +104,7 @@ struct StreamGeo {
 };
 StreamGeo stream_geo(int bits, int K, int N, int C);
 size_t stream_bytes(int bits, int K, int N, int C);
+bool stream_faster(int bits, int K, int N, int C);
 bool stream_supported(int bits, int B, int K, int N, int C, int G);
 hipError_t launch_stream(int bits, const __half *vec, const uint8_t *stream, __half *mul, int K, int N, int C,
                          int accumulate, hipStream_t s);
@@ -128,10 +129,6 @@ hipError_t launch_f32(const float *vec, const uint8_t *qweight, const float *che
 bool fake_quant_supported(int K, int C, int G);
 hipError_t launch_fake_quant(int bits, bool fp32, const void *w, const int32_t *idx, void *out, int K, int N, int C,
                              int G, int ste, hipStream_t stream);
-
-// cq_probe.hip: roofline reference kernels for the measurement script.
-hipError_t launch_probe_read(const void *buf, size_t bytes, void *sink, hipStream_t stream);
-hipError_t launch_probe_empty(hipStream_t stream);
 
 // cq_decode.hip: batch-1 decode-step glue kernels.
 hipError_t launch_add_rmsnorm(__half *h, const __half *delta, const __half *weight, __half *y, int H, float eps,

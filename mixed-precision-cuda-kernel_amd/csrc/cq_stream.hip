@@ -482,14 +482,33 @@ struct StreamCfg {
     int W, T, D, L, S, NB, max_units;
 };
 static constexpr StreamCfg kStreamCfgs[] = {
-    {4, 1, 8, 8, 1, 8, 32}, {4, 1, 8, 12, 2, 8, 48}, {8, 1, 8, 8, 2, 8, 64}, {8, 1, 8, 12, 3, 8, 96}, {8, 1, 8, 16, 4, 8, 128},
+    {4, 1, 8, 8, 1, 8, 32},    // 0: K <= 4096 + cherries, 4-bit, more tiles than compute units
+    {4, 1, 8, 8, 4, 2, 32},    // 1: the same, 3-bit
+    {8, 1, 4, 4, 4, 2, 32},    // 2: K <= 4096 + cherries, about one tile per compute unit
+    {4, 1, 8, 12, 4, 4, 48},   // 3
+    {8, 1, 8, 8, 4, 4, 64},    // 4
+    {8, 1, 8, 12, 6, 4, 96},   // 5
+    {8, 1, 8, 16, 4, 8, 128},  // 6
 };
 constexpr int kStreamCfgCount = sizeof(kStreamCfgs) / sizeof(kStreamCfgs[0]);
 
+
 static int stream_pick(const StreamGeo &geo) {
-    for (int i = 0; i < kStreamCfgCount; i++)
+    // Measured on 4096 -> 11008 / 4096 -> 4096 (us per launch, 4-bit / 3-bit): entry 0 6.54 / 6.53 and
+    // 5.16 / 5.37, entry 1 6.78 / 6.51 and 4.42 / 4.48, entry 2 7.52 / 7.19 and 4.18 / 4.12.
+    if (geo.ng <= 32) return geo.ntiles <= 320 ? 2 : (geo.bits == 4 ? 0 : 1);
+    for (int i = 3; i < kStreamCfgCount; i++)
         if (geo.ng <= kStreamCfgs[i].max_units) return i;
     return -1;
+}
+
+// Where the batch-1 matvec over the stream measured faster than the one over the checkpoint layout
+// (us per launch, 4-bit, weights from HBM): 4096 -> 4096 4.18 against 4.95, 4096 -> 11008 6.54
+// against 7.26-7.46; slower beyond 32 units: 5120 -> 13824 12.1 against 9.1, 11008 -> 4096 7.7
+// against 7.0, 8192 -> 28672 29.4 against 22.8 (several rounds of workgroups, each staging x anew).
+bool stream_faster(int bits, int K, int N, int C) {
+    (void)N;
+    return stream_geo(bits, K, N, C).ng <= 32;
 }
 
 bool stream_supported(int bits, int B, int K, int N, int C, int G) {
@@ -535,6 +554,8 @@ static hipError_t launch_stream_bits(const __half *vec, const uint8_t *stream, _
         case 2: return launch_stream_cfg<BITS, 2>(vec, stream, mul, accumulate, geo, s);
         case 3: return launch_stream_cfg<BITS, 3>(vec, stream, mul, accumulate, geo, s);
         case 4: return launch_stream_cfg<BITS, 4>(vec, stream, mul, accumulate, geo, s);
+        case 5: return launch_stream_cfg<BITS, 5>(vec, stream, mul, accumulate, geo, s);
+        case 6: return launch_stream_cfg<BITS, 6>(vec, stream, mul, accumulate, geo, s);
         default: return hipErrorInvalidValue;
     }
 }

@@ -56,6 +56,8 @@ _lib.cherryq_prepack_bytes.argtypes = [_int, _int, _int, _int]
 _lib.cherryq_prepack_bytes.restype = _sz
 _lib.cherryq_prepack_supported.argtypes = [_int, _int, _int, _int, _int, _int]
 _lib.cherryq_prepack_supported.restype = _int
+_lib.cherryq_prepack_recommended.argtypes = [_int, _int, _int, _int, _int]
+_lib.cherryq_prepack_recommended.restype = _int
 _lib.cherryq_prepack_f16.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _sz, _int, _int, _int, _int, _vp]
 _lib.cherryq_prepack_f16.restype = _int
 _lib.cherryq_unprepack_f16.argtypes = [_int, _vp, _sz, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp]
@@ -332,6 +334,13 @@ def prepack_supported(w_bits, batch, in_features, out_features, num_cherries, gr
     of 128, at most 128 cherry channels and 16384 quantised input channels)."""
     return bool(_lib.cherryq_prepack_supported(int(w_bits), int(batch), int(in_features), int(out_features),
                                                int(num_cherries), int(group_size)))
+
+
+def prepack_recommended(w_bits, in_features, out_features, num_cherries, group_size) -> bool:
+    """Whether the matvec over the repacked stream measured faster on this GPU than the one over
+    the checkpoint layout for this layer shape (what a loader asks before prepack_cherryq)."""
+    return bool(_lib.cherryq_prepack_recommended(int(w_bits), int(in_features), int(out_features),
+                                                 int(num_cherries), int(group_size)))
 
 
 def prepack_cherryq(w_bits, qweight, cherry_weight, cherry_indices, scaling_factors, in_features, group_size):
