@@ -380,11 +380,11 @@ int cherryq_decode_matvec_group_f16(int w_bits, const void *vec, const void *vec
                       reinterpret_cast<const __half *>(l.scales), reinterpret_cast<__half *>(l.mul), l.out_features, 0};
     }
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    if (norm_weight) {
-        int n_total = 0;
-        for (int i = 0; i < n_layers; i++) n_total += outs[i];
-        if (!fast || !matvec_norm_supported(w_bits, K, n_total, C)) return CHERRYQ_E_UNSUPPORTED;
-    }
+    int n_total = 0;
+    for (int i = 0; i < n_layers; i++) n_total += outs[i];
+    // one launch streams all members: its geometry follows their total size
+    fast = fast && matvec_geometry(w_bits, K, n_total, C, 1).splits <= kMaxSplits;
+    if (norm_weight && (!fast || !matvec_norm_supported(w_bits, K, n_total, C))) return CHERRYQ_E_UNSUPPORTED;
     if (fast) {
         const MatvecPrologue pro = {reinterpret_cast<const __half *>(vec_gate),
                                     reinterpret_cast<const __half *>(norm_weight), eps};

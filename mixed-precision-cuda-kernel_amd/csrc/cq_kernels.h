@@ -24,6 +24,12 @@ hipError_t launch_unpack(int bits, const uint8_t *qweight, const __half *cherry_
 // cq_matvec.hip: HBM-streaming matvec for 1..kMatvecMaxRows activation rows.  Returns false when
 // the shape is not one it takes.
 constexpr int kMatvecMaxRows = 4;
+struct MatvecGeometry {
+    int kpl;     // positions per lane and unit: 16 (64-position units) or 32 (128)
+    int nw;      // wavefronts (= units) per workgroup
+    int splits;  // workgroups per column tile; must not exceed 255 (8-bit arrival counter)
+};
+MatvecGeometry matvec_geometry(int bits, int K, int n_total, int C, int rows);
 bool matvec_supported(int bits, int B, int K, int N, int C, int G);
 bool matvec_rows_preferred(int bits, int B, int K, int N, int C, int G);  // 2..4 rows: this kernel rather than the batch one
 hipError_t launch_matvec_rows(int bits, const __half *vec, const uint8_t *qweight, const __half *cherry_weight,

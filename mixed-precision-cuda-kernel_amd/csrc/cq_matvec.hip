@@ -580,8 +580,10 @@ bool matvec_supported(int bits, int B, int K, int N, int C, int G) {
     const long long cbytes = (long long)C * N * 2;
     const long long sbytes = (long long)ceil_div(K - C, G) * N * 2;
     if (wbytes >= 0x7fff0000ll || cbytes >= 0x7fff0000ll || sbytes >= 0x7fff0000ll) return false;
-    if (make_plan(K, N, C, 4, 128).splits > kMaxSplits) return false;
-    return K - C > 0;
+    if (K - C <= 0) return false;
+    // the split count of the geometry the launch will really use (it depends on the size of the
+    // layer and on the row count) must fit the 8-bit arrival counter of the split-K word
+    return matvec_geometry(bits, K, N, C, B).splits <= kMaxSplits;
 }
 
 
@@ -602,6 +604,7 @@ static hipError_t launch_matvec_nw(const __half *vec, const MatvecPrologue &pro,
     if (pro.norm_weight && K > kNormLoads * 8 * 64 * NW) return hipErrorNotSupported;
     if (rows > 1 && (pro.norm_weight || pro.gate || grp.count != 1)) return hipErrorNotSupported;
     Plan plan = make_plan(K, kTileCols, C, NW, 4 * KPL);
+    if (plan.splits > kMaxSplits) return hipErrorNotSupported;  // would wrap the split-K arrival counter
     plan.tiles = tiles;
     const dim3 grid(plan.tiles * plan.splits), block(64 * NW);
     unsigned long long *acc = reinterpret_cast<unsigned long long *>(workspace);
@@ -643,9 +646,28 @@ int matvec_waves_per_wg(int K, int N, int C, int kpl) {
     return nw;
 }
 
+// The launch geometry of a call: positions per lane and unit (16: 64-position units, 32: 128),
+// wavefronts per workgroup, and the resulting workgroups per column tile.  One function for the
+// support checks and the launch, so that they cannot disagree.
+// three and four rows: 128-position units whatever the size -- every row multiplies the split-K
+// atomics (0.85 us per row on the 4096 -> 11008 layer with 64-position units), half as many
+// splits outweigh the coarser grid (4 rows: 13.1 -> 11.5 us; two rows: 9.5 -> 10.1, left alone)
+MatvecGeometry matvec_geometry(int bits, int K, int n_total, int C, int rows) {
+    MatvecGeometry g;
+    g.kpl = rows > 2 ? 32 : matvec_kpl(bits, K, n_total, C);
+    g.nw = matvec_waves_per_wg(K, n_total, C, g.kpl);
+    g.splits = make_plan(K, kTileCols, C, g.nw, 4 * g.kpl).splits;
+    if (g.splits > kMaxSplits && g.kpl == 16) {  // very long rows of a small layer: coarser units
+        g.kpl = 32;
+        g.nw = matvec_waves_per_wg(K, n_total, C, g.kpl);
+        g.splits = make_plan(K, kTileCols, C, g.nw, 4 * g.kpl).splits;
+    }
+    return g;
+}
+
 bool matvec_norm_supported(int bits, int K, int n_total, int C) {
-    const int kpl = matvec_kpl(bits, K, n_total, C);
-    return K <= kNormLoads * 8 * 64 * matvec_waves_per_wg(K, n_total, C, kpl);
+    const MatvecGeometry g = matvec_geometry(bits, K, n_total, C, 1);
+    return g.splits <= kMaxSplits && K <= kNormLoads * 8 * 64 * g.nw;
 }
 
 static hipError_t launch_matvec_rows_group(int bits, const __half *vec, const MatvecPrologue &pro,
@@ -662,11 +684,9 @@ static hipError_t launch_matvec_rows_group(int bits, const __half *vec, const Ma
     }
     for (int i = count; i < kMaxGroup; i++) grp.m[i] = grp.m[0];
     // geometry from the group's total size: the launch streams all members' weights together
-    // three and four rows: 128-position units whatever the size -- every row multiplies the split-K
-    // atomics (0.85 us per row on the 4096 -> 11008 layer with 64-position units), half as many
-    // splits outweigh the coarser grid (4 rows: 13.1 -> 11.5 us; two rows: 9.5 -> 10.1, left alone)
-    const int kpl = rows > 2 ? 32 : matvec_kpl(bits, K, n_total, C);
-    const int nw = matvec_waves_per_wg(K, n_total, C, kpl);
+    const MatvecGeometry geo = matvec_geometry(bits, K, n_total, C, rows);
+    if (geo.splits > kMaxSplits) return hipErrorNotSupported;
+    const int kpl = geo.kpl, nw = geo.nw;
 #define CQ_LAUNCH(B, W, P)                                                                                   \
     return launch_matvec_nw<B, W, P>(vec, pro, grp, tiles, K, C, G, accumulate, workspace, stream, rows)
 #define CQ_PICK_NW(B, P)                                                                                     \
