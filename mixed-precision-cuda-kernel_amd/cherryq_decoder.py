@@ -190,6 +190,7 @@ class CherryLlamaDecoder(nn.Module):
         self.lm_head_t = self.lm_head.t()
         self._graph = None
         self.fuse_norm = True
+        self.layer_trace = None
         self._side = [torch.cuda.Stream(device=self.device_) for _ in range(2)] if self.device_.type == "cuda" else []
 
     # ---- checkpoint schema of the reference's LlamaForCausalLM (llama/modeling_llama_quant.py:
@@ -286,6 +287,8 @@ class CherryLlamaDecoder(nn.Module):
                 self._norm(layer.post_attention_layernorm)
                 matvec_group(gu, self.normed, [self.gate, self.up])
             matvec_group([layer.down_proj], self.up, [self.hid], vec_gate=self.gate, accumulate=True)
+            if self.layer_trace is not None:  # validation only (eager runs): the hidden state after every layer
+                self.layer_trace.append(self.hid.clone())
         self._norm(self.norm)
         self._head()
 

@@ -243,6 +243,41 @@ def test_batch_one_hot_rows_are_bit_exact(qc, bits, k, n):
         np.testing.assert_array_equal(ys, want.astype(np.float16))
 
 
+_ROWS_LAYERS = {}
+
+
+@pytest.mark.parametrize("b", [2, 3, 4])
+@pytest.mark.parametrize("bits,k,n", [(4, 4096, 4096), (3, 4096, 4096), (4, 4096, 11008), (3, 11008, 512)])
+def test_two_to_four_one_hot_rows_are_bit_exact(qc, bits, k, n, b):
+    """2, 3 and 4 one-hot activation rows (the two-row dot2 and the four-row 4x4x4 matrix-core
+    instantiations of the streaming kernel): row i returns dequantised column j_i bit for bit, also
+    with rows of very different power-of-two magnitude, for several placements of the columns."""
+    announce("rows one-hot", bits, k, n, b)
+    if (bits, k, n) not in _ROWS_LAYERS:  # the same layer serves the three row counts
+        p = orc.synthetic_layer(k, n, bits, 128, seed=9)[1]
+        _ROWS_LAYERS[(bits, k, n)] = (p, c_oracle.unpack(p, bits, 128, k))
+    p, dense = _ROWS_LAYERS[(bits, k, n)]
+    idx = p["cherry_indices"].astype(np.int64)
+    nidx = orc.normal_indices(k, idx)
+    pool = [int(nidx[0]), int(nidx[1]), int(nidx[63]), int(nidx[64]), int(nidx[127]), int(nidx[128]), int(nidx[-1]),
+            int(nidx[-65]), int(idx[0]), int(idx[-1]), int(idx[len(idx) // 2]), int(nidx[len(nidx) // 2 + 5])]
+    for start in range(0, len(pool), b):
+        cols = [pool[(start + i) % len(pool)] for i in range(b)]
+        x = np.zeros((b, k), dtype=np.float16)
+        for i, j in enumerate(cols):
+            x[i, j] = 1
+        y = run_fused(qc, bits, x, p, 128)
+        for i, j in enumerate(cols):
+            np.testing.assert_array_equal(y[i], dense[:, j], err_msg=f"row {i} column {j}")
+        # 2^-9 is the smallest factor that keeps every product (down to an fp16-subnormal cherry
+        # weight, 2^-24) a multiple of the split-K accumulator's 2^-34 step
+        scale = np.array([2.0 ** e for e in (-9, 3, -5, 9)][:b])
+        xs = (x.astype(np.float64) * scale[:, None]).astype(np.float16)
+        ys = run_fused(qc, bits, xs, p, 128)
+        with np.errstate(over="ignore"):
+            np.testing.assert_array_equal(ys, c_oracle.fused(xs, p, bits, 128).astype(np.float16))
+
+
 @pytest.mark.parametrize("bits,k,n,b", [(4, 8192, 8192, 16), (4, 8192, 28672, 16), (4, 28672, 8192, 16),
                                         (3, 13824, 5120, 8), (3, 5120, 13824, 4)])
 def test_batch_large_shapes(qc, bits, k, n, b):
