@@ -45,7 +45,8 @@ enum {
     CHERRYQ_E_WORKSPACE = -4,   /* workspace missing, misaligned or too small */
     CHERRYQ_E_BITS = -5,        /* w_bits is not 3 or 4 */
     CHERRYQ_E_ALIGN = -6,       /* a pointer is not aligned as the kernels require */
-    CHERRYQ_E_UNSUPPORTED = -7  /* valid request that this build does not implement */
+    CHERRYQ_E_UNSUPPORTED = -7, /* valid request that this build does not implement */
+    CHERRYQ_E_STATIC_LIMIT = -8 /* beyond the fixed workspace of cherryq_vecquant_matmul_f16_static */
 };
 
 int cherryq_version(void);
@@ -169,6 +170,28 @@ int cherryq_fake_quant_f16(int w_bits, const void *weight, const int32_t *cherry
 int cherryq_fake_quant_f32(int w_bits, const void *weight, const int32_t *cherry_indices, void *out,
                            int in_features, int out_features, int num_cherries, int group_size, int ste,
                            void *stream);
+
+/*
+ * cherryq_vecquant{3,4}matmul_f16 for callers that cannot allocate device memory or carry a
+ * workspace around (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.  Same arguments without workspace / scratch, same
+ * kernels and results for 1 to 4 activation rows; the split-K accumulator words live in a
+ * fixed array of CHERRYQ_STATIC_WORKSPACE_BYTES inside the library's device code (held by every
+ * GPU the library runs on until the process ends), so batch * out_features may not exceed
+ * 131072 and batch may not exceed 4: beyond that the call returns CHERRYQ_E_STATIC_LIMIT and
+ * launches nothing.  The call makes no hipMalloc / hipFree and no allocating library call; its
+ * first call on a device looks the array's address up (hipGetSymbolAddress) and should happen
+ * outside a stream capture.  All calls on one GPU share that GPU's array: calls that may overlap
+ * in time on one GPU (different streams) race -- serialise them or use the entry points above
+ * with workspaces of their own.  The kernels return every word they used to zero; if a launch
+ * is refused by the runtime, the next call clears the whole array first (a fill kernel on the
+ * call's stream, no hipMemset).
+ */
+#define CHERRYQ_STATIC_WORKSPACE_BYTES (1u << 20)
+int cherryq_vecquant_matmul_f16_static(int w_bits, const void *vec, const uint8_t *qweight, const void *cherry_weight,
+                                       const int16_t *cherry_indices, const void *scales, void *mul, int batch,
+                                       int in_features, int out_features, int num_cherries, int group_size,
+                                       int accumulate, void *stream);
 
 /*
  * Load-time repack of a packed layer into a weight stream laid out for this GPU, and the batch-1

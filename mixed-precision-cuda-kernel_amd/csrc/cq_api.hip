@@ -4,6 +4,8 @@
 
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "cq_common.cuh"
 #include "cq_kernels.h"
 
@@ -55,10 +57,9 @@ size_t scratch_bytes(int B, int K, int N, int C) {
 
 static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
-static int check_common(const void *vec, const void *qweight, const void *cherry_weight,
-                        const void *cherry_indices, const void *scales, const void *mul, int B, int K, int N,
-                        int C, int G, void *workspace, size_t workspace_bytes_given, void *scratch,
-                        size_t scratch_bytes_given) {
+static int check_tensors(const void *vec, const void *qweight, const void *cherry_weight,
+                         const void *cherry_indices, const void *scales, const void *mul, int B, int K, int N,
+                         int C, int G) {
     if (B < 0 || K <= 0 || N <= 0 || C < 0 || C > K) return CHERRYQ_E_SHAPE;
     if (K % 8 || N % 8 || C % 8) return CHERRYQ_E_SHAPE;
     if (G <= 0 || G % 32) return CHERRYQ_E_GROUP;
@@ -68,6 +69,15 @@ static int check_common(const void *vec, const void *qweight, const void *cherry
     if (!aligned(qweight, 16) || !aligned(scales, 16) || !aligned(cherry_weight, 16) || !aligned(vec, 4) ||
         !aligned(mul, 16) || !aligned(cherry_indices, 4))
         return CHERRYQ_E_ALIGN;
+    return CHERRYQ_OK;
+}
+
+static int check_common(const void *vec, const void *qweight, const void *cherry_weight,
+                        const void *cherry_indices, const void *scales, const void *mul, int B, int K, int N,
+                        int C, int G, void *workspace, size_t workspace_bytes_given, void *scratch,
+                        size_t scratch_bytes_given) {
+    const int rc = check_tensors(vec, qweight, cherry_weight, cherry_indices, scales, mul, B, K, N, C, G);
+    if (rc) return rc;
     if (!workspace || !aligned(workspace, 256) || workspace_bytes_given < workspace_bytes(B, K, N, C))
         return CHERRYQ_E_WORKSPACE;
     const size_t need = scratch_bytes(B, K, N, C);
@@ -122,6 +132,9 @@ const char *cherryq_status_string(int status) {
         case CHERRYQ_E_BITS: return "w_bits must be 3 or 4";
         case CHERRYQ_E_ALIGN: return "a pointer is not aligned as the kernels require";
         case CHERRYQ_E_UNSUPPORTED: return "request not implemented by this build";
+        case CHERRYQ_E_STATIC_LIMIT:
+            return "request exceeds the fixed workspace of the entry point that does not allocate "
+                   "(at most 4 rows and batch * out_features <= 131072)";
         default: break;
     }
     if (status > 0) return hipGetErrorString((hipError_t)status);
@@ -270,6 +283,104 @@ int cherryq_fake_quant_f32(int w_bits, const void *weight, const int32_t *cherry
                            int out_features, int num_cherries, int group_size, int ste, void *stream) {
     return fake_quant_entry(true, w_bits, weight, cherry_indices, out, in_features, out_features, num_cherries,
                             group_size, ste, stream);
+}
+
+// ---- the entry point that allocates nothing (see include/cherryq.h) -----------------------------
+
+}  // extern "C"
+
+namespace cq {
+
+// The split-K accumulator words of cherryq_vecquant_matmul_f16_static: 4 rows x 32768 columns of
+// 8 bytes.  Zero at load time; the kernels return every word they used to zero.
+constexpr size_t kStaticWorkspaceBytes = CHERRYQ_STATIC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned long long scratch[kStaticWorkspaceBytes / sizeof(unsigned long long)];
+
+constexpr int kStaticMaxDevices = 64;
+static std::mutex g_static_mutex;
+static void *g_static_ptr[kStaticMaxDevices];    // each GPU's own copy of `scratch`, from hipGetSymbolAddress
+static bool g_static_dirty[kStaticMaxDevices];   // a launch failed after the array may have been touched
+
+__global__ __launch_bounds__(256) void static_clear_kernel(unsigned long long *p, unsigned words) {
+    for (unsigned i = blockIdx.x * 256 + threadIdx.x; i < words; i += gridDim.x * 256) p[i] = 0ull;
+}
+
+template <int BITS>
+static int matmul_f16_static(const void *vec, const uint8_t *qweight, const void *cherry_weight,
+                             const int16_t *cherry_indices, const void *scales, void *mul, int B, int K, int N, int C,
+                             int G, int accumulate, void *stream) {
+    if (B < 0 || K <= 0 || N <= 0) return CHERRYQ_E_SHAPE;
+    if (B > kMatvecMaxRows) return CHERRYQ_E_STATIC_LIMIT;
+    const size_t need = ((size_t)(B < 1 ? 1 : B) * (size_t)N * sizeof(unsigned long long) + 255) / 256 * 256;
+    if (need > kStaticWorkspaceBytes) return CHERRYQ_E_STATIC_LIMIT;
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kStaticMaxDevices) return CHERRYQ_E_UNSUPPORTED;
+    void *ws = nullptr;
+    bool dirty = false;
+    {
+        std::lock_guard<std::mutex> lock(g_static_mutex);
+        if (!g_static_ptr[dev]) {  // once per device, with that device current
+            void *ptr = nullptr;
+            e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+            if (e != hipSuccess) return (int)e;
+            if (!ptr) return CHERRYQ_E_NULL;
+            g_static_ptr[dev] = ptr;
+        }
+        ws = g_static_ptr[dev];
+        dirty = g_static_dirty[dev];
+        g_static_dirty[dev] = true;  // until this call's launches are known to have been accepted
+    }
+    // the checks of the entry point this one is a variant of; on rejection nothing was launched
+    int rc = check_tensors(vec, qweight, cherry_weight, cherry_indices, scales, mul, B, K, N, C, G);
+    if (rc == CHERRYQ_OK && C > 0 && K > 32768) rc = CHERRYQ_E_SHAPE;
+    if (rc != CHERRYQ_OK || B == 0) {
+        std::lock_guard<std::mutex> lock(g_static_mutex);
+        g_static_dirty[dev] = dirty;
+        return rc;
+    }
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (dirty) {
+        hipLaunchKernelGGL(static_clear_kernel, dim3(256), dim3(256), 0, s, reinterpret_cast<unsigned long long *>(ws),
+                           (unsigned)(kStaticWorkspaceBytes / sizeof(unsigned long long)));
+        e = hipGetLastError();
+        if (e != hipSuccess) return (int)e;
+    }
+    const __half *x = reinterpret_cast<const __half *>(vec);
+    const __half *cw = reinterpret_cast<const __half *>(cherry_weight);
+    const __half *sc = reinterpret_cast<const __half *>(scales);
+    __half *y = reinterpret_cast<__half *>(mul);
+    if (!force_generic() && B == 1 && matvec_supported(BITS, B, K, N, C, G))
+        e = launch_matvec(BITS, x, qweight, cw, cherry_indices, sc, y, K, N, C, G, accumulate, ws, s);
+    else if (!force_generic() && matvec_rows_preferred(BITS, B, K, N, C, G))
+        e = launch_matvec_rows(BITS, x, qweight, cw, cherry_indices, sc, y, B, K, N, C, G, accumulate, ws, s);
+    else  // the general kernel: same accumulator words, no other buffer
+        e = launch_generic<BITS, __half, int16_t>(x, qweight, cw, cherry_indices, sc, y, B, K, N, C, G, accumulate, ws, s);
+    if (e == hipSuccess) {
+        std::lock_guard<std::mutex> lock(g_static_mutex);
+        g_static_dirty[dev] = false;
+    }
+    return (int)e;
+}
+
+}  // namespace cq
+
+extern "C" {
+
+int cherryq_vecquant_matmul_f16_static(int w_bits, const void *vec, const uint8_t *qweight, const void *cherry_weight,
+                                       const int16_t *cherry_indices, const void *scales, void *mul, int batch,
+                                       int in_features, int out_features, int num_cherries, int group_size,
+                                       int accumulate, void *stream) {
+    if (w_bits == 4) {
+        if (group_size < 128) return CHERRYQ_E_GROUP;
+        return cq::matmul_f16_static<4>(vec, qweight, cherry_weight, cherry_indices, scales, mul, batch, in_features,
+                                        out_features, num_cherries, group_size, accumulate, stream);
+    }
+    if (w_bits == 3)
+        return cq::matmul_f16_static<3>(vec, qweight, cherry_weight, cherry_indices, scales, mul, batch, in_features,
+                                        out_features, num_cherries, group_size, accumulate, stream);
+    return CHERRYQ_E_BITS;
 }
 
 // ---- load-time repacked weight stream (see include/cherryq.h) -----------------------------------

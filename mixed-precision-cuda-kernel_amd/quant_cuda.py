@@ -52,6 +52,8 @@ _lib.cherryq_pack_f16.restype = _int
 for _name in ("cherryq_fake_quant_f16", "cherryq_fake_quant_f32"):
     getattr(_lib, _name).argtypes = [_int, _vp, _vp, _vp, _int, _int, _int, _int, _int, _vp]
     getattr(_lib, _name).restype = _int
+_lib.cherryq_vecquant_matmul_f16_static.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _vp]
+_lib.cherryq_vecquant_matmul_f16_static.restype = _int
 _lib.cherryq_prepack_bytes.argtypes = [_int, _int, _int, _int]
 _lib.cherryq_prepack_bytes.restype = _sz
 _lib.cherryq_prepack_supported.argtypes = [_int, _int, _int, _int, _int, _int]
@@ -235,6 +237,35 @@ def matmul_cherryq(w_bits, vec, qweight, cherry_weight, cherry_indices, scaling_
         raise NotImplementedError(f"{w_bits} bit kernel is not implemented yet.")
     _matmul(fn, f"matmul_cherryq[{w_bits}bit]", vec, qweight, cherry_weight, cherry_indices, scaling_factors,
             out, group_size, w_bits, torch.float16, torch.int16, accumulate=accumulate)
+
+
+def matmul_cherryq_static(w_bits, vec, qweight, cherry_weight, cherry_indices, scaling_factors, out, group_size,
+                          accumulate=False):
+    """matmul_cherryq for 1 to 4 rows without any device allocation or workspace of the caller's:
+    the split-K accumulators live in a fixed 1 MiB array inside the library (so batch *
+    out_features <= 131072), shared by all calls on a GPU -- calls on different streams of one GPU
+    must not overlap.  For code under graph capture and loops that may not allocate."""
+    _check(vec, "vec", torch.float16, 2)
+    dev = vec.device
+    _check(qweight, "qweight", torch.uint8, 2, dev)
+    _check(cherry_weight, "cherry_weight", torch.float16, 2, dev)
+    _check(cherry_indices, "cherry_indices", torch.int16, 1, dev)
+    _check(scaling_factors, "scaling_factors", torch.float16, 2, dev)
+    _check(out, "out", torch.float16, 2, dev)
+    b, k = vec.shape
+    n, c = qweight.shape[1], cherry_indices.shape[0]
+    kn = k - c
+    if qweight.shape[0] * 8 != kn * w_bits or cherry_weight.shape != (c, n) or tuple(out.shape) != (b, n):
+        raise RuntimeError("matmul_cherryq_static: buffer shapes do not match")
+    if int(group_size) <= 0 or tuple(scaling_factors.shape) != (-(-kn // int(group_size)), n):
+        raise RuntimeError(f"scaling_factors shape {tuple(scaling_factors.shape)} does not match group_size={group_size}")
+    with torch.cuda.device(dev):
+        rc = _lib.cherryq_vecquant_matmul_f16_static(int(w_bits), _ptr(vec), _ptr(qweight), _ptr(cherry_weight),
+                                                     _ptr(cherry_indices), _ptr(scaling_factors), _ptr(out), b, k, n, c,
+                                                     int(group_size), 1 if accumulate else 0,
+                                                     _current_stream(dev.index))
+    if rc != 0:
+        _fail(rc, "matmul_cherryq_static")
 
 
 def _dequantize_normal(fn, what, w_bits, qweight, scaling_factors, out, height, cherry_size, group_size):
