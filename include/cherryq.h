@@ -50,6 +50,9 @@ enum {
 };
 
 int cherryq_version(void);
+/* Test hook, not part of the reference interface: on != 0 routes every fused call through the
+ * library's general kernel instead of the specialised ones (the tests compare the two). */
+void cherryq_set_force_generic(int on);
 const char *cherryq_status_string(int status);
 
 /*
@@ -60,7 +63,19 @@ const char *cherryq_status_string(int status);
  *   output element (fixed-point running sum plus an arrival count, added with a single atomic)
  *   and one arrival ticket per 256-column tile.  At least cherryq_workspace_bytes() bytes,
  *   256-byte aligned.  It must be all zero before the first call; every call leaves it all zero
- *   again, whatever the shapes of earlier calls were.
+ *   again, whatever the shapes of earlier calls were.  The one exception: a call that returns a
+ *   positive value (the runtime refused or aborted a launch) may leave words behind -- zero the
+ *   workspace again (hipMemsetAsync, or a fill kernel under capture) before reusing it.
+ *   Numerical contract of the accumulator words (batch 1 to 4, and every shape that takes the
+ *   general kernel): each workgroup's partial sum is rounded to a multiple of 2^-34 and, with fp16
+ *   tensors, clamped to +-(2^21 - 1); the running total must stay within +-2^21 (32 times fp16's
+ *   largest value).  Within that range the sum is exact and independent of the order in which
+ *   workgroups arrive, so results are deterministic; totals beyond fp16's range come out as
+ *   infinities of the right sign.  Outside it -- partial sums of one sign that add up beyond 2^21 --
+ *   the total wraps and the result is unspecified; a NaN activation gives infinite outputs
+ *   (either sign), not NaN.  With fp32 tensors (cherryq_vecquant3matmul_f32) partials of 2^13
+ *   and more, infinities and NaN are carried in a float side accumulator instead: range and
+ *   special values behave as in fp32, the absolute resolution stays 2^-34 per partial.
  * scratch: uninitialised memory for the batched paths (batch >= 2): per-split partial tiles and
  *   the activations laid out in matrix-core operand order.  At least cherryq_scratch_bytes()
  *   bytes (0 for batch 1, then it may be NULL), 256-byte aligned.

@@ -4,18 +4,28 @@
 
 #include <stdlib.h>
 
+#include <atomic>
 #include <mutex>
 
-#include "cq_common.cuh"
+#include "cq_device.h"
 #include "cq_kernels.h"
 
 namespace cq {
 
-// CHERRYQ_FORCE_GENERIC=1 routes every fused call through the generic kernel (a second,
-// independently written HIP path; used by the tests to cross-check the specialised kernels).
+// Test hook: route every fused call through the generic kernel (a second, independently written
+// HIP path that the tests cross-check the specialised kernels against).  Set by
+// cherryq_set_force_generic(); the environment variable CHERRYQ_FORCE_GENERIC=1 is read once,
+// at the first fused call, as the initial value.
+static std::atomic<int> g_force_generic{-1};
 static bool force_generic() {
-    const char *e = getenv("CHERRYQ_FORCE_GENERIC");
-    return e && e[0] == '1';
+    int v = g_force_generic.load(std::memory_order_relaxed);
+    if (v < 0) {
+        const char *e = getenv("CHERRYQ_FORCE_GENERIC");
+        v = e && e[0] == '1' ? 1 : 0;
+        int unset = -1;
+        if (!g_force_generic.compare_exchange_strong(unset, v)) v = unset;  // a setter call came first
+    }
+    return v == 1;
 }
 
 // Size queries answer for any arguments; nonsensical ones are clamped, not rejected.
@@ -30,8 +40,7 @@ static void clamp_dims(int &B, int &K, int &N, int &C) {
 // zero-kept: accumulator words (batch 1 and the generic kernel) and, for batches, the tickets
 size_t workspace_bytes(int B, int K, int N, int C) {
     clamp_dims(B, K, N, C);
-    size_t rows = (size_t)(B < 16 ? B : 16);
-    size_t bytes = (rows * (size_t)N * sizeof(unsigned long long) + 255) / 256 * 256;
+    size_t bytes = splitk_words_bytes(B, N) + splitk_side_bytes(B, N);
     if (B >= 2) {
         size_t b2 = batch_workspace(K, N, C).workspace_total;
         if (b2 > bytes) bytes = b2;
@@ -121,6 +130,8 @@ static int matmul_f16(const void *vec, const uint8_t *qweight, const void *cherr
 extern "C" {
 
 int cherryq_version(void) { return CHERRYQ_VERSION; }
+
+void cherryq_set_force_generic(int on) { cq::g_force_generic.store(on ? 1 : 0); }
 
 const char *cherryq_status_string(int status) {
     switch (status) {

@@ -22,26 +22,14 @@
 //
 // Cherry rows (dense fp16) run through the same MFMA with operands packed by v_perm_b32.
 // Across workgroups the K splits meet, for calls with few outputs, in one 64-bit fixed-point atomic
-// per output element (cq_common.cuh), and for larger ones in per-split partial tiles plus one
+// per output element (cq_device.h), and for larger ones in per-split partial tiles plus one
 // ticket per column tile (agent-scope sc1 stores / loads, no cache-wide fences; the last
 // workgroup adds the partials in split order).  Both are independent of arrival order.
 //
 // Arithmetic contract: csrc/quant_cuda_kernel.cu:797-834 (the reference loops its batch-1 body
 // over the batch rows, re-reading the weights for every row); fp32 accumulation, one rounding.
-#include "cq_common.cuh"
+#include "cq_device.h"
 #include "cq_kernels.h"
-
-// Optional per-wave phase timestamps for a profiling harness; compiled out in the library.
-#ifdef CQ_TRACE
-extern __device__ unsigned long long *g_cq_trace;
-#define CQB_STAMP(slot)                                                                                      \
-    do {                                                                                                     \
-        if (g_cq_trace && (threadIdx.x & 63) == 0)                                                           \
-            g_cq_trace[((size_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 8 + (slot)] = wall_clock64();         \
-    } while (0)
-#else
-#define CQB_STAMP(slot) do { } while (0)
-#endif
 
 namespace cq {
 
@@ -320,7 +308,6 @@ __global__ __launch_bounds__(64 * kBatchWaves) __attribute__((amdgpu_waves_per_e
 
     // this wave's units: u0, u0 + 4, u0 + 8, ...  (the 4 waves interleave).  One register set per
     // wave keeps the kernel at two waves per SIMD, which overlap each other's loads and MFMAs.
-    CQB_STAMP(0);
     const int u0 = split * plan.units_per_wg + wave;
     for (int it = 0; it < units_per_wave; it++) {
         const int ua = u0 + it * kBatchWaves;
@@ -335,7 +322,6 @@ __global__ __launch_bounds__(64 * kBatchWaves) __attribute__((amdgpu_waves_per_e
         if (u >= plan.units_normal && u < plan.units_total) cherry_unit(cx, u, tot);
     }
 
-    CQB_STAMP(1);
     // ---- across the workgroup's wavefronts through LDS.  Column 16 nl + c is stored at
     // 16 nl + ((c + nl) & 15): for a fixed c the 16 lanes of a row then hit 16 different banks.
 #pragma unroll
@@ -355,8 +341,7 @@ __global__ __launch_bounds__(64 * kBatchWaves) __attribute__((amdgpu_waves_per_e
 
     // ---- across workgroups: per-split partial tiles + one ticket per column tile.  (One atomic
     // per output element, as in the batch-1 kernel, is slower here: 16 rows make 16x the atomics.)
-    // Partials travel as agent-scope sc1 stores / loads, no cache-wide fences; see cq_common.cuh.
-    CQB_STAMP(2);
+    // Partials travel as agent-scope sc1 stores / loads, no cache-wide fences; see cq_device.h.
     if (atomic_epilogue) {
         // few enough outputs: one 64-bit fixed-point atomic per output element, as in the batch-1
         // kernel (order-independent, leaves the words zero), instead of partial tiles + ticket
@@ -364,7 +349,6 @@ __global__ __launch_bounds__(64 * kBatchWaves) __attribute__((amdgpu_waves_per_e
 #pragma unroll
         for (int b = 0; b < kBatchRows; b++) v2[b][0] = vals[b];
         splitk_finish<__half, kBatchRows, 1>(v2, B, N, n, active, plan.splits, acc_words, mul, accumulate);
-        CQB_STAMP(4);
         return;
     }
     if (plan.splits > 1) {
@@ -383,7 +367,6 @@ __global__ __launch_bounds__(64 * kBatchWaves) __attribute__((amdgpu_waves_per_e
             *s_last = (old == (unsigned)(plan.splits - 1));
         }
         __syncthreads();
-        CQB_STAMP(3);
         if (!*s_last) return;
         if (tid == 0) __hip_atomic_store(&tickets[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (active) {
@@ -407,7 +390,6 @@ __global__ __launch_bounds__(64 * kBatchWaves) __attribute__((amdgpu_waves_per_e
             }
         }
     }
-    CQB_STAMP(4);
     if (active) {
 #pragma unroll
         for (int b = 0; b < kBatchRows; b++)

@@ -6,23 +6,12 @@
 // rotary embedding :95-147 and apply_rotary_pos_emb :179-210, attention with KV cache :391-402 /
 // :671-696, SiLU-gated MLP :251.  fp16 storage, fp32 arithmetic inside a kernel, roundings at the
 // points where the reference's fp16 tensors are materialised.
-#include "cq_common.cuh"
+#include "cq_device.h"
 #include "cq_kernels.h"
 
 // The rotary embedding rounds every product and every sum to fp16 separately, as the reference's
 // fp16 tensor operations do; contraction would merge a product and a sum into one rounding.
 #pragma clang fp contract(off)
-
-// Optional per-workgroup phase timestamps for a profiling harness; compiled out in the library.
-#ifdef CQ_TRACE
-extern __device__ unsigned long long *g_cq_trace;
-#define CQD_STAMP(slot)                                                                                      \
-    do {                                                                                                     \
-        if (g_cq_trace && threadIdx.x == 0) g_cq_trace[(size_t)blockIdx.x * 8 + (slot)] = wall_clock64();    \
-    } while (0)
-#else
-#define CQD_STAMP(slot) do { } while (0)
-#endif
 
 namespace cq {
 
@@ -119,7 +108,7 @@ __global__ void rope_cache_kernel(__half *__restrict__ q, const __half *__restri
                                   int max_len, RopeBase base) {
     const int pos = *pos_ptr;
     const int head = blockIdx.x, i = threadIdx.x, half_dim = head_dim / 2;
-    if (i >= half_dim || pos >= max_len) return;
+    if (i >= half_dim || (unsigned)pos >= (unsigned)max_len) return;  // also a negative position: nothing is written
     const float inv_freq = rope_inv_freq(i, head_dim, base);
     float sn, cs;
     sincosf((float)pos * inv_freq, &sn, &cs);
@@ -181,7 +170,14 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const __half *__restri
     const int head = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int row = t >> 4, l16 = t & 15;
     const int kvh = head / (n_heads / n_kv_heads);
-    const int len = min(*pos_ptr + 1, max_len);
+    const int pos = *pos_ptr;
+    if ((unsigned)pos >= (unsigned)max_len) {
+        // a position outside the cache (negative, or at / beyond max_len) reads nothing; the
+        // output is NaN so that the caller's mistake shows in everything computed from it
+        if (t < 128) out[(size_t)head * 128 + t] = __ushort_as_half((unsigned short)0x7e00);
+        return;
+    }
+    const int len = pos + 1;
     const uint4 *kb = reinterpret_cast<const uint4 *>(k_cache + (size_t)kvh * max_len * 128);
     const uint4 *vb = reinterpret_cast<const uint4 *>(v_cache + (size_t)kvh * max_len * 128);
     float qf[8];
@@ -249,7 +245,6 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
     __shared__ float s_acc[16][128];
     __shared__ __attribute__((aligned(16))) unsigned short s_qh[128], s_kh[128];  // rotated q, k as fp16
     const int head = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    CQD_STAMP(0);
     const int row = t >> 4, l16 = t & 15;
     const int rep = n_heads / n_kv_heads, kvh = head / rep;
     const uint4 *kb = reinterpret_cast<const uint4 *>(k_cache + (size_t)kvh * max_len * 128);
@@ -279,8 +274,10 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
         inv_freq = rope_inv_freq(i, 128, base);  // does not need the position
     }
     const int pos = *pos_ptr;
-    if (pos >= max_len) return;
-    CQD_STAMP(1);
+    if ((unsigned)pos >= (unsigned)max_len) {  // outside the cache: nothing read or written, the output is NaN
+        if (t < 128) out[(size_t)head * 128 + t] = __ushort_as_half((unsigned short)0x7e00);
+        return;
+    }
     if (t < 128) {
         const int i = t & 63;
         const bool is_k = t >= 64;
@@ -303,7 +300,6 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
         }
     }
     __syncthreads();
-    CQD_STAMP(2);
     // q . k over the lane's 8 dimensions as four packed fp16 dot products (fp32 accumulation), the 16
     // lanes of a row then add up with DPP rotations
     const uint4 qv = *reinterpret_cast<const uint4 *>(&s_qh[8 * l16]);
@@ -345,7 +341,6 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
     m = wave_max_all(m);
     if (lane == 0) s_red[wave] = m;
     __syncthreads();
-    CQD_STAMP(3);
     const int len = pos + 1;
     m = s_red[0];
 #pragma unroll
@@ -359,7 +354,6 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
     sum = wave_sum_all(sum);
     if (lane == 0) s_red[16 + wave] = sum;
     __syncthreads();
-    CQD_STAMP(4);
     float tot = 0.f;
 #pragma unroll
     for (int w = 0; w < 16; w++) tot += s_red[16 + w];
@@ -394,7 +388,6 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
 #pragma unroll
         for (int i = 0; i < 8; i++) acc[i] = fmaf(p, vf[i], acc[i]);
     }
-    CQD_STAMP(5);
     // the four 16-lane rows of a wavefront hold partial sums for the same 128 dimensions: two
     // halving exchanges leave every lane with 2 of its 8 dimensions summed over the four rows
     {
@@ -408,14 +401,12 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
         s_acc[wave][d0 + 1] = q2[1];
     }
     __syncthreads();
-    CQD_STAMP(6);
     if (t < 128) {
         float o = 0.f;
 #pragma unroll
         for (int w = 0; w < 16; w++) o += s_acc[w][t];
         out[(size_t)head * 128 + t] = __float2half_rn(o);
     }
-    CQD_STAMP(7);
 }
 
 // out <- fp16(silu(gate)) * up

@@ -138,14 +138,34 @@ __device__ inline float wave_max_all(float v) {
 // which is thereby ready for the next call.  One memory round trip, no barrier, no second pass.
 //
 // Fixed point loses nothing that fp16 output can show: the resolution 2^-34 is 2^10 times finer
-// than the smallest fp16 subnormal step, and the range +-2^21 is 32 times fp16's largest value
-// (partials are clamped to it; a NaN partial is clamped too and so reads as a huge value).
+// than the smallest fp16 subnormal step, and the range +-2^21 is 32 times fp16's largest value.
+// The contract that follows: every workgroup's partial sum is rounded to a multiple of 2^-34 and,
+// with fp16 tensors, clamped to +-(2^21 - 1) (a NaN partial is clamped too and reads as one end
+// of the range: the output becomes an infinity, not NaN); the running total must stay within +-2^21, which it does whenever the partial sums of
+// one sign add up to less than that -- beyond it the 56-bit field wraps.  With fp32 tensors,
+// whose results may legitimately exceed 2^21, a partial of 2^13 or more (255 smaller ones
+// cannot leave the range) or one that is not finite is instead added to a float side accumulator of the same output (`side`, one float per
+// accumulator word, zero-kept like the words) and joins the total when the output is finished:
+// range and NaN / Inf behave as in fp32, only the 2^-34 absolute resolution remains.
 // Agent-scope release/acquire fences are deliberately not used: on this multi-XCD part they
 // write back and invalidate a whole L2 and serialise the workgroups.
 constexpr float kFixScale = 17179869184.0f;        // 2^34
 constexpr double kFixInvScale = 1.0 / 17179869184.0;
 constexpr float kFixClamp = 2097151.0f;             // 2^21 - 1
 constexpr int kMaxSplits = 255;
+constexpr float kWideEscape = 8192.0f;              // 2^21 / 256: kMaxSplits partials below it cannot leave the range
+
+// Workspace layout of a call with B rows: min(B, 16) * N accumulator words (rounded up to 256
+// bytes), then as many floats: the side accumulators of the fp32-tensor entry point.
+__host__ inline size_t splitk_words_bytes(int B, int N) {
+    return ((size_t)(B < 16 ? (B < 1 ? 1 : B) : 16) * (size_t)N * sizeof(unsigned long long) + 255) / 256 * 256;
+}
+__host__ inline size_t splitk_side_bytes(int B, int N) {
+    return ((size_t)(B < 16 ? (B < 1 ? 1 : B) : 16) * (size_t)N * sizeof(float) + 255) / 256 * 256;
+}
+__host__ inline float *splitk_side(void *workspace, int B, int N) {
+    return reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + splitk_words_bytes(B, N));
+}
 
 __device__ inline unsigned long long splitk_encode(float partial) {
     float p = fminf(fmaxf(partial, -kFixClamp), kFixClamp);
@@ -157,7 +177,8 @@ __device__ inline unsigned long long splitk_encode(float partial) {
 template <typename IO, int MAXB, int COLS>
 __device__ inline void splitk_finish(float (&vals)[MAXB][COLS], int B, int N, int n0, bool active, int splits,
                                      unsigned long long *__restrict__ acc, IO *__restrict__ mul,
-                                     int accumulate) {
+                                     int accumulate, float *__restrict__ side = nullptr) {
+    constexpr bool kWide = sizeof(IO) == 4;  // fp32 tensors: out-of-range partials take the side accumulator
     if (!active) return;
     if (splits > 1) {
         unsigned long long now[MAXB][COLS];
@@ -166,6 +187,14 @@ __device__ inline void splitk_finish(float (&vals)[MAXB][COLS], int B, int N, in
             if (b < B) {
 #pragma unroll
                 for (int c = 0; c < COLS; c++) {
+                    if (kWide && !(fabsf(vals[b][c]) < kWideEscape)) {
+                        // the float add must have completed before this workgroup is counted as
+                        // arrived: wait for its return value
+                        float old = __hip_atomic_fetch_add(side + (size_t)b * N + n0 + c, vals[b][c], __ATOMIC_RELAXED,
+                                                           __HIP_MEMORY_SCOPE_AGENT);
+                        asm volatile("" ::"v"(old) : "memory");
+                        vals[b][c] = 0.f;
+                    }
                     const unsigned long long add = splitk_encode(vals[b][c]);
                     now[b][c] = __hip_atomic_fetch_add(acc + (size_t)b * N + n0 + c, add, __ATOMIC_RELAXED,
                                                        __HIP_MEMORY_SCOPE_AGENT) + add;
@@ -180,6 +209,14 @@ __device__ inline void splitk_finish(float (&vals)[MAXB][COLS], int B, int N, in
                     __hip_atomic_store(acc + (size_t)b * N + n0 + c, 0ull, __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
                     float v = (float)((double)((long long)now[b][c] >> 8) * kFixInvScale);
+                    if (kWide) {
+                        float *sp = side + (size_t)b * N + n0 + c;
+                        const float extra = __hip_atomic_load(sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (!(extra == 0.f)) {
+                            __hip_atomic_store(sp, 0.f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            v += extra;
+                        }
+                    }
                     IO *o = mul + (size_t)b * N + n0 + c;
                     if (accumulate) v += to_float(*o);
                     *o = from_float<IO>(v);

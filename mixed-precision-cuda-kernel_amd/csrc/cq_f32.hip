@@ -21,13 +21,13 @@
 //
 // Cherry rows are further units whose B operands are the fp32 rows themselves.  Across the
 // workgroup's wavefronts the totals meet in LDS, across workgroups in one 64-bit fixed-point
-// atomic per output element (cq_common.cuh).  Up to 16 rows per pass; more rows are further
+// atomic per output element (cq_device.h).  Up to 16 rows per pass; more rows are further
 // passes over the weights.
 //
 // Arithmetic contract: csrc/quant_cuda_kernel.cu:191-314 (group 64) and 441-556 (group 128):
 // fp32 products and sums; the summation order differs (the reference adds 64 or 128 products in
 // sequence per thread and combines blocks with fp32 atomics in arrival order).
-#include "cq_common.cuh"
+#include "cq_device.h"
 #include "cq_kernels.h"
 
 namespace cq {
@@ -79,8 +79,8 @@ __global__ __launch_bounds__(256) void f32_prep_kernel(const float *__restrict__
 // ---- main kernel -------------------------------------------------------------------------------
 __global__ __launch_bounds__(64 * kF32Waves) __attribute__((amdgpu_waves_per_eu(2, 2))) void f32_kernel(
     const uint8_t *__restrict__ qweight, const float *__restrict__ cherry_weight, const float *__restrict__ scales,
-    float *__restrict__ mul, const float4 *__restrict__ xa, unsigned long long *__restrict__ acc_words, int B, int K,
-    int N, int C, int G, int accumulate, Plan plan, int units_per_wave) {
+    float *__restrict__ mul, const float4 *__restrict__ xa, unsigned long long *__restrict__ acc_words,
+    float *__restrict__ side, int B, int K, int N, int C, int G, int accumulate, Plan plan, int units_per_wave) {
     __shared__ float s_red[kF32Waves][kF32Rows][kTileCols];  // 64 KB
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -186,7 +186,7 @@ __global__ __launch_bounds__(64 * kF32Waves) __attribute__((amdgpu_waves_per_eu(
             vals[b][0] = (s_red[0][b][sw] + s_red[1][b][sw]) + (s_red[2][b][sw] + s_red[3][b][sw]);
     }
     const int n = tile * kTileCols + tid;
-    splitk_finish<float, kF32Rows, 1>(vals, B, N, n, n < N, plan.splits, acc_words, mul, accumulate);
+    splitk_finish<float, kF32Rows, 1>(vals, B, N, n, n < N, plan.splits, acc_words, mul, accumulate, side);
 }
 
 bool f32_supported(int B, int K, int N, int C, int G) {
@@ -218,7 +218,7 @@ hipError_t launch_f32(const float *vec, const uint8_t *qweight, const float *che
                            cherry_indices, xa, nb, K, C, plan.units_normal);
         hipLaunchKernelGGL(f32_kernel, dim3(plan.tiles * plan.splits), dim3(64 * kF32Waves), 0, stream, qweight,
                            cherry_weight, scales, mul + (size_t)b0 * N, xa, reinterpret_cast<unsigned long long *>(workspace),
-                           nb, K, N, C, G, accumulate, plan, upv);
+                           splitk_side(workspace, B, N), nb, K, N, C, G, accumulate, plan, upv);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }

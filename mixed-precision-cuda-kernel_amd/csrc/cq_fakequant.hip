@@ -26,7 +26,7 @@
 // the original bits.  A per-chunk "fast path when no cherry and no group boundary falls into the
 // chunk" measured slower than no fast path at all: with 1 chunk in 32 taking the other branch,
 // nearly every wavefront executes both.
-#include "cq_common.cuh"
+#include "cq_device.h"
 #include "cq_kernels.h"
 
 #pragma clang fp contract(off)

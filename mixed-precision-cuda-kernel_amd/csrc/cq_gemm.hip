@@ -39,7 +39,7 @@
 // Arithmetic contract: csrc/quant_cuda_kernel.cu:797-834 (the reference loops its batch-1 body
 // over the rows); here fp16 weights as the dense path's (qlinear.py:183-195), fp32 accumulation,
 // one final rounding.
-#include "cq_common.cuh"
+#include "cq_device.h"
 #include "cq_kernels.h"
 
 namespace cq {

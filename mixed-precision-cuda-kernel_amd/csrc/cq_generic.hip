@@ -7,7 +7,7 @@
 // Arithmetic contract: csrc/quant_cuda_kernel.cu:718-835 (4-bit), 558-672 / 316-438 (3-bit,
 // group multiple of 128 / group 64), 441-556 / 191-314 (fp32 I/O), with fp32 accumulation
 // kept until a single final rounding instead of one fp16 atomic per 128 positions (:833).
-#include "cq_common.cuh"
+#include "cq_device.h"
 #include "cq_kernels.h"
 
 namespace cq {
@@ -41,8 +41,8 @@ template <int BITS, typename IO, typename IDX>
 __global__ __launch_bounds__(64) void generic_kernel(
     const IO *__restrict__ vec, const uint8_t *__restrict__ qweight,
     const IO *__restrict__ cherry_weight, const IDX *__restrict__ cherry_indices,
-    const IO *__restrict__ scales, IO *__restrict__ mul, unsigned long long *__restrict__ acc_words, int B,
-    int K, int N, int C, int G, int accumulate, Plan plan) {
+    const IO *__restrict__ scales, IO *__restrict__ mul, unsigned long long *__restrict__ acc_words,
+    float *__restrict__ side, int B, int K, int N, int C, int G, int accumulate, Plan plan) {
     const int lane = threadIdx.x;
     const int lid = xcd_remap(blockIdx.x, gridDim.x);
     const int tile = lid / plan.splits;
@@ -144,7 +144,7 @@ __global__ __launch_bounds__(64) void generic_kernel(
             }
         }
     }
-    splitk_finish<IO, kMaxB, 4>(acc, B, N, n0, active, plan.splits, acc_words, mul, accumulate);
+    splitk_finish<IO, kMaxB, 4>(acc, B, N, n0, active, plan.splits, acc_words, mul, accumulate, side);
 }
 
 template <int BITS, typename IO, typename IDX>
@@ -155,11 +155,12 @@ hipError_t launch_generic(const IO *vec, const uint8_t *qweight, const IO *cherr
     while (make_plan(K, N, C, upw).splits > kMaxSplits) upw <<= 1;
     Plan plan = make_plan(K, N, C, upw);
     unsigned long long *acc_words = reinterpret_cast<unsigned long long *>(workspace);
+    float *side = sizeof(IO) == 4 ? splitk_side(workspace, B, N) : nullptr;  // fp32 tensors only
     for (int b0 = 0; b0 < B; b0 += kMaxB) {
         int nb = min(kMaxB, B - b0);
         hipLaunchKernelGGL((generic_kernel<BITS, IO, IDX>), dim3(plan.tiles * plan.splits), dim3(64), 0,
                            stream, vec + (size_t)b0 * K, qweight, cherry_weight, cherry_indices, scales,
-                           mul + (size_t)b0 * N, acc_words, nb, K, N, C, G, accumulate, plan);
+                           mul + (size_t)b0 * N, acc_words, side, nb, K, N, C, G, accumulate, plan);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }

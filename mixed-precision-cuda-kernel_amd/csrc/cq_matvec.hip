@@ -1,13 +1,19 @@
-// Batch-1 fused dequant + matvec for gfx950, built as an HBM stream.
+// Fused dequant + matvec for 1 to 4 activation rows on gfx950, built as an HBM stream over the
+// checkpoint layout (matvec_kernel<BITS, NW, KPL, NORM, ROWS>).
 //
-// Work unit: 128 compacted normal positions x 256 output columns (16 KB of 4-bit, 12 KB of
-// 3-bit weights), or 32 cherry rows x 256 columns.  One wavefront owns one unit: the 64 lanes
-// form 4 lane groups (16-lane DPP rows) that split the 128 positions four ways, and the 16
-// lanes of a row each own 16 adjacent columns, so every load is a dwordx4 and a row of lanes
-// reads 256 contiguous bytes of one byte row.  A wavefront issues all 16 (12) weight loads
-// up front and consumes them in order as they land.  Four wavefronts (four consecutive units
-// of one column tile) form a workgroup; the K reduction runs lane -> DPP row -> permlane
-// swaps across rows -> LDS across wavefronts -> split-K partials across workgroups.
+// Work unit: 4 * KPL compacted normal positions (KPL = 16: 64 positions, 8 / 6 KB of 4- / 3-bit
+// weights; KPL = 32: 128 positions) x 256 output columns, or 32 cherry rows x 256 columns.  One
+// wavefront owns one unit: the 64 lanes form 4 lane groups (16-lane DPP rows) that split the
+// positions four ways, and the 16 lanes of a row each own 16 adjacent columns, so every load is
+// a dwordx4 and a row of lanes reads 256 contiguous bytes of one byte row.  A wavefront issues
+// all its weight loads up front and consumes them in order as they land.  NW (1, 2 or 4)
+// wavefronts -- consecutive units of one column tile -- form a workgroup; the K reduction runs
+// lane -> DPP row -> permlane swaps across rows -> LDS across wavefronts -> split-K partials
+// across workgroups (one 64-bit fixed-point atomic per output, cq_device.h).  The launch
+// geometry (KPL, NW) follows the size of the layer: matvec_geometry() below.  NORM fuses an
+// RMSNorm of the activation row into its staging, ROWS = 2 runs two activation rows through the
+// same dot2 sequence, ROWS = 4 up to four through 4x4x4 matrix-core instructions; a gate vector
+// (silu(gate) * x) and several layers per launch are run-time options of the staging.
 //
 // Codes never pass through an int->float conversion.  A code field masked in place inside a
 // 16-bit half is the fp16 subnormal  code * 2^(p-24)  (p = bit position of the field), which
@@ -21,12 +27,8 @@
 //
 // Arithmetic contract: csrc/quant_cuda_kernel.cu:718-835 (4-bit) and 558-672 / 316-438
 // (3-bit); fp32 accumulation throughout, one rounding to fp16 at the end.
-#include "cq_common.cuh"
+#include "cq_device.h"
 #include "cq_kernels.h"
-
-#ifdef CQ_TRACE
-extern __device__ unsigned long long *g_cq_trace;  // defined by the profiling harness
-#endif
 
 namespace cq {
 
@@ -35,17 +37,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
-
-// Optional per-wave phase timestamps for a profiling harness; compiled out in the library.
-#ifdef CQ_TRACE
-#define CQ_STAMP(slot)                                                                                       \
-    do {                                                                                                     \
-        if (g_cq_trace && lane == 0)                                                                         \
-            g_cq_trace[((size_t)blockIdx.x * NW + wave) * 8 + (slot)] = wall_clock64();                      \
-    } while (0)
-#else
-#define CQ_STAMP(slot) do { } while (0)
-#endif
 
 constexpr int kMaxFastCherries = 128;  // two 64-lane chunks of cherry indices
 constexpr uint32_t kRsrcFlags = 0x00020000u;
@@ -183,7 +174,6 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
     for (int r = 0; r < ROWS; r++)
 #pragma unroll
         for (int c = 0; c < 16; c++) tot[r][c] = 0.f;
-    CQ_STAMP(0);
 
     // Fused RMSNorm: the workgroup's threads share one pass over the K activations (16 bytes per
     // load, reads past the end return 0) for the sum of squares.  The loads are issued here, ahead
@@ -335,7 +325,6 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
 #pragma unroll
             for (int i = 0; i < G_::kPairs / 4; i++)
                 xq[r][i] = *reinterpret_cast<const u32x4 *>(&s_pair[wave][ROWS == 4 ? (lane & 3) : r][16 * kq + 4 * i]);
-        CQ_STAMP(1);
 
         if (ROWS == 4) {
             // d[c][r]: this lane's column c, activation row r
@@ -528,7 +517,6 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
         (void)norm_scale<NW>(nchunk, s_ss, wave, lane, K, pro.eps);
     }
 
-    CQ_STAMP(2);
     // ---- reduce over the four lane groups; lane group kq ends up with columns 4kq .. 4kq+3
     float q4[ROWS][4];
 #pragma unroll
@@ -541,9 +529,7 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
     }
     if (NW == 1) {
         const int n = n0 + 4 * kq;
-        CQ_STAMP(3);
         splitk_finish<__half, ROWS, 4>(q4, rows, N, n, n < N, plan.splits, acc_words, mul, accumulate);
-        CQ_STAMP(4);
     } else {
         // ---- across the workgroup's wavefronts through LDS, then 4 / NW columns per thread
         __shared__ float s_red[NW][ROWS][kTileCols];
@@ -563,10 +549,8 @@ __global__ __launch_bounds__(64 * NW) void matvec_kernel(
                 vals[r][c] = v;
             }
         const int n = tile * kTileCols + tid * CPT;
-        CQ_STAMP(3);
         splitk_finish<__half, ROWS, CPT>(vals, rows, N, n, n < N && tid * CPT < kTileCols, plan.splits, acc_words, mul,
                                          accumulate);
-        CQ_STAMP(4);
     }
 }
 

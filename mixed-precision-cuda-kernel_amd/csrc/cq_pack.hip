@@ -9,7 +9,7 @@
 //   q    = rint( clamp( f32( RN16( f32(w) / f32(s) ) ), -qmax, qmax ) - 0.5 ),  qmax = 2^(b-1) - 0.01
 //   code = q + 2^(b-1)
 // (fp32 division followed by rounding to fp16 equals the correctly rounded fp16 quotient: 24 >= 2*11+2.)
-#include "cq_common.cuh"
+#include "cq_device.h"
 #include "cq_kernels.h"
 
 namespace cq {

@@ -31,7 +31,7 @@
 // Arithmetic contract: csrc/quant_cuda_kernel.cu:718-835 (4-bit) and 558-672 (3-bit) of the
 // reference; fp32 accumulation, one rounding to fp16.  Replaces the per-thread decode loops at
 // :811-831 / :649-667 and the serial batch loop :797-834.
-#include "cq_common.cuh"
+#include "cq_device.h"
 #include "cq_kernels.h"
 
 namespace cq {

@@ -54,6 +54,8 @@ for _name in ("cherryq_fake_quant_f16", "cherryq_fake_quant_f32"):
     getattr(_lib, _name).restype = _int
 _lib.cherryq_vecquant_matmul_f16_static.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _vp]
 _lib.cherryq_vecquant_matmul_f16_static.restype = _int
+_lib.cherryq_set_force_generic.argtypes = [_int]
+_lib.cherryq_set_force_generic.restype = None
 _lib.cherryq_prepack_bytes.argtypes = [_int, _int, _int, _int]
 _lib.cherryq_prepack_bytes.restype = _sz
 _lib.cherryq_prepack_supported.argtypes = [_int, _int, _int, _int, _int, _int]
@@ -237,6 +239,12 @@ def matmul_cherryq(w_bits, vec, qweight, cherry_weight, cherry_indices, scaling_
         raise NotImplementedError(f"{w_bits} bit kernel is not implemented yet.")
     _matmul(fn, f"matmul_cherryq[{w_bits}bit]", vec, qweight, cherry_weight, cherry_indices, scaling_factors,
             out, group_size, w_bits, torch.float16, torch.int16, accumulate=accumulate)
+
+
+def force_generic(on: bool) -> None:
+    """Test hook: route every fused call through the library's general kernel (the tests compare it
+    with the specialised ones)."""
+    _lib.cherryq_set_force_generic(1 if on else 0)
 
 
 def matmul_cherryq_static(w_bits, vec, qweight, cherry_weight, cherry_indices, scaling_factors, out, group_size,

@@ -393,3 +393,42 @@ def test_matvec_group_llama7b_shapes_against_the_c_oracle(dec, bits, case):
             got = run(u1, base=base, vec_gate=torch.from_numpy(g1).cuda(), accumulate=True)
             want = f16(base[0].astype(np.float64) + c_oracle.fused(x, packed[0], bits, 128))
             np.testing.assert_array_equal(got[0], want, err_msg=f"column {j}")
+
+
+def test_positions_outside_the_cache_touch_nothing_and_poison_the_output(dec):
+    """A position that is negative or at / beyond max_len must not index the KV cache: the rotary /
+    cache-write kernels write nothing, the attention kernels read nothing and return NaN so that the
+    mistake shows downstream."""
+    print("[case] decode position guards", flush=True)
+    lib = dec._lib
+    nh, nkv, hd, ml = 4, 2, 128, 16
+    torch.manual_seed(3)
+    for bad in (ml, ml + 5, -1, -(2 ** 31)):
+        kc = torch.randn(nkv, ml, hd, device="cuda").half()
+        vc = torch.randn(nkv, ml, hd, device="cuda").half()
+        kc0, vc0 = kc.clone(), vc.clone()
+        q = torch.randn(1, nh * hd, device="cuda").half()
+        k = torch.randn(1, nkv * hd, device="cuda").half()
+        v = torch.randn(1, nkv * hd, device="cuda").half()
+        pos = torch.tensor([bad], dtype=torch.int32, device="cuda")
+        q1 = q.clone()
+        assert lib.cherryq_decode_rope_cache_f16(q1.data_ptr(), k.data_ptr(), v.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+                                                 pos.data_ptr(), nh, nkv, hd, ml, 10000.0, stream()) == 0
+        out = torch.zeros(1, nh * hd, device="cuda").half()
+        assert lib.cherryq_decode_attention_f16(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), out.data_ptr(), pos.data_ptr(),
+                                                nh, nkv, hd, ml, stream()) == 0
+        out2 = torch.zeros(1, nh * hd, device="cuda").half()
+        q2 = q.clone()
+        assert lib.cherryq_decode_rope_attention_f16(q2.data_ptr(), k.data_ptr(), v.data_ptr(), kc.data_ptr(),
+                                                     vc.data_ptr(), out2.data_ptr(), pos.data_ptr(), nh, nkv, hd, ml,
+                                                     10000.0, stream()) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(kc, kc0) and torch.equal(vc, vc0), bad
+        assert torch.isnan(out).all() and torch.isnan(out2).all(), bad
+    # the last valid position still works
+    pos = torch.tensor([ml - 1], dtype=torch.int32, device="cuda")
+    out = torch.zeros(1, nh * hd, device="cuda").half()
+    assert lib.cherryq_decode_rope_attention_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+                                                 out.data_ptr(), pos.data_ptr(), nh, nkv, hd, ml, 10000.0, stream()) == 0
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()

@@ -314,11 +314,11 @@ def test_batch_accumulate_scale_invariance_and_determinism(qc):
         assert orc.rel_l2(y1, want) <= TOL
         np.testing.assert_array_equal(run_fused(qc, bits, x, p, 128), run_fused(qc, bits, x, p, 128))
         # the generic kernel (independent code) agrees
-        os.environ["CHERRYQ_FORCE_GENERIC"] = "1"
+        qc.force_generic(True)
         try:
             yg = run_fused(qc, bits, x, p, 128)
         finally:
-            os.environ["CHERRYQ_FORCE_GENERIC"] = "0"
+            qc.force_generic(False)
         assert orc.rel_l2(run_fused(qc, bits, x, p, 128), yg) <= TOL
 
 
@@ -425,11 +425,11 @@ def test_fp32_variant_against_float64(qc, b, k, n, c, g):
     scale = np.abs(want).max()
     assert np.abs(got - want).max() <= 2e-6 * scale * np.sqrt(k / 1024)
     np.testing.assert_array_equal(got, run())           # order-independent accumulation
-    os.environ["CHERRYQ_FORCE_GENERIC"] = "1"
+    qc.force_generic(True)
     try:
         generic = run()
     finally:
-        os.environ["CHERRYQ_FORCE_GENERIC"] = "0"
+        qc.force_generic(False)
     assert np.abs(generic - want).max() <= 2e-6 * scale * np.sqrt(k / 1024)
 
 
