@@ -259,6 +259,12 @@ def decode_benchmark(prompt_len=128, new_tokens=128, w_bits=4, seed=0):
     cfg = cd.DecoderConfig(w_bits=w_bits, max_position_embeddings=prompt_len + new_tokens)
     model = cd.CherryLlamaDecoder(cfg, seed=seed)
     prompt = torch.randint(0, cfg.vocab_size, (prompt_len,), generator=torch.Generator().manual_seed(seed))
+    # first on the checkpoint layout alone, then as a loader leaves the model: the layers the
+    # library recommends it for repacked into weight streams
+    model.capture(fork=False)
+    model.generate(prompt, 8)
+    _, _, ref_total = model.generate(prompt, new_tokens)
+    repacked = model.prepack()
     model.capture(fork=False)
     model.generate(prompt, 8)                                   # warm-up
     out, _, total = model.generate(prompt, new_tokens)          # throughput: one sync at the end
@@ -285,6 +291,8 @@ def decode_benchmark(prompt_len=128, new_tokens=128, w_bits=4, seed=0):
            "hbm_gbs": round(bytes_per_token * tok_s / 1e9, 1),
            "frac_of_hbm_peak": round(bytes_per_token * tok_s / 1e9 / HBM_PEAK_GBS, 4),
            "launch": "one single-stream HIP graph per token",
+           "layers_repacked_at_load": repacked,
+           "tokens_per_s_checkpoint_layout_only": round(new_tokens / ref_total, 1),
            "prefill_ms_batched": round(prefill_batched * 1e3, 2),
            "prefill_ms_token_steps": round(prefill_steps * 1e3, 2),
            "first_tokens": out[:8].tolist()}

@@ -243,6 +243,25 @@ int cherryq_matvec_prepacked_f16(int w_bits, const void *vec, const void *stream
                                  void *hip_stream);
 
 /*
+ * The decode step's grouped launch over repacked layers (the counterpart of
+ * cherryq_decode_matvec_group_f16 below for layers held as weight streams): 1 to 3 layers that
+ * share w_bits, in_features and num_cherries and read the same (1, in_features) row -- q / k / v,
+ * gate / up, or one projection alone -- in ONE launch; layers[i].mul (+)= act W_i^T with
+ * act = vec, or norm_weight * fp16(vec * rsqrt(mean(vec^2) + eps)) when norm_weight is given
+ * (the RMSNorm in front of the projections, llama/modeling_llama_quant.py:75-89, fused into the
+ * activation staging).  No workspace.  vec and norm_weight 16-byte aligned.
+ */
+typedef struct cherryq_stream_layer {
+    const void *stream;   /* written by cherryq_prepack_f16 */
+    size_t stream_bytes;
+    void *mul;            /* (1, out_features) fp16 */
+    int out_features;
+} cherryq_stream_layer;
+int cherryq_decode_matvec_group_prepacked_f16(int w_bits, const void *vec, const void *norm_weight /* may be NULL */,
+                                              float eps, const cherryq_stream_layer *layers, int n_layers,
+                                              int in_features, int num_cherries, int accumulate, void *hip_stream);
+
+/*
  * One batch-1 launch over 1..4 packed layers that read the SAME activation vector and share
  * in_features, num_cherries, group_size and w_bits: q/k/v_proj (llama/modeling_llama_quant.py
  * :346-348 of the reference) or gate/up_proj (:251).  Arithmetic per layer is that of

@@ -92,6 +92,52 @@ def matvec_group(mods, vec, outs, vec_gate=None, accumulate=False, norm_weight=N
                                              ws.data_ptr(), ws.numel(), stream), "matvec_group")
 
 
+class _StreamLayer(ctypes.Structure):
+    _fields_ = [("stream", _vp), ("stream_bytes", ctypes.c_size_t), ("mul", _vp), ("out_features", _int)]
+
+
+_lib.cherryq_decode_matvec_group_prepacked_f16.argtypes = [_int, _vp, _vp, _f, ctypes.POINTER(_StreamLayer), _int, _int,
+                                                           _int, _int, _vp]
+_lib.cherryq_decode_matvec_group_prepacked_f16.restype = _int
+
+
+def matvec_group_prepacked(mods, vec, outs, accumulate=False, norm_weight=None, eps=1e-6):
+    """matvec_group for 1..3 QuantLinear modules that hold a repacked weight stream
+    (QuantLinear.prepack()): outs[i] (+)= act @ W_i^T in ONE launch without workspace, act = vec or
+    norm_weight * fp16(vec * rsqrt(mean(vec^2) + eps))."""
+    m0 = mods[0]
+    k, c = vec.shape[1], m0.cherry_indices.shape[0]
+    for m, o in zip(mods, outs):
+        st = getattr(m, "_stream", None)
+        if st is None:
+            raise RuntimeError("matvec_group_prepacked: every layer must have been prepack()ed")
+        if (m.w_bits, m.cherry_indices.shape[0], m.in_features) != (m0.w_bits, c, k):
+            raise RuntimeError("matvec_group_prepacked: the layers must share w_bits, num_cherries and in_features")
+        if (not o.is_cuda or o.dtype != torch.float16 or not o.is_contiguous() or o.device != vec.device
+                or tuple(o.shape) != (1, m.out_features) or st.device != vec.device):
+            raise RuntimeError("matvec_group_prepacked: outputs must be contiguous (1, out_features) fp16 tensors on vec's GPU")
+    if tuple(vec.shape) != (1, k) or vec.dtype != torch.float16 or not vec.is_cuda or not vec.is_contiguous():
+        raise RuntimeError("matvec_group_prepacked: vec must be a contiguous (1, in_features) fp16 GPU tensor")
+    if norm_weight is not None and (tuple(norm_weight.shape) != (k,) or norm_weight.dtype != torch.float16
+                                    or not norm_weight.is_cuda or not norm_weight.is_contiguous()):
+        raise RuntimeError("matvec_group_prepacked: norm_weight must be a contiguous (in_features,) fp16 GPU tensor")
+    arr = (_StreamLayer * len(mods))(*[_StreamLayer(m._stream.data_ptr(), m._stream.numel(), o.data_ptr(), m.out_features)
+                                       for m, o in zip(mods, outs)])
+    _ok(_lib.cherryq_decode_matvec_group_prepacked_f16(m0.w_bits, vec.data_ptr(),
+                                                       None if norm_weight is None else norm_weight.data_ptr(), eps, arr,
+                                                       len(mods), k, c, 1 if accumulate else 0, _stream()),
+        "matvec_group_prepacked")
+
+
+def _group(mods, vec, outs, accumulate=False, norm_weight=None, eps=1e-6):
+    """The grouped launch over whichever layout the layers hold: the repacked streams when every
+    layer of the group has one, the checkpoint layout otherwise."""
+    if all(getattr(m, "_stream", None) is not None for m in mods):
+        matvec_group_prepacked(mods, vec, outs, accumulate=accumulate, norm_weight=norm_weight, eps=eps)
+    else:
+        matvec_group(mods, vec, outs, accumulate=accumulate, norm_weight=norm_weight, eps=eps)
+
+
 def _ok(rc, what):
     if rc != 0:
         quant_cuda._fail(rc, what)
@@ -229,6 +275,31 @@ class CherryLlamaDecoder(nn.Module):
                 raise ValueError(f"{k}: checkpoint has {tuple(src.shape)} {src.dtype}, "
                                  f"decoder expects {tuple(dst.shape)} {dst.dtype}")
             dst.copy_(src)
+        for layer in self.layers:  # streams repacked from the previous weights are stale
+            for m in layer.children():
+                m._stream = None
+        self._graph = None
+
+    def prepack(self, only_recommended=True):
+        """Repack, once, every linear whose shape the library recommends it for (those of at most
+        4096 quantised input channels on MI355X: q / k / v / o / gate / up of a 7B model) into the
+        weight stream the batch-1 kernel reads fastest; the token step then uses the stream kernels
+        for them.  The checkpoint-layout buffers stay (the batched prompt pass reads them).
+        Returns the number of layers repacked."""
+        n = 0
+        for layer in self.layers:
+            for m in layer.children():
+                if only_recommended and not quant_cuda.prepack_recommended(m.w_bits, m.in_features, m.out_features,
+                                                                           m.num_cherries, m.group_size):
+                    continue
+                n += bool(m.prepack())
+        self._graph = None
+        return n
+
+    def unprepack(self):
+        for layer in self.layers:
+            for m in layer.children():
+                m.unprepack()
         self._graph = None
 
     # ---- packed bytes a token step must read (for the roofline of tokens/s)
@@ -270,22 +341,22 @@ class CherryLlamaDecoder(nn.Module):
         for li, layer in enumerate(self.layers):
             qkv, gu = [layer.q_proj, layer.k_proj, layer.v_proj], [layer.gate_proj, layer.up_proj]
             if self.fuse_norm:
-                matvec_group(qkv, self.hid, [self.q, self.k, self.v], norm_weight=layer.input_layernorm,
-                             eps=cfg.rms_norm_eps)
+                _group(qkv, self.hid, [self.q, self.k, self.v], norm_weight=layer.input_layernorm,
+                       eps=cfg.rms_norm_eps)
             else:
                 self._norm(layer.input_layernorm)
-                matvec_group(qkv, self.normed, [self.q, self.k, self.v])
+                _group(qkv, self.normed, [self.q, self.k, self.v])
             _ok(_lib.cherryq_decode_rope_attention_f16(self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(),
                                                        self.k_cache[li].data_ptr(), self.v_cache[li].data_ptr(),
                                                        self.attn.data_ptr(), self.pos.data_ptr(), nh, nkv, hd, ml,
                                                        cfg.rope_theta, _stream()), "rope_attention")
-            matvec_group([layer.o_proj], self.attn, [self.hid], accumulate=True)
+            _group([layer.o_proj], self.attn, [self.hid], accumulate=True)
             if self.fuse_norm:
-                matvec_group(gu, self.hid, [self.gate, self.up], norm_weight=layer.post_attention_layernorm,
-                             eps=cfg.rms_norm_eps)
+                _group(gu, self.hid, [self.gate, self.up], norm_weight=layer.post_attention_layernorm,
+                       eps=cfg.rms_norm_eps)
             else:
                 self._norm(layer.post_attention_layernorm)
-                matvec_group(gu, self.normed, [self.gate, self.up])
+                _group(gu, self.normed, [self.gate, self.up])
             matvec_group([layer.down_proj], self.up, [self.hid], vec_gate=self.gate, accumulate=True)
             if self.layer_trace is not None:  # validation only (eager runs): the hidden state after every layer
                 self.layer_trace.append(self.hid.clone())

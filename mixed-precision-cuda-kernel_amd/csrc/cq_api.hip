@@ -464,6 +464,31 @@ int cherryq_matvec_prepacked_f16(int w_bits, const void *vec, const void *stream
                                   reinterpret_cast<hipStream_t>(hip_stream));
 }
 
+int cherryq_decode_matvec_group_prepacked_f16(int w_bits, const void *vec, const void *norm_weight, float eps,
+                                              const cherryq_stream_layer *layers, int n_layers, int in_features,
+                                              int num_cherries, int accumulate, void *hip_stream) {
+    if (w_bits != 3 && w_bits != 4) return CHERRYQ_E_BITS;
+    if (!layers || !vec) return CHERRYQ_E_NULL;
+    if (n_layers < 1 || n_layers > cq::kStreamMaxGroup) return CHERRYQ_E_SHAPE;
+    if (!cq::aligned(vec, 16) || (norm_weight && !cq::aligned(norm_weight, 16))) return CHERRYQ_E_ALIGN;
+    cq::StreamMember members[cq::kStreamMaxGroup];
+    int outs[cq::kStreamMaxGroup];
+    for (int i = 0; i < n_layers; i++) {
+        const cherryq_stream_layer &l = layers[i];
+        const int rc = prepack_check(w_bits, in_features, l.out_features, num_cherries, cq::kStreamUnitK, l.stream_bytes);
+        if (rc) return rc;
+        if (!l.stream || !l.mul) return CHERRYQ_E_NULL;
+        if (!cq::aligned(l.stream, 256) || !cq::aligned(l.mul, 2)) return CHERRYQ_E_ALIGN;
+        members[i] = {reinterpret_cast<const uint8_t *>(l.stream), reinterpret_cast<__half *>(l.mul), l.out_features};
+        outs[i] = l.out_features;
+    }
+    if (!cq::stream_group_supported(w_bits, in_features, num_cherries, cq::kStreamUnitK, outs, n_layers))
+        return CHERRYQ_E_UNSUPPORTED;
+    return (int)cq::launch_stream_group(w_bits, reinterpret_cast<const __half *>(vec),
+                                        reinterpret_cast<const __half *>(norm_weight), eps, members, n_layers,
+                                        in_features, num_cherries, accumulate, reinterpret_cast<hipStream_t>(hip_stream));
+}
+
 // ---- decode-step entry points (see include/cherryq.h) ------------------------------------------
 
 size_t cherryq_group_workspace_bytes(int n_layers, const int *out_features) {

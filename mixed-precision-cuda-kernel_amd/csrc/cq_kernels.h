@@ -108,7 +108,23 @@ struct StreamGeo {
     uint32_t off_cherry, off_units, record_bytes;  // byte offsets inside a tile record, record size
     uint32_t hdr_bytes;                             // gather table + cherry columns in front of the tiles
 };
+constexpr int kStreamMaxGroup = 3;
+struct StreamMember {  // one layer of a group launch
+    const uint8_t *stream;
+    __half *mul;
+    int N;
+};
+struct StreamGroup {  // kernel argument: the members' streams, outputs, widths and first workgroups
+    const uint8_t *stream[kStreamMaxGroup];
+    __half *mul[kStreamMaxGroup];
+    int N[kStreamMaxGroup];
+    int tile_begin[kStreamMaxGroup];
+    int count;
+};
 StreamGeo stream_geo(int bits, int K, int N, int C);
+hipError_t launch_stream_group(int bits, const __half *vec, const __half *norm_w, float eps,
+                               const StreamMember *members, int count, int K, int C, int accumulate, hipStream_t s);
+bool stream_group_supported(int bits, int K, int C, int G, const int *Ns, int count);
 size_t stream_bytes(int bits, int K, int N, int C);
 bool stream_faster(int bits, int K, int N, int C);
 bool stream_supported(int bits, int B, int K, int N, int C, int G);

@@ -46,7 +46,11 @@ typedef _Float16 sh2_t __attribute__((ext_vector_type(2)));
 
 constexpr uint32_t kSFlags = 0x00020000u;
 constexpr uint32_t kSOob = 0x80000000u;
-constexpr int kStreamMaxXLoads = 4;  // 16-byte loads of raw activations per thread
+// 16-byte loads of raw activations per thread that cover the longest row a geometry takes
+// (max_units units of 128 positions plus up to 128 cherry channels) with NT threads
+__host__ __device__ constexpr int stream_x_loads(int max_units, int nt) {
+    return (max_units * 128 + 128 + nt * 8 - 1) / (nt * 8);
+}
 constexpr int kStreamRawPad = 512 + 128 + 8;  // zero halves kept behind the raw activations in LDS
 
 static inline uint32_t align256(uint32_t v) { return (v + 255u) & ~255u; }
@@ -273,6 +277,19 @@ __device__ inline float unit_dot(const su4 w, const unsigned short *xa) {
     }
 }
 
+// weight * fp16(x * rs) on both halves of a pair (the rounding points of add_rmsnorm_kernel)
+__device__ inline uint32_t stream_norm_pair(uint32_t xp, uint32_t wp, float rs) {
+    uint32_t r = 0;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const float xv = __half2float(__ushort_as_half((unsigned short)(xp >> (16 * i))));
+        const float wv = __half2float(__ushort_as_half((unsigned short)(wp >> (16 * i))));
+        const float nv = __half2float(__float2half_rn(xv * rs));
+        r |= (uint32_t)__half_as_ushort(__float2half_rn(wv * nv)) << (16 * i);
+    }
+    return r;
+}
+
 // A workgroup is W computing wavefronts plus S staging wavefronts and owns T tiles (W % T == 0):
 // computing wavefront w works on tile w % T and takes the units g = w / T, w / T + W / T, ... of it
 // (at most L), D loads in flight.  Staging wavefront j prepares NB consecutive blocks of 512
@@ -289,12 +306,37 @@ __device__ inline float unit_dot(const su4 w, const unsigned short *xa) {
 // activations for the grid offset, and raise a counter in LDS; (3) a computing wavefront looks
 // at the counter when its loads are queued, then consumes its units in order, refilling every
 // slot it frees.
-template <int BITS, int W, int T, int D, int L, int S, int NB>
-__global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__restrict__ x,
-                                                              const uint8_t *__restrict__ stream,
-                                                              __half *__restrict__ mul, int accumulate,
-                                                              StreamGeo geo) {
+//
+// Up to kStreamMaxGroup layers that read the same activation row (q / k / v, gate / up) share
+// one launch: consecutive ranges of workgroups belong to consecutive members, each with its own
+// stream (header and tile records) and output.  NORM: the row is RMS-normalised while it is
+// staged -- norm_w * fp16(x * rsqrt(mean(x^2) + eps)), the rounding points of the decoder's
+// separate norm kernel -- at the price of one more workgroup barrier.
+template <int BITS, int W, int T, int D, int L, int S, int NB, int XL, bool NORM, bool GROUP>
+__global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__restrict__ x, StreamGroup grp,
+                                                              const __half *__restrict__ norm_w, float eps,
+                                                              int accumulate, StreamGeo geo) {
     static_assert(L % 4 == 0 && W % T == 0 && D <= L, "");
+    // Which member this workgroup works for.  Every member's fields are first pinned in scalar
+    // registers: left to itself the compiler turns the selects into ONE load at a selected
+    // kernel-argument address, i.e. a second, dependent memory round trip in front of the header
+    // loads (measured: +1.1 us on the 4096 -> 11008 layer).  A single layer skips all of it.
+    const int bid = blockIdx.x;
+    const uint8_t *__restrict__ stream = grp.stream[0];
+    __half *__restrict__ mul = grp.mul[0];
+    int N = grp.N[0], wg = bid;
+    if constexpr (GROUP) {
+        const uint8_t *s1 = grp.stream[1], *s2 = grp.stream[2];
+        __half *o1 = grp.mul[1], *o2 = grp.mul[2];
+        int n1 = grp.N[1], n2 = grp.N[2], t1 = grp.tile_begin[1], t2 = grp.tile_begin[2], cnt = grp.count;
+        asm volatile("" : "+s"(stream), "+s"(s1), "+s"(s2), "+s"(mul), "+s"(o1), "+s"(o2));
+        asm volatile("" : "+s"(N), "+s"(n1), "+s"(n2), "+s"(t1), "+s"(t2), "+s"(cnt));
+        const bool m1 = cnt > 1 && bid >= t1, m2 = cnt > 2 && bid >= t2;
+        stream = m2 ? s2 : m1 ? s1 : stream;
+        mul = m2 ? o2 : m1 ? o1 : mul;
+        N = m2 ? n2 : m1 ? n1 : N;
+        wg = bid - (m2 ? t2 : m1 ? t1 : 0);  // workgroup index within the member
+    }
     constexpr int WT = W / T;
     constexpr int NT = 64 * (W + S);
     constexpr int UB = BITS == 4 ? 1024 : 768;
@@ -304,7 +346,7 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kq = lane >> 4, nn = lane & 15;
     const bool stager = wave >= W;
-    const int K = geo.K, C = geo.C, ng = geo.ng, N = geo.N;
+    const int K = geo.K, C = geo.C, ng = geo.ng;
     const int Knp = ng * kStreamUnitK;
     const int Cp = (C + 31) & ~31;
     const int Knp512 = (Knp + 511) & ~511;
@@ -318,12 +360,12 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
     float *s_red = s_xsum + 4 * nblk;
 
     // ---- (1) raw activations, everyone; gather table and cherry columns, staging wavefronts
-    su4 xr[kStreamMaxXLoads];
+    su4 xr[XL];
     su2 tb[NB];
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, K * 2, kSFlags);
     const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc((void *)stream, 0, (int)geo.hdr_bytes, kSFlags);
 #pragma unroll
-    for (int i = 0; i < kStreamMaxXLoads; i++)
+    for (int i = 0; i < XL; i++)
         if (i * NT * 8 < K) xr[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, (uint32_t)(tid + i * NT) * 16u, 0, 0);
     const int ws = wave - W;  // index among the staging wavefronts
     const int b0 = ws * NB, b1 = min(nblk, b0 + NB);
@@ -337,8 +379,46 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
             ci1 = __builtin_amdgcn_raw_buffer_load_b16(rh, lane + 64 < Cp ? (uint32_t)(Knp512 + (lane + 64) * 2) : kSOob, 0, 0);
         }
     }
+    if constexpr (NORM) {
+        su4 nr[XL];
+        const __amdgpu_buffer_rsrc_t rn = __builtin_amdgcn_make_buffer_rsrc((void *)norm_w, 0, K * 2, kSFlags);
 #pragma unroll
-    for (int i = 0; i < kStreamMaxXLoads; i++)
+        for (int i = 0; i < XL; i++)
+            if (i * NT * 8 < K) nr[i] = __builtin_amdgcn_raw_buffer_load_b128(rn, (uint32_t)(tid + i * NT) * 16u, 0, 0);
+        float ss = 0.f;  // pieces past K read as zeros
+#pragma unroll
+        for (int i = 0; i < XL; i++)
+            if (i * NT * 8 < K) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const float a = __half2float(__ushort_as_half((unsigned short)(xr[i][j] & 0xffffu)));
+                    const float b = __half2float(__ushort_as_half((unsigned short)(xr[i][j] >> 16)));
+                    ss += a * a + b * b;
+                }
+            }
+        ss = wave_sum_all(ss);
+        if (lane == 0) s_red[wave] = ss;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+        float t = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < W + S; wv++) t += s_red[wv];
+        const float rs = rsqrtf(t / (float)K + eps);
+        // one dword at a time (the scheduling barriers keep the temporaries of different dwords
+        // from being live together: this phase must not set the kernel's register count)
+#pragma unroll
+        for (int i = 0; i < XL; i++)
+            if (i * NT * 8 < K) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    xr[i][j] = stream_norm_pair(xr[i][j], nr[i][j], rs);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+    }
+#pragma unroll
+    for (int i = 0; i < XL; i++)
         if (i * NT * 8 < K && (tid + i * NT) * 8 < K) reinterpret_cast<su4 *>(s_raw)[tid + i * NT] = xr[i];
     // zeros behind the activations: what padding positions (and padded cherry columns) read
     if (tid < kStreamRawPad / 8) reinterpret_cast<su4 *>(s_raw)[(K >> 3) + tid] = (su4){0u, 0u, 0u, 0u};
@@ -385,8 +465,8 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
         // quarter of the units; the quarters are added at the end).  Every unit of a tile past the
         // last reads zeros through an empty descriptor.
         const int tl = wave % T, cls = wave / T;
-        const int tile = blockIdx.x * T + tl;
-        const bool tile_ok = tile < geo.ntiles;
+        const int tile = wg * T + tl;
+        const bool tile_ok = tile * kStreamTileCols < N;
         const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(
             (void *)(stream + geo.hdr_bytes + (size_t)(tile_ok ? tile : 0) * geo.record_bytes), 0,
             tile_ok ? (int)geo.record_bytes : 0, kSFlags);
@@ -457,7 +537,7 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     if (tid < 16 * T) {
-        const int otl = tid >> 4, n = (blockIdx.x * T + otl) * 16 + (tid & 15);
+        const int otl = tid >> 4, n = (wg * T + otl) * 16 + (tid & 15);
         if (n < N) {
             float v = 0.f;
 #pragma unroll
@@ -482,8 +562,8 @@ struct StreamCfg {
     int W, T, D, L, S, NB, max_units;
 };
 static constexpr StreamCfg kStreamCfgs[] = {
-    {4, 1, 8, 8, 1, 8, 32},    // 0: K <= 4096 + cherries, 4-bit, more tiles than compute units
-    {4, 1, 8, 8, 4, 2, 32},    // 1: the same, 3-bit
+    {4, 1, 8, 8, 1, 8, 32},    // 0: K <= 4096 + cherries, 4-bit, a few tiles per compute unit
+    {4, 1, 8, 8, 4, 2, 32},    // 1: the same, 3-bit; both widths from about four tiles per compute unit
     {8, 1, 4, 4, 4, 2, 32},    // 2: K <= 4096 + cherries, about one tile per compute unit
     {4, 1, 8, 12, 4, 4, 48},   // 3
     {8, 1, 8, 8, 4, 4, 64},    // 4
@@ -494,9 +574,16 @@ constexpr int kStreamCfgCount = sizeof(kStreamCfgs) / sizeof(kStreamCfgs[0]);
 
 
 static int stream_pick(const StreamGeo &geo) {
-    // Measured on 4096 -> 11008 / 4096 -> 4096 (us per launch, 4-bit / 3-bit): entry 0 6.54 / 6.53 and
-    // 5.16 / 5.37, entry 1 6.78 / 6.51 and 4.42 / 4.48, entry 2 7.52 / 7.19 and 4.18 / 4.12.
-    if (geo.ng <= 32) return geo.ntiles <= 320 ? 2 : (geo.bits == 4 ? 0 : 1);
+    // Measured (us per launch, 4-bit / 3-bit): 4096 -> 11008 (688 tiles): entry 0 6.46 / 6.51, entry 1
+    // 6.74 / 6.51, entry 2 8.36 / 7.70; 4096 -> 4096 (256 tiles): 5.08, 4.32, 4.32 (4-bit); RMSNorm +
+    // 3 x (4096 -> 4096) in one launch (768 tiles): 7.48, 7.56, 9.20; RMSNorm + 2 x (4096 -> 11008)
+    // (1376 tiles, more than one round of entry 0's workgroups): 15.0, 12.7, 14.6.  Two tiles per
+    // workgroup (one staging wavefront for both) measured 12.9 there and 10.6 on 688 tiles.
+    if (geo.ng <= 32) {
+        if (geo.ntiles <= 320) return 2;
+        if (geo.ntiles > 1000) return 1;
+        return geo.bits == 4 ? 0 : 1;
+    }
     for (int i = 3; i < kStreamCfgCount; i++)
         if (geo.ng <= kStreamCfgs[i].max_units) return i;
     return -1;
@@ -523,48 +610,104 @@ bool stream_supported(int bits, int B, int K, int N, int C, int G) {
     return stream_lds_bytes(geo, kStreamCfgs[i].W) <= 160 * 1024;
 }
 
-template <int BITS, int I>
-static hipError_t launch_stream_cfg(const __half *vec, const uint8_t *stream, __half *mul, int accumulate,
-                                    const StreamGeo &geo, hipStream_t s) {
+template <int BITS, int I, bool NORM>
+static hipError_t launch_stream_cfg(const __half *vec, const StreamGroup &grp, const __half *norm_w, float eps,
+                                    int accumulate, const StreamGeo &geo, hipStream_t s) {
     constexpr StreamCfg c = kStreamCfgs[I];
     // what the kernel's fixed-size register arrays assume
-    if (geo.ng * kStreamUnitK > c.NB * 512 * c.S || geo.K > kStreamMaxXLoads * 8 * 64 * (c.W + c.S) ||
+    constexpr int XL = stream_x_loads(c.max_units, 64 * (c.W + c.S));
+    if (geo.ng * kStreamUnitK > c.NB * 512 * c.S || geo.K > XL * 8 * 64 * (c.W + c.S) || geo.ng > c.max_units ||
         ceil_div(geo.ng, c.W / c.T) > c.L)
         return hipErrorInvalidValue;
     const size_t lds = stream_lds_bytes(geo, c.W);
     if (lds > 160 * 1024) return hipErrorInvalidValue;
-    auto kern = stream_kernel<BITS, c.W, c.T, c.D, c.L, c.S, c.NB>;
-    static bool big_lds_enabled = false;  // (per instantiation; the attribute is idempotent, a race only repeats the call)
+    auto kern_one = stream_kernel<BITS, c.W, c.T, c.D, c.L, c.S, c.NB, XL, NORM, false>;
+    auto kern_grp = stream_kernel<BITS, c.W, c.T, c.D, c.L, c.S, c.NB, XL, NORM, true>;
+    static bool big_lds_enabled = false;  // (per instantiation; the attribute is idempotent, a race only repeats the calls)
     if (lds > 48 * 1024 && !big_lds_enabled) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return e;
+        for (const void *k : {reinterpret_cast<const void *>(kern_one), reinterpret_cast<const void *>(kern_grp)}) {
+            hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return e;
+        }
         big_lds_enabled = true;
     }
-    const dim3 grid(ceil_div(geo.ntiles, c.T)), block(64 * (c.W + c.S));
-    hipLaunchKernelGGL(kern, grid, block, lds, s, vec, stream, mul, accumulate, geo);
+    auto kern = grp.count > 1 ? kern_grp : kern_one;
+    // members are told apart by workgroup index: each starts at a workgroup of its own
+    StreamGroup g = grp;
+    int wgs = 0;
+    for (int i = 0; i < kStreamMaxGroup; i++) {
+        g.tile_begin[i] = wgs;
+        if (i < grp.count) wgs += ceil_div(ceil_div(grp.N[i], kStreamTileCols), c.T);
+    }
+    const dim3 grid(wgs), block(64 * (c.W + c.S));
+    hipLaunchKernelGGL(kern, grid, block, lds, s, vec, g, norm_w, eps, accumulate, geo);
     return hipGetLastError();
 }
 
-template <int BITS>
-static hipError_t launch_stream_bits(const __half *vec, const uint8_t *stream, __half *mul, int accumulate,
-                                     const StreamGeo &geo, hipStream_t s) {
+template <int BITS, bool NORM>
+static hipError_t launch_stream_bits(const __half *vec, const StreamGroup &grp, const __half *norm_w, float eps,
+                                     int accumulate, const StreamGeo &geo, hipStream_t s) {
     switch (stream_pick(geo)) {
-        case 0: return launch_stream_cfg<BITS, 0>(vec, stream, mul, accumulate, geo, s);
-        case 1: return launch_stream_cfg<BITS, 1>(vec, stream, mul, accumulate, geo, s);
-        case 2: return launch_stream_cfg<BITS, 2>(vec, stream, mul, accumulate, geo, s);
-        case 3: return launch_stream_cfg<BITS, 3>(vec, stream, mul, accumulate, geo, s);
-        case 4: return launch_stream_cfg<BITS, 4>(vec, stream, mul, accumulate, geo, s);
-        case 5: return launch_stream_cfg<BITS, 5>(vec, stream, mul, accumulate, geo, s);
-        case 6: return launch_stream_cfg<BITS, 6>(vec, stream, mul, accumulate, geo, s);
+        case 0: return launch_stream_cfg<BITS, 0, NORM>(vec, grp, norm_w, eps, accumulate, geo, s);
+        case 1: return launch_stream_cfg<BITS, 1, NORM>(vec, grp, norm_w, eps, accumulate, geo, s);
+        case 2: return launch_stream_cfg<BITS, 2, NORM>(vec, grp, norm_w, eps, accumulate, geo, s);
+        case 3: return launch_stream_cfg<BITS, 3, NORM>(vec, grp, norm_w, eps, accumulate, geo, s);
+        case 4: return launch_stream_cfg<BITS, 4, NORM>(vec, grp, norm_w, eps, accumulate, geo, s);
+        case 5: return launch_stream_cfg<BITS, 5, NORM>(vec, grp, norm_w, eps, accumulate, geo, s);
+        case 6: return launch_stream_cfg<BITS, 6, NORM>(vec, grp, norm_w, eps, accumulate, geo, s);
         default: return hipErrorInvalidValue;
     }
 }
 
+// `count` layers (at most kStreamMaxGroup) of the same bits / K / C that read the same activation
+// row, in one launch; norm_w != nullptr fuses the RMSNorm of that row.
+hipError_t launch_stream_group(int bits, const __half *vec, const __half *norm_w, float eps,
+                               const StreamMember *members, int count, int K, int C, int accumulate, hipStream_t s) {
+    if (count < 1 || count > kStreamMaxGroup) return hipErrorInvalidValue;
+    StreamGroup grp = {};
+    grp.count = count;
+    int tiles = 0, n_total = 0;
+    for (int i = 0; i < kStreamMaxGroup; i++) {
+        const StreamMember &m = members[i < count ? i : 0];
+        grp.stream[i] = m.stream;
+        grp.mul[i] = m.mul;
+        grp.N[i] = m.N;
+        grp.tile_begin[i] = tiles;
+        if (i < count) {
+            tiles += ceil_div(m.N, kStreamTileCols);
+            n_total += m.N;
+        }
+    }
+    // the geometry of one member (records, header) with the launch's total tile count
+    StreamGeo geo = stream_geo(bits, K, members[0].N, C);
+    geo.N = n_total;
+    geo.ntiles = tiles;
+    if (bits == 4)
+        return norm_w ? launch_stream_bits<4, true>(vec, grp, norm_w, eps, accumulate, geo, s)
+                      : launch_stream_bits<4, false>(vec, grp, nullptr, 0.f, accumulate, geo, s);
+    return norm_w ? launch_stream_bits<3, true>(vec, grp, norm_w, eps, accumulate, geo, s)
+                  : launch_stream_bits<3, false>(vec, grp, nullptr, 0.f, accumulate, geo, s);
+}
+
 hipError_t launch_stream(int bits, const __half *vec, const uint8_t *stream, __half *mul, int K, int N, int C,
                          int accumulate, hipStream_t s) {
-    const StreamGeo geo = stream_geo(bits, K, N, C);
-    if (bits == 4) return launch_stream_bits<4>(vec, stream, mul, accumulate, geo, s);
-    return launch_stream_bits<3>(vec, stream, mul, accumulate, geo, s);
+    const StreamMember m = {stream, mul, N};
+    return launch_stream_group(bits, vec, nullptr, 0.f, &m, 1, K, C, accumulate, s);
+}
+
+// Whether a group launch takes these layers (each must be supported on its own; the launch
+// geometry follows the total number of tiles).
+bool stream_group_supported(int bits, int K, int C, int G, const int *Ns, int count) {
+    if (count < 1 || count > kStreamMaxGroup) return false;
+    int tiles = 0;
+    for (int i = 0; i < count; i++) {
+        if (!stream_supported(bits, 1, K, Ns[i], C, G)) return false;
+        tiles += ceil_div(Ns[i], kStreamTileCols);
+    }
+    StreamGeo geo = stream_geo(bits, K, Ns[0], C);
+    geo.ntiles = tiles;
+    const int i = stream_pick(geo);
+    return i >= 0 && stream_lds_bytes(geo, kStreamCfgs[i].W) <= 160 * 1024;
 }
 
 hipError_t launch_stream_pack(int bits, const uint8_t *qweight, const __half *cherry_weight,

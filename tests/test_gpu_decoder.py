@@ -231,6 +231,21 @@ def test_small_decoder_matches_dense_reference(dec, bits):
         _ = model.reference_logits(ids[:4])  # unrelated eager work between replays
         graph2 = model.step_logits(ids, use_graph=True, fork=fork, grouped=grouped)
         assert torch.equal(graph, eager) and torch.equal(graph2, eager), (fork, grouped)
+    # every linear repacked into a weight stream: the stream kernels take the grouped launches
+    model._graph = None
+    model.fuse_norm = True
+    assert model.prepack(only_recommended=False) == 14
+    for fuse_norm in (True, False):
+        model.fuse_norm = fuse_norm
+        model._graph = None
+        eager = model.step_logits(ids, use_graph=False)
+        for t in range(ids.numel()):
+            assert rel(eager[t], want[t]) < 2e-2, (t, "prepacked", fuse_norm)
+        graph = model.step_logits(ids, use_graph=True)
+        _ = model.reference_logits(ids[:4])
+        graph2 = model.step_logits(ids, use_graph=True)
+        assert torch.equal(graph, eager) and torch.equal(graph2, eager), ("prepacked", fuse_norm)
+    model.unprepack()
     model._graph = None
     model.fuse_norm = True
     out, times, total = model.generate(ids[:4], 8, use_graph=True)

@@ -131,6 +131,13 @@ def test_full_size_7b_decoder_against_the_c_oracle():
     r0, r7 = rel(dev_logits[0], want[0]), rel(dev_logits[steps - 1], want[steps - 1])
     print(f"  worst per-layer rel-L2 {worst:.3e}; logits rel-L2 step 0 {r0:.3e}, step {steps - 1} {r7:.3e}", flush=True)
     assert r0 <= LOGIT_TOL and r7 <= LOGIT_TOL
+    # the same model as a loader leaves it (q / k / v / o / gate / up repacked into weight streams):
+    # the captured step now runs the stream kernels for them
+    assert model.prepack() == 6 * cfg.num_hidden_layers
+    pre_logits = model.step_logits(ids, use_graph=True).cpu().numpy()
+    p0, p7 = rel(pre_logits[0], want[0]), rel(pre_logits[steps - 1], want[steps - 1])
+    print(f"  repacked: logits rel-L2 step 0 {p0:.3e}, step {steps - 1} {p7:.3e}", flush=True)
+    assert p0 <= LOGIT_TOL and p7 <= LOGIT_TOL
     # the device's greedy choice is (within the tolerance) the oracle's maximum
     for t in (0, steps - 1):
         j = int(dev_logits[t].argmax())

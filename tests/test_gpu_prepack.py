@@ -220,3 +220,89 @@ def test_prepacked_c_abi_rejections(qc):
     assert f(4, None, buf.data_ptr(), nbytes, y.data_ptr(), 1, 4096, 1024, 16, 0, None) == -1
     assert f(4, x.data_ptr() + 2, buf.data_ptr(), nbytes, y.data_ptr(), 1, 4096, 1024, 16, 0, None) == -6
     assert f(2, x.data_ptr(), buf.data_ptr(), nbytes, y.data_ptr(), 1, 4096, 1024, 16, 0, None) == -5
+
+
+@pytest.mark.parametrize("bits", [4, 3])
+@pytest.mark.parametrize("case", ["qkv_norm", "gate_up_norm", "o_accumulate", "qkv_plain"])
+def test_prepacked_group_llama7b_shapes_against_the_c_oracle(bits, case):
+    """The grouped launch over repacked layers at the decoder's shapes -- 3 x (4096 -> 4096) and
+    2 x (4096 -> 11008) behind the fused RMSNorm, 4096 -> 4096 accumulating into the output -- against
+    the C oracle's fused product of the prologue's result, and bit for bit on activations whose
+    normalised form is one-hot."""
+    import cherryq_decoder as dec
+    print("[case] prepacked group", bits, case, flush=True)
+    K, widths = {"qkv_norm": (4096, (4096, 4096, 4096)), "gate_up_norm": (4096, (11008, 11008)),
+                 "o_accumulate": (4096, (4096,)), "qkv_plain": (4096, (4096, 1024, 1024))}[case]
+    gen = torch.Generator(device="cuda").manual_seed(23 + bits)
+    cfg = dec.DecoderConfig(w_bits=bits, group_size=128, cherry_fraction=1 / 256)
+    mods = [dec.random_packed_linear(cfg, K, n, gen, "cuda") for n in widths]
+    for m in mods:
+        assert m.prepack()
+    packed = [{b: getattr(m, b).cpu().numpy() for b in ("qweight", "scales", "cherry_weight", "cherry_indices")} for m in mods]
+    f16 = lambda a: np.asarray(a).astype(np.float16)
+    rng = np.random.default_rng(9)
+
+    def run(vec, base=None, **kw):
+        outs = [torch.full((1, n), 7.0, dtype=torch.float16, device="cuda") if base is None else
+                torch.from_numpy(base[i]).cuda() for i, n in enumerate(widths)]
+        dec.matvec_group_prepacked(mods, torch.from_numpy(vec).cuda(), outs, **kw)
+        torch.cuda.synchronize()
+        return [o.cpu().numpy() for o in outs]
+
+    if case.endswith("norm"):
+        eps = 1e-6
+        h = f16(rng.standard_normal((1, K)) * 3)
+        nw = f16(rng.random(K) + 0.5)
+        hf = h.astype(np.float64)
+        act = f16(nw.astype(np.float64) * f16(hf / np.sqrt(np.mean(hf * hf) + eps)).astype(np.float64))
+        got = run(h, norm_weight=torch.from_numpy(nw).cuda(), eps=eps)
+        for o, p in zip(got, packed):
+            assert orc.rel_l2(o, c_oracle.fused(act, p, bits, 128)) <= 1e-3
+        # and the launch over the checkpoint layout with the same prologue agrees
+        outs = [torch.empty(1, n, dtype=torch.float16, device="cuda") for n in widths]
+        dec.matvec_group(mods, torch.from_numpy(h).cuda(), outs, norm_weight=torch.from_numpy(nw).cuda(), eps=eps)
+        torch.cuda.synchronize()
+        for o, r in zip(got, outs):
+            assert orc.rel_l2(o, r.cpu().numpy().astype(np.float64)) <= 5e-4
+        # one-hot through the norm: mean(x^2) + eps = 1 for x = e_j and eps = 1 - 1/K
+        nw2 = f16(2.0 ** rng.integers(-2, 3, K))
+        for j in (0, 1, 127, 128, 2049, K - 1, int(packed[0]["cherry_indices"][0]), int(packed[-1]["cherry_indices"][-1])):
+            x = np.zeros((1, K), dtype=np.float16)
+            x[0, j] = 1
+            got = run(x, norm_weight=torch.from_numpy(nw2).cuda(), eps=1.0 - 1.0 / K)
+            xa = np.zeros((1, K), dtype=np.float16)
+            xa[0, j] = nw2[j]
+            for o, p in zip(got, packed):
+                with np.errstate(over="ignore"):
+                    np.testing.assert_array_equal(o[0], f16(c_oracle.fused(xa, p, bits, 128)[0]), err_msg=f"column {j}")
+    else:
+        x = f16(rng.standard_normal((1, K)))
+        acc = case == "o_accumulate"
+        base = [f16(rng.standard_normal((1, n))) for n in widths] if acc else None
+        got = run(x, base=base, accumulate=acc)
+        for i, (o, p) in enumerate(zip(got, packed)):
+            want = c_oracle.fused(x, p, bits, 128) + (base[i].astype(np.float64) if acc else 0.0)
+            assert orc.rel_l2(o, want) <= 1e-3
+        for j in (0, 129, K - 1, int(packed[0]["cherry_indices"][3])):
+            e = np.zeros((1, K), dtype=np.float16)
+            e[0, j] = 1
+            got = run(e, base=base, accumulate=acc)
+            for i, (o, p) in enumerate(zip(got, packed)):
+                want = c_oracle.fused(e, p, bits, 128) + (base[i].astype(np.float64) if acc else 0.0)
+                np.testing.assert_array_equal(o, f16(want), err_msg=f"column {j} member {i}")
+
+
+def test_prepacked_group_rejections():
+    import cherryq_decoder as dec
+    lib = dec._lib
+    fake = 1 << 12
+    one = (dec._StreamLayer * 1)(dec._StreamLayer(fake, 1 << 30, fake, 4096))
+    four = (dec._StreamLayer * 4)(*[dec._StreamLayer(fake, 1 << 30, fake, 4096)] * 4)
+    f = lib.cherryq_decode_matvec_group_prepacked_f16
+    assert f(5, fake, None, 0.0, one, 1, 4096, 16, 0, None) == -5
+    assert f(4, None, None, 0.0, one, 1, 4096, 16, 0, None) == -1
+    assert f(4, fake, None, 0.0, four, 4, 4096, 16, 0, None) == -2
+    assert f(4, fake + 2, None, 0.0, one, 1, 4096, 16, 0, None) == -6
+    small = (dec._StreamLayer * 1)(dec._StreamLayer(fake, 64, fake, 4096))
+    assert f(4, fake, None, 0.0, small, 1, 4096, 16, 0, None) == -4
+    assert f(4, fake, None, 0.0, one, 1, 65536, 0, 0, None) == -7
