@@ -101,10 +101,13 @@ def save_quantized(model: nn.Module, save_dir: str) -> str:
     return path
 
 
-def from_quantized(model_name_or_path: str, model_type: str = "llama", torch_dtype=None, device_map=None):
+def from_quantized(model_name_or_path: str, model_type: str = "llama", torch_dtype=None, device_map=None,
+                   prepack: bool = True):
     """Build this package's decoder from a directory written by `save_quantized` (here or by the
     reference, utils.py:125-149) and load the packed weights.  `device_map` may be None / "cuda" /
-    a device; the whole model lives on that one device."""
+    a device; the whole model lives on that one device.  `prepack` (default) also repacks, once,
+    the layers whose shape the library recommends it for into the weight streams the batch-1
+    kernels read fastest (CherryLlamaDecoder.prepack); the checkpoint-layout buffers stay."""
     if model_type != "llama":
         raise NotImplementedError(f"model_type {model_type!r}")
     if torch_dtype not in (None, torch.float16):
@@ -128,4 +131,6 @@ def from_quantized(model_name_or_path: str, model_type: str = "llama", torch_dty
     path = os.path.normpath(os.path.join(model_name_or_path, _checkpoint_name(cfg.w_bits, cfg.group_size)))
     sd = torch.load(path, map_location="cpu", weights_only=True)
     model.load_reference_state_dict(sd)
+    if prepack and model.device_.type == "cuda":
+        model.prepack()
     return model
