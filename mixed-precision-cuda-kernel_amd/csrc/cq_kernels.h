@@ -114,11 +114,14 @@ struct StreamMember {  // one layer of a group launch
     __half *mul;
     int N;
 };
+struct StreamWalk {  // kernel argument of launches whose workgroups walk several tiles: workgroups per member
+    int wgs[kStreamMaxGroup];
+};
 struct StreamGroup {  // kernel argument: the members' streams, outputs, widths and first workgroups
     const uint8_t *stream[kStreamMaxGroup];
     __half *mul[kStreamMaxGroup];
     int N[kStreamMaxGroup];
-    int tile_begin[kStreamMaxGroup];
+    int tile_begin[kStreamMaxGroup];  // first workgroup of each member
     int count;
 };
 StreamGeo stream_geo(int bits, int K, int N, int C);

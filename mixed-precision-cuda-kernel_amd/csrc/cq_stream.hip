@@ -312,11 +312,12 @@ __device__ inline uint32_t stream_norm_pair(uint32_t xp, uint32_t wp, float rs) 
 // stream (header and tile records) and output.  NORM: the row is RMS-normalised while it is
 // staged -- norm_w * fp16(x * rsqrt(mean(x^2) + eps)), the rounding points of the decoder's
 // separate norm kernel -- at the price of one more workgroup barrier.
-template <int BITS, int W, int T, int D, int L, int S, int NB, int XL, bool NORM, bool GROUP>
+template <int BITS, int W, int T, int D, int L, int S, int NB, int XL, bool NORM, bool GROUP, int P>
 __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__restrict__ x, StreamGroup grp,
                                                               const __half *__restrict__ norm_w, float eps,
-                                                              int accumulate, StreamGeo geo) {
+                                                              int accumulate, StreamGeo geo, StreamWalk walk) {
     static_assert(L % 4 == 0 && W % T == 0 && D <= L, "");
+    static_assert(P == 1 || (T == 1 && L % D == 0 && GROUP), "walking several tiles: one tile at a time, ring slots fixed per unit");
     // Which member this workgroup works for.  Every member's fields are first pinned in scalar
     // registers: left to itself the compiler turns the selects into ONE load at a selected
     // kernel-argument address, i.e. a second, dependent memory round trip in front of the header
@@ -325,6 +326,7 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
     const uint8_t *__restrict__ stream = grp.stream[0];
     __half *__restrict__ mul = grp.mul[0];
     int N = grp.N[0], wg = bid;
+    int member_wgs = 1;  // (P > 1) workgroups that share this member's tiles: this one takes wg, wg + member_wgs, ...
     if constexpr (GROUP) {
         const uint8_t *s1 = grp.stream[1], *s2 = grp.stream[2];
         __half *o1 = grp.mul[1], *o2 = grp.mul[2];
@@ -336,6 +338,11 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
         mul = m2 ? o2 : m1 ? o1 : mul;
         N = m2 ? n2 : m1 ? n1 : N;
         wg = bid - (m2 ? t2 : m1 ? t1 : 0);  // workgroup index within the member
+        if constexpr (P > 1) {
+            int g0 = walk.wgs[0], g1 = walk.wgs[1], g2 = walk.wgs[2];
+            asm volatile("" : "+s"(g0), "+s"(g1), "+s"(g2));
+            member_wgs = m2 ? g2 : m1 ? g1 : g0;
+        }
     }
     constexpr int WT = W / T;
     constexpr int NT = 64 * (W + S);
@@ -464,79 +471,180 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
         // i % 4 == kq (every lane group ends up with the same MFMA results, so each finishes a
         // quarter of the units; the quarters are added at the end).  Every unit of a tile past the
         // last reads zeros through an empty descriptor.
-        const int tl = wave % T, cls = wave / T;
-        const int tile = wg * T + tl;
-        const bool tile_ok = tile * kStreamTileCols < N;
-        const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)(stream + geo.hdr_bytes + (size_t)(tile_ok ? tile : 0) * geo.record_bytes), 0,
-            tile_ok ? (int)geo.record_bytes : 0, kSFlags);
-        uint32_t sc[L / 4];
-        su4 wbuf[D];
-        su4 cw[4];
-        const bool cherry_wave = cls == WT - 1;
-        // cherry rows first: they are consumed first, which frees their registers for the units
-        if (cherry_wave) {
+        if constexpr (P > 1) {
+            // ---- several tiles, one after the other: tile wg, wg + member_wgs, ... of this member.
+            // The ring of D loads runs across tile boundaries (slot i % D always holds unit i of
+            // some tile, L % D == 0), the cherry rows and scales of the next tile are requested as
+            // soon as the registers of the current ones are free, and nothing but the running sum
+            // is kept per tile: its 16 partial outputs per wavefront wait in LDS for the end.
+            const int cls = wave;
+            const int ntl = (N + kStreamTileCols - 1) / kStreamTileCols;
+            const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(
+                (void *)(stream + geo.hdr_bytes), 0, (int)min((unsigned long long)ntl * geo.record_bytes, 0xffffffffull), kSFlags);
+            uint32_t sc[L / 4];
+            su4 wbuf[D];
+            su4 cw[4];
+            const bool cherry_wave = cls == W - 1;
+            int tcur = wg;
+            bool vcur = tcur < ntl;
+            uint32_t tb = (uint32_t)tcur * geo.record_bytes;
+            auto load_cherry = [&](uint32_t base, bool valid) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int lg = 4 * j + kq;
-                cw[j] = __builtin_amdgcn_raw_buffer_load_b128(
-                    rt, 8 * lg < C ? geo.off_cherry + (uint32_t)(lg * 16 + nn) * 16u : kSOob, 0, 2);
-            }
-        }
-        const uint32_t sc_off = (uint32_t)((cls + kq * WT) * 32 + nn * 2);
-#pragma unroll
-        for (int i = 0; i < L / 4; i++)
-            sc[i] = __builtin_amdgcn_raw_buffer_load_b16(rt, cls + (4 * i + kq) * WT < ng ? sc_off : kSOob, 4 * i * WT * 32, 0);
-        const uint32_t w_off = geo.off_units + (uint32_t)(cls * UB + lane * (BITS * 4));
-        auto load_unit = [&](int i) -> su4 {
-            // a unit past the last reads zeros: the vector offset alone lies outside the descriptor
-            const uint32_t off = cls + i * WT < ng ? w_off : kSOob;
-            if constexpr (BITS == 4) {
-                return __builtin_amdgcn_raw_buffer_load_b128(rt, off, i * WT * UB, 2);
-            } else {
-                const su3 v = __builtin_amdgcn_raw_buffer_load_b96(rt, off, i * WT * UB, 2);
-                return (su4){v[0], v[1], v[2], 0u};
-            }
-        };
-#pragma unroll
-        for (int i = 0; i < D; i++) wbuf[i] = load_unit(i);
-        // ---- (3) the staged activations are needed from here on
-        while (__hip_atomic_load(s_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < S) __builtin_amdgcn_s_sleep(1);
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-        float totc = 0.f;
-        if (cherry_wave) {
-            sf4_t dc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-                if (32 * j < C) {
-                    const sh8_t a = *reinterpret_cast<const sh8_t *>(s_xc + 32 * j + 8 * kq);
-                    dc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, as_h8(cw[j]), dc, 0, 0, 0);
+                for (int j = 0; j < 4; j++) {
+                    const int lg = 4 * j + kq;
+                    cw[j] = __builtin_amdgcn_raw_buffer_load_b128(
+                        rt, valid && 8 * lg < C ? geo.off_cherry + (uint32_t)(lg * 16 + nn) * 16u : kSOob, base, 2);
                 }
-            totc = dc[0];
-        }
-        // units, in order; every consumed slot is refilled with the unit D further on
-        const unsigned short *xa0 = s_xs + cls * kStreamUnitK + 32 * kq;
-        const float *xsum0 = s_xsum + cls;
+            };
+            const uint32_t sc_off = (uint32_t)((cls + kq * W) * 32 + nn * 2);
+            auto load_scale = [&](int i4, uint32_t base, bool valid) -> uint32_t {
+                return __builtin_amdgcn_raw_buffer_load_b16(rt, valid && cls + (4 * i4 + kq) * W < ng ? sc_off : kSOob,
+                                                            base + 4 * i4 * W * 32, 0);
+            };
+            const uint32_t w_off = geo.off_units + (uint32_t)(cls * UB + lane * (BITS * 4));
+            auto load_unit = [&](int i, uint32_t base, bool valid) -> su4 {
+                const uint32_t off = valid && cls + i * W < ng ? w_off : kSOob;
+                if constexpr (BITS == 4) {
+                    return __builtin_amdgcn_raw_buffer_load_b128(rt, off, base + i * W * UB, 2);
+                } else {
+                    const su3 v = __builtin_amdgcn_raw_buffer_load_b96(rt, off, base + i * W * UB, 2);
+                    return (su4){v[0], v[1], v[2], 0u};
+                }
+            };
+            if (cherry_wave) load_cherry(tb, vcur);
 #pragma unroll
-        for (int i = 0; i < L; i++) {
-            if (cls + i * WT >= ng) break;
-            const float sf = (i & 3) == kq ? __half2float(__ushort_as_half((unsigned short)sc[i >> 2])) : 0.f;
-            const su4 w = wbuf[i % D];
-            const float v = unit_dot<BITS>(w, xa0 + i * WT * kStreamUnitK);
-            if (i + D < L) wbuf[i % D] = load_unit(i + D);
-            tot += (v + kGrid * xsum0[i * WT]) * sf;
+            for (int i = 0; i < L / 4; i++) sc[i] = load_scale(i, tb, vcur);
+#pragma unroll
+            for (int i = 0; i < D; i++) wbuf[i] = load_unit(i, tb, vcur);
+            while (__hip_atomic_load(s_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < S) __builtin_amdgcn_s_sleep(1);
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+#pragma unroll 1
+            for (int j = 0; j < P; j++) {
+                const int tnext = tcur + member_wgs;
+                const bool vnext = j + 1 < P && tnext < ntl;
+                const uint32_t tbn = (uint32_t)tnext * geo.record_bytes;
+                float totc = 0.f;
+                if (cherry_wave) {
+                    sf4_t dc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+                        if (32 * q < C) {
+                            const sh8_t a = *reinterpret_cast<const sh8_t *>(s_xc + 32 * q + 8 * kq);
+                            dc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, as_h8(cw[q]), dc, 0, 0, 0);
+                        }
+                    totc = dc[0];
+                    load_cherry(tbn, vnext);
+                }
+                float tt = 0.f;
+#pragma unroll
+                for (int i = 0; i < L; i++) {
+                    // a unit past the last one of the column reads zero codes and a zero scale; its
+                    // activations are taken from unit `cls` so that no stale LDS contents (NaN
+                    // patterns) meet the zeros
+                    const bool real = cls + i * W < ng;
+                    const int up = real ? cls + i * W : cls;
+                    const float sf = (i & 3) == kq ? __half2float(__ushort_as_half((unsigned short)sc[i >> 2])) : 0.f;
+                    const su4 w = wbuf[i % D];
+                    const float v = unit_dot<BITS>(w, s_xs + up * kStreamUnitK + 32 * kq);
+                    wbuf[i % D] = i + D < L ? load_unit(i + D, tb, vcur) : load_unit(i + D - L, tbn, vnext);
+                    tt += (v + kGrid * s_xsum[up]) * sf;
+                    if ((i & 3) == 3) sc[i >> 2] = load_scale(i >> 2, tbn, vnext);
+                }
+                tt = swap32_add(tt, tt);
+                tt = swap16_add(tt, tt) + totc;
+                if (kq == 0) s_red[(j * W + wave) * 16 + nn] = tt;
+                tcur = tnext;
+                vcur = vnext;
+                tb = tbn;
+                if (!vcur) break;
+            }
+        } else {
+                const int tl = wave % T, cls = wave / T;
+            const int tile = wg * T + tl;
+            const bool tile_ok = tile * kStreamTileCols < N;
+            const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(
+                (void *)(stream + geo.hdr_bytes + (size_t)(tile_ok ? tile : 0) * geo.record_bytes), 0,
+                tile_ok ? (int)geo.record_bytes : 0, kSFlags);
+            uint32_t sc[L / 4];
+            su4 wbuf[D];
+            su4 cw[4];
+            const bool cherry_wave = cls == WT - 1;
+            // cherry rows first: they are consumed first, which frees their registers for the units
+            if (cherry_wave) {
+    #pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const int lg = 4 * j + kq;
+                    cw[j] = __builtin_amdgcn_raw_buffer_load_b128(
+                        rt, 8 * lg < C ? geo.off_cherry + (uint32_t)(lg * 16 + nn) * 16u : kSOob, 0, 2);
+                }
+            }
+            const uint32_t sc_off = (uint32_t)((cls + kq * WT) * 32 + nn * 2);
+    #pragma unroll
+            for (int i = 0; i < L / 4; i++)
+                sc[i] = __builtin_amdgcn_raw_buffer_load_b16(rt, cls + (4 * i + kq) * WT < ng ? sc_off : kSOob, 4 * i * WT * 32, 0);
+            const uint32_t w_off = geo.off_units + (uint32_t)(cls * UB + lane * (BITS * 4));
+            auto load_unit = [&](int i) -> su4 {
+                // a unit past the last reads zeros: the vector offset alone lies outside the descriptor
+                const uint32_t off = cls + i * WT < ng ? w_off : kSOob;
+                if constexpr (BITS == 4) {
+                    return __builtin_amdgcn_raw_buffer_load_b128(rt, off, i * WT * UB, 2);
+                } else {
+                    const su3 v = __builtin_amdgcn_raw_buffer_load_b96(rt, off, i * WT * UB, 2);
+                    return (su4){v[0], v[1], v[2], 0u};
+                }
+            };
+    #pragma unroll
+            for (int i = 0; i < D; i++) wbuf[i] = load_unit(i);
+            // ---- (3) the staged activations are needed from here on
+            while (__hip_atomic_load(s_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < S) __builtin_amdgcn_s_sleep(1);
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+            float totc = 0.f;
+            if (cherry_wave) {
+                sf4_t dc = {0.f, 0.f, 0.f, 0.f};
+    #pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (32 * j < C) {
+                        const sh8_t a = *reinterpret_cast<const sh8_t *>(s_xc + 32 * j + 8 * kq);
+                        dc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, as_h8(cw[j]), dc, 0, 0, 0);
+                    }
+                totc = dc[0];
+            }
+            // units, in order; every consumed slot is refilled with the unit D further on
+            const unsigned short *xa0 = s_xs + cls * kStreamUnitK + 32 * kq;
+            const float *xsum0 = s_xsum + cls;
+    #pragma unroll
+            for (int i = 0; i < L; i++) {
+                if (cls + i * WT >= ng) break;
+                const float sf = (i & 3) == kq ? __half2float(__ushort_as_half((unsigned short)sc[i >> 2])) : 0.f;
+                const su4 w = wbuf[i % D];
+                const float v = unit_dot<BITS>(w, xa0 + i * WT * kStreamUnitK);
+                if (i + D < L) wbuf[i % D] = load_unit(i + D);
+                tot += (v + kGrid * xsum0[i * WT]) * sf;
+            }
+            // the four lane groups' quarters
+            tot = swap32_add(tot, tot);
+            tot = swap16_add(tot, tot) + totc;
+            if (kq == 0) s_red[wave * 16 + nn] = tot;
         }
-        // the four lane groups' quarters
-        tot = swap32_add(tot, tot);
-        tot = swap16_add(tot, tot) + totc;
-        if (kq == 0) s_red[wave * 16 + nn] = tot;
     }
 
     // ---- across the tile's wavefronts, then one store per output
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-    if (tid < 16 * T) {
+    if constexpr (P > 1) {
+        const int ntl = (N + kStreamTileCols - 1) / kStreamTileCols;
+        for (int o = tid; o < 16 * P; o += NT) {
+            const int j = o >> 4, tile = wg + j * member_wgs, n = tile * 16 + (o & 15);
+            if (tile < ntl && n < N) {
+                float v = 0.f;
+#pragma unroll
+                for (int c = 0; c < W; c++) v += s_red[(j * W + c) * 16 + (o & 15)];
+                if (accumulate) v += __half2float(mul[n]);
+                mul[n] = __float2half_rn(v);
+            }
+        }
+    } else if (tid < 16 * T) {
         const int otl = tid >> 4, n = (wg * T + otl) * 16 + (tid & 15);
         if (n < N) {
             float v = 0.f;
@@ -548,9 +656,12 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
     }
 }
 
-static size_t stream_lds_bytes(const StreamGeo &g, int W) {
+constexpr int kStreamWalk = 8;  // tiles one workgroup takes at most when a launch has more tiles than resident workgroups
+
+static size_t stream_lds_bytes(const StreamGeo &g, int W, int tiles_per_wg = kStreamWalk) {
     const int Knp512 = (g.ng * kStreamUnitK + 511) & ~511, Cp = (g.C + 31) & ~31;
-    return 16 + (size_t)(g.K + kStreamRawPad + Knp512 + Cp) * 2 + (size_t)(Knp512 / 128) * 4 + (size_t)W * 16 * 4;
+    return 16 + (size_t)(g.K + kStreamRawPad + Knp512 + Cp) * 2 + (size_t)(Knp512 / 128) * 4 +
+           (size_t)W * 16 * 4 * tiles_per_wg;
 }
 
 // Launch geometries (W computing wavefronts, T tiles, D loads in flight, L units per wavefront at
@@ -574,6 +685,9 @@ constexpr int kStreamCfgCount = sizeof(kStreamCfgs) / sizeof(kStreamCfgs[0]);
 
 
 static int stream_pick(const StreamGeo &geo) {
+#ifdef CQS_PICK_OVERRIDE  // a tuning harness that includes this file may force an entry of the table
+    if (CQS_PICK_OVERRIDE >= 0) return CQS_PICK_OVERRIDE;
+#endif
     // Measured (us per launch, 4-bit / 3-bit): 4096 -> 11008 (688 tiles): entry 0 6.46 / 6.51, entry 1
     // 6.74 / 6.51, entry 2 8.36 / 7.70; 4096 -> 4096 (256 tiles): 5.08, 4.32, 4.32 (4-bit); RMSNorm +
     // 3 x (4096 -> 4096) in one launch (768 tiles): 7.48, 7.56, 9.20; RMSNorm + 2 x (4096 -> 11008)
@@ -584,18 +698,20 @@ static int stream_pick(const StreamGeo &geo) {
         if (geo.ntiles > 1000) return 1;
         return geo.bits == 4 ? 0 : 1;
     }
-    for (int i = 3; i < kStreamCfgCount; i++)
+    // 33 to 64 units: entry 4 (5120 -> 13824 3-bit: entry 3 11.5 us, entry 4 10.8; 8192 -> 28672: 22.3)
+    for (int i = 4; i < kStreamCfgCount; i++)
         if (geo.ng <= kStreamCfgs[i].max_units) return i;
     return -1;
 }
 
 // Where the batch-1 matvec over the stream measured faster than the one over the checkpoint layout
-// (us per launch, 4-bit, weights from HBM): 4096 -> 4096 4.18 against 4.95, 4096 -> 11008 6.54
-// against 7.26-7.46; slower beyond 32 units: 5120 -> 13824 12.1 against 9.1, 11008 -> 4096 7.7
-// against 7.0, 8192 -> 28672 29.4 against 22.8 (several rounds of workgroups, each staging x anew).
+// (us per launch, 4-bit, weights from HBM): 4096 -> 4096 4.2 against 4.95, 4096 -> 11008 6.5
+// against 7.3-7.5, 8192 -> 28672 (workgroups walking 7 tiles each) 22.3 against 22.8; slower on the
+// other shapes beyond 32 units: 5120 -> 13824 (3-bit) 10.8 against 9.1, 11008 -> 4096 7.6 against
+// 7.0, 8192 -> 8192 9.1 against 8.75.
 bool stream_faster(int bits, int K, int N, int C) {
-    (void)N;
-    return stream_geo(bits, K, N, C).ng <= 32;
+    const StreamGeo g = stream_geo(bits, K, N, C);
+    return g.ng <= 32 || (g.ng <= 64 && g.ntiles >= 1536);
 }
 
 bool stream_supported(int bits, int B, int K, int N, int C, int G) {
@@ -610,37 +726,82 @@ bool stream_supported(int bits, int B, int K, int N, int C, int G) {
     return stream_lds_bytes(geo, kStreamCfgs[i].W) <= 160 * 1024;
 }
 
+constexpr int kStreamCus = 256;  // compute units of an MI355X
+
 template <int BITS, int I, bool NORM>
 static hipError_t launch_stream_cfg(const __half *vec, const StreamGroup &grp, const __half *norm_w, float eps,
                                     int accumulate, const StreamGeo &geo, hipStream_t s) {
     constexpr StreamCfg c = kStreamCfgs[I];
-    // what the kernel's fixed-size register arrays assume
     constexpr int XL = stream_x_loads(c.max_units, 64 * (c.W + c.S));
+    // what the kernel's fixed-size register arrays assume
     if (geo.ng * kStreamUnitK > c.NB * 512 * c.S || geo.K > XL * 8 * 64 * (c.W + c.S) || geo.ng > c.max_units ||
         ceil_div(geo.ng, c.W / c.T) > c.L)
         return hipErrorInvalidValue;
-    const size_t lds = stream_lds_bytes(geo, c.W);
-    if (lds > 160 * 1024) return hipErrorInvalidValue;
-    auto kern_one = stream_kernel<BITS, c.W, c.T, c.D, c.L, c.S, c.NB, XL, NORM, false>;
-    auto kern_grp = stream_kernel<BITS, c.W, c.T, c.D, c.L, c.S, c.NB, XL, NORM, true>;
-    static bool big_lds_enabled = false;  // (per instantiation; the attribute is idempotent, a race only repeats the calls)
-    if (lds > 48 * 1024 && !big_lds_enabled) {
-        for (const void *k : {reinterpret_cast<const void *>(kern_one), reinterpret_cast<const void *>(kern_grp)}) {
+    // More tiles than the chip holds workgroups at a time: every workgroup walks several tiles of
+    // its member (activations staged once, loads streaming across the tile boundaries) instead of
+    // the launch running in rounds that each pay the start-up chain again.
+    constexpr bool kCanWalk = c.T == 1 && c.L % c.D == 0;
+    auto kern_one = stream_kernel<BITS, c.W, c.T, c.D, c.L, c.S, c.NB, XL, NORM, false, 1>;
+    auto kern_grp = stream_kernel<BITS, c.W, c.T, c.D, c.L, c.S, c.NB, XL, NORM, true, 1>;
+    auto kern_walk = stream_kernel<BITS, c.W, c.T, c.D, c.L, c.S, c.NB, XL, NORM, true, kCanWalk ? kStreamWalk : 1>;
+    const size_t lds_walk = stream_lds_bytes(geo, c.W, kStreamWalk);
+    if (stream_lds_bytes(geo, c.W, 1) > 160 * 1024) return hipErrorInvalidValue;
+    // (per instantiation; the calls are idempotent, a race between host threads only repeats them)
+    static bool big_lds_enabled = false;
+    if (lds_walk > 48 * 1024 && !big_lds_enabled) {
+        for (const void *k : {reinterpret_cast<const void *>(kern_one), reinterpret_cast<const void *>(kern_grp),
+                              reinterpret_cast<const void *>(kern_walk)}) {
             hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             if (e != hipSuccess) return e;
         }
         big_lds_enabled = true;
     }
-    auto kern = grp.count > 1 ? kern_grp : kern_one;
+    // Workgroups that the chip holds at a time, of the kernel that takes one tile per workgroup and
+    // of the one that walks (more registers): from the register counts (512 VGPRs per SIMD lane,
+    // allocated in eights, at most 8 wavefronts per SIMD, four SIMDs) and the LDS.  Asked once.
+    static int slots_one = 0, slots_walk = 0;
+    static size_t slots_lds = 0;
+    if (kCanWalk && lds_walk <= 160 * 1024 && (slots_lds != lds_walk || slots_one <= 0)) {
+        auto resident = [&](const void *k, size_t lds_bytes) {
+            hipFuncAttributes attr;
+            int per_cu = 20 / (c.W + c.S);
+            if (hipFuncGetAttributes(&attr, k) == hipSuccess && attr.numRegs > 0) {
+                int per_simd = 512 / ((attr.numRegs + 7) / 8 * 8);
+                if (per_simd > 8) per_simd = 8;
+                per_cu = 4 * per_simd / (c.W + c.S);
+            } else {
+                (void)hipGetLastError();
+            }
+            const int by_lds = (int)((160 * 1024) / lds_bytes);
+            if (per_cu > by_lds) per_cu = by_lds;
+            return kStreamCus * (per_cu < 1 ? 1 : per_cu);
+        };
+        slots_one = resident(reinterpret_cast<const void *>(kern_grp), stream_lds_bytes(geo, c.W, 1));
+        slots_walk = resident(reinterpret_cast<const void *>(kern_walk), lds_walk);
+        slots_lds = lds_walk;
+    }
+    // one round of one-tile workgroups if they all fit; else as few tiles per workgroup as fill the chip once
+    int per_wg = 1;
+    if (kCanWalk && lds_walk <= 160 * 1024 && slots_one > 0 && geo.ntiles > slots_one) per_wg = ceil_div(geo.ntiles, slots_walk);
+    if (per_wg > kStreamWalk) per_wg = kStreamWalk;
+    const bool walk = per_wg > 1;
+    const size_t lds = stream_lds_bytes(geo, c.W, walk ? kStreamWalk : 1);
+    auto kern = walk ? kern_walk : grp.count > 1 ? kern_grp : kern_one;
     // members are told apart by workgroup index: each starts at a workgroup of its own
+    // (The order of the kernel arguments is not free: with the walk fields inside StreamGroup, which
+    // moves everything behind it by 8 bytes, the single-layer kernel measured 7.2 us instead of 6.5
+    // on the 4096 -> 11008 layer, its instructions being the same.)
     StreamGroup g = grp;
+    StreamWalk gw;
     int wgs = 0;
     for (int i = 0; i < kStreamMaxGroup; i++) {
         g.tile_begin[i] = wgs;
-        if (i < grp.count) wgs += ceil_div(ceil_div(grp.N[i], kStreamTileCols), c.T);
+        const int tiles_i = ceil_div(ceil_div(grp.N[i], kStreamTileCols), c.T);
+        gw.wgs[i] = ceil_div(tiles_i, per_wg);
+        if (i < grp.count) wgs += gw.wgs[i];
     }
     const dim3 grid(wgs), block(64 * (c.W + c.S));
-    hipLaunchKernelGGL(kern, grid, block, lds, s, vec, g, norm_w, eps, accumulate, geo);
+    hipLaunchKernelGGL(kern, grid, block, lds, s, vec, g, norm_w, eps, accumulate, geo, gw);
     return hipGetLastError();
 }
 

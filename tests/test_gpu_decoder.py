@@ -296,10 +296,17 @@ def test_saved_checkpoint_reloads_to_identical_logits(dec, tmp_path):
     ids = torch.randint(0, cfg.vocab_size, (6,), generator=torch.Generator().manual_seed(0))
     want = model.step_logits(ids)
     cq_utils.save_quantized(model, str(tmp_path))
-    loaded = cq_utils.from_quantized(str(tmp_path))
+    loaded = cq_utils.from_quantized(str(tmp_path), prepack=False)
     assert loaded.layers[0].q_proj.qweight.is_cuda
     assert torch.equal(loaded.step_logits(ids), want)
     assert rel(want[-1], model.reference_logits(ids)[-1]) < 2e-2
+    # the default: the recommended layers repacked on load (all seven linears of these small layers);
+    # same weights, the stream kernels' rounding
+    repacked = cq_utils.from_quantized(str(tmp_path))
+    assert all(getattr(m, "_stream", None) is not None for m in repacked.layers[0].children())
+    got = repacked.step_logits(ids)
+    for t in range(ids.numel()):
+        assert rel(got[t], want[t]) < 5e-3, t
 
 
 def test_argmax_embed_tail_kernel(dec):

@@ -306,3 +306,39 @@ def test_prepacked_group_rejections():
     small = (dec._StreamLayer * 1)(dec._StreamLayer(fake, 64, fake, 4096))
     assert f(4, fake, None, 0.0, small, 1, 4096, 16, 0, None) == -4
     assert f(4, fake, None, 0.0, one, 1, 65536, 0, 0, None) == -7
+
+
+@pytest.mark.parametrize("bits,k,n", [(4, 4096, 32000), (3, 4096, 32008), (4, 1024, 100000), (3, 2048, 65544)])
+def test_prepacked_layers_with_more_tiles_than_resident_workgroups(bits, k, n):
+    """Wide layers: a workgroup walks several tiles (activations staged once, the load ring running
+    across tile boundaries).  Against the C oracle, one-hot bit for bit (first / last tile, tiles
+    taken second and last by a workgroup), accumulate, and repeatable."""
+    import quant_cuda
+    print("[case] prepacked wide layer", bits, k, n, flush=True)
+    p = orc.synthetic_layer(k, n, bits, 128, seed=60 + bits)[1]
+    t = {name: torch.from_numpy(np.ascontiguousarray(v)).cuda() for name, v in p.items()
+         if name in ("qweight", "scales", "cherry_weight", "cherry_indices")}
+    c = int(p["cherry_indices"].shape[0])
+    stream = quant_cuda.prepack_cherryq(bits, t["qweight"], t["cherry_weight"], t["cherry_indices"], t["scales"], k, 128)
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((1, k)).astype(np.float16)
+
+    def run(xv, base=None):
+        out = torch.full((1, n), 5.0, dtype=torch.float16, device="cuda") if base is None else torch.from_numpy(base).cuda()
+        quant_cuda.matvec_prepacked_cherryq(bits, torch.from_numpy(xv).cuda(), stream, out, k, c, accumulate=base is not None)
+        torch.cuda.synchronize()
+        return out.cpu().numpy()
+
+    want = c_oracle.fused(x, p, bits, 128)
+    got = run(x)
+    assert orc.rel_l2(got, want) <= 1e-3
+    np.testing.assert_array_equal(got, run(x))
+    base = rng.standard_normal((1, n)).astype(np.float16)
+    assert orc.rel_l2(run(x, base), want + base.astype(np.float64)) <= 1e-3
+    idx = p["cherry_indices"].astype(np.int64)
+    nidx = orc.normal_indices(k, idx)
+    probes = [int(nidx[0]), int(nidx[129]), int(nidx[-1])] + ([int(idx[0]), int(idx[-1])] if len(idx) else [])
+    for j in probes:
+        e = np.zeros((1, k), dtype=np.float16)
+        e[0, j] = 1
+        np.testing.assert_array_equal(run(e), c_oracle.fused(e, p, bits, 128).astype(np.float16), err_msg=f"column {j}")
