@@ -43,9 +43,15 @@ def build(force: bool = False, verbose: bool = False) -> Path:
         return LIB
     OBJ.mkdir(exist_ok=True)
 
+    # cq_stream.hip: the dispatcher preloads the first six dwords of the kernel arguments (the
+    # activation pointer, the stream pointer, K and the header size lead stream_kernel's list) into
+    # scalar registers, which takes their load off the start-up chain of every workgroup
+    # (4096 -> 11008: 6.67 -> 6.40 us, 4096 -> 4096: 4.38 -> 4.21 us)
+    extra = {"cq_stream.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=6"]}
+
     def compile_one(src):
         out = OBJ / (src + ".o")
-        cmd = [HIPCC, *FLAGS, "-c", str(CSRC / src), "-o", str(out)]
+        cmd = [HIPCC, *FLAGS, *extra.get(src, []), "-c", str(CSRC / src), "-o", str(out)]
         if verbose:
             print(" ".join(cmd), flush=True)
         r = subprocess.run(cmd, capture_output=True, text=True)

@@ -313,9 +313,15 @@ __device__ inline uint32_t stream_norm_pair(uint32_t xp, uint32_t wp, float rs) 
 // staged -- norm_w * fp16(x * rsqrt(mean(x^2) + eps)), the rounding points of the decoder's
 // separate norm kernel -- at the price of one more workgroup barrier.
 template <int BITS, int W, int T, int D, int L, int S, int NB, int XL, bool NORM, bool GROUP, int P>
-__global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__restrict__ x, StreamGroup grp,
+__global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__restrict__ x,
+                                                              const uint8_t *__restrict__ stream0, int K0,
+                                                              uint32_t hdr_bytes0, StreamGroup grp,
                                                               const __half *__restrict__ norm_w, float eps,
                                                               int accumulate, StreamGeo geo, StreamWalk walk) {
+    // x, stream0 (= grp.stream[0]), K0 (= geo.K) and hdr_bytes0 (= geo.hdr_bytes) lead the argument
+    // list as plain scalars: what the first loads of a workgroup need sits in the first bytes of the
+    // kernel-argument segment (and can be preloaded into scalar registers by the dispatcher when
+    // the file is built with a kernel-argument preload count).
     static_assert(L % 4 == 0 && W % T == 0 && D <= L, "");
     static_assert(P == 1 || (T == 1 && L % D == 0 && GROUP), "walking several tiles: one tile at a time, ring slots fixed per unit");
     // Which member this workgroup works for.  Every member's fields are first pinned in scalar
@@ -323,7 +329,7 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
     // kernel-argument address, i.e. a second, dependent memory round trip in front of the header
     // loads (measured: +1.1 us on the 4096 -> 11008 layer).  A single layer skips all of it.
     const int bid = blockIdx.x;
-    const uint8_t *__restrict__ stream = grp.stream[0];
+    const uint8_t *__restrict__ stream = stream0;
     __half *__restrict__ mul = grp.mul[0];
     int N = grp.N[0], wg = bid;
     int member_wgs = 1;  // (P > 1) workgroups that share this member's tiles: this one takes wg, wg + member_wgs, ...
@@ -353,7 +359,7 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kq = lane >> 4, nn = lane & 15;
     const bool stager = wave >= W;
-    const int K = geo.K, C = geo.C, ng = geo.ng;
+    const int K = K0, C = geo.C, ng = geo.ng;
     const int Knp = ng * kStreamUnitK;
     const int Cp = (C + 31) & ~31;
     const int Knp512 = (Knp + 511) & ~511;
@@ -370,7 +376,7 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
     su4 xr[XL];
     su2 tb[NB];
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, K * 2, kSFlags);
-    const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc((void *)stream, 0, (int)geo.hdr_bytes, kSFlags);
+    const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc((void *)stream, 0, (int)hdr_bytes0, kSFlags);
 #pragma unroll
     for (int i = 0; i < XL; i++)
         if (i * NT * 8 < K) xr[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, (uint32_t)(tid + i * NT) * 16u, 0, 0);
@@ -801,7 +807,7 @@ static hipError_t launch_stream_cfg(const __half *vec, const StreamGroup &grp, c
         if (i < grp.count) wgs += gw.wgs[i];
     }
     const dim3 grid(wgs), block(64 * (c.W + c.S));
-    hipLaunchKernelGGL(kern, grid, block, lds, s, vec, g, norm_w, eps, accumulate, geo, gw);
+    hipLaunchKernelGGL(kern, grid, block, lds, s, vec, g.stream[0], geo.K, geo.hdr_bytes, g, norm_w, eps, accumulate, geo, gw);
     return hipGetLastError();
 }
 
