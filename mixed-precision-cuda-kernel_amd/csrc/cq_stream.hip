@@ -364,8 +364,7 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
     const int Cp = (C + 31) & ~31;
     const int Knp512 = (Knp + 511) & ~511;
     const int nblk = Knp512 >> 9;  // blocks of 512 positions
-    // LDS: counter | raw activations (+ zeros) | compacted activations | cherry activations | unit sums | partial outputs
-    int *s_flag = reinterpret_cast<int *>(smem);
+    // LDS: 16 spare bytes | raw activations (+ zeros) | compacted activations | cherry activations | unit sums | partial outputs
     unsigned short *s_raw = reinterpret_cast<unsigned short *>(smem + 16);
     unsigned short *s_xs = s_raw + K + kStreamRawPad;
     unsigned short *s_xc = s_xs + Knp512;
@@ -380,10 +379,12 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
 #pragma unroll
     for (int i = 0; i < XL; i++)
         if (i * NT * 8 < K) xr[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, (uint32_t)(tid + i * NT) * 16u, 0, 0);
-    const int ws = wave - W;  // index among the staging wavefronts
+    // S == 0: no staging wavefronts -- every computing wavefront stages NB blocks itself, between
+    // queueing its weight loads and using them
+    const int ws = S == 0 ? wave : wave - W;  // index among the wavefronts that stage
     const int b0 = ws * NB, b1 = min(nblk, b0 + NB);
     uint32_t ci0 = 0, ci1 = 0;
-    if (stager) {
+    if (stager || S == 0) {
 #pragma unroll
         for (int i = 0; i < NB; i++)
             tb[i] = __builtin_amdgcn_raw_buffer_load_b64(rh, b0 + i < b1 ? (uint32_t)((b0 + i) * 512 + lane * 8) : kSOob, 0, 0);
@@ -435,14 +436,13 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
         if (i * NT * 8 < K && (tid + i * NT) * 8 < K) reinterpret_cast<su4 *>(s_raw)[tid + i * NT] = xr[i];
     // zeros behind the activations: what padding positions (and padded cherry columns) read
     if (tid < kStreamRawPad / 8) reinterpret_cast<su4 *>(s_raw)[(K >> 3) + tid] = (su4){0u, 0u, 0u, 0u};
-    if (tid == 0) *s_flag = 0;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 
     float tot = 0.f;
-    if (stager) {
-        // ---- (2b) xs[k] = x[k + low(k)] for the positions of blocks [b0, b1), and the sum of every unit
+    // ---- (2b) xs[k] = x[k + low(k)] for the positions of blocks [b0, b1), and the sum of every unit
+    auto stage_blocks = [&]() {
 #pragma unroll
         for (int i = 0; i < NB; i++) {
             const int blk = b0 + i;
@@ -470,8 +470,20 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
             if (lane < Cp) s_xc[lane] = s_raw[ci0 & 0xffffu];
             if (lane + 64 < Cp) s_xc[lane + 64] = s_raw[ci1 & 0xffffu];
         }
+    };
+    // What a computing wavefront does between queueing its loads and using the staged activations:
+    // it meets the staging wavefronts at a workgroup barrier (no polling of LDS, which takes LDS
+    // cycles from the wavefronts that stage); without staging wavefronts it stages its own blocks first.
+    auto staged_wait = [&]() {
+        if constexpr (S == 0) stage_blocks();
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-        if (lane == 0) __hip_atomic_fetch_add(s_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    };
+    if (stager) {
+        stage_blocks();
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
     } else {
         // ---- (2a) computing wavefront.  Lane group kq keeps the scales of the units i with
         // i % 4 == kq (every lane group ends up with the same MFMA results, so each finishes a
@@ -522,8 +534,7 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
             for (int i = 0; i < L / 4; i++) sc[i] = load_scale(i, tb, vcur);
 #pragma unroll
             for (int i = 0; i < D; i++) wbuf[i] = load_unit(i, tb, vcur);
-            while (__hip_atomic_load(s_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < S) __builtin_amdgcn_s_sleep(1);
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+            staged_wait();
 #pragma unroll 1
             for (int j = 0; j < P; j++) {
                 const int tnext = tcur + member_wgs;
@@ -602,8 +613,7 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
     #pragma unroll
             for (int i = 0; i < D; i++) wbuf[i] = load_unit(i);
             // ---- (3) the staged activations are needed from here on
-            while (__hip_atomic_load(s_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < S) __builtin_amdgcn_s_sleep(1);
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+            staged_wait();
             float totc = 0.f;
             if (cherry_wave) {
                 sf4_t dc = {0.f, 0.f, 0.f, 0.f};
@@ -679,13 +689,11 @@ struct StreamCfg {
     int W, T, D, L, S, NB, max_units;
 };
 static constexpr StreamCfg kStreamCfgs[] = {
-    {4, 1, 8, 8, 1, 8, 32},    // 0: K <= 4096 + cherries, 4-bit, a few tiles per compute unit
-    {4, 1, 8, 8, 4, 2, 32},    // 1: the same, 3-bit; both widths from about four tiles per compute unit
-    {8, 1, 4, 4, 4, 2, 32},    // 2: K <= 4096 + cherries, about one tile per compute unit
-    {4, 1, 8, 12, 4, 4, 48},   // 3
-    {8, 1, 8, 8, 4, 4, 64},    // 4
-    {8, 1, 8, 12, 6, 4, 96},   // 5
-    {8, 1, 8, 16, 4, 8, 128},  // 6
+    {4, 1, 8, 8, 4, 2, 32},    // 0: K <= 4096 + cherries, more tiles than compute units
+    {8, 1, 4, 4, 4, 2, 32},    // 1: K <= 4096 + cherries, about one tile per compute unit
+    {8, 1, 8, 8, 0, 2, 64},    // 2: up to 64 units; the computing wavefronts stage the activations themselves
+    {8, 1, 8, 12, 6, 4, 96},   // 3
+    {8, 1, 8, 16, 4, 8, 128},  // 4
 };
 constexpr int kStreamCfgCount = sizeof(kStreamCfgs) / sizeof(kStreamCfgs[0]);
 
@@ -694,27 +702,26 @@ static int stream_pick(const StreamGeo &geo) {
 #ifdef CQS_PICK_OVERRIDE  // a tuning harness that includes this file may force an entry of the table
     if (CQS_PICK_OVERRIDE >= 0) return CQS_PICK_OVERRIDE;
 #endif
-    // Measured (us per launch, 4-bit / 3-bit): 4096 -> 11008 (688 tiles): entry 0 6.46 / 6.51, entry 1
-    // 6.74 / 6.51, entry 2 8.36 / 7.70; 4096 -> 4096 (256 tiles): 5.08, 4.32, 4.32 (4-bit); RMSNorm +
-    // 3 x (4096 -> 4096) in one launch (768 tiles): 7.48, 7.56, 9.20; RMSNorm + 2 x (4096 -> 11008)
-    // (1376 tiles, more than one round of entry 0's workgroups): 15.0, 12.7, 14.6.  Two tiles per
-    // workgroup (one staging wavefront for both) measured 12.9 there and 10.6 on 688 tiles.
-    if (geo.ng <= 32) {
-        if (geo.ntiles <= 320) return 2;
-        if (geo.ntiles > 1000) return 1;
-        return geo.bits == 4 ? 0 : 1;
-    }
-    // 33 to 64 units: entry 4 (5120 -> 13824 3-bit: entry 3 11.5 us, entry 4 10.8; 8192 -> 28672: 22.3)
-    for (int i = 4; i < kStreamCfgCount; i++)
+    // Measured (us per launch, 4-bit / 3-bit; W computing + S staging wavefronts, L units each):
+    // 4096 -> 11008 (688 tiles): entry 0 6.49 / 6.25, entry 1 7.52 / 7.37, W4 L8 S0 6.90 / 6.56,
+    //   W8 L4 S0 6.54 / 6.23, W4 L8 S1 6.39-7.76 (the single staging wavefront is the critical path and
+    //   its speed moved by more than a microsecond with unrelated changes of the code: not used);
+    // 4096 -> 4096 (256 tiles): entry 0 4.25, entry 1 3.93, W8 L4 S0 4.38;
+    // RMSNorm + 3 x (4096 -> 4096) (768 tiles): entry 0 7.37, entry 1 11.6;
+    // RMSNorm + 2 x (4096 -> 11008) (1376 tiles, workgroups walk two tiles): entry 0 10.9, entry 1 12.0;
+    // 8192 -> 28672 (1792 tiles of 64 units, 7 per workgroup): entry 2 21.2, W8 L8 S4 22.2;
+    // 8192 -> 8192: entry 2 9.5, entry 4 8.6; 5120 -> 13824 (3-bit): entry 2 10.4, W8 L12 S0 9.6.
+    if (geo.ng <= 32) return geo.ntiles <= 320 ? 1 : 0;
+    for (int i = 2; i < kStreamCfgCount; i++)
         if (geo.ng <= kStreamCfgs[i].max_units) return i;
     return -1;
 }
 
 // Where the batch-1 matvec over the stream measured faster than the one over the checkpoint layout
 // (us per launch, 4-bit, weights from HBM): 4096 -> 4096 4.2 against 4.95, 4096 -> 11008 6.5
-// against 7.3-7.5, 8192 -> 28672 (workgroups walking 7 tiles each) 22.3 against 22.8; slower on the
-// other shapes beyond 32 units: 5120 -> 13824 (3-bit) 10.8 against 9.1, 11008 -> 4096 7.6 against
-// 7.0, 8192 -> 8192 9.1 against 8.75.
+// against 7.3-7.5, 8192 -> 28672 (workgroups walking 7 tiles each) 21.2 against 22.8; no faster on the
+// other shapes beyond 32 units: 5120 -> 13824 (3-bit) 9.6-10.4 against 9.1, 11008 -> 4096 7.5 against
+// 7.0, 8192 -> 8192 8.6-9.5 against 8.75, 13824 -> 5120 (3-bit) 12.2 against 8.9.
 bool stream_faster(int bits, int K, int N, int C) {
     const StreamGeo g = stream_geo(bits, K, N, C);
     return g.ng <= 32 || (g.ng <= 64 && g.ntiles >= 1536);
@@ -740,7 +747,7 @@ static hipError_t launch_stream_cfg(const __half *vec, const StreamGroup &grp, c
     constexpr StreamCfg c = kStreamCfgs[I];
     constexpr int XL = stream_x_loads(c.max_units, 64 * (c.W + c.S));
     // what the kernel's fixed-size register arrays assume
-    if (geo.ng * kStreamUnitK > c.NB * 512 * c.S || geo.K > XL * 8 * 64 * (c.W + c.S) || geo.ng > c.max_units ||
+    if (geo.ng * kStreamUnitK > c.NB * 512 * (c.S ? c.S : c.W) || geo.K > XL * 8 * 64 * (c.W + c.S) || geo.ng > c.max_units ||
         ceil_div(geo.ng, c.W / c.T) > c.L)
         return hipErrorInvalidValue;
     // More tiles than the chip holds workgroups at a time: every workgroup walks several tiles of
@@ -820,8 +827,6 @@ static hipError_t launch_stream_bits(const __half *vec, const StreamGroup &grp, 
         case 2: return launch_stream_cfg<BITS, 2, NORM>(vec, grp, norm_w, eps, accumulate, geo, s);
         case 3: return launch_stream_cfg<BITS, 3, NORM>(vec, grp, norm_w, eps, accumulate, geo, s);
         case 4: return launch_stream_cfg<BITS, 4, NORM>(vec, grp, norm_w, eps, accumulate, geo, s);
-        case 5: return launch_stream_cfg<BITS, 5, NORM>(vec, grp, norm_w, eps, accumulate, geo, s);
-        case 6: return launch_stream_cfg<BITS, 6, NORM>(vec, grp, norm_w, eps, accumulate, geo, s);
         default: return hipErrorInvalidValue;
     }
 }
