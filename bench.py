@@ -133,7 +133,9 @@ def time_gpu(bits, k, n, group, steps, warmup, batch=1, use_graph=True, path="au
     base, copies = make_copies(bits, k, n, group, 640 << 20)
     c = copies[0]["cherry_indices"].numel()
     if path == "auto":
-        path = "prepacked" if batch == 1 and quant_cuda.prepack_recommended(bits, k, n, c, group) else "reference"
+        path = "prepacked" if (quant_cuda.prepack_recommended(bits, k, n, c, group) and
+                               (batch == 1 or (4 <= batch <= 16 and quant_cuda.prepack_supported(bits, batch, k, n, c, group)))) \
+            else "reference"
     x = torch.from_numpy(np.random.default_rng(1).standard_normal((batch, k)).astype(np.float16)).cuda()
     out = torch.zeros(batch, n, dtype=torch.float16, device="cuda")
     if path == "prepacked":
@@ -446,7 +448,7 @@ def main():
 
     def kernel_name(bits, batch, path):
         if path == "prepacked":
-            return f"cq::stream_kernel<{bits}>"
+            return f"cq::stream_kernel<{bits}>" if batch == 1 else f"cq::stream_rows_prep_kernel + cq::stream_rows_kernel<{bits}>"
         if batch == 1:
             return f"cq::matvec_kernel<{bits}>"
         if batch <= 4:

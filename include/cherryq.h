@@ -243,6 +243,21 @@ int cherryq_matvec_prepacked_f16(int w_bits, const void *vec, const void *stream
                                  void *hip_stream);
 
 /*
+ * The same over 2 to 16 activation rows (vec (batch, in_features), mul (batch, out_features)): the
+ * matrix-core tile that the one-row kernel fills with copies of one row takes 16 different rows
+ * at the same price, still without split-K or workspace.  It needs the compacted activations of
+ * all rows in LDS (batch * in_features * 2 bytes at most about 130 KB: 16 rows of 4096, 8 of 8192)
+ * and an uninitialised scratch buffer of cherryq_prepacked_scratch_bytes() bytes, 256-byte
+ * aligned, that a first small launch fills with them.  batch == 1 forwards to
+ * cherryq_matvec_prepacked_f16 (scratch may then be NULL).  cherryq_prepack_supported(w_bits,
+ * batch, ...) says whether a batch is taken.
+ */
+size_t cherryq_prepacked_scratch_bytes(int w_bits, int batch, int in_features, int out_features, int num_cherries);
+int cherryq_matmul_prepacked_f16(int w_bits, const void *vec, const void *stream, size_t stream_bytes, void *mul,
+                                 int batch, int in_features, int out_features, int num_cherries, int accumulate,
+                                 void *scratch, size_t scratch_bytes, void *hip_stream);
+
+/*
  * The decode step's grouped launch over repacked layers (the counterpart of
  * cherryq_decode_matvec_group_f16 below for layers held as weight streams): 1 to 3 layers that
  * share w_bits, in_features and num_cherries and read the same (1, in_features) row -- q / k / v,

@@ -405,7 +405,16 @@ size_t cherryq_prepack_bytes(int w_bits, int in_features, int out_features, int 
 
 int cherryq_prepack_supported(int w_bits, int batch, int in_features, int out_features, int num_cherries,
                               int group_size) {
+    if (batch >= 2)
+        return cq::stream_rows_supported(w_bits, batch, in_features, out_features, num_cherries, group_size) ? 1 : 0;
     return cq::stream_supported(w_bits, batch, in_features, out_features, num_cherries, group_size) ? 1 : 0;
+}
+
+size_t cherryq_prepacked_scratch_bytes(int w_bits, int batch, int in_features, int out_features, int num_cherries) {
+    if ((w_bits != 3 && w_bits != 4) || batch < 2 || in_features <= 0 || out_features <= 0 || num_cherries < 0 ||
+        num_cherries >= in_features)
+        return 0;
+    return cq::stream_rows_scratch_bytes(w_bits, batch, in_features, out_features, num_cherries);
 }
 
 int cherryq_prepack_recommended(int w_bits, int in_features, int out_features, int num_cherries, int group_size) {
@@ -462,6 +471,28 @@ int cherryq_matvec_prepacked_f16(int w_bits, const void *vec, const void *stream
     return (int)cq::launch_stream(w_bits, reinterpret_cast<const __half *>(vec), reinterpret_cast<const uint8_t *>(stream),
                                   reinterpret_cast<__half *>(mul), in_features, out_features, num_cherries, accumulate,
                                   reinterpret_cast<hipStream_t>(hip_stream));
+}
+
+int cherryq_matmul_prepacked_f16(int w_bits, const void *vec, const void *stream, size_t stream_bytes, void *mul,
+                                 int batch, int in_features, int out_features, int num_cherries, int accumulate,
+                                 void *scratch, size_t scratch_bytes, void *hip_stream) {
+    if (batch == 1)
+        return cherryq_matvec_prepacked_f16(w_bits, vec, stream, stream_bytes, mul, batch, in_features, out_features,
+                                            num_cherries, accumulate, hip_stream);
+    int rc = prepack_check(w_bits, in_features, out_features, num_cherries, cq::kStreamUnitK, stream_bytes);
+    if (rc) return rc;
+    if (batch < 0) return CHERRYQ_E_SHAPE;
+    if (batch == 0) return CHERRYQ_OK;
+    if (!cq::stream_rows_supported(w_bits, batch, in_features, out_features, num_cherries, cq::kStreamUnitK))
+        return CHERRYQ_E_UNSUPPORTED;
+    if (!vec || !stream || !mul) return CHERRYQ_E_NULL;
+    if (!cq::aligned(stream, 256) || !cq::aligned(vec, 2) || !cq::aligned(mul, 2)) return CHERRYQ_E_ALIGN;
+    if (!scratch || !cq::aligned(scratch, 256) ||
+        scratch_bytes < cq::stream_rows_scratch_bytes(w_bits, batch, in_features, out_features, num_cherries))
+        return CHERRYQ_E_WORKSPACE;
+    return (int)cq::launch_stream_rows(w_bits, reinterpret_cast<const __half *>(vec), reinterpret_cast<const uint8_t *>(stream),
+                                       reinterpret_cast<__half *>(mul), batch, in_features, out_features, num_cherries,
+                                       accumulate, scratch, reinterpret_cast<hipStream_t>(hip_stream));
 }
 
 int cherryq_decode_matvec_group_prepacked_f16(int w_bits, const void *vec, const void *norm_weight, float eps,

@@ -672,6 +672,292 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
     }
 }
 
+// ---- 2 to 16 activation rows over the stream --------------------------------------------------
+// The matrix-core tile that the one-row kernel fills with 16 copies of one row takes 16 different
+// rows at the same price: A = the rows' activations (lane (kq, n) reads row n), B = the masked
+// code fields, D = 16 rows x 16 columns (lane (kq, n) ends up with rows 4 kq .. 4 kq + 3 of column n).
+// A workgroup still owns whole columns -- no split-K, no workspace -- but needs the compacted
+// activations of ALL rows in LDS (rows x K x 2 bytes: 128 KB for 16 rows of 4096), so (1) a small
+// launch compacts the rows once into a scratch buffer (x[k + low(k)], the per-unit sums, the
+// cherry activations), (2) the main launch has at most as many workgroups as the chip holds at a
+// time, each copying that buffer into LDS once and then walking tiles wg, wg + G, ...
+
+// one block of 512 compacted positions of one row per wavefront
+__global__ __launch_bounds__(64) void stream_rows_prep_kernel(const __half *__restrict__ x,
+                                                              const uint8_t *__restrict__ hdr,
+                                                              unsigned short *__restrict__ xs,
+                                                              float *__restrict__ xsum,
+                                                              unsigned short *__restrict__ xc, StreamGeo geo) {
+    const int blk = blockIdx.x, row = blockIdx.y, lane = threadIdx.x, kq = lane >> 4, nn = lane & 15;
+    const int K = geo.K, Knp512 = (geo.ng * kStreamUnitK + 511) & ~511, Cp = (geo.C + 31) & ~31, nu = Knp512 >> 7;
+    const unsigned short *xrow = reinterpret_cast<const unsigned short *>(x) + (size_t)row * K;
+    const su2 t = *reinterpret_cast<const su2 *>(hdr + (size_t)blk * 512 + lane * 8);
+    unsigned short h[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int src = blk * 512 + 64 * j + lane + (int)((t[j >> 2] >> (8 * (j & 3))) & 0xffu);
+        h[j] = src < K ? xrow[src] : (unsigned short)0;  // padding positions point beyond the row
+        xs[(size_t)row * Knp512 + blk * 512 + 64 * j + lane] = h[j];
+    }
+    float f[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+        f[u] = __half2float(__ushort_as_half(h[2 * u])) + __half2float(__ushort_as_half(h[2 * u + 1]));
+    const float s01 = swap32_add(f[0], f[1]);
+    const float s23 = swap32_add(f[2], f[3]);
+    const float r = row_sum(swap16_add(s01, s23));
+    if (nn == 0) xsum[(size_t)row * nu + blk * 4 + ((kq >> 1) | ((kq & 1) << 1))] = r;
+    if (blk == 0)
+        for (int c = lane; c < Cp; c += 64) {
+            const int col = reinterpret_cast<const uint16_t *>(hdr + Knp512)[c];
+            xc[(size_t)row * Cp + c] = col < K ? xrow[col] : (unsigned short)0;
+        }
+}
+
+// the four rows (4 kq .. 4 kq + 3) x one column that this lane holds of a unit's 16 x 16 product
+template <int BITS>
+__device__ inline sf4_t unit_dot_rows(const su4 w, const unsigned short *xa) {
+    const sf4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (BITS == 4) {
+        const su4 y = {w[0] >> 8, w[1] >> 8, w[2] >> 8, w[3] >> 8};
+        const sh8_t a0 = *reinterpret_cast<const sh8_t *>(xa);
+        const sh8_t a1 = *reinterpret_cast<const sh8_t *>(xa + 8);
+        const sh8_t a2 = *reinterpret_cast<const sh8_t *>(xa + 16);
+        const sh8_t a3 = *reinterpret_cast<const sh8_t *>(xa + 24);
+        const su4 b0 = {w[0] & 0x000f000fu, y[0] & 0x000f000fu, w[1] & 0x000f000fu, y[1] & 0x000f000fu};
+        const su4 b1 = {w[2] & 0x000f000fu, y[2] & 0x000f000fu, w[3] & 0x000f000fu, y[3] & 0x000f000fu};
+        const su4 b2 = {w[0] & 0x00f000f0u, y[0] & 0x00f000f0u, w[1] & 0x00f000f0u, y[1] & 0x00f000f0u};
+        const su4 b3 = {w[2] & 0x00f000f0u, y[2] & 0x00f000f0u, w[3] & 0x00f000f0u, y[3] & 0x00f000f0u};
+        sf4_t dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, as_h8(b0), zero4, 0, 0, 0);
+        sf4_t dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, as_h8(b2), zero4, 0, 0, 0);
+        dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, as_h8(b1), dl, 0, 0, 0);
+        dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(a3, as_h8(b3), dh, 0, 0, 0);
+        return dl * 16777216.0f + dh * 1048576.0f;
+    } else {
+        const su3 y = {w[0] >> 9, w[1] >> 9, w[2] >> 9};
+        const sh8_t a0 = *reinterpret_cast<const sh8_t *>(xa);
+        const sh8_t a2 = *reinterpret_cast<const sh8_t *>(xa + 8);
+        const sh8_t a4 = *reinterpret_cast<const sh8_t *>(xa + 16);
+        const sh4_t a1 = *reinterpret_cast<const sh4_t *>(xa + 24);
+        const sh4_t a3 = *reinterpret_cast<const sh4_t *>(xa + 28);
+        const uint32_t z = (y[0] & 0x00400040u) | ((y[1] & 0x00400040u) << 1) | ((y[2] & 0x00400040u) << 2);
+        const su4 b0 = {w[0] & 0x00070007u, w[1] & 0x00070007u, w[2] & 0x00070007u, y[0] & 0x00070007u};
+        const su4 b2 = {w[0] & 0x00380038u, w[1] & 0x00380038u, w[2] & 0x00380038u, y[0] & 0x00380038u};
+        const su4 b4 = {w[0] & 0x01c001c0u, w[1] & 0x01c001c0u, w[2] & 0x01c001c0u, z};
+        const su2 b1 = {y[1] & 0x00070007u, y[2] & 0x00070007u};
+        const su2 b3 = {y[1] & 0x00380038u, y[2] & 0x00380038u};
+        sf4_t d0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, as_h8(b0), zero4, 0, 0, 0);
+        sf4_t d3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, as_h8(b2), zero4, 0, 0, 0);
+        const sf4_t d6 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a4, as_h8(b4), zero4, 0, 0, 0);
+        d0 = __builtin_amdgcn_mfma_f32_16x16x16f16(a1, as_h4(b1), d0, 0, 0, 0);
+        d3 = __builtin_amdgcn_mfma_f32_16x16x16f16(a3, as_h4(b3), d3, 0, 0, 0);
+        return d0 * 16777216.0f + d3 * 2097152.0f + d6 * 262144.0f;
+    }
+}
+
+constexpr int kRowsSkew = 8;     // halves added to a row's stride in LDS: 16 rows' 16-byte reads hit 16 different bank groups
+
+// TEAMS teams of W wavefronts, each team on a tile of its own; wavefront c of a team takes units
+// c, c + W, ... (L at most) of every tile the team comes to, all L loads in flight, each slot
+// refilled with the next tile's unit as soon as it is consumed.  Tiles are dealt so that the
+// workgroups' loads stay even: team t of workgroup b takes tiles b + t * G, + TEAMS * G, ...
+// STAGE: the workgroup compacts the rows itself (raw rows and the header's table through LDS)
+// instead of reading rows that stream_rows_prep_kernel compacted -- one launch instead of two,
+// possible while raw and compacted rows fit LDS together (8 rows of 4096).
+template <int BITS, int W, int L, int TEAMS, bool STAGE>
+__global__ __launch_bounds__(64 * W * TEAMS) void stream_rows_kernel(
+    const unsigned short *__restrict__ xs_g, const float *__restrict__ xsum_g, const unsigned short *__restrict__ xc_g,
+    const uint8_t *__restrict__ stream, __half *__restrict__ mul, int B, int accumulate, StreamGeo geo) {
+    constexpr int NW = W * TEAMS, NT = 64 * NW;
+    constexpr int UB = BITS == 4 ? 1024 : 768;
+    constexpr float kGrid = BITS == 4 ? -7.5f : -3.5f;
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int team = wave / W, cls = wave % W;
+    const int kq = lane >> 4, nn = lane & 15;
+    const int K = geo.K, C = geo.C, ng = geo.ng, N = geo.N;
+    const int Knp512 = (ng * kStreamUnitK + 511) & ~511, Cp = (C + 31) & ~31, nu = Knp512 >> 7;
+    const int RS = Knp512 + kRowsSkew, CS = Cp + kRowsSkew;
+    unsigned short *s_x = reinterpret_cast<unsigned short *>(smem);                 // [B][RS]
+    unsigned short *s_xc = s_x + (size_t)B * RS;                                     // [B][CS]
+    float *s_xsum = reinterpret_cast<float *>(s_xc + (size_t)B * CS);                // [16][nu] (rows >= B unused)
+    float *s_red = s_xsum + 16 * nu;                                                 // [NW][256]
+
+    if constexpr (STAGE) {
+        // ---- (1) raw rows (each followed by 8 zeros: what padding positions read), the gather table
+        // and the cherry columns -> LDS; then xs[r][p] = x[r][p + low(p)], unit sums, cherry activations
+        const int XS = K + 8;                                                       // raw row stride
+        unsigned short *s_raw = reinterpret_cast<unsigned short *>(s_red + NW * 256);  // [B][XS]
+        uint8_t *s_tab = reinterpret_cast<uint8_t *>(s_raw + (size_t)B * XS);          // [Knp512]
+        unsigned short *s_col = reinterpret_cast<unsigned short *>(s_tab + Knp512);    // [Cp]
+        const int per_row = K >> 3, total = B * per_row;
+        for (int base = 0; base < total; base += 4 * NT) {
+            su4 v[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int c = base + i * NT + tid;
+                if (c < total) v[i] = reinterpret_cast<const su4 *>(xs_g)[c];  // xs_g: the raw rows here
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int c = base + i * NT + tid;
+                if (c < total) {
+                    const int row = c / per_row, col = c - row * per_row;
+                    *reinterpret_cast<su4 *>(s_raw + (size_t)row * XS + col * 8) = v[i];
+                }
+            }
+        }
+        for (int c = tid; c < B; c += NT) *reinterpret_cast<su4 *>(s_raw + (size_t)c * XS + K) = (su4){0u, 0u, 0u, 0u};
+        for (int c = tid; c < (Knp512 >> 4); c += NT) reinterpret_cast<su4 *>(s_tab)[c] = reinterpret_cast<const su4 *>(stream)[c];
+        for (int c = tid; c < Cp; c += NT) s_col[c] = reinterpret_cast<const unsigned short *>(stream + Knp512)[c];
+        __syncthreads();
+        const int nblk = Knp512 >> 9;
+        for (int q = wave; q < B * nblk; q += NW) {  // (row, block of 512 positions) pairs
+            const int row = q / nblk, blk = q - row * nblk;
+            const su2 t = *reinterpret_cast<const su2 *>(s_tab + blk * 512 + lane * 8);
+            const unsigned short *raw = s_raw + (size_t)row * XS;
+            unsigned short h[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                h[j] = raw[min(blk * 512 + 64 * j + lane + (int)((t[j >> 2] >> (8 * (j & 3))) & 0xffu), K)];
+#pragma unroll
+            for (int j = 0; j < 8; j++) s_x[(size_t)row * RS + blk * 512 + 64 * j + lane] = h[j];
+            float f[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                f[u] = __half2float(__ushort_as_half(h[2 * u])) + __half2float(__ushort_as_half(h[2 * u + 1]));
+            const float s01 = swap32_add(f[0], f[1]);
+            const float s23 = swap32_add(f[2], f[3]);
+            const float r = row_sum(swap16_add(s01, s23));
+            if (nn == 0) s_xsum[row * nu + blk * 4 + ((kq >> 1) | ((kq & 1) << 1))] = r;
+        }
+        for (int c = tid; c < B * Cp; c += NT) {
+            const int row = c / Cp, m = c - row * Cp;
+            s_xc[row * CS + m] = s_raw[(size_t)row * XS + min((int)s_col[m], K)];
+        }
+    } else {
+        // ---- (1) the compacted rows, their unit sums and cherry activations: global -> LDS, 16 bytes a piece
+        const int per_row = Knp512 >> 3, total = B * per_row;
+        for (int base = 0; base < total; base += 8 * NT) {
+            su4 v[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int c = base + i * NT + tid;
+                if (c < total) v[i] = reinterpret_cast<const su4 *>(xs_g)[c];
+            }
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int c = base + i * NT + tid;
+                if (c < total) {
+                    const int row = c / per_row, col = c - row * per_row;
+                    *reinterpret_cast<su4 *>(s_x + (size_t)row * RS + col * 8) = v[i];
+                }
+            }
+        }
+        for (int c = tid; c < B * nu; c += NT) s_xsum[c] = xsum_g[c];
+        for (int c = tid; c < B * Cp; c += NT) s_xc[(c / Cp) * CS + c % Cp] = xc_g[c];
+    }
+    __syncthreads();
+
+    // ---- (2) tiles
+    const int ntl = (N + kStreamTileCols - 1) / kStreamTileCols;
+    const int G = gridDim.x, stride = G * TEAMS;
+    const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(stream + geo.hdr_bytes), 0, (int)min((unsigned long long)ntl * geo.record_bytes, 0xffffffffull), kSFlags);
+    uint32_t sc[L];
+    su4 wbuf[L];
+    su4 cw[4];
+    const bool cherry_wave = cls == W - 1;
+    auto load_cherry = [&](uint32_t base, bool valid) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int lg = 4 * j + kq;
+            cw[j] = __builtin_amdgcn_raw_buffer_load_b128(
+                rt, valid && 8 * lg < C ? geo.off_cherry + (uint32_t)(lg * 16 + nn) * 16u : kSOob, base, 2);
+        }
+    };
+    auto load_scale = [&](int i, uint32_t base, bool valid) -> uint32_t {
+        return __builtin_amdgcn_raw_buffer_load_b16(rt, valid && cls + i * W < ng ? (uint32_t)(cls * 32 + nn * 2) : kSOob,
+                                                    base + i * W * 32, 0);
+    };
+    const uint32_t w_off = geo.off_units + (uint32_t)(cls * UB + lane * (BITS * 4));
+    auto load_unit = [&](int i, uint32_t base, bool valid) -> su4 {
+        const uint32_t off = valid && cls + i * W < ng ? w_off : kSOob;
+        if constexpr (BITS == 4) {
+            return __builtin_amdgcn_raw_buffer_load_b128(rt, off, base + i * W * UB, 2);
+        } else {
+            const su3 v = __builtin_amdgcn_raw_buffer_load_b96(rt, off, base + i * W * UB, 2);
+            return (su4){v[0], v[1], v[2], 0u};
+        }
+    };
+    int tile = blockIdx.x + team * G;
+    bool vcur = tile < ntl;
+    uint32_t tb = (uint32_t)tile * geo.record_bytes;
+    if (cherry_wave) load_cherry(tb, vcur);
+#pragma unroll
+    for (int i = 0; i < L; i++) sc[i] = load_scale(i, tb, vcur);
+#pragma unroll
+    for (int i = 0; i < L; i++) wbuf[i] = load_unit(i, tb, vcur);
+    // lanes of rows that do not exist (n >= B) read row 0: their results are never stored
+    const int arow = nn < B ? nn : 0;
+    const unsigned short *xrow = s_x + (size_t)arow * RS + 32 * kq;
+    const float *xsrow = s_xsum + (4 * kq) * nu;
+    // the loop count is the same for every wavefront of the workgroup (barriers inside): as long as
+    // the workgroup's first team, which has the lowest tile, has one
+    for (int t0 = blockIdx.x; t0 < ntl; t0 += stride) {
+        const int tnext = tile + stride;
+        const bool vnext = tnext < ntl;
+        const uint32_t tbn = (uint32_t)tnext * geo.record_bytes;
+        sf4_t acc = {0.f, 0.f, 0.f, 0.f};
+        if (cherry_wave) {
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+                if (32 * q < C) {
+                    const sh8_t a = *reinterpret_cast<const sh8_t *>(s_xc + arow * CS + 32 * q + 8 * kq);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, as_h8(cw[q]), acc, 0, 0, 0);
+                }
+            load_cherry(tbn, vnext);
+        }
+#pragma unroll
+        for (int i = 0; i < L; i++) {
+            // a unit past the column's last reads zero codes and a zero scale; its activations are
+            // taken from unit `cls`, which exists
+            const int up = cls + i * W < ng ? cls + i * W : cls;
+            const float sf = __half2float(__ushort_as_half((unsigned short)sc[i]));
+            const sf4_t v = unit_dot_rows<BITS>(wbuf[i], xrow + up * kStreamUnitK);
+            wbuf[i] = load_unit(i, tbn, vnext);
+            sc[i] = load_scale(i, tbn, vnext);
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[r] += (v[r] + kGrid * xsrow[r * nu + up]) * sf;
+        }
+        float *red = s_red + (size_t)wave * 256;
+#pragma unroll
+        for (int r = 0; r < 4; r++) red[(4 * kq + r) * 16 + nn] = acc[r];
+        __syncthreads();
+        // 256 outputs per team, summed over its W wavefronts by the team's first 256 threads (all of
+        // them with 4 wavefronts, half of them with 8)
+        {
+            const int t = tid - team * 64 * W;
+            if (t < 256 && vcur) {
+                const int row = t >> 4, n = tile * kStreamTileCols + (t & 15);
+                if (row < B && n < N) {
+                    float v = 0.f;
+#pragma unroll
+                    for (int c = 0; c < W; c++) v += s_red[(size_t)(team * W + c) * 256 + t];
+                    __half *o = mul + (size_t)row * N + n;
+                    if (accumulate) v += __half2float(*o);
+                    *o = __float2half_rn(v);
+                }
+            }
+        }
+        __syncthreads();
+        tile = tnext;
+        vcur = vnext;
+        tb = tbn;
+    }
+}
+
 constexpr int kStreamWalk = 8;  // tiles one workgroup takes at most when a launch has more tiles than resident workgroups
 
 static size_t stream_lds_bytes(const StreamGeo &g, int W, int tiles_per_wg = kStreamWalk) {
@@ -880,6 +1166,106 @@ bool stream_group_supported(int bits, int K, int C, int G, const int *Ns, int co
     geo.ntiles = tiles;
     const int i = stream_pick(geo);
     return i >= 0 && stream_lds_bytes(geo, kStreamCfgs[i].W) <= 160 * 1024;
+}
+
+// ---- 2 to 16 rows: sizes, support, launch
+constexpr int kRowsMax = 16;
+
+struct RowsScratch {
+    size_t xs, xsum, xc, total;  // byte offsets of the compacted rows, their unit sums, their cherry activations
+};
+static RowsScratch rows_scratch(int B, const StreamGeo &g) {
+    const size_t Knp512 = (size_t)((g.ng * kStreamUnitK + 511) & ~511), Cp = (size_t)((g.C + 31) & ~31);
+    RowsScratch r;
+    r.xs = 0;
+    r.xsum = (B * Knp512 * 2 + 255) / 256 * 256;
+    r.xc = r.xsum + (B * (Knp512 / 128) * 4 + 255) / 256 * 256;
+    r.total = r.xc + (B * Cp * 2 + 255) / 256 * 256;
+    return r;
+}
+static size_t rows_lds_bytes(int B, const StreamGeo &g, int waves, bool stage) {
+    const size_t Knp512 = (size_t)((g.ng * kStreamUnitK + 511) & ~511), Cp = (size_t)((g.C + 31) & ~31);
+    size_t bytes = B * (Knp512 + kRowsSkew) * 2 + B * (Cp + kRowsSkew) * 2 + 16 * (Knp512 / 128) * 4 + (size_t)waves * 256 * 4;
+    if (stage) bytes += (size_t)B * (g.K + 8) * 2 + Knp512 + Cp * 2;
+    return bytes;
+}
+
+size_t stream_rows_scratch_bytes(int bits, int B, int K, int N, int C) {
+    if (B < 2) return 0;
+    return rows_scratch(B < kRowsMax ? B : kRowsMax, stream_geo(bits, K, N, C)).total;
+}
+
+bool stream_rows_supported(int bits, int B, int K, int N, int C, int G) {
+    if (B < 2 || B > kRowsMax) return false;
+    if (!stream_supported(bits, 1, K, N, C, G)) return false;
+    const StreamGeo geo = stream_geo(bits, K, N, C);
+    if (geo.ng > 64) return false;  // at most 8 units per wavefront, 8 wavefronts per team
+    return rows_lds_bytes(B, geo, 8, false) <= 160 * 1024;
+}
+
+template <int BITS, int W, int L, int TEAMS, bool STAGE>
+static hipError_t launch_rows_cfg(const unsigned short *xs, const float *xsum, const unsigned short *xc,
+                                  const uint8_t *stream, __half *mul, int B, int accumulate, const StreamGeo &geo,
+                                  hipStream_t s) {
+    auto kern = stream_rows_kernel<BITS, W, L, TEAMS, STAGE>;
+    const size_t lds = rows_lds_bytes(B, geo, W * TEAMS, STAGE);
+    if (lds > 160 * 1024 || ceil_div(geo.ng, W) > L) return hipErrorInvalidValue;
+    static bool big_lds_enabled = false;
+    if (lds > 48 * 1024 && !big_lds_enabled) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        big_lds_enabled = true;
+    }
+    // one workgroup per compute unit (its teams share the rows in LDS); fewer when there are fewer tiles
+    int grid = ceil_div(geo.ntiles, TEAMS);
+    if (grid > kStreamCus) grid = kStreamCus;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * W * TEAMS), lds, s, xs, xsum, xc, stream, mul, B, accumulate, geo);
+    return hipGetLastError();
+}
+
+// vec (B, K), mul (B, N), 2 <= B <= 16; scratch: stream_rows_scratch_bytes(), 256-byte aligned
+hipError_t launch_stream_rows(int bits, const __half *vec, const uint8_t *stream, __half *mul, int B, int K, int N,
+                              int C, int accumulate, void *scratch, hipStream_t s) {
+    const StreamGeo geo = stream_geo(bits, K, N, C);
+    // teams of 8 wavefronts, 4 units each for rows of up to 32 units and 8 beyond; two teams per
+    // workgroup when every compute unit gets at least two tiles
+    const bool l4 = geo.ng <= 32;
+    const int teams = geo.ntiles >= 2 * kStreamCus && rows_lds_bytes(B, geo, 16, false) <= 160 * 1024 ? 2 : 1;
+    // compaction inside the workgroup for a few rows (measured on 4096 -> 11008: 2 rows 10.4 us against
+    // 11.6 with the compaction launch, 4 rows 11.4 against 11.8, 8 rows 13.7 against 12.8)
+    const bool stage = B <= 4 && (K % 8 == 0) && rows_lds_bytes(B, geo, 8 * teams, true) <= 160 * 1024;
+    const unsigned short *xs;
+    const float *xsum = nullptr;
+    const unsigned short *xc = nullptr;
+    if (stage) {
+        xs = reinterpret_cast<const unsigned short *>(vec);
+    } else {
+        const RowsScratch sc = rows_scratch(B, geo);
+        unsigned short *xs_w = reinterpret_cast<unsigned short *>(reinterpret_cast<char *>(scratch) + sc.xs);
+        float *xsum_w = reinterpret_cast<float *>(reinterpret_cast<char *>(scratch) + sc.xsum);
+        unsigned short *xc_w = reinterpret_cast<unsigned short *>(reinterpret_cast<char *>(scratch) + sc.xc);
+        const int nblk = ((geo.ng * kStreamUnitK + 511) & ~511) >> 9;
+        hipLaunchKernelGGL(stream_rows_prep_kernel, dim3(nblk, B), dim3(64), 0, s, vec, stream, xs_w, xsum_w, xc_w, geo);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        xs = xs_w;
+        xsum = xsum_w;
+        xc = xc_w;
+    }
+#define CQ_ROWS_GO(BITS_, W_, L_, T_)                                                                                \
+    return stage ? launch_rows_cfg<BITS_, W_, L_, T_, true>(xs, xsum, xc, stream, mul, B, accumulate, geo, s)        \
+                 : launch_rows_cfg<BITS_, W_, L_, T_, false>(xs, xsum, xc, stream, mul, B, accumulate, geo, s)
+#define CQ_ROWS(BITS_)                                                                                               \
+    do {                                                                                                             \
+        if (l4 && teams == 2) CQ_ROWS_GO(BITS_, 8, 4, 2);                                                            \
+        if (l4) CQ_ROWS_GO(BITS_, 8, 4, 1);                                                                          \
+        if (teams == 2) CQ_ROWS_GO(BITS_, 8, 8, 2);                                                                  \
+        CQ_ROWS_GO(BITS_, 8, 8, 1);                                                                                  \
+    } while (0)
+    if (bits == 4) CQ_ROWS(4);
+    CQ_ROWS(3);
+#undef CQ_ROWS
+#undef CQ_ROWS_GO
 }
 
 hipError_t launch_stream_pack(int bits, const uint8_t *qweight, const __half *cherry_weight,

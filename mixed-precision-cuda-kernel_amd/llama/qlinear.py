@@ -69,6 +69,10 @@ class QuantLinear(nn.Module):
     # instead of the fused dequantise + MFMA kernel (measured crossover on MI355X: the fused kernel
     # is 1.6x faster at 128 rows of a 4096 -> 11008 layer, level at 512, 1.3x slower at 2048).
     prefill_rows = 512
+    # from this many rows (up to 16) a prepack()ed layer runs the rows kernel over the weight stream;
+    # measured on 4096 -> 11008, 4-bit (us, stream / checkpoint layout): 2 rows 9.9 / 9.1, 4 rows
+    # 10.6 / 11.3, 8 rows 13.0 / 16.8, 16 rows 14.4 / 19.1
+    stream_rows_min = 4
 
     @classmethod
     @contextmanager
@@ -217,11 +221,15 @@ class QuantLinear(nn.Module):
                 x2 = x2.to(torch.float16)
             x2 = x2.contiguous()
             stream = getattr(self, "_stream", None)
-            if stream is not None and x2.shape[0] == 1:
-                out = torch.empty(1, self.out_features, dtype=torch.float16, device=stream.device)
+            rows = x2.shape[0]
+            # over the repacked stream: one row, and 4 to 16 rows (the matrix-core tile of the one-row
+            # kernel filled with real rows; 2 and 3 rows are faster on the checkpoint layout's kernel)
+            if stream is not None and (rows == 1 or (self.stream_rows_min <= rows <= 16 and quant_cuda.prepack_supported(
+                    self.w_bits, rows, self.in_features, self.out_features, self.num_cherries, self.group_size))):
+                out = torch.empty(rows, self.out_features, dtype=torch.float16, device=stream.device)
                 quant_cuda.matvec_prepacked_cherryq(self.w_bits, x2, stream, out, self.in_features, self.num_cherries)
             elif getattr(self, "_released", False):
-                raise RuntimeError("prepack(release_reference=True) left only the batch-1 weight stream; "
+                raise RuntimeError("prepack(release_reference=True) left only the weight stream (1 and 4..16 rows); "
                                    "call unprepack() before using other batch sizes")
             elif x2.shape[0] >= self.prefill_rows:
                 # prompt-sized batches: one bit-exact dequantisation pass on the GPU into a transient

@@ -56,6 +56,10 @@ _lib.cherryq_vecquant_matmul_f16_static.argtypes = [_int, _vp, _vp, _vp, _vp, _v
 _lib.cherryq_vecquant_matmul_f16_static.restype = _int
 _lib.cherryq_set_force_generic.argtypes = [_int]
 _lib.cherryq_set_force_generic.restype = None
+_lib.cherryq_prepacked_scratch_bytes.argtypes = [_int, _int, _int, _int, _int]
+_lib.cherryq_prepacked_scratch_bytes.restype = _sz
+_lib.cherryq_matmul_prepacked_f16.argtypes = [_int, _vp, _vp, _sz, _vp, _int, _int, _int, _int, _int, _vp, _sz, _vp]
+_lib.cherryq_matmul_prepacked_f16.restype = _int
 _lib.cherryq_prepack_bytes.argtypes = [_int, _int, _int, _int]
 _lib.cherryq_prepack_bytes.restype = _sz
 _lib.cherryq_prepack_supported.argtypes = [_int, _int, _int, _int, _int, _int]
@@ -431,9 +435,9 @@ def unprepack_cherryq(w_bits, stream, in_features, out_features, num_cherries, g
 
 
 def matvec_prepacked_cherryq(w_bits, vec, stream, out, in_features, num_cherries, accumulate=False):
-    """out (1, N) = (or +=) vec (1, K) @ W^T over a stream made by prepack_cherryq.  Result and
-    arithmetic contract are those of vecquant{3,4}matmul_cherryq at batch 1; no workspace, no
-    atomics."""
+    """out (B, N) = (or +=) vec (B, K) @ W^T over a stream made by prepack_cherryq, 1 <= B <= 16.
+    Result and arithmetic contract are those of vecquant{3,4}matmul_cherryq; no workspace, no
+    atomics (from 2 rows a scratch buffer for the compacted activations, kept by this module)."""
     _check(vec, "vec", torch.float16, 2)
     dev = vec.device
     _check(stream, "stream", torch.uint8, 1, dev)
@@ -444,9 +448,18 @@ def matvec_prepacked_cherryq(w_bits, vec, stream, out, in_features, num_cherries
     if batch == 0:
         return
     with torch.cuda.device(dev):
-        rc = _lib.cherryq_matvec_prepacked_f16(w_bits, vec.data_ptr(), stream.data_ptr(), stream.numel(),
-                                               out.data_ptr(), batch, k, out.shape[1], int(num_cherries),
-                                               1 if accumulate else 0, _current_stream(dev.index))
+        hs = _current_stream(dev.index)
+        if batch == 1:
+            rc = _lib.cherryq_matvec_prepacked_f16(w_bits, vec.data_ptr(), stream.data_ptr(), stream.numel(),
+                                                   out.data_ptr(), batch, k, out.shape[1], int(num_cherries),
+                                                   1 if accumulate else 0, hs)
+        else:
+            # 2 to 16 rows: the compacted activations pass through a scratch buffer kept per (device, stream)
+            nb = _lib.cherryq_prepacked_scratch_bytes(w_bits, batch, k, out.shape[1], int(num_cherries))
+            sc = _scratch(dev, hs, nb)
+            rc = _lib.cherryq_matmul_prepacked_f16(w_bits, vec.data_ptr(), stream.data_ptr(), stream.numel(),
+                                                   out.data_ptr(), batch, k, out.shape[1], int(num_cherries),
+                                                   1 if accumulate else 0, None if sc is None else sc.data_ptr(), nb, hs)
     if rc != 0:
         _fail(rc, "matvec_prepacked_cherryq")
 

@@ -205,7 +205,11 @@ def test_quantlinear_prepack_forward_and_release(qc):
 def test_prepacked_c_abi_rejections(qc):
     lib = qc._lib
     assert lib.cherryq_prepack_bytes(5, 4096, 4096, 16) == 0
-    assert lib.cherryq_prepack_supported(4, 2, 4096, 4096, 16, 128) == 0      # batch 1 only
+    assert lib.cherryq_prepack_supported(4, 2, 4096, 4096, 16, 128) == 1      # 2 to 16 rows: the rows kernel
+    assert lib.cherryq_prepack_supported(4, 17, 4096, 4096, 16, 128) == 0
+    assert lib.cherryq_prepack_supported(4, 16, 8192, 8192, 32, 128) == 0     # 16 rows of 8192 do not fit LDS
+    assert lib.cherryq_prepack_supported(4, 8, 8192, 8192, 32, 128) == 1
+    assert lib.cherryq_prepack_supported(3, 2, 13824, 5120, 48, 128) == 0     # more than 64 units per column
     assert lib.cherryq_prepack_supported(4, 1, 4096, 4096, 16, 64) == 0       # group size a multiple of 128
     assert lib.cherryq_prepack_supported(4, 1, 28672, 8192, 112, 128) == 0    # more than 16384 quantised channels
     assert lib.cherryq_prepack_supported(3, 1, 13824, 5120, 48, 128) == 1
@@ -220,6 +224,20 @@ def test_prepacked_c_abi_rejections(qc):
     assert f(4, None, buf.data_ptr(), nbytes, y.data_ptr(), 1, 4096, 1024, 16, 0, None) == -1
     assert f(4, x.data_ptr() + 2, buf.data_ptr(), nbytes, y.data_ptr(), 1, 4096, 1024, 16, 0, None) == -6
     assert f(2, x.data_ptr(), buf.data_ptr(), nbytes, y.data_ptr(), 1, 4096, 1024, 16, 0, None) == -5
+    # the entry point for 2 to 16 rows: needs its scratch buffer
+    lib.cherryq_prepacked_scratch_bytes.restype = ctypes.c_size_t
+    g = lib.cherryq_matmul_prepacked_f16
+    x4 = torch.zeros(4, 4096, dtype=torch.float16, device="cuda")
+    y4 = torch.zeros(4, 1024, dtype=torch.float16, device="cuda")
+    need = lib.cherryq_prepacked_scratch_bytes(4, 4, 4096, 1024, 16)
+    assert need >= 4 * 4096 * 2 and lib.cherryq_prepacked_scratch_bytes(4, 1, 4096, 1024, 16) == 0
+    sc = torch.empty(need, dtype=torch.uint8, device="cuda")
+    assert g(4, x4.data_ptr(), buf.data_ptr(), nbytes, y4.data_ptr(), 4, 4096, 1024, 16, 0, None, 0, None) == -4
+    assert g(4, x4.data_ptr(), buf.data_ptr(), nbytes, y4.data_ptr(), 4, 4096, 1024, 16, 0, sc.data_ptr(), need - 1, None) == -4
+    assert g(4, x4.data_ptr(), buf.data_ptr(), nbytes, y4.data_ptr(), 17, 4096, 1024, 16, 0, sc.data_ptr(), need, None) == -7
+    assert g(4, x4.data_ptr(), buf.data_ptr(), nbytes, y4.data_ptr(), 4, 4096, 1024, 16, 0, sc.data_ptr(), need, None) == 0
+    assert g(4, x.data_ptr(), buf.data_ptr(), nbytes, y.data_ptr(), 1, 4096, 1024, 16, 0, None, 0, None) == 0
+    torch.cuda.synchronize()
 
 
 @pytest.mark.parametrize("bits", [4, 3])
@@ -342,3 +360,80 @@ def test_prepacked_layers_with_more_tiles_than_resident_workgroups(bits, k, n):
         e = np.zeros((1, k), dtype=np.float16)
         e[0, j] = 1
         np.testing.assert_array_equal(run(e), c_oracle.fused(e, p, bits, 128).astype(np.float16), err_msg=f"column {j}")
+
+
+@pytest.mark.parametrize("bits,k,n,b", [(4, 4096, 11008, 16), (3, 4096, 11008, 16), (4, 4096, 4096, 8), (3, 4096, 4096, 2),
+                                        (4, 8192, 1024, 8), (3, 1160, 264, 5), (4, 4096, 32008, 13), (4, 1024, 520, 16)])
+def test_prepacked_rows_against_the_c_oracle(bits, k, n, b):
+    """2 to 16 activation rows over the repacked stream (compaction launch + matrix-core launch with
+    real rows): against the C oracle, one-hot rows bit for bit (also with rows of very different
+    power-of-two magnitude), accumulate, repeatable, and agreeing with the checkpoint-layout path."""
+    import quant_cuda
+    print("[case] prepacked rows", bits, k, n, b, flush=True)
+    p = orc.synthetic_layer(k, n, bits, 128, seed=70 + bits)[1]
+    t = {name: torch.from_numpy(np.ascontiguousarray(v)).cuda() for name, v in p.items()
+         if name in ("qweight", "scales", "cherry_weight", "cherry_indices")}
+    c = int(p["cherry_indices"].shape[0])
+    assert quant_cuda.prepack_supported(bits, b, k, n, c, 128)
+    stream = quant_cuda.prepack_cherryq(bits, t["qweight"], t["cherry_weight"], t["cherry_indices"], t["scales"], k, 128)
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((b, k)).astype(np.float16)
+
+    def run(xv, base=None):
+        out = torch.full((xv.shape[0], n), 5.0, dtype=torch.float16, device="cuda") if base is None else torch.from_numpy(base).cuda()
+        quant_cuda.matvec_prepacked_cherryq(bits, torch.from_numpy(xv).cuda(), stream, out, k, c, accumulate=base is not None)
+        torch.cuda.synchronize()
+        return out.cpu().numpy()
+
+    want = c_oracle.fused(x, p, bits, 128)
+    got = run(x)
+    for r in range(b):
+        assert orc.rel_l2(got[r], want[r]) <= 1e-3, r
+    np.testing.assert_array_equal(got, run(x))
+    base = rng.standard_normal((b, n)).astype(np.float16)
+    acc = run(x, base)
+    for r in range(b):
+        assert orc.rel_l2(acc[r], want[r] + base[r].astype(np.float64)) <= 1e-3, r
+    ref = torch.empty(b, n, dtype=torch.float16, device="cuda")
+    quant_cuda.matmul_cherryq(bits, torch.from_numpy(x).cuda(), t["qweight"], t["cherry_weight"], t["cherry_indices"],
+                              t["scales"], ref, 128)
+    torch.cuda.synchronize()
+    assert orc.rel_l2(got, ref.cpu().numpy().astype(np.float64)) <= 5e-4
+    idx = p["cherry_indices"].astype(np.int64)
+    nidx = orc.normal_indices(k, idx)
+    pool = [int(nidx[0]), int(nidx[1]), int(nidx[31]), int(nidx[32]), int(nidx[127]), int(nidx[128]), int(nidx[-1]),
+            int(nidx[-33])] + ([int(idx[0]), int(idx[-1]), int(idx[len(idx) // 2])] if len(idx) else [])
+    e = np.zeros((b, k), dtype=np.float16)
+    for r in range(b):
+        e[r, pool[r % len(pool)]] = np.float16(2.0 ** ((r * 5) % 13 - 6))
+    with np.errstate(over="ignore"):
+        np.testing.assert_array_equal(run(e), c_oracle.fused(e, p, bits, 128).astype(np.float16))
+
+
+def test_quantlinear_routes_rows_to_the_stream_after_prepack():
+    """QuantLinear.forward after prepack(): 1 row and 4..16 rows run over the weight stream (also with
+    the checkpoint-layout buffers released), 2 / 3 / 17 rows on the checkpoint layout; all agree with
+    the module before prepack()."""
+    from llama.qlinear import QuantLinear
+    from llama.quantizer import FullSymQuantizer
+    import cherryq_decoder as dec
+    print("[case] QuantLinear rows routing", flush=True)
+    cfg = dec.DecoderConfig(w_bits=4, group_size=128, cherry_fraction=1 / 256)
+    m = dec.random_packed_linear(cfg, 4096, 1024, torch.Generator(device="cuda").manual_seed(2), "cuda")
+    xs = {b: torch.randn(b, 4096, device="cuda", generator=torch.Generator(device="cuda").manual_seed(b)).half()
+          for b in (1, 2, 3, 4, 9, 16, 17)}
+    before = {b: m(x) for b, x in xs.items()}
+    assert m.prepack()
+    for b, x in xs.items():
+        got = m(x)
+        assert got.shape == (b, 1024)
+        assert orc.rel_l2(got.float().cpu().numpy(), before[b].float().cpu().numpy().astype(np.float64)) <= 5e-4, b
+        if b in (2, 3, 17):
+            assert torch.equal(got, before[b]), b   # same kernel as before
+    m.prepack(release_reference=True)
+    for b in (1, 4, 16):
+        assert orc.rel_l2(m(xs[b]).float().cpu().numpy(), before[b].float().cpu().numpy().astype(np.float64)) <= 5e-4
+    with pytest.raises(RuntimeError):
+        m(xs[2])
+    m.unprepack()
+    assert torch.equal(m(xs[2]), before[2])
