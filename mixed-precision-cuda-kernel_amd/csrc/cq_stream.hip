@@ -691,12 +691,22 @@ __global__ __launch_bounds__(64) void stream_rows_prep_kernel(const __half *__re
     const int blk = blockIdx.x, row = blockIdx.y, lane = threadIdx.x, kq = lane >> 4, nn = lane & 15;
     const int K = geo.K, Knp512 = (geo.ng * kStreamUnitK + 511) & ~511, Cp = (geo.C + 31) & ~31, nu = Knp512 >> 7;
     const unsigned short *xrow = reinterpret_cast<const unsigned short *>(x) + (size_t)row * K;
+    // the table and the raw columns the block can touch (its 512 positions + up to 128 cherry
+    // columns in front) are requested together; the gather then runs out of LDS: one memory round
+    // trip instead of two dependent ones
+    __shared__ __align__(16) unsigned short s_seg[512 + 128];
     const su2 t = *reinterpret_cast<const su2 *>(hdr + (size_t)blk * 512 + lane * 8);
+    const int q0 = blk * 512 + lane * 8, q1 = blk * 512 + 512 + lane * 8;
+    const su4 zero = {0u, 0u, 0u, 0u};
+    const su4 v0 = q0 < K ? *reinterpret_cast<const su4 *>(xrow + q0) : zero;        // K % 8 == 0
+    const su4 v1 = lane < 16 && q1 < K ? *reinterpret_cast<const su4 *>(xrow + q1) : zero;
+    *reinterpret_cast<su4 *>(s_seg + lane * 8) = v0;
+    if (lane < 16) *reinterpret_cast<su4 *>(s_seg + 512 + lane * 8) = v1;
+    __syncthreads();
     unsigned short h[8];
 #pragma unroll
     for (int j = 0; j < 8; j++) {
-        const int src = blk * 512 + 64 * j + lane + (int)((t[j >> 2] >> (8 * (j & 3))) & 0xffu);
-        h[j] = src < K ? xrow[src] : (unsigned short)0;  // padding positions point beyond the row
+        h[j] = s_seg[64 * j + lane + (int)((t[j >> 2] >> (8 * (j & 3))) & 0xffu)];  // columns >= K hold zeros
         xs[(size_t)row * Knp512 + blk * 512 + 64 * j + lane] = h[j];
     }
     float f[4];
