@@ -293,19 +293,21 @@ __device__ inline uint32_t stream_norm_pair(uint32_t xp, uint32_t wp, float rs) 
 // A workgroup is W computing wavefronts plus S staging wavefronts and owns T tiles (W % T == 0):
 // computing wavefront w works on tile w % T and takes the units g = w / T, w / T + W / T, ... of it
 // (at most L), D loads in flight.  Staging wavefront j prepares NB consecutive blocks of 512
-// compacted positions (S * NB blocks cover K).
+// compacted positions (S * NB blocks cover K); with S == 0 the computing wavefronts stage NB blocks
+// each themselves.  P > 1: the workgroup walks up to P tiles of its member one after the other
+// (launches with more tiles than the chip holds workgroups), the activations staged once.
 //
 // Order of events.  A CU admits vector loads only as fast as earlier ones return, so whatever a
 // wavefront does after queueing weight loads waits in that queue with them.  Therefore: (1) every
-// wavefront requests its 16 bytes per thread of the activation vector alone (the staging
-// wavefronts also the gather table and the cherry columns from the stream header), copies them
-// to LDS and meets the others -- under a microsecond after the start, nothing else being in the
-// queues; (2) the computing wavefronts queue their cherry rows, scales and first D units, while
-// the staging wavefronts, which never touch the weight stream, gather the activations into MFMA
-// operand order (conflict-free: lane l takes positions l, l + 64, ...), add up every unit's
-// activations for the grid offset, and raise a counter in LDS; (3) a computing wavefront looks
-// at the counter when its loads are queued, then consumes its units in order, refilling every
-// slot it frees.
+// wavefront requests its 16 bytes per thread of the activation vector alone (those that stage
+// also the gather table and the cherry columns from the stream header), copies them to LDS and
+// meets the others -- under a microsecond after the start, nothing else being in the queues;
+// (2) the computing wavefronts queue their cherry rows, scales and first D units, while the
+// staging wavefronts, which never touch the weight stream, gather the activations into MFMA
+// operand order (conflict-free: lane l takes positions l, l + 64, ...) and add up every unit's
+// activations for the grid offset (S == 0: the computing wavefronts do so after queueing their
+// loads -- LDS work does not wait behind vector loads); (3) all meet at a second workgroup
+// barrier, then a computing wavefront consumes its units in order, refilling every slot it frees.
 //
 // Up to kStreamMaxGroup layers that read the same activation row (q / k / v, gate / up) share
 // one launch: consecutive ranges of workgroups belong to consecutive members, each with its own
@@ -576,7 +578,7 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
                 if (!vcur) break;
             }
         } else {
-                const int tl = wave % T, cls = wave / T;
+            const int tl = wave % T, cls = wave / T;
             const int tile = wg * T + tl;
             const bool tile_ok = tile * kStreamTileCols < N;
             const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(
@@ -588,7 +590,7 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
             const bool cherry_wave = cls == WT - 1;
             // cherry rows first: they are consumed first, which frees their registers for the units
             if (cherry_wave) {
-    #pragma unroll
+#pragma unroll
                 for (int j = 0; j < 4; j++) {
                     const int lg = 4 * j + kq;
                     cw[j] = __builtin_amdgcn_raw_buffer_load_b128(
@@ -596,7 +598,7 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
                 }
             }
             const uint32_t sc_off = (uint32_t)((cls + kq * WT) * 32 + nn * 2);
-    #pragma unroll
+#pragma unroll
             for (int i = 0; i < L / 4; i++)
                 sc[i] = __builtin_amdgcn_raw_buffer_load_b16(rt, cls + (4 * i + kq) * WT < ng ? sc_off : kSOob, 4 * i * WT * 32, 0);
             const uint32_t w_off = geo.off_units + (uint32_t)(cls * UB + lane * (BITS * 4));
@@ -610,14 +612,14 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
                     return (su4){v[0], v[1], v[2], 0u};
                 }
             };
-    #pragma unroll
+#pragma unroll
             for (int i = 0; i < D; i++) wbuf[i] = load_unit(i);
             // ---- (3) the staged activations are needed from here on
             staged_wait();
             float totc = 0.f;
             if (cherry_wave) {
                 sf4_t dc = {0.f, 0.f, 0.f, 0.f};
-    #pragma unroll
+#pragma unroll
                 for (int j = 0; j < 4; j++)
                     if (32 * j < C) {
                         const sh8_t a = *reinterpret_cast<const sh8_t *>(s_xc + 32 * j + 8 * kq);
@@ -628,7 +630,7 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
             // units, in order; every consumed slot is refilled with the unit D further on
             const unsigned short *xa0 = s_xs + cls * kStreamUnitK + 32 * kq;
             const float *xsum0 = s_xsum + cls;
-    #pragma unroll
+#pragma unroll
             for (int i = 0; i < L; i++) {
                 if (cls + i * WT >= ng) break;
                 const float sf = (i & 3) == kq ? __half2float(__ushort_as_half((unsigned short)sc[i >> 2])) : 0.f;
