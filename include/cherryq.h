@@ -245,10 +245,11 @@ int cherryq_matvec_prepacked_f16(int w_bits, const void *vec, const void *stream
 /*
  * The same over 2 to 16 activation rows (vec (batch, in_features), mul (batch, out_features)): the
  * matrix-core tile that the one-row kernel fills with copies of one row takes 16 different rows
- * at the same price, still without split-K or workspace.  It needs the compacted activations of
- * all rows in LDS (batch * in_features * 2 bytes at most about 130 KB: 16 rows of 4096, 8 of 8192)
- * and an uninitialised scratch buffer of cherryq_prepacked_scratch_bytes() bytes, 256-byte
- * aligned, that a first small launch fills with them.  batch == 1 forwards to
+ * at the same price, still without split-K or workspace.  The compacted activations of all rows
+ * are brought into matrix-core operand order once (a first small launch into an uninitialised
+ * scratch buffer of cherryq_prepacked_scratch_bytes() bytes, 256-byte aligned; for up to 4 rows
+ * inside the main launch) and then stay in LDS or in registers while a workgroup walks its
+ * tiles; layers of up to 8192 + 128 input channels (64 units of 128 positions) are taken.  batch == 1 forwards to
  * cherryq_matvec_prepacked_f16 (scratch may then be NULL).  cherryq_prepack_supported(w_bits,
  * batch, ...) says whether a batch is taken.
  */

@@ -31,6 +31,8 @@
 // Arithmetic contract: csrc/quant_cuda_kernel.cu:718-835 (4-bit) and 558-672 (3-bit) of the
 // reference; fp32 accumulation, one rounding to fp16.  Replaces the per-thread decode loops at
 // :811-831 / :649-667 and the serial batch loop :797-834.
+#include <type_traits>
+
 #include "cq_device.h"
 #include "cq_kernels.h"
 
@@ -970,6 +972,223 @@ __global__ __launch_bounds__(64 * W * TEAMS) void stream_rows_kernel(
     }
 }
 
+// ---- rows kept in registers -------------------------------------------------------------------
+// The A operands of a wavefront's units do not change from tile to tile, so a wavefront that walks
+// tiles can hold them in registers: 8 units x 4 operands x 4 VGPRs = 128 VGPRs, loaded once from a
+// buffer that a first launch wrote in operand order.  No LDS traffic for the activations, and 16
+// rows of 8192 channels (256 KB, more than LDS holds) become possible.  One workgroup of 8
+// wavefronts per compute unit: teams of W = ceil(units / 8) wavefronts, 8 / W teams.
+
+// grid: one block per unit (+ one for the cherry activations), 256 threads.  xf[unit][m][lane][8]:
+// lane (kq, n) gets row n (zeros from row B on), compacted positions 128 unit + 32 kq + 8 m + 0..7.
+__global__ __launch_bounds__(256) void stream_rows_frag_kernel(const __half *__restrict__ x,
+                                                               const uint8_t *__restrict__ hdr,
+                                                               su4 *__restrict__ xf, float *__restrict__ xsum,
+                                                               su4 *__restrict__ xcf, int B, StreamGeo geo) {
+    __shared__ __align__(16) unsigned short s_seg[16][256 + 8];
+    __shared__ uint8_t s_tab[128];
+    const int u = blockIdx.x, t = threadIdx.x, lane = t & 63, m = t >> 6, kq = lane >> 4, nn = lane & 15;
+    const int K = geo.K, Knp512 = (geo.ng * kStreamUnitK + 511) & ~511;
+    const unsigned short *xh = reinterpret_cast<const unsigned short *>(x);
+    if (u == geo.ng) {  // cherry activations: positions 32 m + 8 kq + 0..7 of the cherry list
+        su4 v = {0u, 0u, 0u, 0u};
+        unsigned short h[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int col = reinterpret_cast<const uint16_t *>(hdr + Knp512)[32 * m + 8 * kq + j];  // padding entries hold K
+            h[j] = nn < B && 32 * m < ((geo.C + 31) & ~31) && col < K ? xh[(size_t)nn * K + col] : (unsigned short)0;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = (uint32_t)h[2 * j] | ((uint32_t)h[2 * j + 1] << 16);
+        xcf[m * 64 + lane] = v;
+        return;
+    }
+    // the unit's raw columns (its 128 positions + up to 128 cherry columns in front) of all rows, and its table bytes
+    for (int c = t; c < 16 * 32; c += 256) {
+        const int row = c >> 5, q = c & 31, pos = u * kStreamUnitK + q * 8;
+        su4 v = {0u, 0u, 0u, 0u};
+        if (row < B && pos < K) v = *reinterpret_cast<const su4 *>(xh + (size_t)row * K + pos);  // K % 8 == 0
+        *reinterpret_cast<su4 *>(&s_seg[row][q * 8]) = v;
+    }
+    if (t < 128) {
+        const int p = u * kStreamUnitK + t;
+        s_tab[t] = hdr[(p >> 9) * 512 + (p & 63) * 8 + ((p & 511) >> 6)];
+    }
+    __syncthreads();
+    {
+        unsigned short h[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int i = 32 * kq + 8 * m + j;
+            h[j] = s_seg[nn][i + s_tab[i]];  // columns >= K hold zeros
+        }
+        su4 v;
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = (uint32_t)h[2 * j] | ((uint32_t)h[2 * j + 1] << 16);
+        xf[((size_t)u * 4 + m) * 64 + lane] = v;
+    }
+    {   // the unit's sum of activations per row: 16 threads per row, 8 positions each
+        const int row = t >> 4, part = t & 15;
+        float sacc = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int i = part * 8 + j;
+            sacc += __half2float(__ushort_as_half(s_seg[row][i + s_tab[i]]));
+        }
+        sacc = row_sum(sacc);
+        if (part == 0) xsum[row * geo.ng + u] = sacc;
+    }
+}
+
+template <int BITS, typename WB>
+__device__ inline sf4_t unit_dot_regs(const WB w, const su4 (&a)[4]) {
+    const sf4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (BITS == 4) {
+        const su4 y = {w[0] >> 8, w[1] >> 8, w[2] >> 8, w[3] >> 8};
+        const su4 b0 = {w[0] & 0x000f000fu, y[0] & 0x000f000fu, w[1] & 0x000f000fu, y[1] & 0x000f000fu};
+        const su4 b1 = {w[2] & 0x000f000fu, y[2] & 0x000f000fu, w[3] & 0x000f000fu, y[3] & 0x000f000fu};
+        const su4 b2 = {w[0] & 0x00f000f0u, y[0] & 0x00f000f0u, w[1] & 0x00f000f0u, y[1] & 0x00f000f0u};
+        const su4 b3 = {w[2] & 0x00f000f0u, y[2] & 0x00f000f0u, w[3] & 0x00f000f0u, y[3] & 0x00f000f0u};
+        sf4_t dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(a[0]), as_h8(b0), zero4, 0, 0, 0);
+        sf4_t dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(a[2]), as_h8(b2), zero4, 0, 0, 0);
+        dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(a[1]), as_h8(b1), dl, 0, 0, 0);
+        dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(a[3]), as_h8(b3), dh, 0, 0, 0);
+        return dl * 16777216.0f + dh * 1048576.0f;
+    } else {
+        const su3 y = {w[0] >> 9, w[1] >> 9, w[2] >> 9};
+        const uint32_t z = (y[0] & 0x00400040u) | ((y[1] & 0x00400040u) << 1) | ((y[2] & 0x00400040u) << 2);
+        const su4 b0 = {w[0] & 0x00070007u, w[1] & 0x00070007u, w[2] & 0x00070007u, y[0] & 0x00070007u};
+        const su4 b2 = {w[0] & 0x00380038u, w[1] & 0x00380038u, w[2] & 0x00380038u, y[0] & 0x00380038u};
+        const su4 b4 = {w[0] & 0x01c001c0u, w[1] & 0x01c001c0u, w[2] & 0x01c001c0u, z};
+        const su2 b1 = {y[1] & 0x00070007u, y[2] & 0x00070007u};
+        const su2 b3 = {y[1] & 0x00380038u, y[2] & 0x00380038u};
+        const su2 a1 = {a[3][0], a[3][1]}, a3 = {a[3][2], a[3][3]};  // positions 24..27 and 28..31
+        sf4_t d0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(a[0]), as_h8(b0), zero4, 0, 0, 0);
+        sf4_t d3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(a[1]), as_h8(b2), zero4, 0, 0, 0);
+        const sf4_t d6 = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(a[2]), as_h8(b4), zero4, 0, 0, 0);
+        d0 = __builtin_amdgcn_mfma_f32_16x16x16f16(as_h4(a1), as_h4(b1), d0, 0, 0, 0);
+        d3 = __builtin_amdgcn_mfma_f32_16x16x16f16(as_h4(a3), as_h4(b3), d3, 0, 0, 0);
+        return d0 * 16777216.0f + d3 * 2097152.0f + d6 * 262144.0f;
+    }
+}
+
+// W wavefronts per team (4: up to 32 units, 8: up to 64), 8 / W teams, 8 units per wavefront.
+template <int BITS, int W>
+__global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restrict__ xf, const float *__restrict__ xsum_g,
+                                                              const su4 *__restrict__ xcf,
+                                                              const uint8_t *__restrict__ stream,
+                                                              __half *__restrict__ mul, int B, int accumulate,
+                                                              StreamGeo geo) {
+    constexpr int L = 8, TEAMS = 8 / W;
+    constexpr int UB = BITS == 4 ? 1024 : 768;
+    constexpr float kGrid = BITS == 4 ? -7.5f : -3.5f;
+    __shared__ float s_red[8][256];
+    extern __shared__ __align__(16) unsigned char smem[];
+    float *s_xsum = reinterpret_cast<float *>(smem);  // [16][ng]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int team = wave / W, cls = wave % W;
+    const int kq = lane >> 4, nn = lane & 15;
+    const int C = geo.C, ng = geo.ng, N = geo.N;
+    // ---- the wavefront's activations: operands of its units, the cherry operands; unit sums to LDS
+    su4 areg[L][4];
+#pragma unroll
+    for (int i = 0; i < L; i++) {
+        const int u = cls + i * W;
+#pragma unroll
+        for (int m = 0; m < 4; m++)
+            areg[i][m] = u < ng ? xf[((size_t)u * 4 + m) * 64 + lane] : (su4){0u, 0u, 0u, 0u};
+    }
+    const bool cherry_wave = cls == W - 1;
+    __shared__ su4 s_acr[4 * 64];  // the cherry operands (read once per tile by each team's last wavefront)
+    if (tid < 4 * 64) s_acr[tid] = xcf[tid];
+    for (int c = tid; c < 16 * ng; c += 512) s_xsum[c] = xsum_g[c];
+    __syncthreads();
+
+    const int ntl = (N + kStreamTileCols - 1) / kStreamTileCols;
+    const int G = gridDim.x, stride = G * TEAMS;
+    const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(stream + geo.hdr_bytes), 0, (int)min((unsigned long long)ntl * geo.record_bytes, 0xffffffffull), kSFlags);
+    typedef typename std::conditional<BITS == 4, su4, su3>::type WB;  // a unit: 4 or 3 dwords per lane
+    uint32_t sc[L];
+    WB wbuf[L];
+    su4 cw[4];
+    auto load_cherry = [&](uint32_t base, bool valid) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int lg = 4 * j + kq;
+            cw[j] = __builtin_amdgcn_raw_buffer_load_b128(
+                rt, valid && 8 * lg < C ? geo.off_cherry + (uint32_t)(lg * 16 + nn) * 16u : kSOob, base, 2);
+        }
+    };
+    auto load_scale = [&](int i, uint32_t base, bool valid) -> uint32_t {
+        return __builtin_amdgcn_raw_buffer_load_b16(rt, valid && cls + i * W < ng ? (uint32_t)(cls * 32 + nn * 2) : kSOob,
+                                                    base + i * W * 32, 0);
+    };
+    const uint32_t w_off = geo.off_units + (uint32_t)(cls * UB + lane * (BITS * 4));
+    auto load_unit = [&](int i, uint32_t base, bool valid) -> WB {
+        const uint32_t off = valid && cls + i * W < ng ? w_off : kSOob;
+        if constexpr (BITS == 4) {
+            return __builtin_amdgcn_raw_buffer_load_b128(rt, off, base + i * W * UB, 2);
+        } else {
+            return __builtin_amdgcn_raw_buffer_load_b96(rt, off, base + i * W * UB, 2);
+        }
+    };
+    int tile = blockIdx.x + team * G;
+    bool vcur = tile < ntl;
+    uint32_t tb = (uint32_t)tile * geo.record_bytes;
+    if (cherry_wave) load_cherry(tb, vcur);
+#pragma unroll
+    for (int i = 0; i < L; i++) sc[i] = load_scale(i, tb, vcur);
+#pragma unroll
+    for (int i = 0; i < L; i++) wbuf[i] = load_unit(i, tb, vcur);
+    const float *xsrow = s_xsum + (4 * kq) * ng;
+    for (int t0 = blockIdx.x; t0 < ntl; t0 += stride) {
+        const int tnext = tile + stride;
+        const bool vnext = tnext < ntl;
+        const uint32_t tbn = (uint32_t)tnext * geo.record_bytes;
+        sf4_t acc = {0.f, 0.f, 0.f, 0.f};
+        if (cherry_wave) {
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+                if (32 * q < C) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(s_acr[q * 64 + lane]), as_h8(cw[q]), acc, 0, 0, 0);
+            load_cherry(tbn, vnext);
+        }
+#pragma unroll
+        for (int i = 0; i < L; i++) {
+            const int up = cls + i * W < ng ? cls + i * W : cls;  // (a unit past the last: zero codes, zero scale, zero operands)
+            const float sf = __half2float(__ushort_as_half((unsigned short)sc[i]));
+            const sf4_t v = unit_dot_regs<BITS, WB>(wbuf[i], areg[i]);
+            wbuf[i] = load_unit(i, tbn, vnext);
+            sc[i] = load_scale(i, tbn, vnext);
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[r] += (v[r] + kGrid * xsrow[r * ng + up]) * sf;
+        }
+        float *red = &s_red[wave][0];
+#pragma unroll
+        for (int r = 0; r < 4; r++) red[(4 * kq + r) * 16 + nn] = acc[r];
+        __syncthreads();
+        {
+            const int t = tid - team * 64 * W;
+            if (t < 256 && vcur) {
+                const int row = t >> 4, n = tile * kStreamTileCols + (t & 15);
+                if (row < B && n < N) {
+                    float v = 0.f;
+#pragma unroll
+                    for (int c = 0; c < W; c++) v += s_red[team * W + c][t];
+                    __half *o = mul + (size_t)row * N + n;
+                    if (accumulate) v += __half2float(*o);
+                    *o = __float2half_rn(v);
+                }
+            }
+        }
+        __syncthreads();
+        tile = tnext;
+        vcur = vnext;
+        tb = tbn;
+    }
+}
+
 constexpr int kStreamWalk = 8;  // tiles one workgroup takes at most when a launch has more tiles than resident workgroups
 
 static size_t stream_lds_bytes(const StreamGeo &g, int W, int tiles_per_wg = kStreamWalk) {
@@ -1202,17 +1421,32 @@ static size_t rows_lds_bytes(int B, const StreamGeo &g, int waves, bool stage) {
     return bytes;
 }
 
+// operand-order buffer of the register variant: units x 4 operands x 64 lanes x 16 bytes, the unit
+// sums of 16 rows, the cherry operands
+struct RowsFrag {
+    size_t xf, xsum, xcf, total;
+};
+static RowsFrag rows_frag(const StreamGeo &g) {
+    RowsFrag r;
+    r.xf = 0;
+    r.xsum = (size_t)g.ng * 4 * 64 * 16;
+    r.xcf = r.xsum + ((size_t)16 * g.ng * 4 + 255) / 256 * 256;
+    r.total = r.xcf + 4 * 64 * 16;
+    return r;
+}
+
 size_t stream_rows_scratch_bytes(int bits, int B, int K, int N, int C) {
     if (B < 2) return 0;
-    return rows_scratch(B < kRowsMax ? B : kRowsMax, stream_geo(bits, K, N, C)).total;
+    const StreamGeo geo = stream_geo(bits, K, N, C);
+    const size_t a = rows_scratch(B < kRowsMax ? B : kRowsMax, geo).total, b = rows_frag(geo).total;
+    return a > b ? a : b;
 }
 
 bool stream_rows_supported(int bits, int B, int K, int N, int C, int G) {
     if (B < 2 || B > kRowsMax) return false;
     if (!stream_supported(bits, 1, K, N, C, G)) return false;
     const StreamGeo geo = stream_geo(bits, K, N, C);
-    if (geo.ng > 64) return false;  // at most 8 units per wavefront, 8 wavefronts per team
-    return rows_lds_bytes(B, geo, 8, false) <= 160 * 1024;
+    return geo.ng <= 64;  // at most 8 units per wavefront, 8 wavefronts per team
 }
 
 template <int BITS, int W, int L, int TEAMS, bool STAGE>
@@ -1239,6 +1473,32 @@ static hipError_t launch_rows_cfg(const unsigned short *xs, const float *xsum, c
 hipError_t launch_stream_rows(int bits, const __half *vec, const uint8_t *stream, __half *mul, int B, int K, int N,
                               int C, int accumulate, void *scratch, hipStream_t s) {
     const StreamGeo geo = stream_geo(bits, K, N, C);
+    // Two main kernels.  Measured (us, whole call, 4-bit; rows in LDS / rows in registers): 4096 -> 11008
+    // 8 rows 12.5 / 13.7, 16 rows 14.1 / 14.0; 4096 -> 4096 8 rows 9.9 / 10.5, 16 rows 12.4 / 10.5;
+    // 8192 -> 28672 8 rows 35.2 / 27.6, 16 rows - / 29.2; 8192 -> 8192 8 rows 16.7 / 14.8.
+    if (B > 8 || geo.ng > 32 || rows_lds_bytes(B, geo, 8, false) > 160 * 1024) {
+        // the rows as matrix-core operands in a buffer, then the kernel that keeps them in registers
+        const RowsFrag f = rows_frag(geo);
+        su4 *xf = reinterpret_cast<su4 *>(reinterpret_cast<char *>(scratch) + f.xf);
+        float *xsum = reinterpret_cast<float *>(reinterpret_cast<char *>(scratch) + f.xsum);
+        su4 *xcf = reinterpret_cast<su4 *>(reinterpret_cast<char *>(scratch) + f.xcf);
+        hipLaunchKernelGGL(stream_rows_frag_kernel, dim3(geo.ng + 1), dim3(256), 0, s, vec, stream, xf, xsum, xcf, B, geo);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        const bool w4 = geo.ng <= 32;
+        const int teams = w4 ? 2 : 1;
+        int grid = ceil_div(geo.ntiles, teams);
+        if (grid > kStreamCus) grid = kStreamCus;
+        const size_t lds = (size_t)16 * geo.ng * 4;
+        if (bits == 4) {
+            if (w4) hipLaunchKernelGGL((stream_rows_reg_kernel<4, 4>), dim3(grid), dim3(512), lds, s, xf, xsum, xcf, stream, mul, B, accumulate, geo);
+            else hipLaunchKernelGGL((stream_rows_reg_kernel<4, 8>), dim3(grid), dim3(512), lds, s, xf, xsum, xcf, stream, mul, B, accumulate, geo);
+        } else {
+            if (w4) hipLaunchKernelGGL((stream_rows_reg_kernel<3, 4>), dim3(grid), dim3(512), lds, s, xf, xsum, xcf, stream, mul, B, accumulate, geo);
+            else hipLaunchKernelGGL((stream_rows_reg_kernel<3, 8>), dim3(grid), dim3(512), lds, s, xf, xsum, xcf, stream, mul, B, accumulate, geo);
+        }
+        return hipGetLastError();
+    }
     // teams of 8 wavefronts, 4 units each for rows of up to 32 units and 8 beyond; two teams per
     // workgroup when every compute unit gets at least two tiles
     const bool l4 = geo.ng <= 32;

@@ -207,8 +207,7 @@ def test_prepacked_c_abi_rejections(qc):
     assert lib.cherryq_prepack_bytes(5, 4096, 4096, 16) == 0
     assert lib.cherryq_prepack_supported(4, 2, 4096, 4096, 16, 128) == 1      # 2 to 16 rows: the rows kernel
     assert lib.cherryq_prepack_supported(4, 17, 4096, 4096, 16, 128) == 0
-    assert lib.cherryq_prepack_supported(4, 16, 8192, 8192, 32, 128) == 0     # 16 rows of 8192 do not fit LDS
-    assert lib.cherryq_prepack_supported(4, 8, 8192, 8192, 32, 128) == 1
+    assert lib.cherryq_prepack_supported(4, 16, 8192, 8192, 32, 128) == 1     # rows kept in registers
     assert lib.cherryq_prepack_supported(3, 2, 13824, 5120, 48, 128) == 0     # more than 64 units per column
     assert lib.cherryq_prepack_supported(4, 1, 4096, 4096, 16, 64) == 0       # group size a multiple of 128
     assert lib.cherryq_prepack_supported(4, 1, 28672, 8192, 112, 128) == 0    # more than 16384 quantised channels
@@ -363,7 +362,8 @@ def test_prepacked_layers_with_more_tiles_than_resident_workgroups(bits, k, n):
 
 
 @pytest.mark.parametrize("bits,k,n,b", [(4, 4096, 11008, 16), (3, 4096, 11008, 16), (4, 4096, 4096, 8), (3, 4096, 4096, 2),
-                                        (4, 8192, 1024, 8), (3, 1160, 264, 5), (4, 4096, 32008, 13), (4, 1024, 520, 16)])
+                                        (4, 8192, 1024, 8), (3, 1160, 264, 5), (4, 4096, 32008, 13), (4, 1024, 520, 16),
+                                        (4, 8192, 4096, 16), (3, 8192, 1032, 9), (4, 4096, 4096, 3)])
 def test_prepacked_rows_against_the_c_oracle(bits, k, n, b):
     """2 to 16 activation rows over the repacked stream (compaction launch + matrix-core launch with
     real rows): against the C oracle, one-hot rows bit for bit (also with rows of very different
