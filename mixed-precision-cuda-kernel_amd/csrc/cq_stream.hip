@@ -1072,14 +1072,15 @@ __device__ inline sf4_t unit_dot_regs(const WB w, const su4 (&a)[4]) {
     }
 }
 
-// W wavefronts per team (4: up to 32 units, 8: up to 64), 8 / W teams, 8 units per wavefront.
-template <int BITS, int W>
+// W wavefronts per team, 8 / W teams, L units per wavefront (W * L units per column at most), the
+// loads of R consecutive tiles of a team in flight (R * L per wavefront).
+template <int BITS, int W, int L, int R>
 __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restrict__ xf, const float *__restrict__ xsum_g,
                                                               const su4 *__restrict__ xcf,
                                                               const uint8_t *__restrict__ stream,
                                                               __half *__restrict__ mul, int B, int accumulate,
                                                               StreamGeo geo) {
-    constexpr int L = 8, TEAMS = 8 / W;
+    constexpr int TEAMS = 8 / W;
     constexpr int UB = BITS == 4 ? 1024 : 768;
     constexpr float kGrid = BITS == 4 ? -7.5f : -3.5f;
     __shared__ float s_red[8][256];
@@ -1110,14 +1111,14 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
     const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(
         (void *)(stream + geo.hdr_bytes), 0, (int)min((unsigned long long)ntl * geo.record_bytes, 0xffffffffull), kSFlags);
     typedef typename std::conditional<BITS == 4, su4, su3>::type WB;  // a unit: 4 or 3 dwords per lane
-    uint32_t sc[L];
-    WB wbuf[L];
-    su4 cw[4];
-    auto load_cherry = [&](uint32_t base, bool valid) {
+    uint32_t sc[R][L];
+    WB wbuf[R][L];
+    su4 cw[R][4];
+    auto load_cherry = [&](su4 (&dst)[4], uint32_t base, bool valid) {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int lg = 4 * j + kq;
-            cw[j] = __builtin_amdgcn_raw_buffer_load_b128(
+            dst[j] = __builtin_amdgcn_raw_buffer_load_b128(
                 rt, valid && 8 * lg < C ? geo.off_cherry + (uint32_t)(lg * 16 + nn) * 16u : kSOob, base, 2);
         }
     };
@@ -1134,58 +1135,69 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
             return __builtin_amdgcn_raw_buffer_load_b96(rt, off, base + i * W * UB, 2);
         }
     };
-    int tile = blockIdx.x + team * G;
-    bool vcur = tile < ntl;
-    uint32_t tb = (uint32_t)tile * geo.record_bytes;
-    if (cherry_wave) load_cherry(tb, vcur);
+    // slot s of the ring holds the tile the team reaches in its (R * j + s)-th step
+    int tile[R];
+    bool valid[R];
 #pragma unroll
-    for (int i = 0; i < L; i++) sc[i] = load_scale(i, tb, vcur);
+    for (int s = 0; s < R; s++) {
+        tile[s] = blockIdx.x + team * G + s * stride;
+        valid[s] = tile[s] < ntl;
+        const uint32_t tb = (uint32_t)tile[s] * geo.record_bytes;
+        if (cherry_wave) load_cherry(cw[s], tb, valid[s]);
 #pragma unroll
-    for (int i = 0; i < L; i++) wbuf[i] = load_unit(i, tb, vcur);
+        for (int i = 0; i < L; i++) sc[s][i] = load_scale(i, tb, valid[s]);
+#pragma unroll
+        for (int i = 0; i < L; i++) wbuf[s][i] = load_unit(i, tb, valid[s]);
+    }
     const float *xsrow = s_xsum + (4 * kq) * ng;
-    for (int t0 = blockIdx.x; t0 < ntl; t0 += stride) {
-        const int tnext = tile + stride;
-        const bool vnext = tnext < ntl;
-        const uint32_t tbn = (uint32_t)tnext * geo.record_bytes;
-        sf4_t acc = {0.f, 0.f, 0.f, 0.f};
-        if (cherry_wave) {
+    // the loop count is the same for every wavefront of the workgroup (barriers inside): as long as
+    // the workgroup's first team, which has the lowest tile, has one in slot 0
+    for (int t0 = blockIdx.x; t0 < ntl; t0 += R * stride) {
 #pragma unroll
-            for (int q = 0; q < 4; q++)
-                if (32 * q < C) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(s_acr[q * 64 + lane]), as_h8(cw[q]), acc, 0, 0, 0);
-            load_cherry(tbn, vnext);
-        }
+        for (int s = 0; s < R; s++) {
+            const int tnext = tile[s] + R * stride;
+            const bool vnext = tnext < ntl;
+            const uint32_t tbn = (uint32_t)tnext * geo.record_bytes;
+            sf4_t acc = {0.f, 0.f, 0.f, 0.f};
+            if (cherry_wave) {
 #pragma unroll
-        for (int i = 0; i < L; i++) {
-            const int up = cls + i * W < ng ? cls + i * W : cls;  // (a unit past the last: zero codes, zero scale, zero operands)
-            const float sf = __half2float(__ushort_as_half((unsigned short)sc[i]));
-            const sf4_t v = unit_dot_regs<BITS, WB>(wbuf[i], areg[i]);
-            wbuf[i] = load_unit(i, tbn, vnext);
-            sc[i] = load_scale(i, tbn, vnext);
+                for (int q = 0; q < 4; q++)
+                    if (32 * q < C)
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(s_acr[q * 64 + lane]), as_h8(cw[s][q]), acc, 0, 0, 0);
+                load_cherry(cw[s], tbn, vnext);
+            }
 #pragma unroll
-            for (int r = 0; r < 4; r++) acc[r] += (v[r] + kGrid * xsrow[r * ng + up]) * sf;
-        }
-        float *red = &s_red[wave][0];
+            for (int i = 0; i < L; i++) {
+                const int up = cls + i * W < ng ? cls + i * W : cls;  // (a unit past the last: zero codes, zero scale, zero operands)
+                const float sf = __half2float(__ushort_as_half((unsigned short)sc[s][i]));
+                const sf4_t v = unit_dot_regs<BITS, WB>(wbuf[s][i], areg[i]);
+                wbuf[s][i] = load_unit(i, tbn, vnext);
+                sc[s][i] = load_scale(i, tbn, vnext);
 #pragma unroll
-        for (int r = 0; r < 4; r++) red[(4 * kq + r) * 16 + nn] = acc[r];
-        __syncthreads();
-        {
-            const int t = tid - team * 64 * W;
-            if (t < 256 && vcur) {
-                const int row = t >> 4, n = tile * kStreamTileCols + (t & 15);
-                if (row < B && n < N) {
-                    float v = 0.f;
+                for (int r = 0; r < 4; r++) acc[r] += (v[r] + kGrid * xsrow[r * ng + up]) * sf;
+            }
+            float *red = &s_red[wave][0];
 #pragma unroll
-                    for (int c = 0; c < W; c++) v += s_red[team * W + c][t];
-                    __half *o = mul + (size_t)row * N + n;
-                    if (accumulate) v += __half2float(*o);
-                    *o = __float2half_rn(v);
+            for (int r = 0; r < 4; r++) red[(4 * kq + r) * 16 + nn] = acc[r];
+            __syncthreads();
+            {
+                const int t = tid - team * 64 * W;
+                if (t < 256 && valid[s]) {
+                    const int row = t >> 4, n = tile[s] * kStreamTileCols + (t & 15);
+                    if (row < B && n < N) {
+                        float v = 0.f;
+#pragma unroll
+                        for (int c = 0; c < W; c++) v += s_red[team * W + c][t];
+                        __half *o = mul + (size_t)row * N + n;
+                        if (accumulate) v += __half2float(*o);
+                        *o = __float2half_rn(v);
+                    }
                 }
             }
+            __syncthreads();
+            tile[s] = tnext;
+            valid[s] = vnext;
         }
-        __syncthreads();
-        tile = tnext;
-        vcur = vnext;
-        tb = tbn;
     }
 }
 
@@ -1474,9 +1486,9 @@ hipError_t launch_stream_rows(int bits, const __half *vec, const uint8_t *stream
                               int C, int accumulate, void *scratch, hipStream_t s) {
     const StreamGeo geo = stream_geo(bits, K, N, C);
     // Two main kernels.  Measured (us, whole call, 4-bit; rows in LDS / rows in registers): 4096 -> 11008
-    // 8 rows 12.5 / 13.7, 16 rows 14.1 / 14.0; 4096 -> 4096 8 rows 9.9 / 10.5, 16 rows 12.4 / 10.5;
-    // 8192 -> 28672 8 rows 35.2 / 27.6, 16 rows - / 29.2; 8192 -> 8192 8 rows 16.7 / 14.8.
-    if (B > 8 || geo.ng > 32 || rows_lds_bytes(B, geo, 8, false) > 160 * 1024) {
+    // 5 rows 12.0 / 12.4, 8 rows 12.4 / 12.5, 16 rows 14.1 / 12.6; 4096 -> 4096 8 rows 9.9 / 9.4, 16 rows
+    // 12.4 / 9.6; 8192 -> 28672 8 rows 35.2 / 27.6, 16 rows - / 29.2; 8192 -> 8192 8 rows 16.7 / 14.8.
+    if (B >= 8 || geo.ng > 32 || rows_lds_bytes(B, geo, 8, false) > 160 * 1024) {
         // the rows as matrix-core operands in a buffer, then the kernel that keeps them in registers
         const RowsFrag f = rows_frag(geo);
         su4 *xf = reinterpret_cast<su4 *>(reinterpret_cast<char *>(scratch) + f.xf);
@@ -1486,17 +1498,21 @@ hipError_t launch_stream_rows(int bits, const __half *vec, const uint8_t *stream
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         const bool w4 = geo.ng <= 32;
-        const int teams = w4 ? 2 : 1;
-        int grid = ceil_div(geo.ntiles, teams);
-        if (grid > kStreamCus) grid = kStreamCus;
+        const int grid = geo.ntiles < kStreamCus ? geo.ntiles : kStreamCus;  // one team of 8 wavefronts per workgroup
         const size_t lds = (size_t)16 * geo.ng * 4;
+#define CQ_REG_GO(BITS_, W_, L_, R_)                                                                                  \
+    hipLaunchKernelGGL((stream_rows_reg_kernel<BITS_, W_, L_, R_>), dim3(grid), dim3(512), lds, s, xf, xsum, xcf, stream, mul,  \
+                       B, accumulate, geo)
+        // up to 32 units: 4 per wavefront and the loads of two tiles in flight (measured on 4096 ->
+        // 11008, 16 rows: 12.6 us against 13.8 with two teams of 4 wavefronts x 8 units); else 8 per wavefront
         if (bits == 4) {
-            if (w4) hipLaunchKernelGGL((stream_rows_reg_kernel<4, 4>), dim3(grid), dim3(512), lds, s, xf, xsum, xcf, stream, mul, B, accumulate, geo);
-            else hipLaunchKernelGGL((stream_rows_reg_kernel<4, 8>), dim3(grid), dim3(512), lds, s, xf, xsum, xcf, stream, mul, B, accumulate, geo);
+            if (w4) CQ_REG_GO(4, 8, 4, 2);
+            else CQ_REG_GO(4, 8, 8, 1);
         } else {
-            if (w4) hipLaunchKernelGGL((stream_rows_reg_kernel<3, 4>), dim3(grid), dim3(512), lds, s, xf, xsum, xcf, stream, mul, B, accumulate, geo);
-            else hipLaunchKernelGGL((stream_rows_reg_kernel<3, 8>), dim3(grid), dim3(512), lds, s, xf, xsum, xcf, stream, mul, B, accumulate, geo);
+            if (w4) CQ_REG_GO(3, 8, 4, 2);
+            else CQ_REG_GO(3, 8, 8, 1);
         }
+#undef CQ_REG_GO
         return hipGetLastError();
     }
     // teams of 8 wavefronts, 4 units each for rows of up to 32 units and 8 beyond; two teams per
