@@ -446,9 +446,13 @@ def main():
                 torch.cuda.empty_cache()
             print(line, file=sys.stderr, flush=True)
 
-    def kernel_name(bits, batch, path):
+    def kernel_name(bits, batch, path, k_in=0):
         if path == "prepacked":
-            return f"cq::stream_kernel<{bits}>" if batch == 1 else f"cq::stream_rows_prep_kernel + cq::stream_rows_kernel<{bits}>"
+            if batch == 1:
+                return f"cq::stream_kernel<{bits}>"
+            if batch >= 8 or k_in > 32 * args.group:  # the rule of launch_stream_rows: activations in registers
+                return f"cq::stream_rows_frag_kernel + cq::stream_rows_reg_kernel<{bits}>"
+            return f"cq::stream_rows_prep_kernel + cq::stream_rows_kernel<{bits}>"
         if batch == 1:
             return f"cq::matvec_kernel<{bits}>"
         if batch <= 4:
@@ -510,7 +514,7 @@ def main():
                                         "bench.py (profiles/); not re-measured in this run") if traffic else
                                        "not measured for this workload / kernel",
                      "algorithmic_bytes_per_launch": ab,
-                     "kernel": kernel_name(bits, args.batch, path)},
+                     "kernel": kernel_name(bits, args.batch, path, k)},
     }
     if main_run["resident_us"] is not None:
         ru = main_run["resident_us"]
