@@ -70,8 +70,8 @@ class QuantLinear(nn.Module):
     # is 1.6x faster at 128 rows of a 4096 -> 11008 layer, level at 512, 1.3x slower at 2048).
     prefill_rows = 512
     # from this many rows (up to 16) a prepack()ed layer runs the rows kernel over the weight stream;
-    # measured on 4096 -> 11008, 4-bit (us, stream / checkpoint layout): 2 rows 9.9 / 9.1, 4 rows
-    # 10.6 / 11.3, 8 rows 13.0 / 16.8, 16 rows 14.4 / 19.1
+    # measured on 4096 -> 11008, 4-bit (us, stream / checkpoint layout): 2 rows 9.8 / 9.2, 4 rows
+    # 10.5 / 11.3, 8 rows 12.5 / 16.8, 16 rows 12.7 / 19.0
     stream_rows_min = 4
 
     @classmethod
