@@ -329,6 +329,19 @@ int cherryq_decode_rope_attention_f16(const void *q, const void *k, const void *
                                       void *out, const int *position, int n_heads, int n_kv_heads,
                                       int head_dim, int max_len, float theta, void *stream);
 /*
+ * Unquantised fp16 head of the decode step: logits (vocab fp16) = act W^T with lm_head W (vocab,
+ * hidden_size) row-major as the reference holds it (llama/modeling_llama_quant.py:1132), fp32
+ * accumulation, one rounding; act = norm_weight * fp16(hidden * rsqrt(mean(hidden^2) + eps)), the
+ * final RMSNorm (:1064, :75-89) fused into the launch, or hidden itself when norm_weight is NULL.
+ * A plain HBM stream over the matrix (the largest single read of a token step).  hidden_size a
+ * multiple of 512, at most 8192 (cherryq_decode_head_supported); hidden, norm_weight, lm_head
+ * 16-byte aligned.
+ */
+int cherryq_decode_head_supported(int vocab, int hidden_size);
+int cherryq_decode_head_f16(const void *hidden, const void *norm_weight /* may be NULL */, float eps,
+                            const void *lm_head, void *logits, int vocab, int hidden_size, void *stream);
+
+/*
  * Tail of a greedy step: *next_token = argmax(logits[0..vocab)) (lowest index among equal maxima),
  * history[*position] = that token when history is non-NULL and the position lies below
  * history_len, hidden_out[0..hidden) = embed[token] (the next step's input), *position += 1.

@@ -39,6 +39,10 @@ _lib.cherryq_decode_silu_mul_f16.argtypes = [_vp, _vp, _vp, _int, _vp]
 _lib.cherryq_decode_argmax_embed_f16.argtypes = [_vp, _int, _vp, _int, _vp, _vp, _vp, _int, _vp, _vp]
 _lib.cherryq_decode_argmax_embed_f16.restype = _int
 _lib.cherryq_decode_rope_attention_f16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _f, _vp]
+_lib.cherryq_decode_head_supported.argtypes = [_int, _int]
+_lib.cherryq_decode_head_supported.restype = _int
+_lib.cherryq_decode_head_f16.argtypes = [_vp, _vp, _f, _vp, _vp, _int, _int, _vp]
+_lib.cherryq_decode_head_f16.restype = _int
 for _n in ("cherryq_decode_add_rmsnorm_f16", "cherryq_decode_rope_cache_f16", "cherryq_decode_attention_f16",
            "cherryq_decode_silu_mul_f16", "cherryq_decode_rope_attention_f16"):
     getattr(_lib, _n).restype = _int
@@ -236,6 +240,7 @@ class CherryLlamaDecoder(nn.Module):
         self.lm_head_t = self.lm_head.t()
         self._graph = None
         self.fuse_norm = True
+        self.fuse_head = True  # final RMSNorm + fp16 head as one launch of the library's own kernel
         self.layer_trace = None
         self._side = [torch.cuda.Stream(device=self.device_) for _ in range(2)] if self.device_.type == "cuda" else []
 
@@ -360,14 +365,23 @@ class CherryLlamaDecoder(nn.Module):
             matvec_group([layer.down_proj], self.up, [self.hid], vec_gate=self.gate, accumulate=True)
             if self.layer_trace is not None:  # validation only (eager runs): the hidden state after every layer
                 self.layer_trace.append(self.hid.clone())
-        self._norm(self.norm)
-        self._head()
+        if self.fuse_head and _lib.cherryq_decode_head_supported(cfg.vocab_size, cfg.hidden_size):
+            self._head(normed=False)
+        else:
+            self._norm(self.norm)
+            self._head()
 
-    def _head(self):
+    def _head(self, normed=True):
         """Unquantised fp16 head, then the greedy tail on the device: next_token = argmax, recorded
-        in history[pos]; its embedding becomes the next step's hidden state; pos += 1."""
+        in history[pos]; its embedding becomes the next step's hidden state; pos += 1.
+        normed=False: the final RMSNorm has not been applied yet and is fused into the head launch."""
         cfg = self.cfg
-        torch.matmul(self.normed, self.lm_head_t, out=self.logits16)
+        if normed:
+            torch.matmul(self.normed, self.lm_head_t, out=self.logits16)
+        else:
+            _ok(_lib.cherryq_decode_head_f16(self.hid.data_ptr(), self.norm.data_ptr(), cfg.rms_norm_eps,
+                                             self.lm_head.data_ptr(), self.logits16.data_ptr(), cfg.vocab_size,
+                                             cfg.hidden_size, _stream()), "head")
         _ok(_lib.cherryq_decode_argmax_embed_f16(self.logits16.data_ptr(), cfg.vocab_size, self.embed_tokens.data_ptr(),
                                                  cfg.hidden_size, self.hid.data_ptr(), self.next_token.data_ptr(),
                                                  self.history.data_ptr(), self.history.numel(), self.pos.data_ptr(),

@@ -638,6 +638,21 @@ int cherryq_decode_rope_attention_f16(const void *q, const void *k, const void *
         reinterpret_cast<hipStream_t>(stream));
 }
 
+int cherryq_decode_head_supported(int vocab, int hidden_size) { return cq::head_supported(vocab, hidden_size) ? 1 : 0; }
+
+int cherryq_decode_head_f16(const void *hidden, const void *norm_weight, float eps, const void *lm_head, void *logits,
+                            int vocab, int hidden_size, void *stream) {
+    if (!hidden || !lm_head || !logits) return CHERRYQ_E_NULL;
+    if (vocab <= 0 || hidden_size <= 0) return CHERRYQ_E_SHAPE;
+    if (!cq::head_supported(vocab, hidden_size)) return CHERRYQ_E_UNSUPPORTED;
+    if (!cq::aligned(hidden, 16) || !cq::aligned(lm_head, 16) || !cq::aligned(logits, 2) ||
+        (norm_weight && !cq::aligned(norm_weight, 16)))
+        return CHERRYQ_E_ALIGN;
+    return (int)cq::launch_head(reinterpret_cast<const __half *>(hidden), reinterpret_cast<const __half *>(norm_weight), eps,
+                                reinterpret_cast<const __half *>(lm_head), reinterpret_cast<__half *>(logits), vocab,
+                                hidden_size, reinterpret_cast<hipStream_t>(stream));
+}
+
 int cherryq_decode_argmax_embed_f16(const void *logits, int vocab, const void *embed, int hidden, void *hidden_out,
                                     long long *next_token, long long *history, int history_len, int *position,
                                     void *stream) {

@@ -419,6 +419,112 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const __half *__restrict_
     out[i] = __float2half_rn(a * __half2float(up[i]));
 }
 
+// Unquantised fp16 head: logits[v] = fp16(sum_k act[k] * W[v][k]) with W (vocab, hidden) row-major
+// as the reference's lm_head holds it (llama/modeling_llama_quant.py:1132), fp32 accumulation, and
+// act = weight * fp16(h * rsqrt(mean(h^2) + eps)) -- the final RMSNorm (:1064), with the rounding
+// points of add_rmsnorm_kernel -- or act = h when no norm weight is given.  The matrix is the
+// largest single read of a token step (262 MB for 32000 x 4096), so the kernel is a plain
+// HBM stream: every wavefront keeps the whole activation row in registers (CH pieces of 16 bytes
+// per lane), normalises it itself (no LDS, no barrier) and then takes rows v = w, w + waves, ...,
+// one row = CH loads of 1 KB, the next row's loads in flight while the current one is multiplied.
+typedef uint32_t hu4 __attribute__((ext_vector_type(4)));
+
+template <int CH>
+__global__ __launch_bounds__(256) void head_kernel(const __half *__restrict__ h, const __half *__restrict__ norm_w,
+                                                   float eps, const __half *__restrict__ W,
+                                                   __half *__restrict__ logits, int V) {
+    constexpr int H = 512 * CH;
+    const int lane = threadIdx.x & 63;
+    const int w = blockIdx.x * 4 + (threadIdx.x >> 6), nw = gridDim.x * 4;
+    auto load_row = [&](hu4 (&dst)[CH], int v) {
+        const hu4 *row = reinterpret_cast<const hu4 *>(W + (size_t)v * H);
+#pragma unroll
+        for (int c = 0; c < CH; c++) dst[c] = __builtin_nontemporal_load(row + c * 64 + lane);
+    };
+    float x[CH][8];
+    {
+        hu4 xr[CH];
+#pragma unroll
+        for (int c = 0; c < CH; c++) xr[c] = reinterpret_cast<const hu4 *>(h)[c * 64 + lane];
+        if (norm_w) {
+            hu4 nr[CH];
+#pragma unroll
+            for (int c = 0; c < CH; c++) nr[c] = reinterpret_cast<const hu4 *>(norm_w)[c * 64 + lane];
+            float ss = 0.f;
+#pragma unroll
+            for (int c = 0; c < CH; c++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const float a = __half2float(__ushort_as_half((unsigned short)(xr[c][j] & 0xffffu)));
+                    const float b = __half2float(__ushort_as_half((unsigned short)(xr[c][j] >> 16)));
+                    ss += a * a + b * b;
+                }
+            ss = wave_sum_all(ss);
+            const float rs = rsqrtf(ss / (float)H + eps);
+#pragma unroll
+            for (int c = 0; c < CH; c++)
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const float xv = __half2float(__ushort_as_half((unsigned short)(xr[c][j >> 1] >> (16 * (j & 1)))));
+                    const float wv = __half2float(__ushort_as_half((unsigned short)(nr[c][j >> 1] >> (16 * (j & 1)))));
+                    const float n = __half2float(__float2half_rn(xv * rs));
+                    x[c][j] = __half2float(__float2half_rn(wv * n));
+                }
+        } else {
+#pragma unroll
+            for (int c = 0; c < CH; c++)
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    x[c][j] = __half2float(__ushort_as_half((unsigned short)(xr[c][j >> 1] >> (16 * (j & 1)))));
+        }
+    }
+    auto finish_row = [&](const hu4 (&r)[CH], int v) {
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; c++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                a0 = fmaf(__half2float(__ushort_as_half((unsigned short)(r[c][j] & 0xffffu))), x[c][2 * j], a0);
+                a1 = fmaf(__half2float(__ushort_as_half((unsigned short)(r[c][j] >> 16))), x[c][2 * j + 1], a1);
+            }
+        const float tot = wave_sum_all(a0 + a1);
+        if (lane == 0) logits[v] = __float2half_rn(tot);
+    };
+    hu4 ra[CH], rb[CH];
+    int v = w;
+    if (v < V) load_row(ra, v);
+    while (v < V) {
+        if (v + nw < V) load_row(rb, v + nw);
+        finish_row(ra, v);
+        v += nw;
+        if (v >= V) break;
+        if (v + nw < V) load_row(ra, v + nw);
+        finish_row(rb, v);
+        v += nw;
+    }
+}
+
+bool head_supported(int vocab, int hidden) { return vocab > 0 && hidden >= 512 && hidden <= 8192 && hidden % 512 == 0; }
+
+hipError_t launch_head(const __half *h, const __half *norm_w, float eps, const __half *W, __half *logits, int vocab,
+                       int hidden, hipStream_t stream) {
+    if (!head_supported(vocab, hidden)) return hipErrorInvalidValue;
+    int grid = ceil_div(vocab, 4);
+    if (grid > 1024) grid = 1024;  // four wavefronts per SIMD
+    switch (hidden / 512) {
+#define CQ_HEAD_CASE(CH_)                                                                                         \
+    case CH_:                                                                                                     \
+        hipLaunchKernelGGL(head_kernel<CH_>, dim3(grid), dim3(256), 0, stream, h, norm_w, eps, W, logits, vocab); \
+        break;
+        CQ_HEAD_CASE(1) CQ_HEAD_CASE(2) CQ_HEAD_CASE(3) CQ_HEAD_CASE(4) CQ_HEAD_CASE(5) CQ_HEAD_CASE(6) CQ_HEAD_CASE(7)
+        CQ_HEAD_CASE(8) CQ_HEAD_CASE(9) CQ_HEAD_CASE(10) CQ_HEAD_CASE(11) CQ_HEAD_CASE(12) CQ_HEAD_CASE(13)
+        CQ_HEAD_CASE(14) CQ_HEAD_CASE(15) CQ_HEAD_CASE(16)
+#undef CQ_HEAD_CASE
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 // Tail of a greedy decoding step, one workgroup: next = argmax(logits) (lowest index among equal
 // maxima), recorded in *next_token and history[*pos]; the next token's embedding row becomes the
 // hidden state of the following step; *pos += 1.  What the reference's generation loop does on

@@ -175,6 +175,10 @@ hipError_t launch_rope_attn_decode(const __half *q, const __half *k, const __hal
 hipError_t launch_argmax_embed(const __half *logits, int vocab, const __half *embed, int hidden, __half *hid,
                                long long *next_token, long long *history, int history_len, int *pos,
                                hipStream_t stream);
+// fp16 head with the final RMSNorm fused (norm_w may be null); hidden a multiple of 512, at most 8192
+bool head_supported(int vocab, int hidden);
+hipError_t launch_head(const __half *h, const __half *norm_w, float eps, const __half *W, __half *logits, int vocab,
+                       int hidden, hipStream_t stream);
 hipError_t launch_silu_mul(const __half *gate, const __half *up, __half *out, int n, hipStream_t stream);
 int attn_max_len();
 

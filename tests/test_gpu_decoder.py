@@ -136,6 +136,54 @@ def test_silu_mul_kernel(dec):
     assert rel(o, torch.nn.functional.silu(g) * u) < 1e-3
 
 
+@pytest.mark.parametrize("V,H", [(32000, 4096), (1000, 1024), (517, 512), (32003, 5120), (4099, 8192)])
+def test_head_kernel_with_fused_final_norm(dec, V, H):
+    """fp16 head (final RMSNorm fused or not) against float64 on the same fp16 operands: one
+    rounding of the fp32-accumulated sum, rel-L2 below 1e-3; a one-hot row returns the matrix
+    column bit for bit; the separate norm launch + this kernel without norm give the same bits."""
+    print("[case] head", V, H, flush=True)
+    lib = dec._lib
+    g = torch.Generator().manual_seed(V + H)
+    h = torch.randn(1, H, generator=g).half().cuda()
+    nw = (1 + 0.1 * torch.randn(H, generator=g)).half().cuda()
+    W = (torch.randn(V, H, generator=g) * 0.02).half().cuda()
+    out = torch.full((1, V), float("nan"), dtype=torch.float16, device="cuda")
+    for norm in (True, False):
+        assert lib.cherryq_decode_head_f16(h.data_ptr(), nw.data_ptr() if norm else None, 1e-6, W.data_ptr(),
+                                           out.data_ptr(), V, H, stream()) == 0
+        hf = h.float()
+        act = (nw.float() * (hf * torch.rsqrt((hf * hf).mean() + 1e-6)).half().float()).half() if norm else h
+        want = act.double() @ W.double().t()
+        assert rel(out, want) < 1e-3, (norm, rel(out, want))
+    onehot = torch.zeros(1, H, dtype=torch.float16, device="cuda")
+    onehot[0, H - 3] = 1.0
+    assert lib.cherryq_decode_head_f16(onehot.data_ptr(), None, 0.0, W.data_ptr(), out.data_ptr(), V, H, stream()) == 0
+    assert torch.equal(out[0], W[:, H - 3])
+    normed = torch.empty_like(h)
+    h2 = h.clone()
+    assert lib.cherryq_decode_add_rmsnorm_f16(h2.data_ptr(), None, nw.data_ptr(), normed.data_ptr(), H, 1e-6, stream()) == 0
+    two = torch.empty_like(out)
+    assert lib.cherryq_decode_head_f16(normed.data_ptr(), None, 0.0, W.data_ptr(), two.data_ptr(), V, H, stream()) == 0
+    assert lib.cherryq_decode_head_f16(h.data_ptr(), nw.data_ptr(), 1e-6, W.data_ptr(), out.data_ptr(), V, H, stream()) == 0
+    # the sum of squares is added up in another order than in the separate launch: the normalised
+    # row may differ by an fp16 ulp here and there, the logits by a few
+    assert rel(out, two.double()) < 1e-3
+
+
+def test_head_validation(dec):
+    lib = dec._lib
+    h = torch.zeros(1, 4096, dtype=torch.float16, device="cuda")
+    W = torch.zeros(8, 4096, dtype=torch.float16, device="cuda")
+    out = torch.zeros(1, 8, dtype=torch.float16, device="cuda")
+    assert lib.cherryq_decode_head_supported(32000, 4096) == 1
+    assert lib.cherryq_decode_head_supported(32000, 256) == 0 and lib.cherryq_decode_head_supported(32000, 8704) == 0
+    assert lib.cherryq_decode_head_supported(32000, 4100) == 0
+    assert lib.cherryq_decode_head_f16(None, None, 0.0, W.data_ptr(), out.data_ptr(), 8, 4096, stream()) == -1
+    assert lib.cherryq_decode_head_f16(h.data_ptr(), None, 0.0, W.data_ptr(), out.data_ptr(), 0, 4096, stream()) == -2
+    assert lib.cherryq_decode_head_f16(h.data_ptr(), None, 0.0, W.data_ptr(), out.data_ptr(), 8, 256, stream()) == -7
+    assert lib.cherryq_decode_head_f16(h.data_ptr() + 2, None, 0.0, W.data_ptr(), out.data_ptr(), 8, 4096, stream()) == -6
+
+
 def test_decode_validation(dec):
     lib = dec._lib
     assert lib.cherryq_decode_add_rmsnorm_f16(None, None, None, None, 4096, 1e-6, None) == -1
