@@ -363,7 +363,8 @@ def test_prepacked_layers_with_more_tiles_than_resident_workgroups(bits, k, n):
 
 @pytest.mark.parametrize("bits,k,n,b", [(4, 4096, 11008, 16), (3, 4096, 11008, 16), (4, 4096, 4096, 8), (3, 4096, 4096, 2),
                                         (4, 8192, 1024, 8), (3, 1160, 264, 5), (4, 4096, 32008, 13), (4, 1024, 520, 16),
-                                        (4, 8192, 4096, 16), (3, 8192, 1032, 9), (4, 4096, 4096, 3)])
+                                        (4, 8192, 4096, 16), (3, 8192, 1032, 9), (4, 4096, 4096, 3),
+                                        (3, 4096, 4112, 8), (4, 2048, 16, 16), (3, 1160, 264, 12), (4, 8192, 8200, 16)])
 def test_prepacked_rows_against_the_c_oracle(bits, k, n, b):
     """2 to 16 activation rows over the repacked stream (compaction launch + matrix-core launch with
     real rows): against the C oracle, one-hot rows bit for bit (also with rows of very different
