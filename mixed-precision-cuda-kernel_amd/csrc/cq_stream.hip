@@ -363,6 +363,13 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kq = lane >> 4, nn = lane & 15;
     const bool stager = wave >= W;
+    // The staging wavefronts are the critical path until the second barrier: they get the issue
+    // slots first.  (Measured on 4096 -> 11008: 6.34 / 6.08 us against 6.48 / 6.24, 4-bit / 3-bit;
+    // with 8 computing wavefronts 4.02 against 3.94 on 4096 -> 4096, and with the fused RMSNorm
+    // 7.51 against 7.21 on the q/k/v group, so only here.)
+    if constexpr (S > 0 && W == 4 && !NORM) {
+        if (stager) __builtin_amdgcn_s_setprio(3);
+    }
     const int K = K0, C = geo.C, ng = geo.ng;
     const int Knp = ng * kStreamUnitK;
     const int Cp = (C + 31) & ~31;
