@@ -1239,6 +1239,7 @@ static int stream_pick(const StreamGeo &geo) {
     if (CQS_PICK_OVERRIDE >= 0) return CQS_PICK_OVERRIDE;
 #endif
     // Measured (us per launch, 4-bit / 3-bit; W computing + S staging wavefronts, L units each):
+    // (entry 0 before its staging wavefronts got issue priority, which took 0.15 us off its single-layer figures)
     // 4096 -> 11008 (688 tiles): entry 0 6.49 / 6.25, entry 1 7.52 / 7.37, W4 L8 S0 6.90 / 6.56,
     //   W8 L4 S0 6.54 / 6.23, W4 L8 S1 6.39-7.76 (the single staging wavefront is the critical path and
     //   its speed moved by more than a microsecond with unrelated changes of the code: not used);
