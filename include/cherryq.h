@@ -223,7 +223,8 @@ int cherryq_vecquant_matmul_f16_static(int w_bits, const void *vec, const uint8_
  * stream: cherryq_prepack_bytes() bytes, 256-byte aligned, written by cherryq_prepack_f16 once
  * per layer.  group_size must be a multiple of 128 (the stream stores one scale row per 128
  * positions); cherryq_prepack_supported() says whether a shape is taken at all (at most 128
- * cherry channels, at most 16384 + 128 input channels, batch 1).  vec must be 16-byte aligned.
+ * cherry channels, at most 16384 + 128 input channels, a stream of less than 2 GiB, batch 1).  vec
+ * must be 16-byte aligned.
  */
 size_t cherryq_prepack_bytes(int w_bits, int in_features, int out_features, int num_cherries);
 int cherryq_prepack_supported(int w_bits, int batch, int in_features, int out_features, int num_cherries,
@@ -251,7 +252,8 @@ int cherryq_matvec_prepacked_f16(int w_bits, const void *vec, const void *stream
  * inside the main launch) and then stay in LDS or in registers while a workgroup walks its
  * tiles; layers of up to 8192 + 128 input channels (64 units of 128 positions) are taken.  batch == 1 forwards to
  * cherryq_matvec_prepacked_f16 (scratch may then be NULL).  cherryq_prepack_supported(w_bits,
- * batch, ...) says whether a batch is taken.
+ * batch, ...) says whether a batch is taken.  vec must be 16-byte aligned (the rows are read as
+ * 16-byte pieces; in_features is a multiple of 8, so every row then is).
  */
 size_t cherryq_prepacked_scratch_bytes(int w_bits, int batch, int in_features, int out_features, int num_cherries);
 int cherryq_matmul_prepacked_f16(int w_bits, const void *vec, const void *stream, size_t stream_bytes, void *mul,

@@ -486,7 +486,7 @@ int cherryq_matmul_prepacked_f16(int w_bits, const void *vec, const void *stream
     if (!cq::stream_rows_supported(w_bits, batch, in_features, out_features, num_cherries, cq::kStreamUnitK))
         return CHERRYQ_E_UNSUPPORTED;
     if (!vec || !stream || !mul) return CHERRYQ_E_NULL;
-    if (!cq::aligned(stream, 256) || !cq::aligned(vec, 2) || !cq::aligned(mul, 2)) return CHERRYQ_E_ALIGN;
+    if (!cq::aligned(stream, 256) || !cq::aligned(vec, 16) || !cq::aligned(mul, 2)) return CHERRYQ_E_ALIGN;
     if (!scratch || !cq::aligned(scratch, 256) ||
         scratch_bytes < cq::stream_rows_scratch_bytes(w_bits, batch, in_features, out_features, num_cherries))
         return CHERRYQ_E_WORKSPACE;

@@ -31,6 +31,7 @@
 // Arithmetic contract: csrc/quant_cuda_kernel.cu:718-835 (4-bit) and 558-672 (3-bit) of the
 // reference; fp32 accumulation, one rounding to fp16.  Replaces the per-thread decode loops at
 // :811-831 / :649-667 and the serial batch loop :797-834.
+#include <mutex>
 #include <type_traits>
 
 #include "cq_device.h"
@@ -567,10 +568,10 @@ __global__ __launch_bounds__(64 * (W + S)) void stream_kernel(const __half *__re
 #pragma unroll
                 for (int i = 0; i < L; i++) {
                     // a unit past the last one of the column reads zero codes and a zero scale; its
-                    // activations are taken from unit `cls` so that no stale LDS contents (NaN
-                    // patterns) meet the zeros
+                    // activations are taken from unit 0, which every layer has and which is always
+                    // staged, so that no stale LDS contents (NaN patterns) meet the zeros
                     const bool real = cls + i * W < ng;
-                    const int up = real ? cls + i * W : cls;
+                    const int up = real ? cls + i * W : 0;
                     const float sf = (i & 3) == kq ? __half2float(__ushort_as_half((unsigned short)sc[i >> 2])) : 0.f;
                     const su4 w = wbuf[i % D];
                     const float v = unit_dot<BITS>(w, s_xs + up * kStreamUnitK + 32 * kq);
@@ -942,9 +943,10 @@ __global__ __launch_bounds__(64 * W * TEAMS) void stream_rows_kernel(
         }
 #pragma unroll
         for (int i = 0; i < L; i++) {
-            // a unit past the column's last reads zero codes and a zero scale; its activations are
-            // taken from unit `cls`, which exists
-            const int up = cls + i * W < ng ? cls + i * W : cls;
+            // a unit past the column's last reads zero codes and a zero scale; its activations and
+            // unit sum are taken from unit 0, which every layer has (unit `cls` need not exist when
+            // a column has fewer units than the team has wavefronts)
+            const int up = cls + i * W < ng ? cls + i * W : 0;
             const float sf = __half2float(__ushort_as_half((unsigned short)sc[i]));
             const sf4_t v = unit_dot_rows<BITS>(wbuf[i], xrow + up * kStreamUnitK);
             wbuf[i] = load_unit(i, tbn, vnext);
@@ -1175,7 +1177,7 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
             }
 #pragma unroll
             for (int i = 0; i < L; i++) {
-                const int up = cls + i * W < ng ? cls + i * W : cls;  // (a unit past the last: zero codes, zero scale, zero operands)
+                const int up = cls + i * W < ng ? cls + i * W : 0;  // (a unit past the last: zero codes, zero scale, zero operands; unit 0's sum, which exists)
                 const float sf = __half2float(__ushort_as_half((unsigned short)sc[s][i]));
                 const sf4_t v = unit_dot_regs<BITS, WB>(wbuf[s][i], areg[i]);
                 wbuf[s][i] = load_unit(i, tbn, vnext);
@@ -1235,9 +1237,6 @@ constexpr int kStreamCfgCount = sizeof(kStreamCfgs) / sizeof(kStreamCfgs[0]);
 
 
 static int stream_pick(const StreamGeo &geo) {
-#ifdef CQS_PICK_OVERRIDE  // a tuning harness that includes this file may force an entry of the table
-    if (CQS_PICK_OVERRIDE >= 0) return CQS_PICK_OVERRIDE;
-#endif
     // Measured (us per launch, 4-bit / 3-bit; W computing + S staging wavefronts, L units each):
     // (entry 0 before its staging wavefronts got issue priority, which took 0.15 us off its single-layer figures)
     // 4096 -> 11008 (688 tiles): entry 0 6.49 / 6.25, entry 1 7.52 / 7.37, W4 L8 S0 6.90 / 6.56,
@@ -1271,12 +1270,28 @@ bool stream_supported(int bits, int B, int K, int N, int C, int G) {
     if (K - C <= 0 || C > 128 || K > 32768) return false;
     if (K % 8 || N % 8 || C % 8) return false;
     const StreamGeo geo = stream_geo(bits, K, N, C);
+    // tile records are addressed with 32-bit byte offsets, and an offset with bit 31 set is how the
+    // kernels read zeros for units that do not exist: the whole stream stays below 2 GiB
+    if ((unsigned long long)geo.hdr_bytes + (unsigned long long)geo.ntiles * geo.record_bytes >= 0x7fff0000ull) return false;
     const int i = stream_pick(geo);
     if (i < 0) return false;
     return stream_lds_bytes(geo, kStreamCfgs[i].W) <= 160 * 1024;
 }
 
 constexpr int kStreamCus = 256;  // compute units of an MI355X
+constexpr int kMaxDevices = 64;  // GPUs of one process that the per-device launch plans cover
+
+struct DevicePlan {
+    bool big_lds = false, asked = false;
+    int regs[2] = {0, 0};
+};
+// vector registers per lane of a kernel (0 if the runtime does not say)
+static int kernel_vgprs(const void *k) {
+    hipFuncAttributes attr;
+    if (hipFuncGetAttributes(&attr, k) == hipSuccess && attr.numRegs > 0) return attr.numRegs;
+    (void)hipGetLastError();
+    return 0;
+}
 
 template <int BITS, int I, bool NORM>
 static hipError_t launch_stream_cfg(const __half *vec, const StreamGroup &grp, const __half *norm_w, float eps,
@@ -1296,39 +1311,50 @@ static hipError_t launch_stream_cfg(const __half *vec, const StreamGroup &grp, c
     auto kern_walk = stream_kernel<BITS, c.W, c.T, c.D, c.L, c.S, c.NB, XL, NORM, true, kCanWalk ? kStreamWalk : 1>;
     const size_t lds_walk = stream_lds_bytes(geo, c.W, kStreamWalk);
     if (stream_lds_bytes(geo, c.W, 1) > 160 * 1024) return hipErrorInvalidValue;
-    // (per instantiation; the calls are idempotent, a race between host threads only repeats them)
-    static bool big_lds_enabled = false;
-    if (lds_walk > 48 * 1024 && !big_lds_enabled) {
-        for (const void *k : {reinterpret_cast<const void *>(kern_one), reinterpret_cast<const void *>(kern_grp),
-                              reinterpret_cast<const void *>(kern_walk)}) {
-            hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-            if (e != hipSuccess) return e;
+    // Per instantiation and device, found once under a lock (the entry points are re-entrant): the
+    // 160 KB dynamic-LDS limit raised, and the register counts of the one-tile and the walking kernel.
+    static std::mutex mu;
+    static DevicePlan plans[kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    int regs_one = 0, regs_walk = 0;
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        DevicePlan &pl = plans[dev];
+        if (lds_walk > 48 * 1024 && !pl.big_lds) {
+            for (const void *k : {reinterpret_cast<const void *>(kern_one), reinterpret_cast<const void *>(kern_grp),
+                                  reinterpret_cast<const void *>(kern_walk)}) {
+                hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (e != hipSuccess) return e;
+            }
+            pl.big_lds = true;
         }
-        big_lds_enabled = true;
+        if (kCanWalk && !pl.asked) {
+            pl.regs[0] = kernel_vgprs(reinterpret_cast<const void *>(kern_grp));
+            pl.regs[1] = kernel_vgprs(reinterpret_cast<const void *>(kern_walk));
+            pl.asked = true;
+        }
+        regs_one = pl.regs[0];
+        regs_walk = pl.regs[1];
     }
     // Workgroups that the chip holds at a time, of the kernel that takes one tile per workgroup and
     // of the one that walks (more registers): from the register counts (512 VGPRs per SIMD lane,
-    // allocated in eights, at most 8 wavefronts per SIMD, four SIMDs) and the LDS.  Asked once.
-    static int slots_one = 0, slots_walk = 0;
-    static size_t slots_lds = 0;
-    if (kCanWalk && lds_walk <= 160 * 1024 && (slots_lds != lds_walk || slots_one <= 0)) {
-        auto resident = [&](const void *k, size_t lds_bytes) {
-            hipFuncAttributes attr;
-            int per_cu = 20 / (c.W + c.S);
-            if (hipFuncGetAttributes(&attr, k) == hipSuccess && attr.numRegs > 0) {
-                int per_simd = 512 / ((attr.numRegs + 7) / 8 * 8);
-                if (per_simd > 8) per_simd = 8;
-                per_cu = 4 * per_simd / (c.W + c.S);
-            } else {
-                (void)hipGetLastError();
-            }
-            const int by_lds = (int)((160 * 1024) / lds_bytes);
-            if (per_cu > by_lds) per_cu = by_lds;
-            return kStreamCus * (per_cu < 1 ? 1 : per_cu);
-        };
-        slots_one = resident(reinterpret_cast<const void *>(kern_grp), stream_lds_bytes(geo, c.W, 1));
-        slots_walk = resident(reinterpret_cast<const void *>(kern_walk), lds_walk);
-        slots_lds = lds_walk;
+    // allocated in eights, at most 8 wavefronts per SIMD, four SIMDs) and the LDS.
+    auto resident = [&](int regs, size_t lds_bytes) {
+        int per_cu = 20 / (c.W + c.S);
+        if (regs > 0) {
+            int per_simd = 512 / ((regs + 7) / 8 * 8);
+            if (per_simd > 8) per_simd = 8;
+            per_cu = 4 * per_simd / (c.W + c.S);
+        }
+        const int by_lds = (int)((160 * 1024) / lds_bytes);
+        if (per_cu > by_lds) per_cu = by_lds;
+        return kStreamCus * (per_cu < 1 ? 1 : per_cu);
+    };
+    int slots_one = 0, slots_walk = 0;
+    if (kCanWalk && lds_walk <= 160 * 1024) {
+        slots_one = resident(regs_one, stream_lds_bytes(geo, c.W, 1));
+        slots_walk = resident(regs_walk, lds_walk);
     }
     // one round of one-tile workgroups if they all fit; else as few tiles per workgroup as fill the chip once
     int per_wg = 1;
@@ -1476,11 +1502,17 @@ static hipError_t launch_rows_cfg(const unsigned short *xs, const float *xsum, c
     auto kern = stream_rows_kernel<BITS, W, L, TEAMS, STAGE>;
     const size_t lds = rows_lds_bytes(B, geo, W * TEAMS, STAGE);
     if (lds > 160 * 1024 || ceil_div(geo.ng, W) > L) return hipErrorInvalidValue;
-    static bool big_lds_enabled = false;
-    if (lds > 48 * 1024 && !big_lds_enabled) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return e;
-        big_lds_enabled = true;
+    if (lds > 48 * 1024) {
+        static std::mutex mu;
+        static bool big_lds[kMaxDevices] = {};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+        std::lock_guard<std::mutex> lock(mu);
+        if (!big_lds[dev]) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return e;
+            big_lds[dev] = true;
+        }
     }
     // one workgroup per compute unit (its teams share the rows in LDS); fewer when there are fewer tiles
     int grid = ceil_div(geo.ntiles, TEAMS);

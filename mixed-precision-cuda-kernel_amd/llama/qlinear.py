@@ -117,6 +117,10 @@ class QuantLinear(nn.Module):
         else:
             self.bias = None
         self.dequantized = False
+        # the repacked weight stream of prepack() (not part of the state dict) and whether the
+        # checkpoint-layout buffers were released in its favour
+        self._stream = None
+        self._released = False
 
     # ---- packing (host logic) ---------------------------------------------------------------
     def _normal_columns(self, device):
@@ -128,6 +132,7 @@ class QuantLinear(nn.Module):
     def pack(self, linear: QuantLinearForTraining):
         """Fill the packed buffers from a fake-quant training module.  llama/qlinear.py:67-118.
         The buffers end up on the CPU, as in the reference."""
+        self._drop_stream()  # a stream made from the old buffers must not outlive them
         if linear.bias is not None:
             self.bias = linear.bias.detach().to(torch.float16).cpu().clone()
         weight = linear.weight
@@ -171,7 +176,37 @@ class QuantLinear(nn.Module):
         return weight
 
     # ---- load-time repack (no counterpart in the reference) -----------------------------------
-    @torch.inference_mode()
+    def _drop_stream(self):
+        self._stream = None
+        self._released = False
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        # new packed buffers: a stream repacked from the old ones is stale
+        self._drop_stream()
+        return super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
+
+    def _apply(self, fn, *args, **kwargs):
+        # .to() / .cuda() / .cpu(): the stream lives on one device and follows the buffers
+        stream = self._stream
+        out = super()._apply(fn, *args, **kwargs)
+        if stream is not None:
+            moved = fn(stream)
+            if moved.dtype != torch.uint8 or not moved.is_cuda:
+                if self._released:
+                    raise RuntimeError("prepack(release_reference=True) left only the weight stream, which exists on "
+                                       "its GPU only; call unprepack() before moving or casting the module")
+                self._stream = None
+            else:
+                self._stream = moved
+        return out
+
+    def state_dict(self, *args, **kwargs):
+        if self._released:
+            raise RuntimeError("prepack(release_reference=True) freed the checkpoint-layout buffers; call unprepack() "
+                               "before state_dict() / saving")
+        return super().state_dict(*args, **kwargs)
+
+    @torch.no_grad()
     def prepack(self, release_reference: bool = False):
         """Rearrange the packed buffers, once, into the weight stream the batch-1 kernel of this
         GPU reads fastest (quant_cuda.prepack_cherryq).  The state-dict buffers stay as they are
@@ -193,14 +228,14 @@ class QuantLinear(nn.Module):
             self._released = True
         return True
 
-    @torch.inference_mode()
+    @torch.no_grad()  # (not inference_mode: the rebuilt buffers must stay loadable with load_state_dict)
     def unprepack(self):
         """Drop the weight stream; if prepack() released the checkpoint-layout buffers, rebuild
         them from it first."""
-        stream = getattr(self, "_stream", None)
+        stream = self._stream
         if stream is None:
             return
-        if getattr(self, "_released", False):
+        if self._released:
             (self.cherry_indices, self.cherry_weight, self.qweight,
              self.scales) = quant_cuda.unprepack_cherryq(self.w_bits, stream, self.in_features, self.out_features,
                                                          self.num_cherries, self.group_size)
@@ -220,17 +255,26 @@ class QuantLinear(nn.Module):
             if x2.dtype != torch.float16:
                 x2 = x2.to(torch.float16)
             x2 = x2.contiguous()
-            stream = getattr(self, "_stream", None)
+            stream = self._stream
             rows = x2.shape[0]
+            rows_min = 2 if self._released else self.stream_rows_min
             # over the repacked stream: one row, and 4 to 16 rows (the matrix-core tile of the one-row
-            # kernel filled with real rows; 2 and 3 rows are faster on the checkpoint layout's kernel)
-            if stream is not None and (rows == 1 or (self.stream_rows_min <= rows <= 16 and quant_cuda.prepack_supported(
+            # kernel filled with real rows; 2 and 3 rows are faster on the checkpoint layout's kernel
+            # while that layout is still there)
+            if stream is not None and (rows == 1 or (rows_min <= rows <= 16 and quant_cuda.prepack_supported(
                     self.w_bits, rows, self.in_features, self.out_features, self.num_cherries, self.group_size))):
                 out = torch.empty(rows, self.out_features, dtype=torch.float16, device=stream.device)
                 quant_cuda.matvec_prepacked_cherryq(self.w_bits, x2, stream, out, self.in_features, self.num_cherries)
-            elif getattr(self, "_released", False):
-                raise RuntimeError("prepack(release_reference=True) left only the weight stream (1 and 4..16 rows); "
-                                   "call unprepack() before using other batch sizes")
+            elif self._released:
+                # only the stream is left: any other number of rows goes over it in pieces of up to 16
+                if rows and not quant_cuda.prepack_supported(self.w_bits, min(rows, 16), self.in_features, self.out_features,
+                                                             self.num_cherries, self.group_size):
+                    raise RuntimeError("prepack(release_reference=True) left only the weight stream, whose kernels do "
+                                       "not take this batch size for this layer; call unprepack() first")
+                out = torch.empty(rows, self.out_features, dtype=torch.float16, device=stream.device)
+                for r0 in range(0, rows, 16):
+                    quant_cuda.matvec_prepacked_cherryq(self.w_bits, x2[r0:r0 + 16], stream, out[r0:r0 + 16],
+                                                        self.in_features, self.num_cherries)
             elif x2.shape[0] >= self.prefill_rows:
                 # prompt-sized batches: one bit-exact dequantisation pass on the GPU into a transient
                 # dense weight, then a library fp16 GEMM -- the arithmetic of the dequantised branch

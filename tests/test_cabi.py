@@ -64,6 +64,22 @@ def test_workspace_sizes(lib):
     assert lib.cherryq_scratch_bytes_f32(16, 4096, 13824, 16) >= lib.cherryq_scratch_bytes(16, 4096, 13824, 16)
 
 
+def test_weight_stream_shapes_taken_and_refused(lib):
+    """cherryq_prepack_supported is host arithmetic: the shapes a loader may repack, and the bound
+    that keeps every byte offset inside a stream below 2 GiB (offsets are 32-bit, and one with bit 31
+    set is how the kernels read zeros)."""
+    lib.cherryq_prepack_bytes.restype = ctypes.c_size_t
+    f = lib.cherryq_prepack_supported
+    assert f(4, 1, 4096, 11008, 16, 128) == 1 and f(3, 1, 4096, 11008, 16, 128) == 1
+    assert f(4, 1, 4096, 11008, 16, 64) == 0 and f(4, 1, 4096, 11004, 16, 128) == 0
+    size = lambda n: lib.cherryq_prepack_bytes(4, 4096, n, 16)
+    record = size(32) - size(16)
+    n_ok = (0x7fff0000 - (size(16) - record)) // record * 16   # widest layer below the bound, or 16 columns more
+    assert size(n_ok - 16) < 0x7fff0000 <= size(n_ok + 16)
+    assert f(4, 1, 4096, n_ok - 16, 16, 128) == 1
+    assert f(4, 1, 4096, n_ok + 16, 16, 128) == 0
+
+
 def _call(fn, *, vec=0x1000, qw=0x1000, cw=0x1000, idx=0x1000, sc=0x1000, mul=0x1000, b=1, k=4096, n=4096,
           c=16, g=128, acc=1, ws=0x1000, wsb=1 << 30, scr=None, scrb=0, stream=None):
     fn.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 6 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
