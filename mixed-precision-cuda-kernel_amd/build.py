@@ -18,7 +18,7 @@ CSRC = HERE / "csrc"
 OBJ = HERE / "build"
 LIB = HERE / "libcherryq.so"
 PROBE_LIB = HERE / "libcherryq_probe.so"  # bench-only roofline reference kernels, not part of the product library
-SOURCES = ["cq_api.hip", "cq_generic.hip", "cq_matvec.hip", "cq_stream.hip", "cq_batch.hip", "cq_gemm.hip", "cq_f32.hip", "cq_decode.hip", "cq_pack.hip", "cq_fakequant.hip"]
+SOURCES = ["cq_api.hip", "cq_generic.hip", "cq_matvec.hip", "cq_stream.hip", "cq_stream_cu.hip", "cq_batch.hip", "cq_gemm.hip", "cq_f32.hip", "cq_decode.hip", "cq_pack.hip", "cq_fakequant.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
@@ -47,7 +47,10 @@ def build(force: bool = False, verbose: bool = False) -> Path:
     # activation pointer, the stream pointer, K and the header size lead stream_kernel's list) into
     # scalar registers, which takes their load off the start-up chain of every workgroup
     # (4096 -> 11008: 6.67 -> 6.40 us, 4096 -> 4096: 4.38 -> 4.21 us)
-    extra = {"cq_stream.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=6"]}
+    # cq_stream_cu.hip: likewise the first 14 dwords of stream_cu_kernel's list (pointers, shape and
+    # record geometry: everything a wavefront needs for its first requests)
+    extra = {"cq_stream.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=6"],
+             "cq_stream_cu.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=14"]}
 
     def compile_one(src):
         out = OBJ / (src + ".o")

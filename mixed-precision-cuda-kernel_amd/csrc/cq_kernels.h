@@ -133,6 +133,10 @@ size_t stream_rows_scratch_bytes(int bits, int B, int K, int N, int C);
 bool stream_rows_supported(int bits, int B, int K, int N, int C, int G);
 hipError_t launch_stream_rows(int bits, const __half *vec, const uint8_t *stream, __half *mul, int B, int K, int N,
                               int C, int accumulate, void *scratch, hipStream_t s);
+// cq_stream_cu.hip: the same launch with one workgroup per compute unit (up to 64 units per column)
+bool stream_cu_supported(int bits, int K, int C, const int *Ns, int count);
+hipError_t launch_stream_cu(int bits, const __half *vec, const __half *norm_w, float eps, const StreamMember *members,
+                            int count, int K, int C, int accumulate, hipStream_t s);
 size_t stream_bytes(int bits, int K, int N, int C);
 bool stream_faster(int bits, int K, int N, int C);
 bool stream_supported(int bits, int B, int K, int N, int C, int G);

@@ -31,30 +31,14 @@
 // Arithmetic contract: csrc/quant_cuda_kernel.cu:718-835 (4-bit) and 558-672 (3-bit) of the
 // reference; fp32 accumulation, one rounding to fp16.  Replaces the per-thread decode loops at
 // :811-831 / :649-667 and the serial batch loop :797-834.
+#include <stdlib.h>
+
 #include <mutex>
 #include <type_traits>
 
-#include "cq_device.h"
-#include "cq_kernels.h"
+#include "cq_stream_dev.h"
 
 namespace cq {
-
-typedef _Float16 sh8_t __attribute__((ext_vector_type(8)));
-typedef _Float16 sh4_t __attribute__((ext_vector_type(4)));
-typedef float sf4_t __attribute__((ext_vector_type(4)));
-typedef uint32_t su4 __attribute__((ext_vector_type(4)));
-typedef uint32_t su3 __attribute__((ext_vector_type(3)));
-typedef uint32_t su2 __attribute__((ext_vector_type(2)));
-typedef _Float16 sh2_t __attribute__((ext_vector_type(2)));
-
-constexpr uint32_t kSFlags = 0x00020000u;
-constexpr uint32_t kSOob = 0x80000000u;
-// 16-byte loads of raw activations per thread that cover the longest row a geometry takes
-// (max_units units of 128 positions plus up to 128 cherry channels) with NT threads
-__host__ __device__ constexpr int stream_x_loads(int max_units, int nt) {
-    return (max_units * 128 + 128 + nt * 8 - 1) / (nt * 8);
-}
-constexpr int kStreamRawPad = 512 + 128 + 8;  // zero halves kept behind the raw activations in LDS
 
 static inline uint32_t align256(uint32_t v) { return (v + 255u) & ~255u; }
 
@@ -231,53 +215,6 @@ __global__ __launch_bounds__(256) void stream_header_unpack_kernel(const uint8_t
     const int Knp512 = (geo.ng * kStreamUnitK + 511) & ~511;
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i < geo.C) cherry_indices[i] = (int16_t)reinterpret_cast<const uint16_t *>(hdr + Knp512)[i];
-}
-
-// ---- the matvec --------------------------------------------------------------------------------
-__device__ inline sh8_t as_h8(su4 v) { return __builtin_bit_cast(sh8_t, v); }
-__device__ inline sh4_t as_h4(su2 v) { return __builtin_bit_cast(sh4_t, v); }
-
-// One unit (128 positions x 16 columns) against the activations of the same positions: the
-// sum over the unit of x * code for the lane's column (row 0 of the MFMA tile, which every lane
-// group receives because every row of A holds the same activations).
-template <int BITS>
-__device__ inline float unit_dot(const su4 w, const unsigned short *xa) {
-    const sf4_t zero4 = {0.f, 0.f, 0.f, 0.f};
-    if constexpr (BITS == 4) {
-        const su4 y = {w[0] >> 8, w[1] >> 8, w[2] >> 8, w[3] >> 8};
-        const sh8_t a0 = *reinterpret_cast<const sh8_t *>(xa);
-        const sh8_t a1 = *reinterpret_cast<const sh8_t *>(xa + 8);
-        const sh8_t a2 = *reinterpret_cast<const sh8_t *>(xa + 16);
-        const sh8_t a3 = *reinterpret_cast<const sh8_t *>(xa + 24);
-        const su4 b0 = {w[0] & 0x000f000fu, y[0] & 0x000f000fu, w[1] & 0x000f000fu, y[1] & 0x000f000fu};
-        const su4 b1 = {w[2] & 0x000f000fu, y[2] & 0x000f000fu, w[3] & 0x000f000fu, y[3] & 0x000f000fu};
-        const su4 b2 = {w[0] & 0x00f000f0u, y[0] & 0x00f000f0u, w[1] & 0x00f000f0u, y[1] & 0x00f000f0u};
-        const su4 b3 = {w[2] & 0x00f000f0u, y[2] & 0x00f000f0u, w[3] & 0x00f000f0u, y[3] & 0x00f000f0u};
-        sf4_t dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, as_h8(b0), zero4, 0, 0, 0);
-        sf4_t dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, as_h8(b2), zero4, 0, 0, 0);
-        dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, as_h8(b1), dl, 0, 0, 0);
-        dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(a3, as_h8(b3), dh, 0, 0, 0);
-        return dl[0] * 16777216.0f + dh[0] * 1048576.0f;
-    } else {
-        const su3 y = {w[0] >> 9, w[1] >> 9, w[2] >> 9};
-        const sh8_t a0 = *reinterpret_cast<const sh8_t *>(xa);        // positions 0..7: fields at bit 0
-        const sh8_t a2 = *reinterpret_cast<const sh8_t *>(xa + 8);    // 8..15: bit 3
-        const sh8_t a4 = *reinterpret_cast<const sh8_t *>(xa + 16);   // 16..23: bit 6
-        const sh4_t a1 = *reinterpret_cast<const sh4_t *>(xa + 24);   // 24..27: bit 0
-        const sh4_t a3 = *reinterpret_cast<const sh4_t *>(xa + 28);   // 28..31: bit 3
-        const uint32_t z = (y[0] & 0x00400040u) | ((y[1] & 0x00400040u) << 1) | ((y[2] & 0x00400040u) << 2);
-        const su4 b0 = {w[0] & 0x00070007u, w[1] & 0x00070007u, w[2] & 0x00070007u, y[0] & 0x00070007u};
-        const su4 b2 = {w[0] & 0x00380038u, w[1] & 0x00380038u, w[2] & 0x00380038u, y[0] & 0x00380038u};
-        const su4 b4 = {w[0] & 0x01c001c0u, w[1] & 0x01c001c0u, w[2] & 0x01c001c0u, z};
-        const su2 b1 = {y[1] & 0x00070007u, y[2] & 0x00070007u};
-        const su2 b3 = {y[1] & 0x00380038u, y[2] & 0x00380038u};
-        sf4_t d0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, as_h8(b0), zero4, 0, 0, 0);
-        sf4_t d3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, as_h8(b2), zero4, 0, 0, 0);
-        const sf4_t d6 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a4, as_h8(b4), zero4, 0, 0, 0);
-        d0 = __builtin_amdgcn_mfma_f32_16x16x16f16(a1, as_h4(b1), d0, 0, 0, 0);
-        d3 = __builtin_amdgcn_mfma_f32_16x16x16f16(a3, as_h4(b3), d3, 0, 0, 0);
-        return d0[0] * 16777216.0f + d3[0] * 2097152.0f + d6[0] * 262144.0f;
-    }
 }
 
 // weight * fp16(x * rs) on both halves of a pair (the rounding points of add_rmsnorm_kernel)
@@ -1394,11 +1331,31 @@ static hipError_t launch_stream_bits(const __half *vec, const StreamGroup &grp, 
     }
 }
 
+// Which of the two launch shapes takes a call: the one with one workgroup per compute unit
+// (cq_stream_cu.hip) wherever it measured faster.
+static bool stream_cu_preferred(int bits, int K, int C, const int *Ns, int count, bool norm) {
+    // measurement switch, read once: CHERRYQ_STREAM_CU=0 never, =1 wherever the shape is supported
+    static const int forced = [] {
+        const char *e = getenv("CHERRYQ_STREAM_CU");
+        return e && e[0] == '0' ? 0 : e && e[0] == '1' ? 1 : -1;
+    }();
+    if (forced == 0) return false;
+    if (forced == 1) return stream_cu_supported(bits, K, C, Ns, count);
+    if (count != 1 || norm) return false;
+    return stream_cu_supported(bits, K, C, Ns, count);
+}
+
 // `count` layers (at most kStreamMaxGroup) of the same bits / K / C that read the same activation
 // row, in one launch; norm_w != nullptr fuses the RMSNorm of that row.
 hipError_t launch_stream_group(int bits, const __half *vec, const __half *norm_w, float eps,
                                const StreamMember *members, int count, int K, int C, int accumulate, hipStream_t s) {
     if (count < 1 || count > kStreamMaxGroup) return hipErrorInvalidValue;
+    {
+        int Ns[kStreamMaxGroup];
+        for (int i = 0; i < count; i++) Ns[i] = members[i].N;
+        if (stream_cu_preferred(bits, K, C, Ns, count, norm_w != nullptr))
+            return launch_stream_cu(bits, vec, norm_w, eps, members, count, K, C, accumulate, s);
+    }
     StreamGroup grp = {};
     grp.count = count;
     int tiles = 0, n_total = 0;
