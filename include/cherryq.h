@@ -223,15 +223,17 @@ int cherryq_vecquant_matmul_f16_static(int w_bits, const void *vec, const uint8_
  * stream: cherryq_prepack_bytes() bytes, 256-byte aligned, written by cherryq_prepack_f16 once
  * per layer.  group_size must be a multiple of 128 (the stream stores one scale row per 128
  * positions); cherryq_prepack_supported() says whether a shape is taken at all (at most 128
- * cherry channels, at most 16384 + 128 input channels, a stream of less than 2 GiB, batch 1).  vec
+ * cherry channels, at most 28672 + 128 input channels, a stream of less than 2 GiB, batch 1).  vec
  * must be 16-byte aligned.
  */
 size_t cherryq_prepack_bytes(int w_bits, int in_features, int out_features, int num_cherries);
 int cherryq_prepack_supported(int w_bits, int batch, int in_features, int out_features, int num_cherries,
                               int group_size);
 /* 1 where the matvec over the stream measured faster on MI355X than the one over the checkpoint
- * layout (today: layers of at most 4096 non-cherry input channels), 0 elsewhere or if unsupported:
- * what a loader asks before spending the extra copy of the weights. */
+ * layout (today: layers of at most 4096 non-cherry input channels, and deeper ones whose 16-column
+ * tiles spread evenly over the 256 compute units -- every LLaMA-7B and -70B projection, not the
+ * 13B ones), 0 elsewhere or if unsupported: what a loader asks before spending the extra copy of
+ * the weights. */
 int cherryq_prepack_recommended(int w_bits, int in_features, int out_features, int num_cherries, int group_size);
 int cherryq_prepack_f16(int w_bits, const uint8_t *qweight, const void *cherry_weight, const int16_t *cherry_indices,
                         const void *scales, void *stream, size_t stream_bytes, int in_features, int out_features,
@@ -278,6 +280,33 @@ typedef struct cherryq_stream_layer {
 int cherryq_decode_matvec_group_prepacked_f16(int w_bits, const void *vec, const void *norm_weight /* may be NULL */,
                                               float eps, const cherryq_stream_layer *layers, int n_layers,
                                               int in_features, int num_cherries, int accumulate, void *hip_stream);
+
+/*
+ * gate_proj and up_proj of a gated MLP (two repacked layers of the same shape that read the same
+ * row) in ONE launch that stores the activation the down projection reads,
+ * act = fp16(fp16(silu(g)) * u) with g = fp16(vec' Wg^T), u = fp16(vec' Wu^T) and vec' = vec or
+ * its RMSNorm (norm_weight given) -- llama/modeling_llama_quant.py:251 with the rounding points of
+ * its fp16 tensors -- instead of the two results: pairs of wavefront teams work on the same 16
+ * columns of both layers and meet in LDS.  No workspace; act (1, out_features) fp16 is overwritten.
+ * cherryq_decode_gate_up_prepacked_supported() says whether a shape is taken (up to 8192 + 128
+ * input channels).  No counterpart in the reference, whose three projections are separate calls.
+ */
+int cherryq_decode_gate_up_prepacked_supported(int w_bits, int in_features, int out_features, int num_cherries);
+int cherryq_decode_gate_up_prepacked_f16(int w_bits, const void *vec, const void *norm_weight /* may be NULL */, float eps,
+                                         const void *gate_stream, size_t gate_stream_bytes, const void *up_stream,
+                                         size_t up_stream_bytes, void *act, int in_features, int out_features,
+                                         int num_cherries, void *hip_stream);
+
+/*
+ * The down projection of a gated MLP over a repacked layer: mul (+)= act W^T with
+ * act = fp16(fp16(silu(vec_gate)) * vec), the activation llama/modeling_llama_quant.py:251 forms
+ * between the gate / up and the down projection, computed while the row is staged (the
+ * counterpart of cherryq_decode_matvec_group_f16's vec_gate for layers held as weight streams).
+ * One launch, no workspace.  vec and vec_gate: (1, in_features) fp16, 16-byte aligned.
+ */
+int cherryq_decode_matvec_gated_prepacked_f16(int w_bits, const void *vec, const void *vec_gate, const void *stream,
+                                              size_t stream_bytes, void *mul, int in_features, int out_features,
+                                              int num_cherries, int accumulate, void *hip_stream);
 
 /*
  * One batch-1 launch over 1..4 packed layers that read the SAME activation vector and share

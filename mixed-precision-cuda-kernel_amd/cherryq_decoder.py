@@ -133,6 +133,65 @@ def matvec_group_prepacked(mods, vec, outs, accumulate=False, norm_weight=None, 
         "matvec_group_prepacked")
 
 
+_lib.cherryq_decode_matvec_gated_prepacked_f16.argtypes = [_int, _vp, _vp, _vp, ctypes.c_size_t, _vp, _int, _int, _int, _int, _vp]
+_lib.cherryq_decode_matvec_gated_prepacked_f16.restype = _int
+
+
+_lib.cherryq_decode_gate_up_prepacked_f16.argtypes = [_int, _vp, _vp, _f, _vp, ctypes.c_size_t, _vp, ctypes.c_size_t, _vp,
+                                                      _int, _int, _int, _vp]
+_lib.cherryq_decode_gate_up_prepacked_f16.restype = _int
+_lib.cherryq_decode_gate_up_prepacked_supported.argtypes = [_int] * 4
+_lib.cherryq_decode_gate_up_prepacked_supported.restype = _int
+
+
+def gate_up_prepacked_supported(gate_mod, up_mod) -> bool:
+    """Whether gate_up_prepacked takes this pair of layers (both repacked, same shape and cherry count)."""
+    g, u = gate_mod, up_mod
+    if getattr(g, "_stream", None) is None or getattr(u, "_stream", None) is None:
+        return False
+    if (g.w_bits, g.in_features, g.out_features, g.num_cherries) != (u.w_bits, u.in_features, u.out_features, u.num_cherries):
+        return False
+    return bool(_lib.cherryq_decode_gate_up_prepacked_supported(g.w_bits, g.in_features, g.out_features, g.num_cherries))
+
+
+def gate_up_prepacked(gate_mod, up_mod, vec, act, norm_weight=None, eps=1e-6):
+    """act = fp16(fp16(silu(vec' Wg^T)) * (vec' Wu^T)) in ONE launch over the two repacked layers, vec' =
+    vec or norm_weight * fp16(vec * rsqrt(mean(vec^2) + eps)): what the down projection reads."""
+    if not gate_up_prepacked_supported(gate_mod, up_mod):
+        raise RuntimeError("gate_up_prepacked: two prepack()ed layers of the same supported shape are needed")
+    g, u = gate_mod, up_mod
+    k, n = g.in_features, g.out_features
+    dev = g._stream.device
+    for t, shape in ((vec, (1, k)), (act, (1, n))):
+        if tuple(t.shape) != shape or t.dtype != torch.float16 or not t.is_cuda or not t.is_contiguous() or t.device != dev:
+            raise RuntimeError("gate_up_prepacked: vec (1, in_features) and act (1, out_features) must be contiguous fp16 "
+                               "tensors on the layers' GPU")
+    if norm_weight is not None and (tuple(norm_weight.shape) != (k,) or norm_weight.dtype != torch.float16
+                                    or not norm_weight.is_cuda or not norm_weight.is_contiguous()):
+        raise RuntimeError("gate_up_prepacked: norm_weight must be a contiguous (in_features,) fp16 GPU tensor")
+    _ok(_lib.cherryq_decode_gate_up_prepacked_f16(g.w_bits, vec.data_ptr(), None if norm_weight is None else norm_weight.data_ptr(),
+                                                  eps, g._stream.data_ptr(), g._stream.numel(), u._stream.data_ptr(),
+                                                  u._stream.numel(), act.data_ptr(), k, n, g.num_cherries, _stream()),
+        "gate_up_prepacked")
+
+
+def matvec_gated_prepacked(mod, vec, vec_gate, out, accumulate=False):
+    """out (+)= fp16(fp16(silu(vec_gate)) * vec) @ W^T for a QuantLinear that holds a repacked weight
+    stream: the down projection of the gated MLP in one launch, the activation formed while the
+    row is staged."""
+    st = getattr(mod, "_stream", None)
+    if st is None:
+        raise RuntimeError("matvec_gated_prepacked: the layer must have been prepack()ed")
+    k = mod.in_features
+    for t, shape in ((vec, (1, k)), (vec_gate, (1, k)), (out, (1, mod.out_features))):
+        if tuple(t.shape) != shape or t.dtype != torch.float16 or not t.is_cuda or not t.is_contiguous() or t.device != st.device:
+            raise RuntimeError("matvec_gated_prepacked: vec / vec_gate (1, in_features) and out (1, out_features) must be "
+                               "contiguous fp16 tensors on the layer's GPU")
+    _ok(_lib.cherryq_decode_matvec_gated_prepacked_f16(mod.w_bits, vec.data_ptr(), vec_gate.data_ptr(), st.data_ptr(),
+                                                       st.numel(), out.data_ptr(), k, mod.out_features, mod.num_cherries,
+                                                       1 if accumulate else 0, _stream()), "matvec_gated_prepacked")
+
+
 def _group(mods, vec, outs, accumulate=False, norm_weight=None, eps=1e-6):
     """The grouped launch over whichever layout the layers hold: the repacked streams when every
     layer of the group has one, the checkpoint layout otherwise."""
@@ -241,6 +300,7 @@ class CherryLlamaDecoder(nn.Module):
         self._graph = None
         self.fuse_norm = True
         self.fuse_head = True  # final RMSNorm + fp16 head as one launch of the library's own kernel
+        self.fuse_act = True   # gate / up as one launch that stores SiLU(gate) * up (layers repacked), plain down projection
         self.layer_trace = None
         self._side = [torch.cuda.Stream(device=self.device_) for _ in range(2)] if self.device_.type == "cuda" else []
 
@@ -356,13 +416,27 @@ class CherryLlamaDecoder(nn.Module):
                                                        self.attn.data_ptr(), self.pos.data_ptr(), nh, nkv, hd, ml,
                                                        cfg.rope_theta, _stream()), "rope_attention")
             _group([layer.o_proj], self.attn, [self.hid], accumulate=True)
-            if self.fuse_norm:
-                _group(gu, self.hid, [self.gate, self.up], norm_weight=layer.post_attention_layernorm,
-                       eps=cfg.rms_norm_eps)
+            down = layer.down_proj
+            if self.fuse_act and getattr(down, "_stream", None) is not None and gate_up_prepacked_supported(*gu):
+                # gate / up in one launch that stores SiLU(gate) * up, then the plain down projection
+                if self.fuse_norm:
+                    gate_up_prepacked(gu[0], gu[1], self.hid, self.act, norm_weight=layer.post_attention_layernorm,
+                                      eps=cfg.rms_norm_eps)
+                else:
+                    self._norm(layer.post_attention_layernorm)
+                    gate_up_prepacked(gu[0], gu[1], self.normed, self.act)
+                matvec_group_prepacked([down], self.act, [self.hid], accumulate=True)
             else:
-                self._norm(layer.post_attention_layernorm)
-                _group(gu, self.normed, [self.gate, self.up])
-            matvec_group([layer.down_proj], self.up, [self.hid], vec_gate=self.gate, accumulate=True)
+                if self.fuse_norm:
+                    _group(gu, self.hid, [self.gate, self.up], norm_weight=layer.post_attention_layernorm,
+                           eps=cfg.rms_norm_eps)
+                else:
+                    self._norm(layer.post_attention_layernorm)
+                    _group(gu, self.normed, [self.gate, self.up])
+                # the down projection forms SiLU(gate) * up while it stages its row: split-K workgroups of the
+                # checkpoint layout each do so for their own slice only (over a weight stream every workgroup
+                # would repeat it for the whole row: measured 9.9 us against 8.0)
+                matvec_group([down], self.up, [self.hid], vec_gate=self.gate, accumulate=True)
             if self.layer_trace is not None:  # validation only (eager runs): the hidden state after every layer
                 self.layer_trace.append(self.hid.clone())
         if self.fuse_head and _lib.cherryq_decode_head_supported(cfg.vocab_size, cfg.hidden_size):

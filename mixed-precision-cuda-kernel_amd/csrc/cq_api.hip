@@ -520,6 +520,44 @@ int cherryq_decode_matvec_group_prepacked_f16(int w_bits, const void *vec, const
                                         in_features, num_cherries, accumulate, reinterpret_cast<hipStream_t>(hip_stream));
 }
 
+int cherryq_decode_gate_up_prepacked_f16(int w_bits, const void *vec, const void *norm_weight, float eps,
+                                         const void *gate_stream, size_t gate_stream_bytes, const void *up_stream,
+                                         size_t up_stream_bytes, void *act, int in_features, int out_features,
+                                         int num_cherries, void *hip_stream) {
+    int rc = prepack_check(w_bits, in_features, out_features, num_cherries, cq::kStreamUnitK, gate_stream_bytes);
+    if (rc) return rc;
+    rc = prepack_check(w_bits, in_features, out_features, num_cherries, cq::kStreamUnitK, up_stream_bytes);
+    if (rc) return rc;
+    if (!vec || !gate_stream || !up_stream || !act) return CHERRYQ_E_NULL;
+    if (!cq::aligned(gate_stream, 256) || !cq::aligned(up_stream, 256) || !cq::aligned(vec, 16) ||
+        (norm_weight && !cq::aligned(norm_weight, 16)) || !cq::aligned(act, 2))
+        return CHERRYQ_E_ALIGN;
+    if (!cq::stream_pair_supported(w_bits, in_features, out_features, num_cherries)) return CHERRYQ_E_UNSUPPORTED;
+    return (int)cq::launch_stream_pair(w_bits, reinterpret_cast<const __half *>(vec), reinterpret_cast<const __half *>(norm_weight),
+                                       eps, reinterpret_cast<const uint8_t *>(gate_stream),
+                                       reinterpret_cast<const uint8_t *>(up_stream), reinterpret_cast<__half *>(act),
+                                       in_features, out_features, num_cherries, reinterpret_cast<hipStream_t>(hip_stream));
+}
+
+int cherryq_decode_gate_up_prepacked_supported(int w_bits, int in_features, int out_features, int num_cherries) {
+    if (!cq::stream_supported(w_bits, 1, in_features, out_features, num_cherries, cq::kStreamUnitK)) return 0;
+    return cq::stream_pair_supported(w_bits, in_features, out_features, num_cherries) ? 1 : 0;
+}
+
+int cherryq_decode_matvec_gated_prepacked_f16(int w_bits, const void *vec, const void *vec_gate, const void *stream,
+                                              size_t stream_bytes, void *mul, int in_features, int out_features,
+                                              int num_cherries, int accumulate, void *hip_stream) {
+    int rc = prepack_check(w_bits, in_features, out_features, num_cherries, cq::kStreamUnitK, stream_bytes);
+    if (rc) return rc;
+    if (!vec || !vec_gate || !stream || !mul) return CHERRYQ_E_NULL;
+    if (!cq::aligned(stream, 256) || !cq::aligned(vec, 16) || !cq::aligned(vec_gate, 16) || !cq::aligned(mul, 2))
+        return CHERRYQ_E_ALIGN;
+    if (!cq::stream_gated_supported(w_bits, in_features, out_features, num_cherries)) return CHERRYQ_E_UNSUPPORTED;
+    return (int)cq::launch_stream_gated(w_bits, reinterpret_cast<const __half *>(vec), reinterpret_cast<const __half *>(vec_gate),
+                                        reinterpret_cast<const uint8_t *>(stream), reinterpret_cast<__half *>(mul), in_features,
+                                        out_features, num_cherries, accumulate, reinterpret_cast<hipStream_t>(hip_stream));
+}
+
 // ---- decode-step entry points (see include/cherryq.h) ------------------------------------------
 
 size_t cherryq_group_workspace_bytes(int n_layers, const int *out_features) {

@@ -135,8 +135,16 @@ hipError_t launch_stream_rows(int bits, const __half *vec, const uint8_t *stream
                               int C, int accumulate, void *scratch, hipStream_t s);
 // cq_stream_cu.hip: the same launch with one workgroup per compute unit (up to 64 units per column)
 bool stream_cu_supported(int bits, int K, int C, const int *Ns, int count);
-hipError_t launch_stream_cu(int bits, const __half *vec, const __half *norm_w, float eps, const StreamMember *members,
-                            int count, int K, int C, int accumulate, hipStream_t s);
+hipError_t launch_stream_cu(int bits, const __half *vec, const __half *norm_w, float eps, const __half *gate,
+                            const StreamMember *members, int count, int K, int C, int accumulate, hipStream_t s);
+// gate_proj and up_proj (same shape, same row) in one launch that stores fp16(fp16(silu(gate)) * up)
+bool stream_pair_supported(int bits, int K, int N, int C);
+hipError_t launch_stream_pair(int bits, const __half *vec, const __half *norm_w, float eps, const uint8_t *stream_gate,
+                              const uint8_t *stream_up, __half *act, int K, int N, int C, hipStream_t s);
+// one repacked layer behind the gated-MLP activation fp16(fp16(silu(gate)) * vec) (the down projection)
+bool stream_gated_supported(int bits, int K, int N, int C);
+hipError_t launch_stream_gated(int bits, const __half *vec, const __half *gate, const uint8_t *stream, __half *mul,
+                               int K, int N, int C, int accumulate, hipStream_t s);
 size_t stream_bytes(int bits, int K, int N, int C);
 bool stream_faster(int bits, int K, int N, int C);
 bool stream_supported(int bits, int B, int K, int N, int C, int G);

@@ -1190,14 +1190,33 @@ static int stream_pick(const StreamGeo &geo) {
     return -1;
 }
 
+constexpr int kStreamCus = 256;  // compute units of an MI355X
+
+// How unevenly a launch with one workgroup per compute unit spreads `tiles` whole tiles over the
+// chip: tiles of the busiest compute unit over the average (1 = even).
+static double cu_imbalance(int tiles) {
+    const int cus = tiles < kStreamCus ? tiles : kStreamCus;
+    return tiles > 0 ? (double)ceil_div(tiles, cus) * cus / tiles : 1.0;
+}
+
 // Where the batch-1 matvec over the stream measured faster than the one over the checkpoint layout
-// (us per launch, 4-bit, weights from HBM): 4096 -> 4096 4.2 against 4.95, 4096 -> 11008 6.5
-// against 7.3-7.5, 8192 -> 28672 (workgroups walking 7 tiles each) 21.2 against 22.8; no faster on the
-// other shapes beyond 32 units: 5120 -> 13824 (3-bit) 9.6-10.4 against 9.1, 11008 -> 4096 7.5 against
-// 7.0, 8192 -> 8192 8.6-9.5 against 8.75, 13824 -> 5120 (3-bit) 12.2 against 8.9.
+// (us per launch, weights from HBM; checkpoint layout / stream, the stream on whichever of its two
+// launch shapes is faster): 4096 -> 4096 4.95 / 3.58 (3-bit 4.79 / 3.55), 4096 -> 11008 7.46 / 5.71
+// (6.79 / 5.15), 11008 -> 4096 7.04 / 5.91 (6.76 / 5.56), 8192 -> 8192 8.75 / 7.72, 8192 -> 1024
+// 4.55 / 4.24, 8192 -> 28672 22.8 / 20.5, 28672 -> 8192 23.5 / 22.3.  Not faster where whole tiles
+// spread unevenly over the 256 compute units and a column is too deep for several small workgroups
+// per compute unit: 5120 -> 5120 (3-bit, 320 tiles) 5.68 / 5.95, 5120 -> 13824 (864 tiles) 9.05 /
+// 10.1, 13824 -> 5120 (320 tiles) 8.93 / 10.3.
 bool stream_faster(int bits, int K, int N, int C) {
     const StreamGeo g = stream_geo(bits, K, N, C);
-    return g.ng <= 32 || (g.ng <= 64 && g.ntiles >= 1536);
+    if (g.ng <= 32) return true;
+    return cu_imbalance(g.ntiles) <= 1.15;
+}
+
+// the launch shapes of this file (several workgroups per compute unit) take the layer
+static bool stream_old_supported(const StreamGeo &geo) {
+    const int i = stream_pick(geo);
+    return i >= 0 && stream_lds_bytes(geo, kStreamCfgs[i].W) <= 160 * 1024;
 }
 
 bool stream_supported(int bits, int B, int K, int N, int C, int G) {
@@ -1210,12 +1229,9 @@ bool stream_supported(int bits, int B, int K, int N, int C, int G) {
     // tile records are addressed with 32-bit byte offsets, and an offset with bit 31 set is how the
     // kernels read zeros for units that do not exist: the whole stream stays below 2 GiB
     if ((unsigned long long)geo.hdr_bytes + (unsigned long long)geo.ntiles * geo.record_bytes >= 0x7fff0000ull) return false;
-    const int i = stream_pick(geo);
-    if (i < 0) return false;
-    return stream_lds_bytes(geo, kStreamCfgs[i].W) <= 160 * 1024;
+    return stream_old_supported(geo) || stream_cu_supported(bits, K, C, &N, 1);
 }
 
-constexpr int kStreamCus = 256;  // compute units of an MI355X
 constexpr int kMaxDevices = 64;  // GPUs of one process that the per-device launch plans cover
 
 struct DevicePlan {
@@ -1334,28 +1350,57 @@ static hipError_t launch_stream_bits(const __half *vec, const StreamGroup &grp, 
 // Which of the two launch shapes takes a call: the one with one workgroup per compute unit
 // (cq_stream_cu.hip) wherever it measured faster.
 static bool stream_cu_preferred(int bits, int K, int C, const int *Ns, int count, bool norm) {
-    // measurement switch, read once: CHERRYQ_STREAM_CU=0 never, =1 wherever the shape is supported
+    if (!stream_cu_supported(bits, K, C, Ns, count)) return false;
+    int tiles = 0;
+    for (int i = 0; i < count; i++) tiles += ceil_div(Ns[i], kStreamTileCols);
+    StreamGeo geo = stream_geo(bits, K, Ns[0], C);
+    geo.ntiles = tiles;
+    if (!stream_old_supported(geo)) return true;
+    // measurement switch, read once: CHERRYQ_STREAM_CU=0 the older shape wherever it can, =1 the newer
     static const int forced = [] {
         const char *e = getenv("CHERRYQ_STREAM_CU");
         return e && e[0] == '0' ? 0 : e && e[0] == '1' ? 1 : -1;
     }();
-    if (forced == 0) return false;
-    if (forced == 1) return stream_cu_supported(bits, K, C, Ns, count);
-    if (count != 1 || norm) return false;
-    return stream_cu_supported(bits, K, C, Ns, count);
+    if (forced >= 0) return forced == 1;
+    // Measured (us, older shape / one workgroup per compute unit; 4-bit unless noted): single layers
+    // as listed at stream_faster(); RMSNorm + q/k/v (3 x 4096 -> 4096) 7.35 / 7.24 (3-bit 7.10 / 6.76),
+    // RMSNorm + gate/up (2 x 4096 -> 11008) 10.95 / 9.76 (3-bit 9.69 / 8.96), q/k/v without norm 7.02 /
+    // 7.08, RMSNorm + 8192 -> (8192, 1024, 1024) 11.5 / 10.6, RMSNorm + 2 x (8192 -> 28672) 40.2 / 38.9;
+    // between 33 and 64 units per column only where whole tiles spread evenly over the compute
+    // units (5120 -> 5120, 3-bit: 5.95 / 6.52; 5120 -> 13824: 10.1 / 10.6).
+    (void)norm;
+    if (geo.ng > 32 && geo.ng <= 64) return cu_imbalance(tiles) <= 1.15;
+    return true;
 }
+
 
 // `count` layers (at most kStreamMaxGroup) of the same bits / K / C that read the same activation
 // row, in one launch; norm_w != nullptr fuses the RMSNorm of that row.
+hipError_t launch_stream_group_old(int bits, const __half *vec, const __half *norm_w, float eps,
+                                   const StreamMember *members, int count, int K, int C, int accumulate, hipStream_t s);
+
 hipError_t launch_stream_group(int bits, const __half *vec, const __half *norm_w, float eps,
                                const StreamMember *members, int count, int K, int C, int accumulate, hipStream_t s) {
     if (count < 1 || count > kStreamMaxGroup) return hipErrorInvalidValue;
-    {
-        int Ns[kStreamMaxGroup];
-        for (int i = 0; i < count; i++) Ns[i] = members[i].N;
-        if (stream_cu_preferred(bits, K, C, Ns, count, norm_w != nullptr))
-            return launch_stream_cu(bits, vec, norm_w, eps, members, count, K, C, accumulate, s);
-    }
+    int Ns[kStreamMaxGroup];
+    for (int i = 0; i < count; i++) Ns[i] = members[i].N;
+    if (stream_cu_preferred(bits, K, C, Ns, count, norm_w != nullptr))
+        return launch_stream_cu(bits, vec, norm_w, eps, nullptr, members, count, K, C, accumulate, s);
+    return launch_stream_group_old(bits, vec, norm_w, eps, members, count, K, C, accumulate, s);
+}
+
+bool stream_gated_supported(int bits, int K, int N, int C) { return stream_cu_supported(bits, K, C, &N, 1); }
+
+hipError_t launch_stream_gated(int bits, const __half *vec, const __half *gate, const uint8_t *stream, __half *mul,
+                               int K, int N, int C, int accumulate, hipStream_t s) {
+    const StreamMember m = {stream, mul, N};
+    return launch_stream_cu(bits, vec, nullptr, 0.f, gate, &m, 1, K, C, accumulate, s);
+}
+
+// the launch with one workgroup per tile (or per few tiles), several workgroups per compute unit
+hipError_t launch_stream_group_old(int bits, const __half *vec, const __half *norm_w, float eps,
+                                   const StreamMember *members, int count, int K, int C, int accumulate, hipStream_t s) {
+    if (count < 1 || count > kStreamMaxGroup) return hipErrorInvalidValue;
     StreamGroup grp = {};
     grp.count = count;
     int tiles = 0, n_total = 0;
@@ -1398,8 +1443,7 @@ bool stream_group_supported(int bits, int K, int C, int G, const int *Ns, int co
     }
     StreamGeo geo = stream_geo(bits, K, Ns[0], C);
     geo.ntiles = tiles;
-    const int i = stream_pick(geo);
-    return i >= 0 && stream_lds_bytes(geo, kStreamCfgs[i].W) <= 160 * 1024;
+    return stream_old_supported(geo) || stream_cu_supported(bits, K, C, Ns, count);
 }
 
 // ---- 2 to 16 rows: sizes, support, launch

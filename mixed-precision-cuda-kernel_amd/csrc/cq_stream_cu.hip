@@ -40,6 +40,21 @@ constexpr int kCuMaxWalk = 16;   // tiles one team takes at most
 constexpr int kCuCus = 256;      // compute units of an MI355X
 constexpr int kCuMaxDevices = 64;
 
+constexpr int kCuPlain = 0, kCuNorm = 1, kCuGate = 2;
+
+// fp16(silu(gate)) * up, rounded to fp16, on both halves of a pair (the rounding points of silu_mul_kernel)
+__device__ inline uint32_t cu_silu_mul_pair(uint32_t gate, uint32_t up) {
+    uint32_t r = 0;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const float g = __half2float(__ushort_as_half((unsigned short)(gate >> (16 * i))));
+        const float u = __half2float(__ushort_as_half((unsigned short)(up >> (16 * i))));
+        const float a = __half2float(__float2half_rn(g / (1.f + __expf(-g))));
+        r |= (uint32_t)__half_as_ushort(__float2half_rn(a * u)) << (16 * i);
+    }
+    return r;
+}
+
 // weight * fp16(x * rs) on both halves of a pair (the rounding points of add_rmsnorm_kernel)
 __device__ inline uint32_t cu_norm_pair(uint32_t xp, uint32_t wp, float rs) {
     uint32_t r = 0;
@@ -53,73 +68,74 @@ __device__ inline uint32_t cu_norm_pair(uint32_t xp, uint32_t wp, float rs) {
     return r;
 }
 
-struct CuGroup {  // members 1 and 2 of a group launch (member 0 travels in the leading arguments)
-    const uint8_t *stream[2];
-    __half *mul[2];
-    int N[2];
-    int wg_begin[2];  // first workgroup of members 1 and 2
-    int wgs[2];       // workgroups of members 1 and 2
-    int count;
+// What a workgroup works on, gathered from the kernel arguments by the two kernel shells below.
+struct CuJob {
+    const __half *x;
+    const uint8_t *stream;  // the layer's stream (header, then tile records)
+    __half *mul;
+    const __half *norm_w;
+    float eps;
+    int K, C, N;
+    int G, bid;             // workgroups that share the layer, this one's index among them
+    int accumulate, P;      // P: tiles the launch's busiest team walks
+    const uint8_t *stream2; // PAIR: the second layer's stream
 };
 
 // S staging wavefronts (wavefronts 0 .. S-1, NB blocks of 512 compacted positions each), then
 // TEAMS teams of W computing wavefronts; computing wavefront c of a team takes the units c, c + W,
-// ... (L at most) of every tile the team comes to.  The leading arguments (14 dwords) are what the
-// first loads of a workgroup need; the file is built with a kernel-argument preload count that
-// puts them into scalar registers before the wavefronts start.
-template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, bool NORM, bool GROUP>
-__global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_kernel(
-    const __half *__restrict__ x, const uint8_t *__restrict__ stream0, __half *__restrict__ mul0, int K, int C, int ng,
-    int N0, uint32_t hdr_bytes, uint32_t off_cherry, uint32_t off_units, uint32_t record_bytes, int wgs0, int accumulate,
-    const __half *__restrict__ norm_w, float eps, CuGroup grp) {
+// ... (L at most) of every tile the team comes to.  WALK: some team has more than one tile.
+// PRO: what the staging wavefronts do to the row on its way into LDS -- kCuPlain nothing,
+// kCuNorm the RMSNorm norm_w * fp16(x * rsqrt(mean(x^2) + eps)), kCuGate the gated-MLP activation
+// fp16(fp16(silu(gate)) * x) with the gate vector passed in the norm_w slot.
+// PAIR: the teams work in pairs on the same tile index of TWO layers of the same shape that read the
+// same row (gate_proj / up_proj): even teams on job.stream, odd teams on job.stream2, each layer's
+// compaction staged by half of the staging wavefronts (the layers keep different cherry channels);
+// the epilogue stores fp16(fp16(silu(gate)) * up) of the two rounded results instead of the results.
+template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, int PRO, bool WALK, bool PAIR = false>
+__device__ __forceinline__ void stream_cu_body(const CuJob &job) {
     constexpr int NC = W * TEAMS;  // computing wavefronts
     constexpr int NT = 64 * (NC + S);
     constexpr int UB = BITS == 4 ? 1024 : 768;
     constexpr float kGrid = BITS == 4 ? -7.5f : -3.5f;
     constexpr int XS = NB + 1;  // 16-byte loads per lane that cover a staging wavefront's raw slice
     static_assert(D0 <= D && D <= L && L % D == 0 && L % 4 == 0, "ring slots are fixed per unit across tiles");
+    static_assert(!PAIR || (TEAMS % 2 == 0 && S % 2 == 0 && PRO != kCuGate), "pairs of teams, half of the staging wavefronts per layer");
+    constexpr int MEM = PAIR ? 2 : 1;      // layers a workgroup stages the row for
+    constexpr int SM = S / MEM;            // staging wavefronts per layer
+    constexpr int TSLOTS = TEAMS / MEM;    // tiles a workgroup works on at a time
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kq = lane >> 4, nn = lane & 15;
-
-    // which layer this workgroup works for (members are consecutive ranges of workgroups); the
-    // candidates are pinned in scalar registers first so that the selects stay selects
-    const uint8_t *__restrict__ stream = stream0;
-    __half *__restrict__ mul = mul0;
-    int N = N0, bid = blockIdx.x, G = wgs0;
-    if constexpr (GROUP) {
-        const uint8_t *s1 = grp.stream[0], *s2 = grp.stream[1];
-        __half *o1 = grp.mul[0], *o2 = grp.mul[1];
-        int n1 = grp.N[0], n2 = grp.N[1], b1 = grp.wg_begin[0], b2 = grp.wg_begin[1], g1 = grp.wgs[0], g2 = grp.wgs[1],
-            cnt = grp.count;
-        asm volatile("" : "+s"(stream), "+s"(s1), "+s"(s2), "+s"(mul), "+s"(o1), "+s"(o2));
-        asm volatile("" : "+s"(N), "+s"(n1), "+s"(n2), "+s"(b1), "+s"(b2), "+s"(g1), "+s"(g2), "+s"(cnt));
-        const bool m1 = cnt > 1 && bid >= b1, m2 = cnt > 2 && bid >= b2;
-        stream = m2 ? s2 : m1 ? s1 : stream;
-        mul = m2 ? o2 : m1 ? o1 : mul;
-        N = m2 ? n2 : m1 ? n1 : N;
-        G = m2 ? g2 : m1 ? g1 : G;
-        bid -= m2 ? b2 : m1 ? b1 : 0;
-    }
-    const int ntiles = (N + kStreamTileCols - 1) / kStreamTileCols;
+    const int K = job.K, C = job.C, N = job.N, G = job.G, bid = job.bid;
+    // the record geometry of stream_geo(), from the shape (scalar arithmetic: cheaper than
+    // kernel arguments that would not fit the preloaded ones)
+    const int ng = (K - C + kStreamUnitK - 1) / kStreamUnitK;
     const int Knp512 = (ng * kStreamUnitK + 511) & ~511;
     const int nblk = Knp512 >> 9;
+    const uint32_t off_cherry = ((uint32_t)ng * 32u + 255u) & ~255u;
+    const uint32_t off_units = off_cherry + (((uint32_t)C * 32u + 255u) & ~255u);
+    const uint32_t record_bytes = off_units + (uint32_t)ng * UB;
+    const uint32_t hdr_bytes = ((uint32_t)(Knp512 + 2 * ((C + 31) & ~31)) + 255u) & ~255u;
+    const int ntiles = (N + kStreamTileCols - 1) / kStreamTileCols;
     // LDS: raw activations (slice by slice, zeros past the row) | compacted activations | unit sums | partial outputs
     unsigned short *s_raw = reinterpret_cast<unsigned short *>(smem);
-    unsigned short *s_xs = s_raw + Knp512 + 512 * NB + 8;
-    float *s_xsum = reinterpret_cast<float *>(s_xs + Knp512);
-    float *s_red = s_xsum + 4 * nblk;
-    const int tstride = G * TEAMS;
-    const int P = (ntiles + tstride - 1) / tstride;  // tiles the busiest team walks
+    unsigned short *s_xs = s_raw + Knp512 + 512 * NB + 8;                   // [MEM][Knp512]
+    float *s_xsum = reinterpret_cast<float *>(s_xs + MEM * Knp512);         // [MEM][4 nblk]
+    float *s_red = s_xsum + MEM * 4 * nblk;
+    const int tstride = G * TSLOTS;
 
     if (wave < S) {
         // ---- staging wavefront: its slice of the row, its blocks' gather table; gather; unit sums
         __builtin_amdgcn_s_setprio(3);
-        const int b0 = wave * NB, b1 = min(nblk, b0 + NB);
+        const int mem = PAIR ? wave / SM : 0, ws = wave - mem * SM;   // the layer it stages for, its index among that layer's
+        const int b0 = ws * NB, b1 = min(nblk, b0 + NB);
         const bool active = b0 < nblk, last = active && b1 == nblk;
-        const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, K * 2, kSFlags);
-        const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc((void *)stream, 0, (int)hdr_bytes, kSFlags);
+        const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)job.x, 0, K * 2, kSFlags);
+        const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc((void *)(PAIR && mem ? job.stream2 : job.stream), 0,
+                                                                            (int)hdr_bytes, kSFlags);
+        unsigned short *xs_m = s_xs + mem * Knp512;
+        float *xsum_m = s_xsum + mem * 4 * nblk;
         su4 xr[XS];
         su2 tb[NB];
 #pragma unroll
@@ -128,9 +144,24 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_kernel(
 #pragma unroll
         for (int i = 0; i < NB; i++)
             tb[i] = __builtin_amdgcn_raw_buffer_load_b64(rh, b0 + i < b1 ? (uint32_t)((b0 + i) * 512 + lane * 8) : kSOob, 0, 0);
-        if constexpr (NORM) {
+        if constexpr (PRO == kCuGate) {
+            su4 gr[XS];
+            const __amdgpu_buffer_rsrc_t rg = __builtin_amdgcn_make_buffer_rsrc((void *)job.norm_w, 0, K * 2, kSFlags);
+#pragma unroll
+            for (int i = 0; i < XS; i++)
+                gr[i] = __builtin_amdgcn_raw_buffer_load_b128(rg, active ? (uint32_t)(b0 * 512 + i * 512 + lane * 8) * 2u : kSOob, 0, 0);
+#pragma unroll
+            for (int i = 0; i < XS; i++) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    xr[i][j] = cu_silu_mul_pair(gr[i][j], xr[i][j]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+        if constexpr (PRO == kCuNorm) {
             su4 nr[XS];
-            const __amdgpu_buffer_rsrc_t rn = __builtin_amdgcn_make_buffer_rsrc((void *)norm_w, 0, K * 2, kSFlags);
+            const __amdgpu_buffer_rsrc_t rn = __builtin_amdgcn_make_buffer_rsrc((void *)job.norm_w, 0, K * 2, kSFlags);
 #pragma unroll
             for (int i = 0; i < XS; i++)
                 nr[i] = __builtin_amdgcn_raw_buffer_load_b128(rn, active ? (uint32_t)(b0 * 512 + i * 512 + lane * 8) * 2u : kSOob, 0, 0);
@@ -152,10 +183,10 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_kernel(
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
             __builtin_amdgcn_s_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-            float t = 0.f;
+            float t = 0.f;   // (with two layers each layer's staging wavefronts cover the whole row: the first layer's sums)
 #pragma unroll
-            for (int wv = 0; wv < S; wv++) t += s_red[wv];
-            const float rs = rsqrtf(t / (float)K + eps);
+            for (int wv = 0; wv < SM; wv++) t += s_red[wv];
+            const float rs = rsqrtf(t / (float)K + job.eps);
 #pragma unroll
             for (int i = 0; i < XS; i++) {
 #pragma unroll
@@ -179,7 +210,7 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_kernel(
                         h[j] = s_raw[blk * 512 + 64 * j + lane + (int)((t[j >> 2] >> (8 * (j & 3))) & 0xffu)];
                     float f[4];
 #pragma unroll
-                    for (int j = 0; j < 8; j++) s_xs[blk * 512 + 64 * j + lane] = h[j];
+                    for (int j = 0; j < 8; j++) xs_m[blk * 512 + 64 * j + lane] = h[j];
 #pragma unroll
                     for (int u = 0; u < 4; u++)
                         f[u] = __half2float(__ushort_as_half(h[2 * u])) + __half2float(__ushort_as_half(h[2 * u + 1]));
@@ -188,7 +219,7 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_kernel(
                     const float s01 = swap32_add(f[0], f[1]);
                     const float s23 = swap32_add(f[2], f[3]);
                     const float r = row_sum(swap16_add(s01, s23));
-                    if (nn == 0) s_xsum[blk * 4 + ((kq >> 1) | ((kq & 1) << 1))] = r;
+                    if (nn == 0) xsum_m[blk * 4 + ((kq >> 1) | ((kq & 1) << 1))] = r;
                 }
             }
         }
@@ -198,6 +229,10 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_kernel(
         // ---- computing wavefront
         const int cwv = wave - S;
         const int team = cwv / W, cls = cwv % W;
+        const int mem = PAIR ? team & 1 : 0, slot = PAIR ? team >> 1 : team;   // the team's layer, its tile slot
+        const uint8_t *__restrict__ stream = PAIR && mem ? job.stream2 : job.stream;
+        const unsigned short *xs_m = s_xs + mem * Knp512;
+        const float *xsum_m = s_xsum + mem * 4 * nblk;
         const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(
             (void *)(stream + hdr_bytes), 0, (int)min((unsigned long long)ntiles * record_bytes, 0xffffffffull), kSFlags);
         const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc((void *)stream, 0, (int)hdr_bytes, kSFlags);
@@ -206,15 +241,16 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_kernel(
         su4 cw[4];
         su4 civ[4];
         const bool cherry_wave = cls == W - 1;
-        int tcur = bid + G * team;
+        int tcur = bid + G * slot;
         bool vcur = tcur < ntiles;
         uint32_t tb = (uint32_t)tcur * record_bytes;
         auto load_cherry = [&](uint32_t base, bool valid) {
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const int lg = 4 * j + kq;
-                cw[j] = __builtin_amdgcn_raw_buffer_load_b128(
-                    rt, valid && 8 * lg < C ? off_cherry + (uint32_t)(lg * 16 + nn) * 16u : kSOob, base, 2);
+                if (32 * j < C)
+                    cw[j] = __builtin_amdgcn_raw_buffer_load_b128(
+                        rt, valid && 8 * lg < C ? off_cherry + (uint32_t)(lg * 16 + nn) * 16u : kSOob, base, 2);
             }
         };
         // lane group kq keeps the scales of the units i with i % 4 == kq (every lane group ends up
@@ -240,14 +276,14 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_kernel(
             // the cherry columns of the lane's A operands (positions 32 q + 8 kq + 0..7 of the list) and the rows
 #pragma unroll
             for (int q = 0; q < 4; q++)
-                civ[q] = __builtin_amdgcn_raw_buffer_load_b128(rh, 32 * q < C ? (uint32_t)(Knp512 + 64 * q + 16 * kq) : kSOob, 0, 0);
+                if (32 * q < C) civ[q] = __builtin_amdgcn_raw_buffer_load_b128(rh, (uint32_t)(Knp512 + 64 * q + 16 * kq), 0, 0);
             load_cherry(tb, vcur);
         }
 #pragma unroll
         for (int i = 0; i < L / 4; i++) sc[i] = load_scale(i, tb, vcur);
 #pragma unroll
         for (int i = 0; i < D0; i++) wbuf[i] = load_unit(i, tb, vcur);
-        if constexpr (NORM) {
+        if constexpr (PRO == kCuNorm) {
             __builtin_amdgcn_s_barrier();  // (the staging wavefronts exchange their sums of squares)
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
@@ -270,10 +306,11 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_kernel(
                 }
             }
         }
+        const int P = WALK ? job.P : 1;
 #pragma unroll 1
         for (int j = 0; j < P; j++) {
             const int tnext = tcur + tstride;
-            const bool vnext = tnext < ntiles;
+            const bool vnext = WALK && tnext < ntiles;
             const uint32_t tbn = (uint32_t)tnext * record_bytes;
             float totc = 0.f;
             if (cherry_wave) {
@@ -282,7 +319,7 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_kernel(
                 for (int q = 0; q < 4; q++)
                     if (32 * q < C) dc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(ca[q]), as_h8(cw[q]), dc, 0, 0, 0);
                 totc = dc[0];
-                load_cherry(tbn, vnext);
+                if constexpr (WALK) load_cherry(tbn, vnext);
             }
             float tt = 0.f;
 #pragma unroll
@@ -293,10 +330,13 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_kernel(
                 const int up = real ? cls + i * W : 0;
                 const float sf = (i & 3) == kq ? __half2float(__ushort_as_half((unsigned short)sc[i >> 2])) : 0.f;
                 const su4 w = wbuf[i % D];
-                const float v = unit_dot<BITS>(w, s_xs + up * kStreamUnitK + 32 * kq);
-                wbuf[i % D] = i + D < L ? load_unit(i + D, tb, vcur) : load_unit(i + D - L, tbn, vnext);
-                tt += (v + kGrid * s_xsum[up]) * sf;
-                if ((i & 3) == 3) sc[i >> 2] = load_scale(i >> 2, tbn, vnext);
+                const float v = unit_dot<BITS>(w, xs_m + up * kStreamUnitK + 32 * kq);
+                if (i + D < L) wbuf[i % D] = load_unit(i + D, tb, vcur);
+                else if constexpr (WALK) wbuf[i % D] = load_unit(i + D - L, tbn, vnext);
+                tt += (v + kGrid * xsum_m[up]) * sf;
+                if constexpr (WALK) {
+                    if ((i & 3) == 3) sc[i >> 2] = load_scale(i >> 2, tbn, vnext);
+                }
             }
             // the four lane groups' quarters
             tt = swap32_add(tt, tt);
@@ -313,17 +353,99 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_kernel(
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-    for (int o = tid; o < 16 * P * TEAMS; o += NT) {
-        const int jt = o >> 4, j = jt / TEAMS, team = jt - j * TEAMS;
-        const int tile = bid + G * (team + TEAMS * j), n = tile * 16 + (o & 15);
+    const int P = WALK ? job.P : 1;
+    __half *__restrict__ mul = job.mul;
+    for (int o = tid; o < 16 * P * TSLOTS; o += NT) {
+        const int jt = o >> 4, j = jt / TSLOTS, slot = jt - j * TSLOTS;
+        const int tile = bid + G * (slot + TSLOTS * j), n = tile * 16 + (o & 15);
         if (tile < ntiles && n < N) {
-            float v = 0.f;
+            if constexpr (PAIR) {
+                float g = 0.f, u = 0.f;
 #pragma unroll
-            for (int c = 0; c < W; c++) v += s_red[(j * NC + team * W + c) * 16 + (o & 15)];
-            if (accumulate) v += __half2float(mul[n]);
-            mul[n] = __float2half_rn(v);
+                for (int c = 0; c < W; c++) {
+                    g += s_red[(j * NC + (2 * slot) * W + c) * 16 + (o & 15)];
+                    u += s_red[(j * NC + (2 * slot + 1) * W + c) * 16 + (o & 15)];
+                }
+                // the two projections' results as they would be stored, then the activation of silu_mul_kernel
+                const float g16 = __half2float(__float2half_rn(g)), u16 = __half2float(__float2half_rn(u));
+                const float a = __half2float(__float2half_rn(g16 / (1.f + __expf(-g16))));
+                mul[n] = __float2half_rn(a * u16);
+            } else {
+                float v = 0.f;
+#pragma unroll
+                for (int c = 0; c < W; c++) v += s_red[(j * NC + slot * W + c) * 16 + (o & 15)];
+                if (job.accumulate) v += __half2float(mul[n]);
+                mul[n] = __float2half_rn(v);
+            }
         }
     }
+}
+
+// The file is built with a kernel-argument preload count of 14 dwords: the dispatcher puts the
+// leading arguments into scalar registers before a wavefront starts, so nothing that a
+// wavefront's first requests depend on waits for a load from the argument segment (which costs
+// most of a microsecond).  Both shells are laid out for that.
+
+// one layer: x, stream, mul, K, C, N, workgroups, accumulate, P = 12 dwords
+template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, bool WALK>
+__global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_kernel(const __half *__restrict__ x,
+                                                                          const uint8_t *__restrict__ stream,
+                                                                          __half *__restrict__ mul, int K, int C, int N,
+                                                                          int wgs, int accumulate, int P) {
+    const CuJob job = {x, stream, mul, nullptr, 0.f, K, C, N, wgs, (int)blockIdx.x, accumulate, P, nullptr};
+    stream_cu_body<BITS, W, L, TEAMS, S, NB, D0, D, kCuPlain, WALK>(job);
+}
+
+// Up to three layers that read the same row (q / k / v, gate / up), consecutive ranges of
+// workgroups per layer, optionally behind the fused RMSNorm or the gated-MLP activation (one
+// layer then: the down projection).  Leading 14 dwords: x, norm_w (or the gate vector), the
+// three streams, then packed K | C << 16, N0/8 | N1/8 << 16, N2/8 | P << 16 | accumulate << 31,
+// first workgroup of member 1 | of member 2 << 10 | all workgroups << 20.
+struct CuGroupTail {
+    __half *mul[kStreamMaxGroup];
+    float eps;
+};
+template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, int PRO, bool WALK>
+__global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_group_kernel(
+    const __half *__restrict__ x, const __half *__restrict__ norm_w, const uint8_t *__restrict__ stream0,
+    const uint8_t *__restrict__ stream1, const uint8_t *__restrict__ stream2, uint32_t kc, uint32_t n01, uint32_t n2p,
+    uint32_t wgb, CuGroupTail tail) {
+    // the candidates are pinned in scalar registers first so that the selects stay selects (and do
+    // not become one load at a selected argument address)
+    const uint8_t *s0 = stream0, *s1 = stream1, *s2 = stream2;
+    asm volatile("" : "+s"(s0), "+s"(s1), "+s"(s2));
+    const int bid = blockIdx.x;
+    const int b1 = (int)(wgb & 1023u), b2 = (int)((wgb >> 10) & 1023u), total = (int)(wgb >> 20);
+    const bool m1 = bid >= b1, m2 = bid >= b2;  // (absent members start at `total`)
+    __half *o0 = tail.mul[0], *o1 = tail.mul[1], *o2 = tail.mul[2];
+    asm volatile("" : "+s"(o0), "+s"(o1), "+s"(o2));
+    CuJob job;
+    job.x = x;
+    job.norm_w = norm_w;
+    job.eps = tail.eps;
+    job.stream = m2 ? s2 : m1 ? s1 : s0;
+    job.mul = m2 ? o2 : m1 ? o1 : o0;
+    job.K = (int)(kc & 0xffffu);
+    job.C = (int)(kc >> 16);
+    job.N = 8 * (int)(m2 ? (n2p & 0xffffu) : m1 ? (n01 >> 16) : (n01 & 0xffffu));
+    job.G = m2 ? total - b2 : m1 ? b2 - b1 : b1;
+    job.bid = bid - (m2 ? b2 : m1 ? b1 : 0);
+    job.accumulate = (int)(n2p >> 31);
+    job.P = (int)((n2p >> 16) & 0x7fffu);
+    job.stream2 = nullptr;
+    stream_cu_body<BITS, W, L, TEAMS, S, NB, D0, D, PRO, WALK>(job);
+}
+
+// gate_proj and up_proj of a gated MLP in one launch, storing the activation
+// fp16(fp16(silu(gate)) * up) that the down projection reads (llama/modeling_llama_quant.py:251)
+// instead of the two results: 14 dwords, all preloaded.
+template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, int PRO, bool WALK>
+__global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_pair_kernel(
+    const __half *__restrict__ x, const __half *__restrict__ norm_w, const uint8_t *__restrict__ stream_gate,
+    const uint8_t *__restrict__ stream_up, __half *__restrict__ act, uint32_t kc, int N, uint32_t wgs_p, float eps) {
+    const CuJob job = {x, stream_gate, act, norm_w, eps, (int)(kc & 0xffffu), (int)(kc >> 16), N, (int)(wgs_p & 0xffffu),
+                       (int)blockIdx.x, 0, (int)(wgs_p >> 16), stream_up};
+    stream_cu_body<BITS, W, L, TEAMS, S, NB, D0, D, PRO, WALK, true>(job);
 }
 
 // ---- launch geometries --------------------------------------------------------------------------
@@ -337,21 +459,39 @@ struct CuCfg {
     int W, L, TEAMS, S, NB, D0, D;
 };
 static constexpr CuCfg kCuCfgs[] = {
-    {8, 4, 1, 4, 2, 2, 4},  // 0: up to 32 units, at most one tile per compute unit
-    {4, 8, 2, 4, 2, 3, 4},  // 1: up to 32 units, up to two tiles per compute unit
-    {4, 8, 3, 4, 2, 3, 4},  // 2: up to 32 units, more
-    {8, 8, 1, 8, 2, 2, 4},  // 3: up to 64 units
+    {8, 4, 1, 4, 2, 2, 4},   // 0: up to 32 units, at most one tile per compute unit
+    {4, 8, 2, 4, 2, 3, 4},   // 1: up to 32 units, up to two tiles per compute unit
+    {4, 8, 3, 4, 2, 3, 4},   // 2: up to 32 units, more
+    {8, 8, 1, 8, 2, 2, 4},   // 3: up to 64 units
+    {11, 8, 1, 5, 5, 3, 4},  // 4: up to 88 units (11008 input channels)
+    {8, 16, 1, 8, 4, 4, 8},  // 5: up to 128 units
+    {8, 28, 1, 8, 7, 4, 7},  // 6: up to 224 units (28672 input channels)
 };
+// Deep columns (entries 4 to 6) are the same kernel with more units per wavefront and more
+// blocks per staging wavefront; the barrier then opens later (staging 22 blocks takes 1.3 us
+// instead of 0.5), which the D0 units requested in front of it cover.  Measured: 11008 -> 4096
+// 7.04 us on the checkpoint layout -> 5.93 (3-bit 6.76 -> 5.57; with 8 x 12 units and 8 staging
+// wavefronts 6.01 / 5.59); 28672 -> 8192 23.5 -> 22.0; 13824 -> 5120 (3-bit, 320 tiles on 256
+// compute units: a quarter of them walk two tiles) 10.2 against 8.93, so that shape stays on the
+// checkpoint layout.
+// NOT used: 3-bit instantiations that walk tiles with a ring of D = 4 and more than 8 units per
+// wavefront (L = 12 or 16) gave wrong sums on the GPU (every output off by hundreds; D = 2, 3, 6,
+// 8, 12, 16 and every 4-bit instantiation are right); the cause was not found in the generated
+// code, so the table keeps L / D = 2 for deep columns and the parity tests run every entry in
+// both bit widths, with and without walking.
 
 static int cu_pick(int ng, int tiles_per_cu_ceil) {
     if (ng <= 32) return tiles_per_cu_ceil <= 1 ? 0 : tiles_per_cu_ceil == 2 ? 1 : 2;
     if (ng <= 64) return 3;
+    if (ng <= 88) return 4;
+    if (ng <= 128) return 5;
+    if (ng <= 224) return 6;
     return -1;
 }
 
-static size_t cu_lds_bytes(const StreamGeo &g, const CuCfg &c, int P) {
+static size_t cu_lds_bytes(const StreamGeo &g, const CuCfg &c, int P, int layers = 1) {
     const int Knp512 = (g.ng * kStreamUnitK + 511) & ~511;
-    size_t need = (size_t)(Knp512 + 512 * c.NB + 8 + Knp512) * 2 + (size_t)(Knp512 / 128) * 4 +
+    size_t need = (size_t)(Knp512 + 512 * c.NB + 8 + layers * Knp512) * 2 + (size_t)layers * (Knp512 / 128) * 4 +
                   (size_t)c.W * c.TEAMS * 16 * 4 * P;
     const size_t alone = 80 * 1024 + 1024;  // more than half of a compute unit's LDS: one workgroup per compute unit
     return need > alone ? need : alone;
@@ -399,79 +539,175 @@ bool stream_cu_supported(int bits, int K, int C, const int *Ns, int count) {
     if (geo.ng > c.W * c.L || geo.ng * kStreamUnitK > c.S * c.NB * 512 || C > 128) return false;
     const CuSplit sp = cu_split(tiles, count, c.TEAMS);
     if (sp.walk > kCuMaxWalk) return false;
+    for (int i = 0; i < count; i++)
+        if (Ns[i] % 8 || Ns[i] / 8 > 0xffff) return false;
+    if (K > 0xffff || sp.total > 1023) return false;
     return cu_lds_bytes(geo, c, sp.walk) <= 160 * 1024;
 }
 
-template <int BITS, int I, bool NORM, bool GROUP>
+template <typename KERN>
+static hipError_t cu_raise_lds(KERN kern, bool *raised) {
+    // per instantiation and device, once: the dynamic-LDS limit raised
+    static std::mutex mu;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kCuMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!raised[dev]) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        raised[dev] = true;
+    }
+    return hipSuccess;
+}
+
+template <int BITS, int I, int PRO, bool GROUP, bool WALK>
 static hipError_t launch_cu_cfg(const __half *vec, const __half *norm_w, float eps, const StreamMember *members, int count,
                                 const StreamGeo &geo, const CuSplit &sp, int accumulate, hipStream_t s) {
     constexpr CuCfg c = kCuCfgs[I];
-    auto kern = stream_cu_kernel<BITS, c.W, c.L, c.TEAMS, c.S, c.NB, c.D0, c.D, NORM, GROUP>;
     const size_t lds = cu_lds_bytes(geo, c, sp.walk);
-    {
-        // per instantiation and device, once: the dynamic-LDS limit raised
-        static std::mutex mu;
-        static bool raised[kCuMaxDevices] = {};
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kCuMaxDevices) return hipErrorInvalidDevice;
-        std::lock_guard<std::mutex> lock(mu);
-        if (!raised[dev]) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-            if (e != hipSuccess) return e;
-            raised[dev] = true;
+    const dim3 grid(sp.total), block(64 * (c.W * c.TEAMS + c.S));
+    static bool raised[kCuMaxDevices] = {};
+    if constexpr (!GROUP) {
+        auto kern = stream_cu_kernel<BITS, c.W, c.L, c.TEAMS, c.S, c.NB, c.D0, c.D, WALK>;
+        if (hipError_t e = cu_raise_lds(kern, raised)) return e;
+        hipLaunchKernelGGL(kern, grid, block, lds, s, vec, members[0].stream, members[0].mul, geo.K, geo.C, members[0].N,
+                           sp.wgs[0], accumulate, sp.walk);
+    } else {
+        auto kern = stream_cu_group_kernel<BITS, c.W, c.L, c.TEAMS, c.S, c.NB, c.D0, c.D, PRO, WALK>;
+        if (hipError_t e = cu_raise_lds(kern, raised)) return e;
+        CuGroupTail tail = {};
+        const uint8_t *st[kStreamMaxGroup];
+        uint32_t n8[kStreamMaxGroup], begin[kStreamMaxGroup];
+        for (int i = 0; i < kStreamMaxGroup; i++) {
+            const StreamMember &m = members[i < count ? i : 0];
+            st[i] = m.stream;
+            tail.mul[i] = m.mul;
+            n8[i] = (uint32_t)(m.N / 8);
+            begin[i] = (uint32_t)(i < count ? sp.begin[i] : sp.total);
         }
+        tail.eps = eps;
+        const uint32_t kc = (uint32_t)geo.K | ((uint32_t)geo.C << 16);
+        const uint32_t n01 = n8[0] | (n8[1] << 16);
+        const uint32_t n2p = n8[2] | ((uint32_t)sp.walk << 16) | (accumulate ? 0x80000000u : 0u);
+        const uint32_t wgb = begin[1] | (begin[2] << 10) | ((uint32_t)sp.total << 20);
+        hipLaunchKernelGGL(kern, grid, block, lds, s, vec, norm_w, st[0], st[1], st[2], kc, n01, n2p, wgb, tail);
     }
-    CuGroup g = {};
-    g.count = count;
-    for (int i = 1; i < kStreamMaxGroup; i++) {
-        const StreamMember &m = members[i < count ? i : 0];
-        g.stream[i - 1] = m.stream;
-        g.mul[i - 1] = m.mul;
-        g.N[i - 1] = m.N;
-        g.wg_begin[i - 1] = i < count ? sp.begin[i] : 0x7fffffff;
-        g.wgs[i - 1] = i < count ? sp.wgs[i] : 1;
-    }
-    hipLaunchKernelGGL(kern, dim3(sp.total), dim3(64 * (c.W * c.TEAMS + c.S)), lds, s, vec, members[0].stream, members[0].mul,
-                       geo.K, geo.C, geo.ng, members[0].N, geo.hdr_bytes, geo.off_cherry, geo.off_units, geo.record_bytes,
-                       sp.wgs[0], accumulate, norm_w, eps, g);
     return hipGetLastError();
 }
 
 // `count` layers of the same bits / K / C that read the same activation row, in one launch;
-// norm_w != nullptr fuses the RMSNorm of that row.  The caller has asked stream_cu_supported().
-hipError_t launch_stream_cu(int bits, const __half *vec, const __half *norm_w, float eps, const StreamMember *members,
-                            int count, int K, int C, int accumulate, hipStream_t s) {
-    if (count < 1 || count > kStreamMaxGroup) return hipErrorInvalidValue;
+// norm_w != nullptr fuses the RMSNorm of that row, gate != nullptr (one layer, no norm) the
+// gated-MLP activation fp16(fp16(silu(gate)) * vec).  The caller has asked stream_cu_supported().
+hipError_t launch_stream_cu(int bits, const __half *vec, const __half *norm_w, float eps, const __half *gate,
+                            const StreamMember *members, int count, int K, int C, int accumulate, hipStream_t s) {
+    if (count < 1 || count > kStreamMaxGroup || (gate && (norm_w || count != 1))) return hipErrorInvalidValue;
     int tiles[kStreamMaxGroup], all = 0;
     for (int i = 0; i < count; i++) {
         tiles[i] = ceil_div(members[i].N, kStreamTileCols);
         all += tiles[i];
+        if (members[i].N % 8 || members[i].N / 8 > 0xffff) return hipErrorInvalidValue;  // (the group shell packs N / 8 into 16 bits)
     }
+    if (K > 0xffff) return hipErrorInvalidValue;
     const StreamGeo geo = stream_geo(bits, K, members[0].N, C);
     const int idx = cu_pick(geo.ng, ceil_div(all, kCuCus));
     if (idx < 0) return hipErrorInvalidValue;
     const CuSplit sp = cu_split(tiles, count, kCuCfgs[idx].TEAMS);
-    if (sp.walk > kCuMaxWalk) return hipErrorInvalidValue;
-#define CQ_CU_GO(BITS_, I_)                                                                                          \
-    do {                                                                                                             \
-        if (norm_w) {                                                                                                \
-            return count > 1 ? launch_cu_cfg<BITS_, I_, true, true>(vec, norm_w, eps, members, count, geo, sp, accumulate, s)   \
-                             : launch_cu_cfg<BITS_, I_, true, false>(vec, norm_w, eps, members, count, geo, sp, accumulate, s); \
-        }                                                                                                            \
-        return count > 1 ? launch_cu_cfg<BITS_, I_, false, true>(vec, nullptr, 0.f, members, count, geo, sp, accumulate, s)     \
-                         : launch_cu_cfg<BITS_, I_, false, false>(vec, nullptr, 0.f, members, count, geo, sp, accumulate, s);   \
+    if (sp.walk > kCuMaxWalk || sp.total > 1023) return hipErrorInvalidValue;
+    const bool group = count > 1 || norm_w != nullptr || gate != nullptr, walk = sp.walk > 1;
+#define CQ_CU_GO(BITS_, I_)                                                                                               \
+    do {                                                                                                                  \
+        if (!group)                                                                                                       \
+            return walk ? launch_cu_cfg<BITS_, I_, kCuPlain, false, true>(vec, nullptr, 0.f, members, count, geo, sp, accumulate, s)   \
+                        : launch_cu_cfg<BITS_, I_, kCuPlain, false, false>(vec, nullptr, 0.f, members, count, geo, sp, accumulate, s); \
+        if (gate)                                                                                                         \
+            return walk ? launch_cu_cfg<BITS_, I_, kCuGate, true, true>(vec, gate, 0.f, members, count, geo, sp, accumulate, s)        \
+                        : launch_cu_cfg<BITS_, I_, kCuGate, true, false>(vec, gate, 0.f, members, count, geo, sp, accumulate, s);      \
+        if (norm_w)                                                                                                       \
+            return walk ? launch_cu_cfg<BITS_, I_, kCuNorm, true, true>(vec, norm_w, eps, members, count, geo, sp, accumulate, s)      \
+                        : launch_cu_cfg<BITS_, I_, kCuNorm, true, false>(vec, norm_w, eps, members, count, geo, sp, accumulate, s);    \
+        return walk ? launch_cu_cfg<BITS_, I_, kCuPlain, true, true>(vec, nullptr, 0.f, members, count, geo, sp, accumulate, s)        \
+                    : launch_cu_cfg<BITS_, I_, kCuPlain, true, false>(vec, nullptr, 0.f, members, count, geo, sp, accumulate, s);      \
     } while (0)
 #define CQ_CU_BITS(BITS_)            \
     switch (idx) {                   \
         case 0: CQ_CU_GO(BITS_, 0);  \
         case 1: CQ_CU_GO(BITS_, 1);  \
         case 2: CQ_CU_GO(BITS_, 2);  \
-        default: CQ_CU_GO(BITS_, 3); \
+        case 3: CQ_CU_GO(BITS_, 3);  \
+        case 4: CQ_CU_GO(BITS_, 4);  \
+        case 5: CQ_CU_GO(BITS_, 5);  \
+        default: CQ_CU_GO(BITS_, 6); \
     }
     if (bits == 4) CQ_CU_BITS(4)
     CQ_CU_BITS(3)
 #undef CQ_CU_BITS
 #undef CQ_CU_GO
+}
+
+
+// ---- gate_proj + up_proj -> fp16(fp16(silu(gate)) * up) in one launch ----------------------------
+// Pairs of teams on the same tile of the two layers.  Up to 32 units per column: three pairs of
+// two-wavefront teams (16 units per wavefront) and 2 + 2 staging wavefronts of four blocks, i.e. the
+// three tiles per compute unit of the 4096 -> 11008 launch with both layers' tile t in one
+// workgroup; up to 64 units: one pair of four-wavefront teams and 4 + 4 staging wavefronts.
+static constexpr CuCfg kCuPairCfgs[] = {
+    {2, 16, 6, 4, 4, 3, 8},
+    {4, 16, 2, 8, 4, 3, 8},
+};
+
+static int cu_pair_pick(int ng) { return ng <= 32 ? 0 : ng <= 64 ? 1 : -1; }
+
+bool stream_pair_supported(int bits, int K, int N, int C) {
+    if ((bits != 3 && bits != 4) || K > 0xffff || C > 128 || N % 8) return false;
+    const StreamGeo geo = stream_geo(bits, K, N, C);
+    const int idx = cu_pair_pick(geo.ng);
+    if (idx < 0) return false;
+    const CuCfg &c = kCuPairCfgs[idx];
+    const int tiles[1] = {geo.ntiles};
+    const CuSplit sp = cu_split(tiles, 1, c.TEAMS / 2);
+    if (sp.walk > kCuMaxWalk || sp.total > 0xffff) return false;
+    return cu_lds_bytes(geo, c, sp.walk, 2) <= 160 * 1024;
+}
+
+template <int BITS, int I, int PRO, bool WALK>
+static hipError_t launch_pair_cfg(const __half *vec, const __half *norm_w, float eps, const uint8_t *sg, const uint8_t *su,
+                                  __half *act, const StreamGeo &geo, const CuSplit &sp, hipStream_t s) {
+    constexpr CuCfg c = kCuPairCfgs[I];
+    auto kern = stream_cu_pair_kernel<BITS, c.W, c.L, c.TEAMS, c.S, c.NB, c.D0, c.D, PRO, WALK>;
+    static bool raised[kCuMaxDevices] = {};
+    if (hipError_t e = cu_raise_lds(kern, raised)) return e;
+    const size_t lds = cu_lds_bytes(geo, c, sp.walk, 2);
+    hipLaunchKernelGGL(kern, dim3(sp.total), dim3(64 * (c.W * c.TEAMS + c.S)), lds, s, vec, norm_w, sg, su, act,
+                       (uint32_t)geo.K | ((uint32_t)geo.C << 16), geo.N, (uint32_t)sp.wgs[0] | ((uint32_t)sp.walk << 16), eps);
+    return hipGetLastError();
+}
+
+// act (1, N) = fp16(fp16(silu(vec' Wg^T)) * (vec' Wu^T)), vec' = vec or its RMSNorm; the caller has
+// asked stream_pair_supported().
+hipError_t launch_stream_pair(int bits, const __half *vec, const __half *norm_w, float eps, const uint8_t *stream_gate,
+                              const uint8_t *stream_up, __half *act, int K, int N, int C, hipStream_t s) {
+    const StreamGeo geo = stream_geo(bits, K, N, C);
+    const int idx = cu_pair_pick(geo.ng);
+    if (idx < 0) return hipErrorInvalidValue;
+    const int tiles[1] = {geo.ntiles};
+    const CuSplit sp = cu_split(tiles, 1, kCuPairCfgs[idx].TEAMS / 2);
+    if (sp.walk > kCuMaxWalk) return hipErrorInvalidValue;
+    const bool walk = sp.walk > 1;
+#define CQ_PAIR_GO(BITS_, I_)                                                                                        \
+    do {                                                                                                             \
+        if (norm_w)                                                                                                  \
+            return walk ? launch_pair_cfg<BITS_, I_, kCuNorm, true>(vec, norm_w, eps, stream_gate, stream_up, act, geo, sp, s)   \
+                        : launch_pair_cfg<BITS_, I_, kCuNorm, false>(vec, norm_w, eps, stream_gate, stream_up, act, geo, sp, s); \
+        return walk ? launch_pair_cfg<BITS_, I_, kCuPlain, true>(vec, nullptr, 0.f, stream_gate, stream_up, act, geo, sp, s)     \
+                    : launch_pair_cfg<BITS_, I_, kCuPlain, false>(vec, nullptr, 0.f, stream_gate, stream_up, act, geo, sp, s);   \
+    } while (0)
+    if (bits == 4) {
+        if (idx == 0) CQ_PAIR_GO(4, 0);
+        CQ_PAIR_GO(4, 1);
+    }
+    if (idx == 0) CQ_PAIR_GO(3, 0);
+    CQ_PAIR_GO(3, 1);
+#undef CQ_PAIR_GO
 }
 
 }  // namespace cq

@@ -15,8 +15,8 @@ from oracle import c_oracle
 
 pytestmark = pytest.mark.gpu
 
-LAYER_TOL = 1e-2    # rel-L2 of the hidden state after any layer, step 0 (measured: 3.9e-3 at worst)
-LOGIT_TOL = 2e-2    # rel-L2 of a step's logits (measured: 4.0e-3 at step 0, 6.5e-3 at step 7)
+LAYER_TOL = 6e-3    # rel-L2 of the hidden state after any layer, step 0 (measured: 3.9e-3 at worst)
+LOGIT_TOL = 1e-2    # rel-L2 of a step's logits (measured: 4.0e-3 at step 0, 6.5-6.8e-3 at step 7)
 
 
 def f16(a):
@@ -131,9 +131,9 @@ def test_full_size_7b_decoder_against_the_c_oracle():
     r0, r7 = rel(dev_logits[0], want[0]), rel(dev_logits[steps - 1], want[steps - 1])
     print(f"  worst per-layer rel-L2 {worst:.3e}; logits rel-L2 step 0 {r0:.3e}, step {steps - 1} {r7:.3e}", flush=True)
     assert r0 <= LOGIT_TOL and r7 <= LOGIT_TOL
-    # the same model as a loader leaves it (q / k / v / o / gate / up repacked into weight streams):
-    # the captured step now runs the stream kernels for them
-    assert model.prepack() == 6 * cfg.num_hidden_layers
+    # the same model as a loader leaves it (all seven projections repacked into weight streams): the
+    # captured step now runs the stream kernels for them, the down projection behind the fused SiLU * up
+    assert model.prepack() == 7 * cfg.num_hidden_layers
     pre_logits = model.step_logits(ids, use_graph=True).cpu().numpy()
     p0, p7 = rel(pre_logits[0], want[0]), rel(pre_logits[steps - 1], want[steps - 1])
     print(f"  repacked: logits rel-L2 step 0 {p0:.3e}, step {steps - 1} {p7:.3e}", flush=True)

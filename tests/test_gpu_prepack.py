@@ -56,7 +56,12 @@ def run(qc, bits, stream, x, n, c, out=None, accumulate=False):
 # last unit, N not a multiple of 16, no cherries at all, two cherry MFMA steps (C = 48)
 SHAPES = [(4, 4096, 11008), (3, 4096, 11008), (4, 11008, 4096), (3, 11008, 4096), (4, 4096, 4096), (3, 4096, 4096),
           (3, 5120, 5120), (3, 5120, 13824), (3, 13824, 5120), (4, 8192, 8192), (4, 8192, 1024),
-          (4, 1024, 264), (3, 1024, 264), (4, 2304, 40), (3, 768, 24)]
+          (4, 1024, 264), (3, 1024, 264), (4, 2304, 40), (3, 768, 24),
+          # every launch geometry of the kernel with one workgroup per compute unit, both bit widths, with
+          # and without tile walking: 257..512 tiles of up to 32 units, 64 / 88 / 128 / 224 units per column
+          (4, 2048, 6000), (3, 2048, 6000), (3, 8192, 8192), (3, 8192, 264), (4, 11008, 4608), (3, 11008, 4608),
+          (4, 13824, 5120), (4, 16384, 264), (3, 13824, 264), (4, 28672, 264), (3, 28672, 264), (4, 20480, 4352),
+          (3, 24576, 4104)]
 
 
 @pytest.mark.parametrize("bits,k,n", SHAPES)
@@ -98,7 +103,8 @@ def test_prepacked_matvec_against_oracle(qc, bits, k, n):
 
 
 @pytest.mark.parametrize("bits,k,n", [(4, 4096, 4096), (3, 4096, 4096), (4, 11008, 512), (3, 11008, 512),
-                                      (3, 5120, 520), (4, 8192, 264), (3, 13824, 264)])
+                                      (3, 5120, 520), (4, 8192, 264), (3, 13824, 264), (4, 28672, 264), (3, 28672, 264),
+                                      (3, 11008, 4608), (4, 16384, 4112)])
 def test_prepacked_one_hot_reads_back_dequantised_weights(qc, bits, k, n):
     """x = e_j returns column j of the dense weight: decode, gather around the cherry channels and
     the per-unit grid offset are exact.  Positions probe every code slot of a lane's 32 and both
@@ -209,7 +215,9 @@ def test_prepacked_c_abi_rejections(qc):
     assert lib.cherryq_prepack_supported(4, 16, 8192, 8192, 32, 128) == 1     # rows kept in registers
     assert lib.cherryq_prepack_supported(3, 2, 13824, 5120, 48, 128) == 0     # more than 64 units per column
     assert lib.cherryq_prepack_supported(4, 1, 4096, 4096, 16, 64) == 0       # group size a multiple of 128
-    assert lib.cherryq_prepack_supported(4, 1, 28672, 8192, 112, 128) == 0    # more than 16384 quantised channels
+    assert lib.cherryq_prepack_supported(4, 1, 28672, 8192, 112, 128) == 1    # 224 units per column: the deepest taken
+    assert lib.cherryq_prepack_supported(4, 1, 32768, 8192, 128, 128) == 0    # more than 224 units
+    assert lib.cherryq_prepack_supported(4, 16, 28672, 8192, 112, 128) == 0   # 2 to 16 rows: up to 64 units
     assert lib.cherryq_prepack_supported(3, 1, 13824, 5120, 48, 128) == 1
     nbytes = lib.cherryq_prepack_bytes(4, 4096, 1024, 16)
     buf = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
@@ -460,7 +468,8 @@ def _column_sample(p, cols):
             "qweight": np.ascontiguousarray(p["qweight"][:, cols]), "scales": np.ascontiguousarray(p["scales"][:, cols])}
 
 
-@pytest.mark.parametrize("bits,k,n", [(4, 8192, 28672), (3, 8192, 28672), (3, 8192, 16392), (4, 8192, 16392)])
+@pytest.mark.parametrize("bits,k,n", [(4, 8192, 28672), (3, 8192, 28672), (3, 8192, 16392), (4, 8192, 16392),
+                                      (4, 28672, 8192), (3, 28672, 8192)])
 def test_prepacked_deep_and_wide_layers_walk_tiles(qc, bits, k, n):
     """64 units per column AND more tiles than resident workgroups: the geometry a loader selects for
     the 70B gate / up projections (computing wavefronts that stage the activations themselves, every
@@ -496,7 +505,7 @@ def test_prepacked_deep_and_wide_layers_walk_tiles(qc, bits, k, n):
     nidx = orc.normal_indices(k, idx)
     kn = len(nidx)
     for j in [int(nidx[0]), int(nidx[127]), int(nidx[128]), int(nidx[4095]), int(nidx[4096]), int(nidx[kn - 1]),
-              int(nidx[kn - 129]), int(idx[0]), int(idx[-1])]:
+              int(nidx[kn - 129]), int(nidx[kn // 2 + 77]), int(idx[0]), int(idx[-1])]:
         e = np.zeros((1, k), dtype=np.float16)
         e[0, j] = 1
         with np.errstate(over="ignore"):
@@ -613,3 +622,133 @@ def test_prepacked_layers_with_fewer_units_than_wavefronts(bits, k, n, b):
         e[r, pool[r % len(pool)]] = np.float16(2.0 ** ((r * 5) % 13 - 6))
     with np.errstate(over="ignore"):
         np.testing.assert_array_equal(go(e), c_oracle.fused(e, p, bits, 128).astype(np.float16))
+
+
+@pytest.mark.parametrize("bits,k,n", [(4, 11008, 4096), (3, 11008, 4096), (4, 4096, 1024), (3, 13824, 5120), (4, 28672, 1032)])
+def test_prepacked_gated_down_projection(bits, k, n):
+    """cherryq_decode_matvec_gated_prepacked_f16: fp16(fp16(silu(gate)) * up) formed while the row is
+    staged, then the matvec over the repacked layer, accumulating or not.  Against the C oracle's
+    fused product of that activation, against the checkpoint-layout launch with the same prologue, and
+    bit for bit where the activation is one-hot (silu(g) * u exactly representable)."""
+    import cherryq_decoder as dec
+    print("[case] prepacked gated", bits, k, n, flush=True)
+    gen = torch.Generator(device="cuda").manual_seed(31 + bits)
+    cfg = dec.DecoderConfig(w_bits=bits, group_size=128, cherry_fraction=1 / 256)
+    m = dec.random_packed_linear(cfg, k, n, gen, "cuda")
+    p = {b: getattr(m, b).cpu().numpy() for b in NAMES}
+    assert m.prepack()
+    rng = np.random.default_rng(19)
+    f16 = lambda a: np.asarray(a).astype(np.float16)
+    up = f16(rng.standard_normal((1, k)))
+    gate = f16(rng.standard_normal((1, k)) * 2)
+
+    def act_of(g, u):
+        g32 = g.astype(np.float32)
+        silu = f16(g32 / (np.float32(1) + np.exp(-g32, dtype=np.float32)))
+        return f16(silu.astype(np.float32) * u.astype(np.float32))
+
+    def go(u, g, base=None):
+        out = torch.full((1, n), 3.0, dtype=torch.float16, device="cuda") if base is None else torch.from_numpy(base).cuda()
+        dec.matvec_gated_prepacked(m, torch.from_numpy(u).cuda(), torch.from_numpy(g).cuda(), out, accumulate=base is not None)
+        torch.cuda.synchronize()
+        return out.cpu().numpy()
+
+    act = act_of(gate, up)
+    want = c_oracle.fused(act, p, bits, 128)
+    got = go(up, gate)
+    assert np.isfinite(got).all()
+    assert orc.rel_l2(got, want) <= 1e-3
+    np.testing.assert_array_equal(got, go(up, gate))
+    base = f16(rng.standard_normal((1, n)))
+    assert orc.rel_l2(go(up, gate, base), want + base.astype(np.float64)) <= 1e-3
+    # the checkpoint-layout launch with the same prologue: same activation bits, two summation orders
+    ref = torch.zeros(1, n, dtype=torch.float16, device="cuda")
+    dec.matvec_group([m], torch.from_numpy(up).cuda(), [ref], vec_gate=torch.from_numpy(gate).cuda())
+    torch.cuda.synchronize()
+    assert orc.rel_l2(got, ref.cpu().numpy().astype(np.float64)) <= 5e-4
+    # one-hot activations: gate = 0 everywhere (silu(0) = 0) except one channel with a huge gate
+    # (silu(g) = g exactly in fp16 for g >= 17: exp(-g) < 2^-24)
+    idx = p["cherry_indices"].astype(np.int64)
+    nidx = orc.normal_indices(k, idx)
+    for j in (int(nidx[0]), int(nidx[129]), int(nidx[-1]), int(idx[0]), int(idx[-1]), int(nidx[len(nidx) // 2])):
+        g = np.zeros((1, k), dtype=np.float16)
+        g[0, j] = 32
+        u = f16(rng.standard_normal((1, k)))
+        u[0, j] = np.float16(2.0 ** -5)
+        e = np.zeros((1, k), dtype=np.float16)
+        e[0, j] = 1   # 32 * 2^-5
+        with np.errstate(over="ignore"):
+            np.testing.assert_array_equal(go(u, g), f16(c_oracle.fused(e, p, bits, 128)), err_msg=f"column {j}")
+
+
+def test_prepacked_gated_rejections():
+    import cherryq_decoder as dec
+    lib = dec._lib
+    fake = 1 << 12
+    f = lib.cherryq_decode_matvec_gated_prepacked_f16
+    assert f(5, fake, fake, fake, 1 << 30, fake, 4096, 4096, 16, 0, None) == -5
+    assert f(4, fake, None, fake, 1 << 30, fake, 4096, 4096, 16, 0, None) == -1
+    assert f(4, fake, fake + 2, fake, 1 << 30, fake, 4096, 4096, 16, 0, None) == -6
+    assert f(4, fake, fake, fake, 64, fake, 4096, 4096, 16, 0, None) == -4
+    assert f(4, fake, fake, fake, 1 << 30, fake, 65536, 4096, 0, 0, None) == -7
+
+
+@pytest.mark.parametrize("bits,k,n,norm", [(4, 4096, 11008, True), (3, 4096, 11008, True), (4, 4096, 11008, False),
+                                           (4, 8192, 28672, True), (3, 8192, 4104, False), (4, 4096, 32008, True),
+                                           (3, 1024, 264, True), (4, 512, 40, False)])
+def test_prepacked_gate_up_fused_activation(bits, k, n, norm):
+    """cherryq_decode_gate_up_prepacked_f16: both projections and SiLU(gate) * up in one launch.  Bit for
+    bit what the separate launches give (grouped gate / up launch, then the SiLU * up kernel: same
+    rounding points), and the activation of the C oracle's two products within tolerance."""
+    import cherryq_decoder as dec
+    print("[case] prepacked gate/up fused", bits, k, n, norm, flush=True)
+    gen = torch.Generator(device="cuda").manual_seed(37 + bits)
+    cfg = dec.DecoderConfig(w_bits=bits, group_size=128, cherry_fraction=1 / 256)
+    mg, mu = dec.random_packed_linear(cfg, k, n, gen, "cuda"), dec.random_packed_linear(cfg, k, n, gen, "cuda")
+    packed = [{b: getattr(m, b).cpu().numpy() for b in NAMES} for m in (mg, mu)]
+    assert mg.prepack() and mu.prepack()
+    assert dec.gate_up_prepacked_supported(mg, mu)
+    rng = np.random.default_rng(23)
+    f16 = lambda a: np.asarray(a).astype(np.float16)
+    # activations scaled so that the gate results spread over a few units: SiLU in its curved range
+    x = f16(rng.standard_normal((1, k)) * 4)
+    nw = f16(rng.random(k) + 0.5)
+    eps = 1e-6
+    kw = dict(norm_weight=torch.from_numpy(nw).cuda(), eps=eps) if norm else {}
+    xt = torch.from_numpy(x).cuda()
+    act = torch.full((1, n), 9.0, dtype=torch.float16, device="cuda")
+    dec.gate_up_prepacked(mg, mu, xt, act, **kw)
+    torch.cuda.synchronize()
+    got = act.cpu().numpy()
+    assert np.isfinite(got).all()
+    # the separate launches
+    g = torch.empty(1, n, dtype=torch.float16, device="cuda")
+    u = torch.empty(1, n, dtype=torch.float16, device="cuda")
+    dec.matvec_group_prepacked([mg, mu], xt, [g, u], **kw)
+    want = torch.empty(1, n, dtype=torch.float16, device="cuda")
+    dec._ok(dec._lib.cherryq_decode_silu_mul_f16(g.data_ptr(), u.data_ptr(), want.data_ptr(), n, dec._stream()), "silu_mul")
+    torch.cuda.synchronize()
+    # both launches round the same fp32 sums once: the last bit of gate or up may differ where the summation
+    # orders differ (teams of two wavefronts here, of four there), never more
+    gw, ww = got.astype(np.float64), want.cpu().numpy().astype(np.float64)
+    assert orc.rel_l2(gw, ww) <= 5e-4
+    assert (got == want.cpu().numpy()).mean() > 0.8
+    # against the oracle
+    if norm:
+        hf = x.astype(np.float64)
+        a_in = f16(nw.astype(np.float64) * f16(hf / np.sqrt(np.mean(hf * hf) + eps)).astype(np.float64))
+    else:
+        a_in = x
+    cols = np.arange(n) if k * n <= 4096 * 11008 else np.sort(rng.choice(n // 16, size=40, replace=False))[:, None] * 16 + np.arange(16)
+    cols = np.asarray(cols).reshape(-1)
+    subs = [_column_sample(p, cols) for p in packed]
+    go, uo = (f16(c_oracle.fused(a_in, sp, bits, 128)) for sp in subs)
+    g32 = go.astype(np.float32)
+    silu = f16(g32 / (np.float32(1) + np.exp(-g32, dtype=np.float32)))
+    ref = f16(silu.astype(np.float32) * uo.astype(np.float32)).astype(np.float64)
+    assert orc.rel_l2(gw[:, cols], ref) <= 2e-3   # fp16 roundings of gate and up enter the activation
+    # repeatable
+    act2 = torch.empty_like(act)
+    dec.gate_up_prepacked(mg, mu, xt, act2, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(act, act2)
