@@ -51,6 +51,15 @@ MEASURED_TRAFFIC = {("llama7b_gate_up_w4", 1, "reference"): 25320960,
                     ("llama7b_gate_up_w4", 1, "prepacked"): 23824998}
 
 
+# Matrix-core busy share of the 16-row kernels from rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES runs (busy
+# cycles / (kernel time x 2.4 GHz x 1024 SIMDs)); like the traffic figure it cannot be read while timing.
+MFMA_BUSY = {"llama70b_gate_up_w4": {"frac": 0.123, "kernel": "cq::stream_rows_reg_kernel<4, 8, 8, 1>",
+                                     "profile": "profiles/rows16_w4_llama70b_gate_up_8192x28672_stream.md"},
+             "llama70b_down_w4": {"frac": 0.084, "kernel": "cq::batch_kernel<4>",
+                                  "profile": "profiles/batch_w4_llama70b_gate_up_8192x28672_b16_mfma_counters.md",
+                                  "note": "measured on the 8192 -> 28672 layer, same kernel and unit count per byte"}}
+
+
 def algorithmic_bytes(bits, k, n, batch=1, group=128):
     """Bytes one call must move: packed codes + scales + cherry rows + indices + x + y."""
     c = -(-k // 256) // 8 * 8
@@ -446,10 +455,12 @@ def main():
                 torch.cuda.empty_cache()
             print(line, file=sys.stderr, flush=True)
 
-    def kernel_name(bits, batch, path, k_in=0):
+    def kernel_name(bits, batch, path, k_in=0, n_out=0):
         if path == "prepacked":
             if batch == 1:
-                return f"cq::stream_kernel<{bits}>"
+                import quant_cuda
+                base_name = quant_cuda.prepacked_kernel_name(bits, k_in, n_out, -(-k_in // 256) // 8 * 8) if k_in and n_out else ""
+                return f"{base_name or 'cq::stream_cu_kernel'}<{bits}>"
             if batch >= 8 or k_in > 32 * args.group:  # the rule of launch_stream_rows: activations in registers
                 return f"cq::stream_rows_frag_kernel + cq::stream_rows_reg_kernel<{bits}>"
             return f"cq::stream_rows_prep_kernel + cq::stream_rows_kernel<{bits}>"
@@ -461,6 +472,25 @@ def main():
             return f"cq::batch_prep_kernel<{bits}> + cq::batch_kernel<{bits}>"
         return f"cq::gemm_prep_kernel<{bits}> + cq::gemm_kernel<{bits}, {32 if batch <= 32 else 64 if batch <= 64 else 128}>"
 
+    side_steps = min(args.steps, 500)
+
+    def batch_record(name, batch, mfma=None):
+        """A small-batch call (2..16 rows) on the path a loader gets for the layer: whole-call device time
+        (preparation launch included), bytes, flops; `mfma`: matrix-core busy share from a recorded PMC run."""
+        b_, k_, n_ = WORKLOADS[name]
+        r = time_gpu(b_, k_, n_, args.group, side_steps, min(args.warmup, 50), batch=batch, use_graph=not args.no_graph)
+        ab_ = algorithmic_bytes(b_, k_, n_, batch, args.group)
+        fl = 2.0 * batch * k_ * n_
+        rec = {"workload": name, "batch": batch, "us": round(r["us"], 3), "path": r["path"],
+               "kernel": kernel_name(b_, batch, r["path"], k_, n_), "algorithmic_bytes_per_call": ab_,
+               "achieved": round(ab_ / r["us"] / 1e3, 1), "unit": "GB/s", "frac": round(ab_ / r["us"] / 1e3 / HBM_PEAK_GBS, 4),
+               "tflops": round(fl / r["us"] / 1e6, 1), "frac_of_fp16_mfma_peak": round(fl / r["us"] / 1e6 / 2500, 4)}
+        if mfma:
+            rec["mfma_busy"] = mfma
+        del r
+        torch.cuda.empty_cache()
+        return rec
+
     def side_record(name, with_cpu=False):
         """One more layer in the same JSON line: both paths' device time, achieved bandwidth of the faster."""
         b_, k_, n_ = WORKLOADS[name]
@@ -471,7 +501,7 @@ def main():
             import quant_cuda
             if path == "prepacked" and not quant_cuda.prepack_supported(b_, 1, k_, n_, -(-k_ // 256) // 8 * 8, args.group):
                 continue
-            r = time_gpu(b_, k_, n_, args.group, args.steps, args.warmup, use_graph=not args.no_graph, path=path)
+            r = time_gpu(b_, k_, n_, args.group, side_steps, min(args.warmup, 50), use_graph=not args.no_graph, path=path)
             rec[f"{path}_us"] = round(r["us"], 3)
             if best is None or r["us"] < best[0]:
                 best = (r["us"], path)
@@ -479,7 +509,7 @@ def main():
                 rec["cpu_baseline"] = cpu_baseline(b_, k_, n_, args.group, r["base"], r["x"].cpu().numpy(), seconds=4.0)
             del r
             torch.cuda.empty_cache()
-        rec.update({"us": round(best[0], 3), "path": best[1], "kernel": kernel_name(b_, 1, best[1]),
+        rec.update({"us": round(best[0], 3), "path": best[1], "kernel": kernel_name(b_, 1, best[1], k_, n_),
                     "achieved": round(ab_ / best[0] / 1e3, 1), "unit": "GB/s", "peak": HBM_PEAK_GBS,
                     "frac": round(ab_ / best[0] / 1e3 / HBM_PEAK_GBS, 4)})
         return rec
@@ -514,7 +544,7 @@ def main():
                                         "bench.py (profiles/); not re-measured in this run") if traffic else
                                        "not measured for this workload / kernel",
                      "algorithmic_bytes_per_launch": ab,
-                     "kernel": kernel_name(bits, args.batch, path, k)},
+                     "kernel": kernel_name(bits, args.batch, path, k, n)},
     }
     if main_run["resident_us"] is not None:
         ru = main_run["resident_us"]
@@ -530,12 +560,23 @@ def main():
             del other
             torch.cuda.empty_cache()
         result["roofline"]["reference"] = roofline_reference(ab, args.steps)
+        if not args.no_decode:
+            result["decode"] = decode_benchmark()
         if args.workload == "llama7b_gate_up_w4":
             # the other half of the headline metric (3-bit, same layer) and config 0 (4096 -> 4096,
             # 4-bit, with the reference's CPU path on that layer)
             result["roofline_w3"] = side_record("llama7b_gate_up_w3")
             result["config0"] = side_record("llama7b_attn_w4", with_cpu=True)
-    if not args.no_decode:
+            # the rest of the configurations: the down projection of config 1, the LLaMA-13B shapes in
+            # 3 bits at batch 1 / 4 / 8 (config 3), the LLaMA-70B shapes in 4 bits at batch 1 / 16 (config 4)
+            result["config1_down"] = [side_record("llama7b_down_w4"), side_record("llama7b_down_w3")]
+            result["config3"] = {"batch1": [side_record(w) for w in ("llama13b_attn_w3", "llama13b_gate_up_w3", "llama13b_down_w3")],
+                                 "batched": [batch_record(w, b) for w in ("llama13b_attn_w3", "llama13b_gate_up_w3") for b in (4, 8)]}
+            result["config4"] = {"batch1": [side_record(w) for w in ("llama70b_attn_w4", "llama70b_kv_w4", "llama70b_gate_up_w4",
+                                                                     "llama70b_down_w4")],
+                                 "batch16": [batch_record("llama70b_gate_up_w4", 16, MFMA_BUSY.get("llama70b_gate_up_w4")),
+                                             batch_record("llama70b_down_w4", 16, MFMA_BUSY.get("llama70b_down_w4"))]}
+    if not args.no_decode and "decode" not in result:
         result["decode"] = decode_benchmark()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(bits, k, n, args.group, base, x_host)

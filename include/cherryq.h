@@ -235,6 +235,10 @@ int cherryq_prepack_supported(int w_bits, int batch, int in_features, int out_fe
  * 13B ones), 0 elsewhere or if unsupported: what a loader asks before spending the extra copy of
  * the weights. */
 int cherryq_prepack_recommended(int w_bits, int in_features, int out_features, int num_cherries, int group_size);
+/* The kernel cherryq_matvec_prepacked_f16 launches for a layer, as it appears in a profiler's
+ * kernel trace (without template arguments): "cq::stream_cu_kernel" (one workgroup per compute
+ * unit) or "cq::stream_kernel"; "" for shapes the entry point does not take. */
+const char *cherryq_matvec_prepacked_kernel_name(int w_bits, int in_features, int out_features, int num_cherries);
 int cherryq_prepack_f16(int w_bits, const uint8_t *qweight, const void *cherry_weight, const int16_t *cherry_indices,
                         const void *scales, void *stream, size_t stream_bytes, int in_features, int out_features,
                         int num_cherries, int group_size, void *hip_stream);

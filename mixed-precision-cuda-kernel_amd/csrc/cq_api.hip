@@ -422,6 +422,11 @@ int cherryq_prepack_recommended(int w_bits, int in_features, int out_features, i
     return cq::stream_faster(w_bits, in_features, out_features, num_cherries) ? 1 : 0;
 }
 
+const char *cherryq_matvec_prepacked_kernel_name(int w_bits, int in_features, int out_features, int num_cherries) {
+    if (!cq::stream_supported(w_bits, 1, in_features, out_features, num_cherries, cq::kStreamUnitK)) return "";
+    return cq::stream_uses_cu(w_bits, in_features, out_features, num_cherries) ? "cq::stream_cu_kernel" : "cq::stream_kernel";
+}
+
 static int prepack_check(int w_bits, int K, int N, int C, int G, size_t stream_bytes_given) {
     if (w_bits != 3 && w_bits != 4) return CHERRYQ_E_BITS;
     if (K <= 0 || N <= 0 || C < 0 || C >= K || K % 8 || N % 8 || C % 8) return CHERRYQ_E_SHAPE;

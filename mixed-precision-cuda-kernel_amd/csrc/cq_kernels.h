@@ -147,6 +147,7 @@ hipError_t launch_stream_gated(int bits, const __half *vec, const __half *gate, 
                                int K, int N, int C, int accumulate, hipStream_t s);
 size_t stream_bytes(int bits, int K, int N, int C);
 bool stream_faster(int bits, int K, int N, int C);
+bool stream_uses_cu(int bits, int K, int N, int C);
 bool stream_supported(int bits, int B, int K, int N, int C, int G);
 hipError_t launch_stream(int bits, const __half *vec, const uint8_t *stream, __half *mul, int K, int N, int C,
                          int accumulate, hipStream_t s);

@@ -1389,6 +1389,9 @@ hipError_t launch_stream_group(int bits, const __half *vec, const __half *norm_w
     return launch_stream_group_old(bits, vec, norm_w, eps, members, count, K, C, accumulate, s);
 }
 
+// which of the two launch shapes cherryq_matvec_prepacked_f16 uses for a layer (for profiles and benchmarks)
+bool stream_uses_cu(int bits, int K, int N, int C) { return stream_cu_preferred(bits, K, C, &N, 1, false); }
+
 bool stream_gated_supported(int bits, int K, int N, int C) { return stream_cu_supported(bits, K, C, &N, 1); }
 
 hipError_t launch_stream_gated(int bits, const __half *vec, const __half *gate, const uint8_t *stream, __half *mul,

@@ -386,6 +386,13 @@ def prepack_recommended(w_bits, in_features, out_features, num_cherries, group_s
                                                  int(num_cherries), int(group_size)))
 
 
+def prepacked_kernel_name(w_bits, in_features, out_features, num_cherries) -> str:
+    """The kernel matvec_prepacked_cherryq launches for a one-row call on this layer, as a profiler names it."""
+    _lib.cherryq_matvec_prepacked_kernel_name.restype = ctypes.c_char_p
+    return _lib.cherryq_matvec_prepacked_kernel_name(int(w_bits), int(in_features), int(out_features),
+                                                     int(num_cherries)).decode()
+
+
 def prepack_cherryq(w_bits, qweight, cherry_weight, cherry_indices, scaling_factors, in_features, group_size):
     """The packed buffers of one layer rearranged, once, into the weight stream the batch-1 matvec
     of this GPU reads fastest (16 output columns' whole input range contiguous, codes placed
