@@ -1562,7 +1562,9 @@ hipError_t launch_stream_rows(int bits, const __half *vec, const uint8_t *stream
     // teams of 8 wavefronts, 4 units each for rows of up to 32 units and 8 beyond; two teams per
     // workgroup when every compute unit gets at least two tiles
     const bool l4 = geo.ng <= 32;
-    const int teams = geo.ntiles >= 2 * kStreamCus && rows_lds_bytes(B, geo, 16, false) <= 160 * 1024 ? 2 : 1;
+    // (two teams of 8 units per wavefront do not fit the 128 registers of a 1024-thread workgroup: they
+    // spilled, and a kernel with scratch memory also launches several microseconds slower)
+    const int teams = l4 && geo.ntiles >= 2 * kStreamCus && rows_lds_bytes(B, geo, 16, false) <= 160 * 1024 ? 2 : 1;
     // compaction inside the workgroup for a few rows (measured on 4096 -> 11008: 2 rows 10.4 us against
     // 11.6 with the compaction launch, 4 rows 11.4 against 11.8, 8 rows 13.7 against 12.8)
     const bool stage = B <= 4 && (K % 8 == 0) && rows_lds_bytes(B, geo, 8 * teams, true) <= 160 * 1024;
@@ -1591,7 +1593,6 @@ hipError_t launch_stream_rows(int bits, const __half *vec, const uint8_t *stream
     do {                                                                                                             \
         if (l4 && teams == 2) CQ_ROWS_GO(BITS_, 8, 4, 2);                                                            \
         if (l4) CQ_ROWS_GO(BITS_, 8, 4, 1);                                                                          \
-        if (teams == 2) CQ_ROWS_GO(BITS_, 8, 8, 2);                                                                  \
         CQ_ROWS_GO(BITS_, 8, 8, 1);                                                                                  \
     } while (0)
     if (bits == 4) CQ_ROWS(4);

@@ -73,13 +73,16 @@ struct CuJob {
     const __half *x;
     const uint8_t *stream;  // the layer's stream (header, then tile records)
     __half *mul;
-    const __half *norm_w;
+    const __half *norm_w;   // kCuNorm: the norm weight; kCuGate: the gate vector
     float eps;
     int K, C, N;
     int G, bid;             // workgroups that share the layer, this one's index among them
     int accumulate, P;      // P: tiles the launch's busiest team walks
-    const uint8_t *stream2; // PAIR: the second layer's stream
+    const uint8_t *stream2, *stream3;  // MEM > 1: the second and third layer's stream
+    __half *mul2, *mul3;               // ... and output
 };
+
+constexpr int kCuSeparate = 0, kCuSiluPair = 1;  // epilogues: every layer's result | fp16(fp16(silu(layer 0)) * layer 1)
 
 // S staging wavefronts (wavefronts 0 .. S-1, NB blocks of 512 compacted positions each), then
 // TEAMS teams of W computing wavefronts; computing wavefront c of a team takes the units c, c + W,
@@ -87,11 +90,13 @@ struct CuJob {
 // PRO: what the staging wavefronts do to the row on its way into LDS -- kCuPlain nothing,
 // kCuNorm the RMSNorm norm_w * fp16(x * rsqrt(mean(x^2) + eps)), kCuGate the gated-MLP activation
 // fp16(fp16(silu(gate)) * x) with the gate vector passed in the norm_w slot.
-// PAIR: the teams work in pairs on the same tile index of TWO layers of the same shape that read the
-// same row (gate_proj / up_proj): even teams on job.stream, odd teams on job.stream2, each layer's
-// compaction staged by half of the staging wavefronts (the layers keep different cherry channels);
-// the epilogue stores fp16(fp16(silu(gate)) * up) of the two rounded results instead of the results.
-template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, int PRO, bool WALK, bool PAIR = false>
+// MEM > 1: MEM layers of the same shape that read the same row share a workgroup (2: gate_proj /
+// up_proj, 3: q / k / v of equal widths): team t works on layer t % MEM, on the same tile index as
+// the other teams of its slot t / MEM, so the tiles of all layers spread evenly over the compute
+// units; each layer's compaction is staged by S / MEM of the staging wavefronts (the layers keep
+// different cherry channels).  EPI: kCuSeparate stores every layer's result, kCuSiluPair (MEM 2)
+// fp16(fp16(silu(layer 0)) * layer 1) of the two rounded results instead.
+template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, int PRO, bool WALK, int MEM = 1, int EPI = kCuSeparate>
 __device__ __forceinline__ void stream_cu_body(const CuJob &job) {
     constexpr int NC = W * TEAMS;  // computing wavefronts
     constexpr int NT = 64 * (NC + S);
@@ -99,8 +104,8 @@ __device__ __forceinline__ void stream_cu_body(const CuJob &job) {
     constexpr float kGrid = BITS == 4 ? -7.5f : -3.5f;
     constexpr int XS = NB + 1;  // 16-byte loads per lane that cover a staging wavefront's raw slice
     static_assert(D0 <= D && D <= L && L % D == 0 && L % 4 == 0, "ring slots are fixed per unit across tiles");
-    static_assert(!PAIR || (TEAMS % 2 == 0 && S % 2 == 0 && PRO != kCuGate), "pairs of teams, half of the staging wavefronts per layer");
-    constexpr int MEM = PAIR ? 2 : 1;      // layers a workgroup stages the row for
+    static_assert(MEM >= 1 && MEM <= 3 && TEAMS % MEM == 0 && S % MEM == 0 && (MEM == 1 || PRO != kCuGate), "teams and staging wavefronts per layer");
+    static_assert(EPI == kCuSeparate || MEM == 2, "");
     constexpr int SM = S / MEM;            // staging wavefronts per layer
     constexpr int TSLOTS = TEAMS / MEM;    // tiles a workgroup works on at a time
     extern __shared__ __align__(16) unsigned char smem[];
@@ -108,6 +113,12 @@ __device__ __forceinline__ void stream_cu_body(const CuJob &job) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kq = lane >> 4, nn = lane & 15;
     const int K = job.K, C = job.C, N = job.N, G = job.G, bid = job.bid;
+    // the layers' streams, pinned in scalar registers so that picking one by a wavefront's layer
+    // stays a scalar select (left alone the compiler builds a table in scratch memory and indexes
+    // it: a kernel with scratch launches microseconds slower and starts with a memory round trip)
+    const uint8_t *st0 = job.stream, *st1 = MEM > 1 ? job.stream2 : job.stream, *st2 = MEM > 2 ? job.stream3 : job.stream;
+    if constexpr (MEM > 1) asm volatile("" : "+s"(st0), "+s"(st1), "+s"(st2));
+    auto stream_of = [&](int m) -> const uint8_t * { return MEM > 2 && m == 2 ? st2 : MEM > 1 && m == 1 ? st1 : st0; };
     // the record geometry of stream_geo(), from the shape (scalar arithmetic: cheaper than
     // kernel arguments that would not fit the preloaded ones)
     const int ng = (K - C + kStreamUnitK - 1) / kStreamUnitK;
@@ -128,11 +139,11 @@ __device__ __forceinline__ void stream_cu_body(const CuJob &job) {
     if (wave < S) {
         // ---- staging wavefront: its slice of the row, its blocks' gather table; gather; unit sums
         __builtin_amdgcn_s_setprio(3);
-        const int mem = PAIR ? wave / SM : 0, ws = wave - mem * SM;   // the layer it stages for, its index among that layer's
+        const int mem = MEM > 1 ? wave / SM : 0, ws = wave - mem * SM;   // the layer it stages for, its index among that layer's
         const int b0 = ws * NB, b1 = min(nblk, b0 + NB);
         const bool active = b0 < nblk, last = active && b1 == nblk;
         const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)job.x, 0, K * 2, kSFlags);
-        const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc((void *)(PAIR && mem ? job.stream2 : job.stream), 0,
+        const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc((void *)stream_of(mem), 0,
                                                                             (int)hdr_bytes, kSFlags);
         unsigned short *xs_m = s_xs + mem * Knp512;
         float *xsum_m = s_xsum + mem * 4 * nblk;
@@ -229,8 +240,8 @@ __device__ __forceinline__ void stream_cu_body(const CuJob &job) {
         // ---- computing wavefront
         const int cwv = wave - S;
         const int team = cwv / W, cls = cwv % W;
-        const int mem = PAIR ? team & 1 : 0, slot = PAIR ? team >> 1 : team;   // the team's layer, its tile slot
-        const uint8_t *__restrict__ stream = PAIR && mem ? job.stream2 : job.stream;
+        const int mem = MEM > 1 ? team % MEM : 0, slot = MEM > 1 ? team / MEM : team;   // the team's layer, its tile slot
+        const uint8_t *__restrict__ stream = stream_of(mem);
         const unsigned short *xs_m = s_xs + mem * Knp512;
         const float *xsum_m = s_xsum + mem * 4 * nblk;
         const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(
@@ -354,26 +365,31 @@ __device__ __forceinline__ void stream_cu_body(const CuJob &job) {
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     const int P = WALK ? job.P : 1;
-    __half *__restrict__ mul = job.mul;
-    for (int o = tid; o < 16 * P * TSLOTS; o += NT) {
-        const int jt = o >> 4, j = jt / TSLOTS, slot = jt - j * TSLOTS;
-        const int tile = bid + G * (slot + TSLOTS * j), n = tile * 16 + (o & 15);
+    constexpr int OUTS = EPI == kCuSiluPair ? TSLOTS : TEAMS;   // 16-column pieces of output per walk step
+    __half *mu0 = job.mul, *mu1 = MEM > 1 ? job.mul2 : job.mul, *mu2 = MEM > 2 ? job.mul3 : job.mul;
+    if constexpr (MEM > 1) asm volatile("" : "+s"(mu0), "+s"(mu1), "+s"(mu2));
+    for (int o = tid; o < 16 * P * OUTS; o += NT) {
+        const int jt = o >> 4, j = jt / OUTS, t = jt - j * OUTS, col = o & 15;
+        const int slot = EPI == kCuSiluPair ? t : t / MEM, mem = EPI == kCuSiluPair ? 0 : t - slot * MEM;
+        const int tile = bid + G * (slot + TSLOTS * j), n = tile * 16 + col;
         if (tile < ntiles && n < N) {
-            if constexpr (PAIR) {
+            const float *red = s_red + (j * NC + (slot * MEM + mem) * W) * 16 + col;
+            if constexpr (EPI == kCuSiluPair) {
                 float g = 0.f, u = 0.f;
 #pragma unroll
                 for (int c = 0; c < W; c++) {
-                    g += s_red[(j * NC + (2 * slot) * W + c) * 16 + (o & 15)];
-                    u += s_red[(j * NC + (2 * slot + 1) * W + c) * 16 + (o & 15)];
+                    g += red[c * 16];
+                    u += red[(W + c) * 16];
                 }
                 // the two projections' results as they would be stored, then the activation of silu_mul_kernel
                 const float g16 = __half2float(__float2half_rn(g)), u16 = __half2float(__float2half_rn(u));
                 const float a = __half2float(__float2half_rn(g16 / (1.f + __expf(-g16))));
-                mul[n] = __float2half_rn(a * u16);
+                mu0[n] = __float2half_rn(a * u16);
             } else {
                 float v = 0.f;
 #pragma unroll
-                for (int c = 0; c < W; c++) v += s_red[(j * NC + slot * W + c) * 16 + (o & 15)];
+                for (int c = 0; c < W; c++) v += red[c * 16];
+                __half *__restrict__ mul = MEM > 2 && mem == 2 ? mu2 : MEM > 1 && mem == 1 ? mu1 : mu0;  // (per-lane select: vector registers)
                 if (job.accumulate) v += __half2float(mul[n]);
                 mul[n] = __float2half_rn(v);
             }
@@ -392,7 +408,7 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_kernel(const _
                                                                           const uint8_t *__restrict__ stream,
                                                                           __half *__restrict__ mul, int K, int C, int N,
                                                                           int wgs, int accumulate, int P) {
-    const CuJob job = {x, stream, mul, nullptr, 0.f, K, C, N, wgs, (int)blockIdx.x, accumulate, P, nullptr};
+    const CuJob job = {x, stream, mul, nullptr, 0.f, K, C, N, wgs, (int)blockIdx.x, accumulate, P, nullptr, nullptr, nullptr, nullptr};
     stream_cu_body<BITS, W, L, TEAMS, S, NB, D0, D, kCuPlain, WALK>(job);
 }
 
@@ -432,20 +448,28 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_group_kernel(
     job.bid = bid - (m2 ? b2 : m1 ? b1 : 0);
     job.accumulate = (int)(n2p >> 31);
     job.P = (int)((n2p >> 16) & 0x7fffu);
-    job.stream2 = nullptr;
+    job.stream2 = job.stream3 = nullptr;
+    job.mul2 = job.mul3 = nullptr;
     stream_cu_body<BITS, W, L, TEAMS, S, NB, D0, D, PRO, WALK>(job);
 }
 
-// gate_proj and up_proj of a gated MLP in one launch, storing the activation
-// fp16(fp16(silu(gate)) * up) that the down projection reads (llama/modeling_llama_quant.py:251)
-// instead of the two results: 14 dwords, all preloaded.
-template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, int PRO, bool WALK>
-__global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_pair_kernel(
-    const __half *__restrict__ x, const __half *__restrict__ norm_w, const uint8_t *__restrict__ stream_gate,
-    const uint8_t *__restrict__ stream_up, __half *__restrict__ act, uint32_t kc, int N, uint32_t wgs_p, float eps) {
-    const CuJob job = {x, stream_gate, act, norm_w, eps, (int)(kc & 0xffffu), (int)(kc >> 16), N, (int)(wgs_p & 0xffffu),
-                       (int)blockIdx.x, 0, (int)(wgs_p >> 16), stream_up};
-    stream_cu_body<BITS, W, L, TEAMS, S, NB, D0, D, PRO, WALK, true>(job);
+// MEM = 2 or 3 layers of the SAME shape that read the same row, every workgroup working on the same
+// columns of all of them.  EPI = kCuSiluPair (MEM 2): gate_proj and up_proj of a gated MLP, storing
+// the activation fp16(fp16(silu(gate)) * up) that the down projection reads
+// (llama/modeling_llama_quant.py:251) into mul[0] instead of the two results.  EPI = kCuSeparate
+// with MEM 3 was measured for q / k / v and not kept.  Leading 14 dwords: x, norm_w, three streams, K | C << 16, N,
+// workgroups | P << 16, eps; the outputs behind them.
+struct CuMultiTail {
+    __half *mul[kStreamMaxGroup];
+};
+template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, int PRO, bool WALK, int MEM, int EPI>
+__global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_multi_kernel(
+    const __half *__restrict__ x, const __half *__restrict__ norm_w, const uint8_t *__restrict__ stream0,
+    const uint8_t *__restrict__ stream1, const uint8_t *__restrict__ stream2, uint32_t kc, int N, uint32_t wgs_p, float eps,
+    CuMultiTail tail) {
+    const CuJob job = {x, stream0, tail.mul[0], norm_w, eps, (int)(kc & 0xffffu), (int)(kc >> 16), N, (int)(wgs_p & 0xffffu),
+                       (int)blockIdx.x, 0, (int)(wgs_p >> 16), stream1, stream2, tail.mul[1], tail.mul[2]};
+    stream_cu_body<BITS, W, L, TEAMS, S, NB, D0, D, PRO, WALK, MEM, EPI>(job);
 }
 
 // ---- launch geometries --------------------------------------------------------------------------
@@ -645,11 +669,15 @@ hipError_t launch_stream_cu(int bits, const __half *vec, const __half *norm_w, f
 }
 
 
-// ---- gate_proj + up_proj -> fp16(fp16(silu(gate)) * up) in one launch ----------------------------
-// Pairs of teams on the same tile of the two layers.  Up to 32 units per column: three pairs of
+// ---- several layers of one shape in every workgroup -----------------------------------------------
+// gate_proj + up_proj -> fp16(fp16(silu(gate)) * up).  Up to 32 units per column: three pairs of
 // two-wavefront teams (16 units per wavefront) and 2 + 2 staging wavefronts of four blocks, i.e. the
 // three tiles per compute unit of the 4096 -> 11008 launch with both layers' tile t in one
 // workgroup; up to 64 units: one pair of four-wavefront teams and 4 + 4 staging wavefronts.
+// (Measured and not kept: q / k / v of equal widths the same way, three teams of three wavefronts
+// and 2 + 2 + 2 staging wavefronts, one tile of each layer per compute unit instead of consecutive
+// ranges of 85 / 85 / 86 workgroups: 8.25 us behind the RMSNorm against 7.24, 7.00 against 7.08
+// without -- the later barrier costs what the even spread gains.)
 static constexpr CuCfg kCuPairCfgs[] = {
     {2, 16, 6, 4, 4, 3, 8},
     {4, 16, 2, 8, 4, 3, 8},
@@ -669,16 +697,18 @@ bool stream_pair_supported(int bits, int K, int N, int C) {
     return cu_lds_bytes(geo, c, sp.walk, 2) <= 160 * 1024;
 }
 
-template <int BITS, int I, int PRO, bool WALK>
-static hipError_t launch_pair_cfg(const __half *vec, const __half *norm_w, float eps, const uint8_t *sg, const uint8_t *su,
-                                  __half *act, const StreamGeo &geo, const CuSplit &sp, hipStream_t s) {
-    constexpr CuCfg c = kCuPairCfgs[I];
-    auto kern = stream_cu_pair_kernel<BITS, c.W, c.L, c.TEAMS, c.S, c.NB, c.D0, c.D, PRO, WALK>;
+template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, int PRO, bool WALK, int MEM, int EPI>
+static hipError_t launch_multi_cfg(const __half *vec, const __half *norm_w, float eps, const uint8_t *const *streams,
+                                   __half *const *muls, const StreamGeo &geo, const CuSplit &sp, hipStream_t s) {
+    constexpr CuCfg c = {W, L, TEAMS, S, NB, D0, D};
+    auto kern = stream_cu_multi_kernel<BITS, W, L, TEAMS, S, NB, D0, D, PRO, WALK, MEM, EPI>;
     static bool raised[kCuMaxDevices] = {};
     if (hipError_t e = cu_raise_lds(kern, raised)) return e;
-    const size_t lds = cu_lds_bytes(geo, c, sp.walk, 2);
-    hipLaunchKernelGGL(kern, dim3(sp.total), dim3(64 * (c.W * c.TEAMS + c.S)), lds, s, vec, norm_w, sg, su, act,
-                       (uint32_t)geo.K | ((uint32_t)geo.C << 16), geo.N, (uint32_t)sp.wgs[0] | ((uint32_t)sp.walk << 16), eps);
+    const size_t lds = cu_lds_bytes(geo, c, sp.walk, MEM);
+    CuMultiTail tail = {{muls[0], muls[1], muls[MEM > 2 ? 2 : 1]}};
+    hipLaunchKernelGGL(kern, dim3(sp.total), dim3(64 * (W * TEAMS + S)), lds, s, vec, norm_w, streams[0], streams[1],
+                       streams[MEM > 2 ? 2 : 1], (uint32_t)geo.K | ((uint32_t)geo.C << 16), geo.N,
+                       (uint32_t)sp.wgs[0] | ((uint32_t)sp.walk << 16), eps, tail);
     return hipGetLastError();
 }
 
@@ -693,13 +723,18 @@ hipError_t launch_stream_pair(int bits, const __half *vec, const __half *norm_w,
     const CuSplit sp = cu_split(tiles, 1, kCuPairCfgs[idx].TEAMS / 2);
     if (sp.walk > kCuMaxWalk) return hipErrorInvalidValue;
     const bool walk = sp.walk > 1;
-#define CQ_PAIR_GO(BITS_, I_)                                                                                        \
-    do {                                                                                                             \
-        if (norm_w)                                                                                                  \
-            return walk ? launch_pair_cfg<BITS_, I_, kCuNorm, true>(vec, norm_w, eps, stream_gate, stream_up, act, geo, sp, s)   \
-                        : launch_pair_cfg<BITS_, I_, kCuNorm, false>(vec, norm_w, eps, stream_gate, stream_up, act, geo, sp, s); \
-        return walk ? launch_pair_cfg<BITS_, I_, kCuPlain, true>(vec, nullptr, 0.f, stream_gate, stream_up, act, geo, sp, s)     \
-                    : launch_pair_cfg<BITS_, I_, kCuPlain, false>(vec, nullptr, 0.f, stream_gate, stream_up, act, geo, sp, s);   \
+    const uint8_t *streams[2] = {stream_gate, stream_up};
+    __half *muls[2] = {act, act};
+#define CQ_MULTI(BITS_, C_, PRO_, WALK_, MEM_, EPI_) \
+    launch_multi_cfg<BITS_, C_.W, C_.L, C_.TEAMS, C_.S, C_.NB, C_.D0, C_.D, PRO_, WALK_, MEM_, EPI_>
+#define CQ_PAIR_GO(BITS_, I_)                                                                                            \
+    do {                                                                                                                 \
+        constexpr CuCfg c = kCuPairCfgs[I_];                                                                             \
+        if (norm_w)                                                                                                      \
+            return walk ? CQ_MULTI(BITS_, c, kCuNorm, true, 2, kCuSiluPair)(vec, norm_w, eps, streams, muls, geo, sp, s)  \
+                        : CQ_MULTI(BITS_, c, kCuNorm, false, 2, kCuSiluPair)(vec, norm_w, eps, streams, muls, geo, sp, s); \
+        return walk ? CQ_MULTI(BITS_, c, kCuPlain, true, 2, kCuSiluPair)(vec, nullptr, 0.f, streams, muls, geo, sp, s)   \
+                    : CQ_MULTI(BITS_, c, kCuPlain, false, 2, kCuSiluPair)(vec, nullptr, 0.f, streams, muls, geo, sp, s);  \
     } while (0)
     if (bits == 4) {
         if (idx == 0) CQ_PAIR_GO(4, 0);
@@ -709,5 +744,7 @@ hipError_t launch_stream_pair(int bits, const __half *vec, const __half *norm_w,
     CQ_PAIR_GO(3, 1);
 #undef CQ_PAIR_GO
 }
+
+#undef CQ_MULTI
 
 }  // namespace cq
