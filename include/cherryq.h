@@ -313,6 +313,18 @@ int cherryq_decode_matvec_gated_prepacked_f16(int w_bits, const void *vec, const
                                               int num_cherries, int accumulate, void *hip_stream);
 
 /*
+ * The output projection of the attention block over a repacked layer, reading the partial results
+ * of cherryq_decode_rope_attention_split_f16 (slices must be cherryq_decode_attention_projection_slices();
+ * in_features = n_heads * 128): mul (+)= act W^T with act the combined heads' results, formed with
+ * the arithmetic of cherryq_decode_attention_combine_f16 while the row is staged.  One launch, no
+ * workspace.  partial 16-byte, max_sum 8-byte aligned.
+ */
+int cherryq_decode_matvec_attention_prepacked_supported(int w_bits, int in_features, int out_features, int num_cherries);
+int cherryq_decode_matvec_attention_prepacked_f16(int w_bits, const void *partial, const float *max_sum, int slices,
+                                                  const void *stream, size_t stream_bytes, void *mul, int in_features,
+                                                  int out_features, int num_cherries, int accumulate, void *hip_stream);
+
+/*
  * One batch-1 launch over 1..4 packed layers that read the SAME activation vector and share
  * in_features, num_cherries, group_size and w_bits: q/k/v_proj (llama/modeling_llama_quant.py
  * :346-348 of the reference) or gate/up_proj (:251).  Arithmetic per layer is that of
@@ -363,6 +375,30 @@ int cherryq_decode_attention_f16(const void *q, const void *k_cache, const void 
 int cherryq_decode_rope_attention_f16(const void *q, const void *k, const void *v, void *k_cache, void *v_cache,
                                       void *out, const int *position, int n_heads, int n_kv_heads,
                                       int head_dim, int max_len, float theta, void *stream);
+/*
+ * The same with a head's positions dealt to `slices` workgroups (1 .. cherryq_decode_attention_max_slices(),
+ * which is 8): slice s takes the blocks of 64 positions s, s + slices, s + 2 slices, ..., is a softmax
+ * of its own, and stores its result into
+ * partial[s][n_heads * head_dim] (fp16) and the maximum of its scores and the sum of their
+ * exponentials into max_sum[s][n_heads][2] (fp32).  A head's result is sum_s c_s partial[s] with
+ * c_s = exp(max_s - max) sum_s / sum_t exp(max_t - max) sum_t; cherryq_decode_attention_combine_f16
+ * forms it (fp16), and cherryq_decode_matvec_attention_prepacked_f16 is an output projection
+ * (llama/modeling_llama_quant.py:404, o_proj) over a repacked layer that forms it while it stages its
+ * input (for cherryq_decode_attention_projection_slices() = 4 slices), so that split attention +
+ * projection stay two launches.  With slices = 1, and up to position 63 with any number, the combined
+ * result equals cherryq_decode_rope_attention_f16's bit for bit; otherwise it differs by the
+ * roundings of the partial results (about 4e-4 relative).  One workgroup per head reads the
+ * head's whole cache through one compute unit: 50 us per layer at 4000 positions of 32 heads
+ * against 22 us with 4 slices (18 against 11 at 1000 positions; at 256 positions the two are within
+ * 0.5 us and the combining costs more than that).  No counterpart in the reference.
+ */
+int cherryq_decode_attention_max_slices(void);
+int cherryq_decode_attention_projection_slices(void);
+int cherryq_decode_rope_attention_split_f16(const void *q, const void *k, const void *v, void *k_cache, void *v_cache,
+                                            void *partial, float *max_sum, int slices, const int *position, int n_heads,
+                                            int n_kv_heads, int head_dim, int max_len, float theta, void *stream);
+int cherryq_decode_attention_combine_f16(const void *partial, const float *max_sum, int slices, void *out, int n_heads,
+                                         int head_dim, void *stream);
 /*
  * Unquantised fp16 head of the decode step: logits (vocab fp16) = act W^T with lm_head W (vocab,
  * hidden_size) row-major as the reference holds it (llama/modeling_llama_quant.py:1132), fp32

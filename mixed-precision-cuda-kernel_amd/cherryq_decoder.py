@@ -39,6 +39,20 @@ _lib.cherryq_decode_silu_mul_f16.argtypes = [_vp, _vp, _vp, _int, _vp]
 _lib.cherryq_decode_argmax_embed_f16.argtypes = [_vp, _int, _vp, _int, _vp, _vp, _vp, _int, _vp, _vp]
 _lib.cherryq_decode_argmax_embed_f16.restype = _int
 _lib.cherryq_decode_rope_attention_f16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _f, _vp]
+_lib.cherryq_decode_attention_max_slices.argtypes = []
+_lib.cherryq_decode_attention_max_slices.restype = _int
+_lib.cherryq_decode_attention_projection_slices.argtypes = []
+_lib.cherryq_decode_attention_projection_slices.restype = _int
+_lib.cherryq_decode_rope_attention_split_f16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _int, _int,
+                                                         _int, _f, _vp]
+_lib.cherryq_decode_rope_attention_split_f16.restype = _int
+_lib.cherryq_decode_attention_combine_f16.argtypes = [_vp, _vp, _int, _vp, _int, _int, _vp]
+_lib.cherryq_decode_attention_combine_f16.restype = _int
+_lib.cherryq_decode_matvec_attention_prepacked_supported.argtypes = [_int, _int, _int, _int]
+_lib.cherryq_decode_matvec_attention_prepacked_supported.restype = _int
+_lib.cherryq_decode_matvec_attention_prepacked_f16.argtypes = [_int, _vp, _vp, _int, _vp, ctypes.c_size_t, _vp, _int, _int,
+                                                               _int, _int, _vp]
+_lib.cherryq_decode_matvec_attention_prepacked_f16.restype = _int
 _lib.cherryq_decode_head_supported.argtypes = [_int, _int]
 _lib.cherryq_decode_head_supported.restype = _int
 _lib.cherryq_decode_head_f16.argtypes = [_vp, _vp, _f, _vp, _vp, _int, _int, _vp]
@@ -192,6 +206,65 @@ def matvec_gated_prepacked(mod, vec, vec_gate, out, accumulate=False):
                                                        1 if accumulate else 0, _stream()), "matvec_gated_prepacked")
 
 
+ATTN_SLICES = _lib.cherryq_decode_attention_projection_slices()   # what a repacked output projection combines
+
+
+def rope_attention_split(q, k, v, k_cache, v_cache, partial, max_sum, pos, n_heads, n_kv_heads, head_dim, max_len,
+                         theta, slices=ATTN_SLICES):
+    """Rotary embedding + cache write + attention for one token with every head's positions dealt
+    to `slices` workgroups: partial (slices, n_heads * head_dim) fp16 and max_sum (slices, n_heads, 2)
+    fp32 receive the slices' results (attention_combine / matvec_attention_prepacked read them)."""
+    for t, shape, dt in ((q, (1, n_heads * head_dim), torch.float16), (k, (1, n_kv_heads * head_dim), torch.float16),
+                         (v, (1, n_kv_heads * head_dim), torch.float16),
+                         (k_cache, (n_kv_heads, max_len, head_dim), torch.float16),
+                         (v_cache, (n_kv_heads, max_len, head_dim), torch.float16),
+                         (partial, (slices, n_heads * head_dim), torch.float16), (max_sum, (slices, n_heads, 2), torch.float32),
+                         (pos, (1,), torch.int32)):
+        if tuple(t.shape) != shape or t.dtype != dt or not t.is_cuda or not t.is_contiguous() or t.device != q.device:
+            raise RuntimeError("rope_attention_split: expected a contiguous %s tensor of shape %s on the GPU, got %s %s"
+                               % (dt, shape, t.dtype, tuple(t.shape)))
+    _ok(_lib.cherryq_decode_rope_attention_split_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), k_cache.data_ptr(),
+                                                     v_cache.data_ptr(), partial.data_ptr(), max_sum.data_ptr(), slices,
+                                                     pos.data_ptr(), n_heads, n_kv_heads, head_dim, max_len, theta,
+                                                     _stream()), "rope_attention_split")
+
+
+def attention_combine(partial, max_sum, out, head_dim=128):
+    """out (1, n_heads * head_dim) <- the heads' results from the slices' partial results."""
+    slices, n = partial.shape
+    n_heads = n // head_dim
+    for t, shape, dt in ((partial, (slices, n), torch.float16), (max_sum, (slices, n_heads, 2), torch.float32),
+                         (out, (1, n), torch.float16)):
+        if tuple(t.shape) != shape or t.dtype != dt or not t.is_cuda or not t.is_contiguous() or t.device != partial.device:
+            raise RuntimeError("attention_combine: expected a contiguous %s tensor of shape %s on the GPU" % (dt, shape))
+    _ok(_lib.cherryq_decode_attention_combine_f16(partial.data_ptr(), max_sum.data_ptr(), slices, out.data_ptr(), n_heads,
+                                                  head_dim, _stream()), "attention_combine")
+
+
+def matvec_attention_prepacked_supported(mod) -> bool:
+    return (getattr(mod, "_stream", None) is not None and
+            bool(_lib.cherryq_decode_matvec_attention_prepacked_supported(mod.w_bits, mod.in_features, mod.out_features,
+                                                                          mod.num_cherries)))
+
+
+def matvec_attention_prepacked(mod, partial, max_sum, out, accumulate=False):
+    """out (+)= heads @ W^T for a QuantLinear that holds a repacked weight stream (the output
+    projection), `heads` formed from rope_attention_split's partial results while the row is staged."""
+    st = getattr(mod, "_stream", None)
+    if st is None:
+        raise RuntimeError("matvec_attention_prepacked: the layer must have been prepack()ed")
+    k = mod.in_features
+    for t, shape, dt in ((partial, (ATTN_SLICES, k), torch.float16), (max_sum, (ATTN_SLICES, k // 128, 2), torch.float32),
+                         (out, (1, mod.out_features), torch.float16)):
+        if tuple(t.shape) != shape or t.dtype != dt or not t.is_cuda or not t.is_contiguous() or t.device != st.device:
+            raise RuntimeError("matvec_attention_prepacked: expected a contiguous %s tensor of shape %s on the layer's GPU"
+                               % (dt, shape))
+    _ok(_lib.cherryq_decode_matvec_attention_prepacked_f16(mod.w_bits, partial.data_ptr(), max_sum.data_ptr(), ATTN_SLICES,
+                                                           st.data_ptr(), st.numel(), out.data_ptr(), k, mod.out_features,
+                                                           mod.num_cherries, 1 if accumulate else 0, _stream()),
+        "matvec_attention_prepacked")
+
+
 def _group(mods, vec, outs, accumulate=False, norm_weight=None, eps=1e-6):
     """The grouped launch over whichever layout the layers hold: the repacked streams when every
     layer of the group has one, the checkpoint layout otherwise."""
@@ -294,12 +367,19 @@ class CherryLlamaDecoder(nn.Module):
         self.gate = torch.zeros(1, cfg.intermediate_size, **f16)
         self.up = torch.zeros(1, cfg.intermediate_size, **f16)
         self.act = torch.zeros(1, cfg.intermediate_size, **f16)
+        self.attn_part = torch.zeros(ATTN_SLICES, h, **f16)   # split attention: the slices' results ...
+        self.attn_ml = torch.zeros(ATTN_SLICES, cfg.num_attention_heads, 2, dtype=torch.float32, device=self.device_)  # ... and (maximum, sum)
         self.logits16 = torch.zeros(1, cfg.vocab_size, **f16)
         self.history = torch.zeros(ml, dtype=torch.int64, device=self.device_)  # history[p]: token predicted at position p
         self.lm_head_t = self.lm_head.t()
         self._graph = None
         self.fuse_norm = True
         self.fuse_head = True  # final RMSNorm + fp16 head as one launch of the library's own kernel
+        # Attention dealt to ATTN_SLICES workgroups per head, combined by a repacked o_proj's staging: None =
+        # for caches of 1024 positions and more.  (Measured per layer: 256-position cache 5.5 -> 5.0 us for
+        # the attention but 4.3 -> 6.5 us for the projection; 1000 of 4096 positions 18.1 -> 11.3 us, 4000
+        # positions 50 -> 22 us for the attention.)
+        self.split_attn = None
         self.fuse_act = True   # gate / up as one launch that stores SiLU(gate) * up (layers repacked), plain down projection
         self.layer_trace = None
         self._side = [torch.cuda.Stream(device=self.device_) for _ in range(2)] if self.device_.type == "cuda" else []
@@ -411,11 +491,19 @@ class CherryLlamaDecoder(nn.Module):
             else:
                 self._norm(layer.input_layernorm)
                 _group(qkv, self.normed, [self.q, self.k, self.v])
-            _ok(_lib.cherryq_decode_rope_attention_f16(self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(),
-                                                       self.k_cache[li].data_ptr(), self.v_cache[li].data_ptr(),
-                                                       self.attn.data_ptr(), self.pos.data_ptr(), nh, nkv, hd, ml,
-                                                       cfg.rope_theta, _stream()), "rope_attention")
-            _group([layer.o_proj], self.attn, [self.hid], accumulate=True)
+            split = ml >= 1024 if self.split_attn is None else self.split_attn
+            if split and hd == 128 and matvec_attention_prepacked_supported(layer.o_proj):
+                # every head's positions on ATTN_SLICES compute units; o_proj combines the slices' results
+                # while it stages its row
+                rope_attention_split(self.q, self.k, self.v, self.k_cache[li], self.v_cache[li], self.attn_part,
+                                     self.attn_ml, self.pos, nh, nkv, hd, ml, cfg.rope_theta)
+                matvec_attention_prepacked(layer.o_proj, self.attn_part, self.attn_ml, self.hid, accumulate=True)
+            else:
+                _ok(_lib.cherryq_decode_rope_attention_f16(self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(),
+                                                           self.k_cache[li].data_ptr(), self.v_cache[li].data_ptr(),
+                                                           self.attn.data_ptr(), self.pos.data_ptr(), nh, nkv, hd, ml,
+                                                           cfg.rope_theta, _stream()), "rope_attention")
+                _group([layer.o_proj], self.attn, [self.hid], accumulate=True)
             down = layer.down_proj
             if self.fuse_act and getattr(down, "_stream", None) is not None and gate_up_prepacked_supported(*gu):
                 # gate / up in one launch that stores SiLU(gate) * up, then the plain down projection

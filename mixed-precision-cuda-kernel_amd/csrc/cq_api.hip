@@ -563,6 +563,28 @@ int cherryq_decode_matvec_gated_prepacked_f16(int w_bits, const void *vec, const
                                         out_features, num_cherries, accumulate, reinterpret_cast<hipStream_t>(hip_stream));
 }
 
+int cherryq_decode_matvec_attention_prepacked_supported(int w_bits, int in_features, int out_features, int num_cherries) {
+    if ((w_bits != 3 && w_bits != 4) || in_features <= 0 || out_features <= 0 || num_cherries < 0) return 0;
+    if (in_features % 8 || out_features % 8 || num_cherries % 8 || num_cherries >= in_features) return 0;
+    return cq::stream_attn_out_supported(w_bits, in_features, num_cherries, out_features) ? 1 : 0;
+}
+
+int cherryq_decode_matvec_attention_prepacked_f16(int w_bits, const void *partial, const float *max_sum, int slices,
+                                                  const void *stream, size_t stream_bytes, void *mul, int in_features,
+                                                  int out_features, int num_cherries, int accumulate, void *hip_stream) {
+    int rc = prepack_check(w_bits, in_features, out_features, num_cherries, cq::kStreamUnitK, stream_bytes);
+    if (rc) return rc;
+    if (!partial || !max_sum || !stream || !mul) return CHERRYQ_E_NULL;
+    if (slices != cq::attn_out_slices() || in_features % 128) return CHERRYQ_E_SHAPE;
+    if (!cq::aligned(stream, 256) || !cq::aligned(partial, 16) || !cq::aligned(max_sum, 8) || !cq::aligned(mul, 2))
+        return CHERRYQ_E_ALIGN;
+    if (!cq::stream_attn_out_supported(w_bits, in_features, num_cherries, out_features)) return CHERRYQ_E_UNSUPPORTED;
+    return (int)cq::launch_stream_attn_out(w_bits, reinterpret_cast<const __half *>(partial), max_sum,
+                                           reinterpret_cast<const uint8_t *>(stream), reinterpret_cast<__half *>(mul),
+                                           in_features, out_features, num_cherries, accumulate,
+                                           reinterpret_cast<hipStream_t>(hip_stream));
+}
+
 // ---- decode-step entry points (see include/cherryq.h) ------------------------------------------
 
 size_t cherryq_group_workspace_bytes(int n_layers, const int *out_features) {
@@ -679,6 +701,38 @@ int cherryq_decode_rope_attention_f16(const void *q, const void *k, const void *
         reinterpret_cast<__half *>(k_cache), reinterpret_cast<__half *>(v_cache), reinterpret_cast<__half *>(out),
         position, n_heads, n_kv_heads, max_len, theta, 1.0f / sqrtf((float)head_dim),
         reinterpret_cast<hipStream_t>(stream));
+}
+
+int cherryq_decode_attention_max_slices(void) { return cq::attn_max_slices(); }
+int cherryq_decode_attention_projection_slices(void) { return cq::attn_out_slices(); }
+
+int cherryq_decode_rope_attention_split_f16(const void *q, const void *k, const void *v, void *k_cache, void *v_cache,
+                                            void *partial, float *max_sum, int slices, const int *position, int n_heads,
+                                            int n_kv_heads, int head_dim, int max_len, float theta, void *stream) {
+    if (!q || !k || !v || !k_cache || !v_cache || !partial || !max_sum || !position) return CHERRYQ_E_NULL;
+    if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads || max_len <= 0 || max_len > cq::attn_max_len() ||
+        slices < 1 || slices > cq::attn_max_slices())
+        return CHERRYQ_E_SHAPE;
+    if (head_dim != 128) return CHERRYQ_E_UNSUPPORTED;
+    if (!cq::aligned(q, 16) || !cq::aligned(k, 16) || !cq::aligned(v, 16) || !cq::aligned(k_cache, 16) ||
+        !cq::aligned(v_cache, 16) || !cq::aligned(partial, 16) || !cq::aligned(max_sum, 8))
+        return CHERRYQ_E_ALIGN;
+    return (int)cq::launch_rope_attn_split(
+        reinterpret_cast<const __half *>(q), reinterpret_cast<const __half *>(k), reinterpret_cast<const __half *>(v),
+        reinterpret_cast<__half *>(k_cache), reinterpret_cast<__half *>(v_cache), reinterpret_cast<__half *>(partial),
+        max_sum, position, n_heads, n_kv_heads, max_len, slices, theta, 1.0f / sqrtf((float)head_dim),
+        reinterpret_cast<hipStream_t>(stream));
+}
+
+int cherryq_decode_attention_combine_f16(const void *partial, const float *max_sum, int slices, void *out, int n_heads,
+                                         int head_dim, void *stream) {
+    if (!partial || !max_sum || !out) return CHERRYQ_E_NULL;
+    if (n_heads <= 0 || slices < 1 || slices > cq::attn_max_slices()) return CHERRYQ_E_SHAPE;
+    if (head_dim != 128) return CHERRYQ_E_UNSUPPORTED;
+    if (!cq::aligned(partial, 2) || !cq::aligned(max_sum, 4) || !cq::aligned(out, 2)) return CHERRYQ_E_ALIGN;
+    return (int)cq::launch_attn_combine(reinterpret_cast<const __half *>(partial), max_sum,
+                                        reinterpret_cast<__half *>(out), n_heads, slices,
+                                        reinterpret_cast<hipStream_t>(stream));
 }
 
 int cherryq_decode_head_supported(int vocab, int hidden_size) { return cq::head_supported(vocab, hidden_size) ? 1 : 0; }

@@ -409,6 +409,240 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
     }
 }
 
+// rope_attn_decode_kernel with a head's positions dealt to `slices` workgroups (grid = n_heads *
+// slices; workgroup b works on head b % n_heads, slice b / n_heads = the blocks of 64 positions
+// slice, slice + slices, slice + 2 slices, ... so that the slices stay balanced at every position).
+// One workgroup per head requests the head's whole K and V (128 KB at 256 positions, 4 MB at 4096)
+// through ONE compute unit, which accepts about 32 KB at a time; with 32 heads only 32 of the 256
+// compute units pull data.  A slice is a softmax of its own: it stores
+// fp16(sum_j fp16(e_j / l) v_j) with e_j = exp(score_j - m), m and l its scores' maximum and sum of
+// e_j, and (m, l) as two floats; a slice without positions stores zeros and (-inf, 0).
+// attn_combine_weights() turns the (m, l) of a head's slices into the factors of the slices'
+// results; the reader of the partial results (the output projection while it stages its input, or
+// attn_combine_kernel) applies them.  With one slice the stored result is rope_attn_decode_kernel's,
+// bit for bit, and its factor is exactly 1.  The slice that owns the new position attends to it
+// from LDS and (first query head of a kv group) stores the rotated k and the v row into the caches.
+__global__ __launch_bounds__(1024) void rope_attn_split_kernel(
+    const __half *__restrict__ q, const __half *__restrict__ k, const __half *__restrict__ v,
+    __half *__restrict__ k_cache, __half *__restrict__ v_cache, __half *__restrict__ part, float *__restrict__ ml,
+    const int *__restrict__ pos_ptr, int n_heads, int n_kv_heads, int max_len, int slices, RopeBase base, float scale) {
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    __shared__ float s_score[kMaxAttnLen];   // indexed by 64 * (the slice's block number) + position % 64
+    __shared__ float s_red[32];
+    __shared__ float s_acc[16][128];
+    __shared__ __attribute__((aligned(16))) unsigned short s_qh[128], s_kh[128];  // rotated q, k as fp16
+    const int head = blockIdx.x % n_heads, slice = blockIdx.x / n_heads;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int row = t >> 4, l16 = t & 15;
+    const int rep = n_heads / n_kv_heads, kvh = head / rep;
+    const uint4 *kb = reinterpret_cast<const uint4 *>(k_cache + (size_t)kvh * max_len * 128);
+    const uint4 *vb = reinterpret_cast<const uint4 *>(v_cache + (size_t)kvh * max_len * 128);
+    auto position = [&](int lb) { return 64 * (slice + slices * lb) + row; };  // this thread's row of the slice's block lb
+    // A cache that four blocks per slice cover is requested whole before the position is known (one
+    // memory round trip in front of the arithmetic); of a longer one only the rows up to the
+    // position are read, after it has arrived (rows beyond it would be most of the traffic).
+    const bool early = max_len <= 256 * slices;
+    uint4 k_first[4], v_first[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const int j = position(u);
+        k_first[u] = early && j < max_len ? kb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
+        v_first[u] = early && j < max_len ? vb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
+    }
+    float x1 = 0.f, x2 = 0.f, inv_freq = 0.f;
+    __half v1 = __float2half(0.f), v2 = v1;
+    if (t < 128) {
+        const int i = t & 63;
+        const __half *src = t >= 64 ? k + (size_t)kvh * 128 : q + (size_t)head * 128;
+        x1 = __half2float(src[i]);
+        x2 = __half2float(src[i + 64]);
+        if (t >= 64) {
+            v1 = v[(size_t)kvh * 128 + i];
+            v2 = v[(size_t)kvh * 128 + i + 64];
+        }
+        inv_freq = rope_inv_freq(i, 128, base);
+    }
+    const int pos = *pos_ptr;
+    __half *pdst = part + ((size_t)slice * n_heads + head) * 128;
+    float *mdst = ml + ((size_t)slice * n_heads + head) * 2;
+    if ((unsigned)pos >= (unsigned)max_len) {  // outside the cache: nothing read or written, the output is NaN
+        if (t < 128) pdst[t] = __ushort_as_half((unsigned short)0x7e00);
+        if (t == 0) {
+            mdst[0] = 0.f;
+            mdst[1] = 1.f;
+        }
+        return;
+    }
+    const int used = pos / 64 + 1;  // blocks that hold positions 0 .. pos
+    if (slice >= used) {            // nothing to attend to in this slice
+        if (t < 128) pdst[t] = __float2half(0.f);
+        if (t == 0) {
+            mdst[0] = -INFINITY;
+            mdst[1] = 0.f;
+        }
+        return;
+    }
+    const bool has_new = (used - 1) % slices == slice;  // the new position lies in this slice's last block
+    const int nblk = (used - slice + slices - 1) / slices;
+    const int len = 64 * nblk - (has_new ? 63 - pos % 64 : 0);  // positions of this slice, the new one included
+    const int cached = len - (has_new ? 1 : 0);
+    if (!early) {
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int j = position(u);
+            k_first[u] = j < pos ? kb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
+            v_first[u] = j < pos ? vb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
+        }
+    }
+    if (t < 128) {
+        const int i = t & 63;
+        const bool is_k = t >= 64;
+        float sn, cs;
+        sincosf((float)pos * inv_freq, &sn, &cs);
+        const float c = __half2float(__float2half_rn(cs)), sr = __half2float(__float2half_rn(sn));
+        const float a1 = __half2float(__float2half_rn(x1 * c)), b1 = __half2float(__float2half_rn(-x2 * sr));
+        const float a2 = __half2float(__float2half_rn(x2 * c)), b2 = __half2float(__float2half_rn(x1 * sr));
+        const __half o1 = __float2half_rn(a1 + b1), o2 = __float2half_rn(a2 + b2);
+        unsigned short *dst = is_k ? s_kh : s_qh;
+        dst[i] = __half_as_ushort(o1);
+        dst[i + 64] = __half_as_ushort(o2);
+        if (is_k && has_new && head % rep == 0) {
+            __half *kd = k_cache + ((size_t)kvh * max_len + pos) * 128;
+            __half *vd = v_cache + ((size_t)kvh * max_len + pos) * 128;
+            kd[i] = o1;
+            kd[i + 64] = o2;
+            vd[i] = v1;
+            vd[i + 64] = v2;
+        }
+    }
+    __syncthreads();
+    const uint4 qv = *reinterpret_cast<const uint4 *>(&s_qh[8 * l16]);
+    auto dot8 = [&](const uint4 &kv) {
+        float d = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, kv.x), __builtin_bit_cast(half2_t, qv.x), 0.f, false);
+        d = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, kv.y), __builtin_bit_cast(half2_t, qv.y), d, false);
+        d = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, kv.z), __builtin_bit_cast(half2_t, qv.z), d, false);
+        d = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, kv.w), __builtin_bit_cast(half2_t, qv.w), d, false);
+        return row_sum(d);
+    };
+    float m = -INFINITY;
+    for (int lb0 = 0; 64 * lb0 < cached; lb0 += 4) {
+        uint4 kk[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int j = position(lb0 + u);
+            if (lb0 == 0)
+                kk[u] = k_first[u];
+            else
+                kk[u] = j < pos ? kb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const float sc = __half2float(__float2half_rn(dot8(kk[u]))) * scale;
+            if (position(lb0 + u) < pos) {
+                m = fmaxf(m, sc);
+                if (l16 == 0) s_score[64 * (lb0 + u) + row] = sc;
+            }
+        }
+    }
+    if (has_new && row == 0) {  // the new position, from LDS
+        const float sc = __half2float(__float2half_rn(dot8(*reinterpret_cast<const uint4 *>(&s_kh[8 * l16])))) * scale;
+        m = fmaxf(m, sc);
+        if (l16 == 0) s_score[len - 1] = sc;
+    }
+    m = wave_max_all(m);
+    if (lane == 0) s_red[wave] = m;
+    __syncthreads();
+    m = s_red[0];
+#pragma unroll
+    for (int w = 1; w < 16; w++) m = fmaxf(m, s_red[w]);
+    float sum = 0.f;
+    for (int j = t; j < len; j += 1024) {
+        const float e = __expf(s_score[j] - m);
+        s_score[j] = e;
+        sum += e;
+    }
+    sum = wave_sum_all(sum);
+    if (lane == 0) s_red[16 + wave] = sum;
+    __syncthreads();
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < 16; w++) tot += s_red[16 + w];
+    const float inv = 1.f / tot;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = 0.f;
+    for (int lb0 = 0; 64 * lb0 < cached; lb0 += 4) {
+        uint4 vv[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int j = position(lb0 + u);
+            if (lb0 == 0)
+                vv[u] = j < pos ? v_first[u] : make_uint4(0, 0, 0, 0);  // rows past the position may hold anything
+            else
+                vv[u] = j < pos ? vb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const float p = position(lb0 + u) < pos ? __half2float(__float2half_rn(s_score[64 * (lb0 + u) + row] * inv)) : 0.f;
+            float vf[8];
+            unpack8(vv[u], vf);
+#pragma unroll
+            for (int i = 0; i < 8; i++) acc[i] = fmaf(p, vf[i], acc[i]);
+        }
+    }
+    if (has_new && row == 0) {
+        const float p = __half2float(__float2half_rn(s_score[len - 1] * inv));
+        float vf[8];
+        unpack8(reinterpret_cast<const uint4 *>(v + (size_t)kvh * 128)[l16], vf);
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[i] = fmaf(p, vf[i], acc[i]);
+    }
+    {
+        float h4[4], q2[2];
+#pragma unroll
+        for (int i = 0; i < 4; i++) h4[i] = swap32_add(acc[i], acc[4 + i]);
+#pragma unroll
+        for (int i = 0; i < 2; i++) q2[i] = swap16_add(h4[i], h4[2 + i]);
+        const int d0 = 8 * l16 + 4 * (lane >> 5) + 2 * ((lane >> 4) & 1);
+        s_acc[wave][d0] = q2[0];
+        s_acc[wave][d0 + 1] = q2[1];
+    }
+    __syncthreads();
+    if (t < 128) {
+        float o = 0.f;
+#pragma unroll
+        for (int w = 0; w < 16; w++) o += s_acc[w][t];
+        pdst[t] = __float2half_rn(o);
+    }
+    if (t == 0) {
+        mdst[0] = m;
+        mdst[1] = tot;
+    }
+}
+
+// out[head][d] <- fp16(sum_s c_s * part[s][head][d]) with the factors of attn_combine_weights();
+// one thread per output element.  (The output projection over a weight stream applies the same
+// factors while it stages its input; this kernel serves every other reader.)
+__global__ __launch_bounds__(256) void attn_combine_kernel(const __half *__restrict__ part, const float *__restrict__ ml,
+                                                           __half *__restrict__ out, int n_heads, int slices) {
+    const int i = blockIdx.x * 256 + threadIdx.x, n = n_heads * 128;
+    if (i >= n) return;
+    const int head = i >> 7;
+    float mv[kAttnMaxSlices], lv[kAttnMaxSlices], c[kAttnMaxSlices];
+#pragma unroll
+    for (int s = 0; s < kAttnMaxSlices; s++) {
+        const bool on = s < slices;
+        mv[s] = on ? ml[((size_t)s * n_heads + head) * 2] : -INFINITY;
+        lv[s] = on ? ml[((size_t)s * n_heads + head) * 2 + 1] : 0.f;
+    }
+    attn_combine_weights(mv, lv, c);
+    float o = 0.f;
+#pragma unroll
+    for (int s = 0; s < kAttnMaxSlices; s++)
+        if (s < slices) o = fmaf(c[s], __half2float(part[(size_t)s * n + i]), o);
+    out[i] = __float2half_rn(o);
+}
+
 // out <- fp16(silu(gate)) * up
 __global__ __launch_bounds__(256) void silu_mul_kernel(const __half *__restrict__ gate, const __half *__restrict__ up,
                                                        __half *__restrict__ out, int n) {
@@ -627,6 +861,23 @@ hipError_t launch_rope_attn_decode(const __half *q, const __half *k, const __hal
                                    int max_len, float theta, float scale, hipStream_t stream) {
     hipLaunchKernelGGL(rope_attn_decode_kernel, dim3(n_heads), dim3(1024), 0, stream, q, k, v, k_cache, v_cache, out,
                        pos, n_heads, n_kv_heads, max_len, rope_base(theta), scale);
+    return hipGetLastError();
+}
+
+hipError_t launch_rope_attn_split(const __half *q, const __half *k, const __half *v, __half *k_cache, __half *v_cache,
+                                  __half *part, float *ml, const int *pos, int n_heads, int n_kv_heads, int max_len,
+                                  int slices, float theta, float scale, hipStream_t stream) {
+    // 60 KB of unused dynamic LDS on top of the 25 KB the kernel declares: more than half of a compute
+    // unit's, so that the workgroups spread one per compute unit instead of sharing one's memory pipeline
+    hipLaunchKernelGGL(rope_attn_split_kernel, dim3(n_heads * slices), dim3(1024), 60 * 1024, stream, q, k, v, k_cache, v_cache,
+                       part, ml, pos, n_heads, n_kv_heads, max_len, slices, rope_base(theta), scale);
+    return hipGetLastError();
+}
+
+hipError_t launch_attn_combine(const __half *part, const float *ml, __half *out, int n_heads, int slices,
+                               hipStream_t stream) {
+    hipLaunchKernelGGL(attn_combine_kernel, dim3(ceil_div(n_heads * 128, 256)), dim3(256), 0, stream, part, ml, out,
+                       n_heads, slices);
     return hipGetLastError();
 }
 

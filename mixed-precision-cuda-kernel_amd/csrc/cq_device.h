@@ -237,4 +237,25 @@ __device__ inline void splitk_finish(float (&vals)[MAXB][COLS], int B, int N, in
         }
 }
 
+// Attention over a head's positions dealt to several workgroups: slice s of a head leaves the
+// maximum m[s] of its scores, the sum l[s] of exp(score - m[s]) and its own softmax-weighted sum of
+// value rows; the head's result is sum_s c[s] * result[s] with c[s] = exp(m[s] - M) l[s] / sum of
+// the same over the slices, M the largest m.  An empty slice has l = 0 (and m = -inf): factor 0.
+// One slice alone gets exactly 1.
+constexpr int kAttnMaxSlices = 8;
+template <int NS>
+__device__ inline void attn_combine_weights(const float (&m)[NS], const float (&l)[NS], float (&c)[NS]) {
+    float M = m[0];
+#pragma unroll
+    for (int s = 1; s < NS; s++) M = fmaxf(M, m[s]);
+    float w[NS], L = 0.f;
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        w[s] = l[s] > 0.f ? __expf(m[s] - M) * l[s] : 0.f;
+        L += w[s];
+    }
+#pragma unroll
+    for (int s = 0; s < NS; s++) c[s] = L > 0.f ? w[s] / L : 0.f;
+}
+
 }  // namespace cq

@@ -136,7 +136,15 @@ hipError_t launch_stream_rows(int bits, const __half *vec, const uint8_t *stream
 // cq_stream_cu.hip: the same launch with one workgroup per compute unit (up to 64 units per column)
 bool stream_cu_supported(int bits, int K, int C, const int *Ns, int count);
 hipError_t launch_stream_cu(int bits, const __half *vec, const __half *norm_w, float eps, const __half *gate,
-                            const StreamMember *members, int count, int K, int C, int accumulate, hipStream_t s);
+                            const StreamMember *members, int count, int K, int C, int accumulate, hipStream_t s,
+                            const float *attn_ml = nullptr);
+// one repacked layer whose input row is formed from the partial results of launch_rope_attn_split
+// with attn_out_slices() slices (part [slices][K] fp16, ml [slices][K / 128][2] fp32): the output projection
+bool stream_attn_out_supported(int bits, int K, int C, int N);
+hipError_t launch_stream_attn_out(int bits, const __half *part, const float *ml, const uint8_t *stream, __half *mul,
+                                  int K, int N, int C, int accumulate, hipStream_t s);
+int attn_max_slices();
+int attn_out_slices();  // slices launch_stream_attn_out combines
 // gate_proj and up_proj (same shape, same row) in one launch that stores fp16(fp16(silu(gate)) * up)
 bool stream_pair_supported(int bits, int K, int N, int C);
 hipError_t launch_stream_pair(int bits, const __half *vec, const __half *norm_w, float eps, const uint8_t *stream_gate,
@@ -185,6 +193,14 @@ hipError_t launch_attn_decode(const __half *q, const __half *k_cache, const __ha
 hipError_t launch_rope_attn_decode(const __half *q, const __half *k, const __half *v, __half *k_cache,
                                    __half *v_cache, __half *out, const int *pos, int n_heads, int n_kv_heads,
                                    int max_len, float theta, float scale, hipStream_t stream);
+// Attention with a head's positions dealt to `slices` workgroups (1 .. kAttnMaxSlices): partial results
+// part[slices][n_heads * 128] fp16 and (maximum, sum) pairs ml[slices][n_heads][2] fp32; the combine
+// kernel (or the output projection's staging, launch_stream_attn_out) forms the heads' results.
+hipError_t launch_rope_attn_split(const __half *q, const __half *k, const __half *v, __half *k_cache, __half *v_cache,
+                                  __half *part, float *ml, const int *pos, int n_heads, int n_kv_heads, int max_len,
+                                  int slices, float theta, float scale, hipStream_t stream);
+hipError_t launch_attn_combine(const __half *part, const float *ml, __half *out, int n_heads, int slices,
+                               hipStream_t stream);
 hipError_t launch_argmax_embed(const __half *logits, int vocab, const __half *embed, int hidden, __half *hid,
                                long long *next_token, long long *history, int history_len, int *pos,
                                hipStream_t stream);

@@ -1400,6 +1400,15 @@ hipError_t launch_stream_gated(int bits, const __half *vec, const __half *gate, 
     return launch_stream_cu(bits, vec, nullptr, 0.f, gate, &m, 1, K, C, accumulate, s);
 }
 
+hipError_t launch_stream_attn_out(int bits, const __half *part, const float *ml, const uint8_t *stream, __half *mul,
+                                  int K, int N, int C, int accumulate, hipStream_t s) {
+    const StreamMember m = {stream, mul, N};
+    return launch_stream_cu(bits, part, nullptr, 0.f, nullptr, &m, 1, K, C, accumulate, s, ml);
+}
+
+int attn_max_slices() { return kAttnMaxSlices; }
+int attn_out_slices() { return 4; }  // kCuAttnSlices of cq_stream_cu.hip
+
 // the launch with one workgroup per tile (or per few tiles), several workgroups per compute unit
 hipError_t launch_stream_group_old(int bits, const __half *vec, const __half *norm_w, float eps,
                                    const StreamMember *members, int count, int K, int C, int accumulate, hipStream_t s) {

@@ -40,7 +40,8 @@ constexpr int kCuMaxWalk = 16;   // tiles one team takes at most
 constexpr int kCuCus = 256;      // compute units of an MI355X
 constexpr int kCuMaxDevices = 64;
 
-constexpr int kCuPlain = 0, kCuNorm = 1, kCuGate = 2;
+constexpr int kCuPlain = 0, kCuNorm = 1, kCuGate = 2, kCuAttn = 3;
+constexpr int kCuAttnSlices = 4;  // slices of a split attention that the kCuAttn prologue combines
 
 // fp16(silu(gate)) * up, rounded to fp16, on both halves of a pair (the rounding points of silu_mul_kernel)
 __device__ inline uint32_t cu_silu_mul_pair(uint32_t gate, uint32_t up) {
@@ -73,7 +74,7 @@ struct CuJob {
     const __half *x;
     const uint8_t *stream;  // the layer's stream (header, then tile records)
     __half *mul;
-    const __half *norm_w;   // kCuNorm: the norm weight; kCuGate: the gate vector
+    const __half *norm_w;   // kCuNorm: the norm weight; kCuGate: the gate vector; kCuAttn: the slices' (maximum, sum) pairs
     float eps;
     int K, C, N;
     int G, bid;             // workgroups that share the layer, this one's index among them
@@ -89,7 +90,11 @@ constexpr int kCuSeparate = 0, kCuSiluPair = 1;  // epilogues: every layer's res
 // ... (L at most) of every tile the team comes to.  WALK: some team has more than one tile.
 // PRO: what the staging wavefronts do to the row on its way into LDS -- kCuPlain nothing,
 // kCuNorm the RMSNorm norm_w * fp16(x * rsqrt(mean(x^2) + eps)), kCuGate the gated-MLP activation
-// fp16(fp16(silu(gate)) * x) with the gate vector passed in the norm_w slot.
+// fp16(fp16(silu(gate)) * x) with the gate vector passed in the norm_w slot, kCuAttn the row
+// formed from the partial results of an attention dealt to kCuAttnSlices workgroups per head
+// (rope_attn_split_kernel): x holds [slices][K] fp16 partial results, the norm_w slot
+// [slices][K / 128][2] floats, the row is fp16(sum_s c_s * partial_s) with attn_combine_weights()
+// (the arithmetic of attn_combine_kernel, for an output projection that reads the heads' results).
 // MEM > 1: MEM layers of the same shape that read the same row share a workgroup (2: gate_proj /
 // up_proj, 3: q / k / v of equal widths): team t works on layer t % MEM, on the same tile index as
 // the other teams of its slot t / MEM, so the tiles of all layers spread evenly over the compute
@@ -167,6 +172,49 @@ __device__ __forceinline__ void stream_cu_body(const CuJob &job) {
                 for (int j = 0; j < 4; j++) {
                     xr[i][j] = cu_silu_mul_pair(gr[i][j], xr[i][j]);
                     __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+        if constexpr (PRO == kCuAttn) {
+            su4 pr[kCuAttnSlices - 1][XS];
+            su2 mlr[kCuAttnSlices][XS];
+            const int heads = K >> 7;
+            const __amdgpu_buffer_rsrc_t rm = __builtin_amdgcn_make_buffer_rsrc((void *)job.norm_w, 0, kCuAttnSlices * heads * 8, kSFlags);
+#pragma unroll
+            for (int sl = 1; sl < kCuAttnSlices; sl++) {
+                const __amdgpu_buffer_rsrc_t rp = __builtin_amdgcn_make_buffer_rsrc((void *)(job.x + (size_t)sl * K), 0, K * 2, kSFlags);
+#pragma unroll
+                for (int i = 0; i < XS; i++)
+                    pr[sl - 1][i] = __builtin_amdgcn_raw_buffer_load_b128(rp, active ? (uint32_t)(b0 * 512 + i * 512 + lane * 8) * 2u : kSOob, 0, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < XS; i++) {
+                const int col = b0 * 512 + i * 512 + lane * 8;
+#pragma unroll
+                for (int sl = 0; sl < kCuAttnSlices; sl++)
+                    mlr[sl][i] = __builtin_amdgcn_raw_buffer_load_b64(rm, active && col < K ? (uint32_t)(sl * heads + (col >> 7)) * 8u : kSOob, 0, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < XS; i++) {
+                float mv[kCuAttnSlices], lv[kCuAttnSlices], cf[kCuAttnSlices];
+#pragma unroll
+                for (int sl = 0; sl < kCuAttnSlices; sl++) {
+                    mv[sl] = __uint_as_float(mlr[sl][i][0]);
+                    lv[sl] = __uint_as_float(mlr[sl][i][1]);
+                }
+                attn_combine_weights(mv, lv, cf);
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    uint32_t r = 0;
+#pragma unroll
+                    for (int hf = 0; hf < 2; hf++) {
+                        float o = fmaf(cf[0], __half2float(__ushort_as_half((unsigned short)(xr[i][j] >> (16 * hf)))), 0.f);
+#pragma unroll
+                        for (int sl = 1; sl < kCuAttnSlices; sl++)
+                            o = fmaf(cf[sl], __half2float(__ushort_as_half((unsigned short)(pr[sl - 1][i][j] >> (16 * hf)))), o);
+                        r |= (uint32_t)__half_as_ushort(__float2half_rn(o)) << (16 * hf);
+                    }
+                    xr[i][j] = r;
                 }
             }
         }
@@ -504,6 +552,8 @@ static constexpr CuCfg kCuCfgs[] = {
 // code, so the table keeps L / D = 2 for deep columns and the parity tests run every entry in
 // both bit widths, with and without walking.
 
+constexpr int kCuAttnMaxCfg = 3;  // the attention-combining prologue exists for entries 0 .. 3 (output projections up to 64 units)
+
 static int cu_pick(int ng, int tiles_per_cu_ceil) {
     if (ng <= 32) return tiles_per_cu_ceil <= 1 ? 0 : tiles_per_cu_ceil == 2 ? 1 : 2;
     if (ng <= 64) return 3;
@@ -569,6 +619,14 @@ bool stream_cu_supported(int bits, int K, int C, const int *Ns, int count) {
     return cu_lds_bytes(geo, c, sp.walk) <= 160 * 1024;
 }
 
+// an output projection that forms its input row from split-attention partial results
+bool stream_attn_out_supported(int bits, int K, int C, int N) {
+    const int Ns[1] = {N};
+    if (K % 128 || !stream_cu_supported(bits, K, C, Ns, 1)) return false;
+    const StreamGeo geo = stream_geo(bits, K, N, C);
+    return cu_pick(geo.ng, ceil_div(geo.ntiles, kCuCus)) <= kCuAttnMaxCfg;
+}
+
 template <typename KERN>
 static hipError_t cu_raise_lds(KERN kern, bool *raised) {
     // per instantiation and device, once: the dynamic-LDS limit raised
@@ -623,8 +681,10 @@ static hipError_t launch_cu_cfg(const __half *vec, const __half *norm_w, float e
 // norm_w != nullptr fuses the RMSNorm of that row, gate != nullptr (one layer, no norm) the
 // gated-MLP activation fp16(fp16(silu(gate)) * vec).  The caller has asked stream_cu_supported().
 hipError_t launch_stream_cu(int bits, const __half *vec, const __half *norm_w, float eps, const __half *gate,
-                            const StreamMember *members, int count, int K, int C, int accumulate, hipStream_t s) {
+                            const StreamMember *members, int count, int K, int C, int accumulate, hipStream_t s,
+                            const float *attn_ml) {
     if (count < 1 || count > kStreamMaxGroup || (gate && (norm_w || count != 1))) return hipErrorInvalidValue;
+    if (attn_ml && (gate || norm_w || count != 1 || K % 128)) return hipErrorInvalidValue;
     int tiles[kStreamMaxGroup], all = 0;
     for (int i = 0; i < count; i++) {
         tiles[i] = ceil_div(members[i].N, kStreamTileCols);
@@ -638,8 +698,16 @@ hipError_t launch_stream_cu(int bits, const __half *vec, const __half *norm_w, f
     const CuSplit sp = cu_split(tiles, count, kCuCfgs[idx].TEAMS);
     if (sp.walk > kCuMaxWalk || sp.total > 1023) return hipErrorInvalidValue;
     const bool group = count > 1 || norm_w != nullptr || gate != nullptr, walk = sp.walk > 1;
+    const __half *ml_slot = reinterpret_cast<const __half *>(attn_ml);
 #define CQ_CU_GO(BITS_, I_)                                                                                               \
     do {                                                                                                                  \
+        if (attn_ml) {                                                                                                    \
+            if constexpr (I_ <= kCuAttnMaxCfg)                                                                            \
+                return walk ? launch_cu_cfg<BITS_, I_, kCuAttn, true, true>(vec, ml_slot, 0.f, members, count, geo, sp, accumulate, s)   \
+                            : launch_cu_cfg<BITS_, I_, kCuAttn, true, false>(vec, ml_slot, 0.f, members, count, geo, sp, accumulate, s); \
+            else                                                                                                          \
+                return hipErrorInvalidValue;                                                                              \
+        }                                                                                                                 \
         if (!group)                                                                                                       \
             return walk ? launch_cu_cfg<BITS_, I_, kCuPlain, false, true>(vec, nullptr, 0.f, members, count, geo, sp, accumulate, s)   \
                         : launch_cu_cfg<BITS_, I_, kCuPlain, false, false>(vec, nullptr, 0.f, members, count, geo, sp, accumulate, s); \
