@@ -143,7 +143,7 @@ def time_gpu(bits, k, n, group, steps, warmup, batch=1, use_graph=True, path="au
     c = copies[0]["cherry_indices"].numel()
     if path == "auto":
         path = "prepacked" if (quant_cuda.prepack_recommended(bits, k, n, c, group) and
-                               (batch == 1 or (4 <= batch <= 16 and quant_cuda.prepack_supported(bits, batch, k, n, c, group)))) \
+                               (batch == 1 or (batch <= 16 and quant_cuda.prepacked_rows_recommended(bits, batch, k, n, c, group)))) \
             else "reference"
     x = torch.from_numpy(np.random.default_rng(1).standard_normal((batch, k)).astype(np.float16)).cuda()
     out = torch.zeros(batch, n, dtype=torch.float16, device="cuda")

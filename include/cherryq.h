@@ -230,10 +230,9 @@ size_t cherryq_prepack_bytes(int w_bits, int in_features, int out_features, int 
 int cherryq_prepack_supported(int w_bits, int batch, int in_features, int out_features, int num_cherries,
                               int group_size);
 /* 1 where the matvec over the stream measured faster on MI355X than the one over the checkpoint
- * layout (today: layers of at most 4096 non-cherry input channels, and deeper ones whose 16-column
- * tiles spread evenly over the 256 compute units -- every LLaMA-7B and -70B projection, not the
- * 13B ones), 0 elsewhere or if unsupported: what a loader asks before spending the extra copy of
- * the weights. */
+ * layout (today: every shape the launch with one workgroup per compute unit takes -- every
+ * LLaMA-7B, -13B and -70B projection among them; within 3 % at worst on the shapes measured), 0
+ * elsewhere or if unsupported: what a loader asks before spending the extra copy of the weights. */
 int cherryq_prepack_recommended(int w_bits, int in_features, int out_features, int num_cherries, int group_size);
 /* The kernel cherryq_matvec_prepacked_f16 launches for a layer, as it appears in a profiler's
  * kernel trace (without template arguments): "cq::stream_cu_kernel" (one workgroup per compute

@@ -426,11 +426,11 @@ class CherryLlamaDecoder(nn.Module):
         self._graph = None
 
     def prepack(self, only_recommended=True):
-        """Repack, once, every linear whose shape the library recommends it for (those of at most
-        4096 quantised input channels on MI355X: q / k / v / o / gate / up of a 7B model) into the
-        weight stream the batch-1 kernel reads fastest; the token step then uses the stream kernels
-        for them.  The checkpoint-layout buffers stay (the batched prompt pass reads them).
-        Returns the number of layers repacked."""
+        """Repack, once, every linear whose shape the library recommends it for (on MI355X: all
+        seven projections of the LLaMA-7B, -13B and -70B shapes) into the weight stream the batch-1
+        kernel reads fastest; the token step then uses the stream kernels for them.  The
+        checkpoint-layout buffers stay (the batched prompt pass reads them).  Returns the number of
+        layers repacked."""
         n = 0
         for layer in self.layers:
             for m in layer.children():

@@ -18,9 +18,10 @@
 //     operand: a field masked in place at bit p <= 8 of a 16-bit half IS the fp16 subnormal
 //     code * 2^(p-24).  4-bit: fields at bit 0 and 4 of each half directly, the other two after
 //     one shift by 8 (5 VALU instructions per 8 codes, no v_perm).  3-bit: fields at bit 0, 3, 6
-//     directly, two more after one shift by 9, and the 6 left-over bits of the three dwords form
-//     the last two codes (23 instructions per 32 codes) -- here the values truly straddle dwords.
-//   * v_mfma_f32_16x16x32_f16 (and 16x16x16 for the 3-bit remainders) multiplies: B = the lane's
+//     directly, two more after one shift by 9 (and, for the last four positions, by 3 more), and
+//     the 6 left-over bits of the three dwords form the last two codes (25 instructions per 32
+//     codes) -- here the values truly straddle dwords.
+//   * v_mfma_f32_16x16x32_f16 multiplies (4 steps per unit at either width): B = the lane's
 //     masked fields, A = the activations of the same positions from LDS, and the MFMA's K
 //     dimension runs across the four lane groups, so the reduction over a unit's 128 positions
 //     costs nothing.  Fields of different bit positions go to different accumulators (scaled by
@@ -697,19 +698,17 @@ __device__ inline sf4_t unit_dot_rows(const su4 w, const unsigned short *xa) {
         const sh8_t a0 = *reinterpret_cast<const sh8_t *>(xa);
         const sh8_t a2 = *reinterpret_cast<const sh8_t *>(xa + 8);
         const sh8_t a4 = *reinterpret_cast<const sh8_t *>(xa + 16);
-        const sh4_t a1 = *reinterpret_cast<const sh4_t *>(xa + 24);
-        const sh4_t a3 = *reinterpret_cast<const sh4_t *>(xa + 28);
+        const sh8_t a1 = *reinterpret_cast<const sh8_t *>(xa + 24);
         const uint32_t z = (y[0] & 0x00400040u) | ((y[1] & 0x00400040u) << 1) | ((y[2] & 0x00400040u) << 2);
         const su4 b0 = {w[0] & 0x00070007u, w[1] & 0x00070007u, w[2] & 0x00070007u, y[0] & 0x00070007u};
         const su4 b2 = {w[0] & 0x00380038u, w[1] & 0x00380038u, w[2] & 0x00380038u, y[0] & 0x00380038u};
         const su4 b4 = {w[0] & 0x01c001c0u, w[1] & 0x01c001c0u, w[2] & 0x01c001c0u, z};
-        const su2 b1 = {y[1] & 0x00070007u, y[2] & 0x00070007u};
-        const su2 b3 = {y[1] & 0x00380038u, y[2] & 0x00380038u};
+        // positions 24..27 sit at bit 0, 28..31 at bit 3: moved to bit 0 so that one 16x16x32 step takes all eight
+        const su4 b1 = {y[1] & 0x00070007u, y[2] & 0x00070007u, (y[1] >> 3) & 0x00070007u, (y[2] >> 3) & 0x00070007u};
         sf4_t d0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, as_h8(b0), zero4, 0, 0, 0);
-        sf4_t d3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, as_h8(b2), zero4, 0, 0, 0);
+        const sf4_t d3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, as_h8(b2), zero4, 0, 0, 0);
         const sf4_t d6 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a4, as_h8(b4), zero4, 0, 0, 0);
-        d0 = __builtin_amdgcn_mfma_f32_16x16x16f16(a1, as_h4(b1), d0, 0, 0, 0);
-        d3 = __builtin_amdgcn_mfma_f32_16x16x16f16(a3, as_h4(b3), d3, 0, 0, 0);
+        d0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, as_h8(b1), d0, 0, 0, 0);
         return d0 * 16777216.0f + d3 * 2097152.0f + d6 * 262144.0f;
     }
 }
@@ -1006,14 +1005,12 @@ __device__ inline sf4_t unit_dot_regs(const WB w, const su4 (&a)[4]) {
         const su4 b0 = {w[0] & 0x00070007u, w[1] & 0x00070007u, w[2] & 0x00070007u, y[0] & 0x00070007u};
         const su4 b2 = {w[0] & 0x00380038u, w[1] & 0x00380038u, w[2] & 0x00380038u, y[0] & 0x00380038u};
         const su4 b4 = {w[0] & 0x01c001c0u, w[1] & 0x01c001c0u, w[2] & 0x01c001c0u, z};
-        const su2 b1 = {y[1] & 0x00070007u, y[2] & 0x00070007u};
-        const su2 b3 = {y[1] & 0x00380038u, y[2] & 0x00380038u};
-        const su2 a1 = {a[3][0], a[3][1]}, a3 = {a[3][2], a[3][3]};  // positions 24..27 and 28..31
+        // positions 24..27 sit at bit 0, 28..31 at bit 3: moved to bit 0 so that one 16x16x32 step takes all eight
+        const su4 b1 = {y[1] & 0x00070007u, y[2] & 0x00070007u, (y[1] >> 3) & 0x00070007u, (y[2] >> 3) & 0x00070007u};
         sf4_t d0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(a[0]), as_h8(b0), zero4, 0, 0, 0);
-        sf4_t d3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(a[1]), as_h8(b2), zero4, 0, 0, 0);
+        const sf4_t d3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(a[1]), as_h8(b2), zero4, 0, 0, 0);
         const sf4_t d6 = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(a[2]), as_h8(b4), zero4, 0, 0, 0);
-        d0 = __builtin_amdgcn_mfma_f32_16x16x16f16(as_h4(a1), as_h4(b1), d0, 0, 0, 0);
-        d3 = __builtin_amdgcn_mfma_f32_16x16x16f16(as_h4(a3), as_h4(b3), d3, 0, 0, 0);
+        d0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(a[3]), as_h8(b1), d0, 0, 0, 0);
         return d0 * 16777216.0f + d3 * 2097152.0f + d6 * 262144.0f;
     }
 }
@@ -1037,7 +1034,17 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
     const int team = wave / W, cls = wave % W;
     const int kq = lane >> 4, nn = lane & 15;
     const int C = geo.C, ng = geo.ng, N = geo.N;
-    // ---- the wavefront's activations: operands of its units, the cherry operands; unit sums to LDS
+    // ---- requests, in the order their data is needed: the small shared operands (cherry
+    // activations, unit sums: they go through LDS and gate the barrier), the wavefront's own A
+    // operands, then the first R tiles' weights -- all queued BEFORE the barrier, so that the weight
+    // stream is under way while the workgroup still waits for its activations
+    const bool cherry_wave = cls == W - 1;
+    __shared__ su4 s_acr[4 * 64];  // the cherry operands (read once per tile by each team's last wavefront)
+    su4 acr_v = {0u, 0u, 0u, 0u};
+    if (tid < 4 * 64) acr_v = xcf[tid];
+    float xs_v[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) xs_v[j] = tid + 512 * j < 16 * ng ? xsum_g[tid + 512 * j] : 0.f;
     su4 areg[L][4];
 #pragma unroll
     for (int i = 0; i < L; i++) {
@@ -1046,11 +1053,7 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
         for (int m = 0; m < 4; m++)
             areg[i][m] = u < ng ? xf[((size_t)u * 4 + m) * 64 + lane] : (su4){0u, 0u, 0u, 0u};
     }
-    const bool cherry_wave = cls == W - 1;
-    __shared__ su4 s_acr[4 * 64];  // the cherry operands (read once per tile by each team's last wavefront)
-    if (tid < 4 * 64) s_acr[tid] = xcf[tid];
-    for (int c = tid; c < 16 * ng; c += 512) s_xsum[c] = xsum_g[c];
-    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
 
     const int ntl = (N + kStreamTileCols - 1) / kStreamTileCols;
     const int G = gridDim.x, stride = G * TEAMS;
@@ -1095,6 +1098,12 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
 #pragma unroll
         for (int i = 0; i < L; i++) wbuf[s][i] = load_unit(i, tb, valid[s]);
     }
+    __builtin_amdgcn_sched_barrier(0);
+    if (tid < 4 * 64) s_acr[tid] = acr_v;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        if (tid + 512 * j < 16 * ng) s_xsum[tid + 512 * j] = xs_v[j];
+    __syncthreads();
     const float *xsrow = s_xsum + (4 * kq) * ng;
     // the loop count is the same for every wavefront of the workgroup (barriers inside): as long as
     // the workgroup's first team, which has the lowest tile, has one in slot 0
@@ -1192,25 +1201,18 @@ static int stream_pick(const StreamGeo &geo) {
 
 constexpr int kStreamCus = 256;  // compute units of an MI355X
 
-// How unevenly a launch with one workgroup per compute unit spreads `tiles` whole tiles over the
-// chip: tiles of the busiest compute unit over the average (1 = even).
-static double cu_imbalance(int tiles) {
-    const int cus = tiles < kStreamCus ? tiles : kStreamCus;
-    return tiles > 0 ? (double)ceil_div(tiles, cus) * cus / tiles : 1.0;
-}
-
 // Where the batch-1 matvec over the stream measured faster than the one over the checkpoint layout
-// (us per launch, weights from HBM; checkpoint layout / stream, the stream on whichever of its two
-// launch shapes is faster): 4096 -> 4096 4.95 / 3.58 (3-bit 4.79 / 3.55), 4096 -> 11008 7.46 / 5.71
-// (6.79 / 5.15), 11008 -> 4096 7.04 / 5.91 (6.76 / 5.56), 8192 -> 8192 8.75 / 7.72, 8192 -> 1024
-// 4.55 / 4.24, 8192 -> 28672 22.8 / 20.5, 28672 -> 8192 23.5 / 22.3.  Not faster where whole tiles
-// spread unevenly over the 256 compute units and a column is too deep for several small workgroups
-// per compute unit: 5120 -> 5120 (3-bit, 320 tiles) 5.68 / 5.95, 5120 -> 13824 (864 tiles) 9.05 /
-// 10.1, 13824 -> 5120 (320 tiles) 8.93 / 10.3.
+// (us per launch, weights from HBM; checkpoint layout / stream): 4096 -> 4096 4.95 / 3.58 (3-bit
+// 4.79 / 3.55), 4096 -> 11008 7.46 / 5.71 (6.79 / 5.15), 11008 -> 4096 7.04 / 5.91 (6.76 / 5.56),
+// 8192 -> 8192 8.75 / 7.72, 8192 -> 1024 4.55 / 4.24, 8192 -> 28672 22.8 / 20.5, 28672 -> 8192 23.5 /
+// 22.3, 5120 -> 5120 5.87 / 4.52 (5.57 / 4.65), 5120 -> 13824 10.15 / 8.2 (8.80 / 8.1), 13824 -> 5120
+// 10.24 / 8.9 (8.81 / 8.5), 12288 -> 4096 7.90 / 6.5 (6.93 / 6.1), 8192 -> 5120 7.03 / 6.88 (6.50 / 6.71),
+// 6144 -> 6144 6.75 / 6.40 (6.45 / 6.42), 5120 -> 20480 (3-bit) 12.3 / 10.2: everywhere the launch with
+// one workgroup per compute unit takes the layer, within 3 % at worst.
 bool stream_faster(int bits, int K, int N, int C) {
     const StreamGeo g = stream_geo(bits, K, N, C);
     if (g.ng <= 32) return true;
-    return cu_imbalance(g.ntiles) <= 1.15;
+    return stream_cu_supported(bits, K, C, &N, 1);
 }
 
 // the launch shapes of this file (several workgroups per compute unit) take the layer
@@ -1363,13 +1365,13 @@ static bool stream_cu_preferred(int bits, int K, int C, const int *Ns, int count
     }();
     if (forced >= 0) return forced == 1;
     // Measured (us, older shape / one workgroup per compute unit; 4-bit unless noted): single layers
-    // as listed at stream_faster(); RMSNorm + q/k/v (3 x 4096 -> 4096) 7.35 / 7.24 (3-bit 7.10 / 6.76),
-    // RMSNorm + gate/up (2 x 4096 -> 11008) 10.95 / 9.76 (3-bit 9.69 / 8.96), q/k/v without norm 7.02 /
-    // 7.08, RMSNorm + 8192 -> (8192, 1024, 1024) 11.5 / 10.6, RMSNorm + 2 x (8192 -> 28672) 40.2 / 38.9;
-    // between 33 and 64 units per column only where whole tiles spread evenly over the compute
-    // units (5120 -> 5120, 3-bit: 5.95 / 6.52; 5120 -> 13824: 10.1 / 10.6).
+    // 4096 -> 11008 6.35 / 5.68, 4096 -> 4096 3.99 / 3.58, 8192 -> 8192 8.9 / 7.7, 5120 -> 5120 6.0 / 4.5,
+    // 5120 -> 13824 10.7 / 8.2, 13824 -> 5120 11.6 / 8.9; RMSNorm + q/k/v (3 x 4096 -> 4096) 7.35 / 7.24
+    // (3-bit 7.10 / 6.76), RMSNorm + gate/up (2 x 4096 -> 11008) 10.95 / 9.76 (3-bit 9.69 / 8.96), q/k/v
+    // without norm 7.02 / 7.08, RMSNorm + 8192 -> (8192, 1024, 1024) 11.5 / 10.6, RMSNorm + 2 x (8192 ->
+    // 28672) 40.2 / 38.9: the newer shape wherever it takes the launch.
     (void)norm;
-    if (geo.ng > 32 && geo.ng <= 64) return cu_imbalance(tiles) <= 1.15;
+    (void)geo;
     return true;
 }
 

@@ -538,7 +538,19 @@ static constexpr CuCfg kCuCfgs[] = {
     {11, 8, 1, 5, 5, 3, 4},  // 4: up to 88 units (11008 input channels)
     {8, 16, 1, 8, 4, 4, 8},  // 5: up to 128 units
     {8, 28, 1, 8, 7, 4, 7},  // 6: up to 224 units (28672 input channels)
+    {5, 8, 2, 6, 2, 3, 4},   // 7: up to 40 units (5120 input channels), two teams
+    {4, 28, 2, 8, 4, 4, 7},  // 8: up to 112 units (13824 input channels), two tiles per compute unit
+    {12, 8, 1, 4, 6, 3, 4},  // 9: up to 96 units, one team of 12 (12288 -> 4096: 6.5 / 6.1 us against 7.2 / 6.7 for entry 5)
 };
+// The LLaMA-13B widths (entries 7 and 8), us per launch, 4-bit / 3-bit, against the checkpoint layout's
+// 5.87 / 5.57 (5120 -> 5120), 10.15 / 8.80 (5120 -> 13824), 10.24 / 8.81 (13824 -> 5120):
+// 5120 -> 5120 (320 tiles): entry 7 4.52 / 4.65 (entry 3: 6.0 / 6.0; three teams of 4 x 12 units 5.4 / 5.9;
+//   four teams of 3 x 16 units 6.2 / 6.5);
+// 5120 -> 13824 (864 tiles): entry 7, teams walking two tiles, 8.2-8.3 / 8.1-8.2 (four teams of 3 x 16
+//   units without walking 8.0 / 8.2 with a ring of 4, 9.0 / 8.7 with a ring of 8; 4 x 12 units x 3 teams
+//   8.8 / 8.3; 2 x 20 units x 6 teams 8.6-8.8 / 8.8);
+// 13824 -> 5120 (320 tiles of 108 units): entry 8 9.2 / 8.95 (entry 5, walking: 10.3; 6 x 20 units x 2
+//   teams with 4 staging wavefronts 9.6 / 9.4; 7 x 16 units and 2 staging wavefronts of 14 blocks 11.7 / 11.6).
 // Deep columns (entries 4 to 6) are the same kernel with more units per wavefront and more
 // blocks per staging wavefront; the barrier then opens later (staging 22 blocks takes 1.3 us
 // instead of 0.5), which the D0 units requested in front of it cover.  Measured: 11008 -> 4096
@@ -546,18 +558,20 @@ static constexpr CuCfg kCuCfgs[] = {
 // wavefronts 6.01 / 5.59); 28672 -> 8192 23.5 -> 22.0; 13824 -> 5120 (3-bit, 320 tiles on 256
 // compute units: a quarter of them walk two tiles) 10.2 against 8.93, so that shape stays on the
 // checkpoint layout.
-// NOT used: 3-bit instantiations that walk tiles with a ring of D = 4 and more than 8 units per
-// wavefront (L = 12 or 16) gave wrong sums on the GPU (every output off by hundreds; D = 2, 3, 6,
-// 8, 12, 16 and every 4-bit instantiation are right); the cause was not found in the generated
-// code, so the table keeps L / D = 2 for deep columns and the parity tests run every entry in
-// both bit widths, with and without walking.
+// (While a 3-bit unit still ended in two 16x16x16 MFMAs chained onto 16x16x32 results, tile-walking
+// 3-bit instantiations with more than 8 units per wavefront and a short ring -- L = 12 or 16 with
+// D = 4, L = 20 with D = 2, 4 or 5 -- returned wrong sums; unit_dot() explains.  The parity tests run
+// every entry in both bit widths, with and without walking.)
 
 constexpr int kCuAttnMaxCfg = 3;  // the attention-combining prologue exists for entries 0 .. 3 (output projections up to 64 units)
 
 static int cu_pick(int ng, int tiles_per_cu_ceil) {
     if (ng <= 32) return tiles_per_cu_ceil <= 1 ? 0 : tiles_per_cu_ceil == 2 ? 1 : 2;
+    if (ng <= 40) return 7;
     if (ng <= 64) return 3;
     if (ng <= 88) return 4;
+    if (ng <= 96) return 9;
+    if (ng <= 112 && tiles_per_cu_ceil == 2) return 8;
     if (ng <= 128) return 5;
     if (ng <= 224) return 6;
     return -1;
@@ -728,7 +742,10 @@ hipError_t launch_stream_cu(int bits, const __half *vec, const __half *norm_w, f
         case 3: CQ_CU_GO(BITS_, 3);  \
         case 4: CQ_CU_GO(BITS_, 4);  \
         case 5: CQ_CU_GO(BITS_, 5);  \
-        default: CQ_CU_GO(BITS_, 6); \
+        case 6: CQ_CU_GO(BITS_, 6);  \
+        case 7: CQ_CU_GO(BITS_, 7);  \
+        case 8: CQ_CU_GO(BITS_, 8);  \
+        default: CQ_CU_GO(BITS_, 9); \
     }
     if (bits == 4) CQ_CU_BITS(4)
     CQ_CU_BITS(3)

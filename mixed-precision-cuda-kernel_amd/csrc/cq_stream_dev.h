@@ -51,23 +51,26 @@ __device__ inline float unit_dot(const su4 w, const unsigned short *xa) {
         dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(a3, as_h8(b3), dh, 0, 0, 0);
         return dl[0] * 16777216.0f + dh[0] * 1048576.0f;
     } else {
+        // Every step is a 16x16x32 MFMA.  (The last 8 positions were two 16x16x16 steps once, chained
+        // onto the 16x16x32 results through their accumulators: kernels whose schedule packed
+        // those chains tightly -- tile-walking ones with more than 8 units per wavefront and a short
+        // ring -- then returned sums that were off by hundreds and changed from run to run, while a
+        // scheduling barrier around each unit, or this form, made them right.  The shift that
+        // brings positions 28..31 to bit 0 costs two instructions and no MFMA time.)
         const su3 y = {w[0] >> 9, w[1] >> 9, w[2] >> 9};
         const sh8_t a0 = *reinterpret_cast<const sh8_t *>(xa);        // positions 0..7: fields at bit 0
         const sh8_t a2 = *reinterpret_cast<const sh8_t *>(xa + 8);    // 8..15: bit 3
         const sh8_t a4 = *reinterpret_cast<const sh8_t *>(xa + 16);   // 16..23: bit 6
-        const sh4_t a1 = *reinterpret_cast<const sh4_t *>(xa + 24);   // 24..27: bit 0
-        const sh4_t a3 = *reinterpret_cast<const sh4_t *>(xa + 28);   // 28..31: bit 3
+        const sh8_t a1 = *reinterpret_cast<const sh8_t *>(xa + 24);   // 24..27: bit 0, 28..31: bit 3 (moved to bit 0 below)
         const uint32_t z = (y[0] & 0x00400040u) | ((y[1] & 0x00400040u) << 1) | ((y[2] & 0x00400040u) << 2);
         const su4 b0 = {w[0] & 0x00070007u, w[1] & 0x00070007u, w[2] & 0x00070007u, y[0] & 0x00070007u};
         const su4 b2 = {w[0] & 0x00380038u, w[1] & 0x00380038u, w[2] & 0x00380038u, y[0] & 0x00380038u};
         const su4 b4 = {w[0] & 0x01c001c0u, w[1] & 0x01c001c0u, w[2] & 0x01c001c0u, z};
-        const su2 b1 = {y[1] & 0x00070007u, y[2] & 0x00070007u};
-        const su2 b3 = {y[1] & 0x00380038u, y[2] & 0x00380038u};
+        const su4 b1 = {y[1] & 0x00070007u, y[2] & 0x00070007u, (y[1] >> 3) & 0x00070007u, (y[2] >> 3) & 0x00070007u};
         sf4_t d0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, as_h8(b0), zero4, 0, 0, 0);
-        sf4_t d3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, as_h8(b2), zero4, 0, 0, 0);
+        const sf4_t d3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, as_h8(b2), zero4, 0, 0, 0);
         const sf4_t d6 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a4, as_h8(b4), zero4, 0, 0, 0);
-        d0 = __builtin_amdgcn_mfma_f32_16x16x16f16(a1, as_h4(b1), d0, 0, 0, 0);
-        d3 = __builtin_amdgcn_mfma_f32_16x16x16f16(a3, as_h4(b3), d3, 0, 0, 0);
+        d0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, as_h8(b1), d0, 0, 0, 0);
         return d0[0] * 16777216.0f + d3[0] * 2097152.0f + d6[0] * 262144.0f;
     }
 }

@@ -257,12 +257,14 @@ class QuantLinear(nn.Module):
             x2 = x2.contiguous()
             stream = self._stream
             rows = x2.shape[0]
-            rows_min = 2 if self._released else self.stream_rows_min
-            # over the repacked stream: one row, and 4 to 16 rows (the matrix-core tile of the one-row
-            # kernel filled with real rows; 2 and 3 rows are faster on the checkpoint layout's kernel
-            # while that layout is still there)
-            if stream is not None and (rows == 1 or (rows_min <= rows <= 16 and quant_cuda.prepack_supported(
-                    self.w_bits, rows, self.in_features, self.out_features, self.num_cherries, self.group_size))):
+            # over the repacked stream: one row, and the small batches that measured faster there than on
+            # the checkpoint layout's kernels (the matrix-core tile of the one-row kernel filled with real
+            # rows: from 4 rows, from 8 on layers of more than 32 units); with the checkpoint buffers
+            # released, everything the stream kernels take
+            shape = (self.w_bits, rows, self.in_features, self.out_features, self.num_cherries, self.group_size)
+            if stream is not None and (rows == 1 or (2 <= rows <= 16 and (
+                    quant_cuda.prepack_supported(*shape) if self._released else
+                    rows >= self.stream_rows_min and quant_cuda.prepacked_rows_recommended(*shape)))):
                 out = torch.empty(rows, self.out_features, dtype=torch.float16, device=stream.device)
                 quant_cuda.matvec_prepacked_cherryq(self.w_bits, x2, stream, out, self.in_features, self.num_cherries)
             elif self._released:

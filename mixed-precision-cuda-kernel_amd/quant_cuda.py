@@ -386,6 +386,21 @@ def prepack_recommended(w_bits, in_features, out_features, num_cherries, group_s
                                                  int(num_cherries), int(group_size)))
 
 
+def prepacked_rows_recommended(w_bits, rows, in_features, out_features, num_cherries, group_size) -> bool:
+    """Whether `rows` activation rows run faster over a layer's repacked stream than over its
+    checkpoint buffers (for a caller that holds both).  One row: prepack_recommended().  Several:
+    from 4 rows on layers of up to 32 units of 128 input channels, from 8 rows on deeper ones
+    (measured on MI355X, checkpoint layout / stream in us: 4096 -> 11008 4-bit 2 rows 9.1 / 9.9, 4 rows
+    11.2 / 10.6, 8 rows 16.8 / 12.4; 5120 -> 5120 3-bit 4 rows 7.9 / 11.9, 8 rows 13.7 / 11.9;
+    5120 -> 13824 3-bit 4 rows 14.5 / 16.0, 8 rows 19.6 / 16.1)."""
+    if rows == 1:
+        return prepack_recommended(w_bits, in_features, out_features, num_cherries, group_size)
+    if rows < 1 or not prepack_supported(w_bits, rows, in_features, out_features, num_cherries, group_size):
+        return False
+    units = -(-(int(in_features) - int(num_cherries)) // 128)
+    return rows >= (4 if units <= 32 else 8)
+
+
 def prepacked_kernel_name(w_bits, in_features, out_features, num_cherries) -> str:
     """The kernel matvec_prepacked_cherryq launches for a one-row call on this layer, as a profiler names it."""
     _lib.cherryq_matvec_prepacked_kernel_name.restype = ctypes.c_char_p

@@ -61,7 +61,9 @@ SHAPES = [(4, 4096, 11008), (3, 4096, 11008), (4, 11008, 4096), (3, 11008, 4096)
           # and without tile walking: 257..512 tiles of up to 32 units, 64 / 88 / 128 / 224 units per column
           (4, 2048, 6000), (3, 2048, 6000), (3, 8192, 8192), (3, 8192, 264), (4, 11008, 4608), (3, 11008, 4608),
           (4, 13824, 5120), (4, 16384, 264), (3, 13824, 264), (4, 28672, 264), (3, 28672, 264), (4, 20480, 4352),
-          (3, 24576, 4104)]
+          (3, 24576, 4104),
+          # the geometries of the LLaMA-13B widths in the other bit width, and the 96-unit one (12 wavefronts on a tile)
+          (4, 5120, 5120), (4, 5120, 13824), (3, 12288, 4096), (4, 12288, 4104), (3, 13824, 8200)]
 
 
 @pytest.mark.parametrize("bits,k,n", SHAPES)
@@ -104,7 +106,8 @@ def test_prepacked_matvec_against_oracle(qc, bits, k, n):
 
 @pytest.mark.parametrize("bits,k,n", [(4, 4096, 4096), (3, 4096, 4096), (4, 11008, 512), (3, 11008, 512),
                                       (3, 5120, 520), (4, 8192, 264), (3, 13824, 264), (4, 28672, 264), (3, 28672, 264),
-                                      (3, 11008, 4608), (4, 16384, 4112)])
+                                      (3, 11008, 4608), (4, 16384, 4112), (4, 5120, 8200), (3, 5120, 8200),
+                                      (3, 12288, 264), (4, 13824, 8200), (3, 13824, 8200)])
 def test_prepacked_one_hot_reads_back_dequantised_weights(qc, bits, k, n):
     """x = e_j returns column j of the dense weight: decode, gather around the cherry channels and
     the per-unit grid offset are exact.  Positions probe every code slot of a lane's 32 and both
