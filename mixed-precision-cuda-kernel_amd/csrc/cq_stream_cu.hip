@@ -763,12 +763,16 @@ hipError_t launch_stream_cu(int bits, const __half *vec, const __half *norm_w, f
 // and 2 + 2 + 2 staging wavefronts, one tile of each layer per compute unit instead of consecutive
 // ranges of 85 / 85 / 86 workgroups: 8.25 us behind the RMSNorm against 7.24, 7.00 against 7.08
 // without -- the later barrier costs what the even spread gains.)
+// Measured, RMSNorm + gate/up + SiLU, 4-bit / 3-bit us (ring of 8 -> ring of 4): 2 x (4096 -> 11008) 10.67 /
+// 9.72 -> 10.25 / 9.23; 2 x (8192 -> 28672) 41.2 / 33.9 -> 39.3 / 32.6; 2 x (5120 -> 13824) on the 64-unit
+// entry 18.2 / 17.7, on the 48-unit entry 15.4 / 14.8 (two teams of 5 x 8 units: 15.8 / 14.8).
 static constexpr CuCfg kCuPairCfgs[] = {
-    {2, 16, 6, 4, 4, 3, 8},
-    {4, 16, 2, 8, 4, 3, 8},
+    {2, 16, 6, 4, 4, 3, 4},   // up to 32 units: three pairs of two-wavefront teams
+    {3, 16, 4, 4, 6, 2, 4},   // up to 48 units: two pairs of three-wavefront teams
+    {4, 16, 2, 8, 4, 2, 4},   // up to 64 units: one pair of four-wavefront teams
 };
 
-static int cu_pair_pick(int ng) { return ng <= 32 ? 0 : ng <= 64 ? 1 : -1; }
+static int cu_pair_pick(int ng) { return ng <= 32 ? 0 : ng <= 48 ? 1 : ng <= 64 ? 2 : -1; }
 
 bool stream_pair_supported(int bits, int K, int N, int C) {
     if ((bits != 3 && bits != 4) || K > 0xffff || C > 128 || N % 8) return false;
@@ -776,6 +780,7 @@ bool stream_pair_supported(int bits, int K, int N, int C) {
     const int idx = cu_pair_pick(geo.ng);
     if (idx < 0) return false;
     const CuCfg &c = kCuPairCfgs[idx];
+    if (geo.ng > c.W * c.L || geo.ng * kStreamUnitK > (c.S / 2) * c.NB * 512) return false;
     const int tiles[1] = {geo.ntiles};
     const CuSplit sp = cu_split(tiles, 1, c.TEAMS / 2);
     if (sp.walk > kCuMaxWalk || sp.total > 0xffff) return false;
@@ -823,10 +828,12 @@ hipError_t launch_stream_pair(int bits, const __half *vec, const __half *norm_w,
     } while (0)
     if (bits == 4) {
         if (idx == 0) CQ_PAIR_GO(4, 0);
-        CQ_PAIR_GO(4, 1);
+        if (idx == 1) CQ_PAIR_GO(4, 1);
+        CQ_PAIR_GO(4, 2);
     }
     if (idx == 0) CQ_PAIR_GO(3, 0);
-    CQ_PAIR_GO(3, 1);
+    if (idx == 1) CQ_PAIR_GO(3, 1);
+    CQ_PAIR_GO(3, 2);
 #undef CQ_PAIR_GO
 }
 

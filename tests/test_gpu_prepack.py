@@ -698,7 +698,10 @@ def test_prepacked_gated_rejections():
 
 @pytest.mark.parametrize("bits,k,n,norm", [(4, 4096, 11008, True), (3, 4096, 11008, True), (4, 4096, 11008, False),
                                            (4, 8192, 28672, True), (3, 8192, 4104, False), (4, 4096, 32008, True),
-                                           (3, 1024, 264, True), (4, 512, 40, False)])
+                                           (3, 1024, 264, True), (4, 512, 40, False),
+                                           # the 48-unit geometry (LLaMA-13B: 5120 -> 13824), both widths, walking and not
+                                           (3, 5120, 13824, True), (4, 5120, 13824, False), (4, 6144, 4104, True),
+                                           (3, 6144, 264, False), (3, 8192, 28672, True)])
 def test_prepacked_gate_up_fused_activation(bits, k, n, norm):
     """cherryq_decode_gate_up_prepacked_f16: both projections and SiLU(gate) * up in one launch.  Bit for
     bit what the separate launches give (grouped gate / up launch, then the SiLU * up kernel: same
