@@ -235,9 +235,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const __half *__restri
 // a cache row that another one writes in the same launch; the first query head of each kv group
 // stores the rotated k and the v row into the caches for later tokens.  Arithmetic and rounding
 // points are those of rope_cache_kernel followed by attn_decode_kernel.
+// (No __restrict__ on the inputs: loads through a read-only restrict pointer may be moved anywhere,
+// and the order of this kernel's first requests matters.)
 __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
-    const __half *__restrict__ q, const __half *__restrict__ k, const __half *__restrict__ v,
-    __half *__restrict__ k_cache, __half *__restrict__ v_cache, __half *__restrict__ out,
+    const __half *q, const __half *k, const __half *v, __half *k_cache, __half *v_cache, __half *__restrict__ out,
     const int *__restrict__ pos_ptr, int n_heads, int n_kv_heads, int max_len, RopeBase base, float scale) {
     typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
     __shared__ float s_score[kMaxAttnLen];
@@ -249,30 +250,40 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
     const int rep = n_heads / n_kv_heads, kvh = head / rep;
     const uint4 *kb = reinterpret_cast<const uint4 *>(k_cache + (size_t)kvh * max_len * 128);
     const uint4 *vb = reinterpret_cast<const uint4 *>(v_cache + (size_t)kvh * max_len * 128);
-    // The cache rows of the first pass are requested before the position is known (rows up to
-    // max_len exist; those at or beyond the position are ignored below), so that the position,
-    // q/k/v and the cache rows travel together: one memory round trip in front of the arithmetic.
+    // Order of the requests = order of use: the new token's q (threads 0..63), k and v (threads
+    // 64..127) and the position, every K row of the first pass; the V rows behind the first barrier.
+    // The cache rows are requested before the position is known (rows up to max_len exist; those
+    // at or beyond the position are ignored below): one memory round trip in front of the arithmetic.
+    // Every request is an unconditional buffer load (rows past the cache read zeros through the
+    // descriptor; every thread requests the small values, threads from 128 on drop them): all of
+    // them sit in one basic block in this order, so the wait in front of the rotation counts only
+    // the requests issued before it -- behind a branch the compiler waits for everything that is
+    // outstanding, V rows included, and plain loads it moves next to their first use.
+    typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
+    constexpr uint32_t kFlags = 0x00020000u;
+    const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc((void *)(q + (size_t)head * 128), 0, 256, kFlags);
+    const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void *)(k + (size_t)kvh * 128), 0, 256, kFlags);
+    const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void *)(v + (size_t)kvh * 128), 0, 256, kFlags);
+    const __amdgpu_buffer_rsrc_t rkc = __builtin_amdgcn_make_buffer_rsrc((void *)kb, 0, max_len * 256, kFlags);
+    const __amdgpu_buffer_rsrc_t rvc = __builtin_amdgcn_make_buffer_rsrc((void *)vb, 0, max_len * 256, kFlags);
+    const int ci = t & 63;
+    const unsigned short q1 = __builtin_amdgcn_raw_buffer_load_b16(rq, ci * 2, 0, 0), q2 = __builtin_amdgcn_raw_buffer_load_b16(rq, ci * 2 + 128, 0, 0);
+    const unsigned short k1 = __builtin_amdgcn_raw_buffer_load_b16(rk, ci * 2, 0, 0), k2 = __builtin_amdgcn_raw_buffer_load_b16(rk, ci * 2 + 128, 0, 0);
+    const __half v1 = __ushort_as_half(__builtin_amdgcn_raw_buffer_load_b16(rv, ci * 2, 0, 0));
+    const __half v2 = __ushort_as_half(__builtin_amdgcn_raw_buffer_load_b16(rv, ci * 2 + 128, 0, 0));
+    asm volatile("" ::: "memory");   // (keeps the groups of requests in this order through the compiler)
+    __builtin_amdgcn_sched_barrier(0);
     uint4 k_first[4], v_first[4];
 #pragma unroll
     for (int u = 0; u < 4; u++) {
-        const int j = row + 64 * u;
-        k_first[u] = j < max_len ? kb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
-        v_first[u] = j < max_len ? vb[(size_t)j * 16 + l16] : make_uint4(0, 0, 0, 0);
+        const u4_t r = __builtin_amdgcn_raw_buffer_load_b128(rkc, (row + 64 * u) * 256 + l16 * 16, 0, 0);
+        k_first[u] = make_uint4(r[0], r[1], r[2], r[3]);
     }
-    // likewise the new token's q (threads 0..63), k and v (threads 64..127)
-    float x1 = 0.f, x2 = 0.f, inv_freq = 0.f;
-    __half v1 = __float2half(0.f), v2 = v1;
-    if (t < 128) {
-        const int i = t & 63;
-        const __half *src = t >= 64 ? k + (size_t)kvh * 128 : q + (size_t)head * 128;
-        x1 = __half2float(src[i]);
-        x2 = __half2float(src[i + 64]);
-        if (t >= 64) {
-            v1 = v[(size_t)kvh * 128 + i];
-            v2 = v[(size_t)kvh * 128 + i + 64];
-        }
-        inv_freq = rope_inv_freq(i, 128, base);  // does not need the position
-    }
+    asm volatile("" ::: "memory");   // (keeps the groups of requests in this order through the compiler)
+    __builtin_amdgcn_sched_barrier(0);
+    const __half r1 = __ushort_as_half((t & 64) ? k1 : q1), r2 = __ushort_as_half((t & 64) ? k2 : q2);
+    const float x1 = __half2float(r1), x2 = __half2float(r2);
+    const float inv_freq = rope_inv_freq(t & 63, 128, base);  // does not need the position
     const int pos = *pos_ptr;
     if ((unsigned)pos >= (unsigned)max_len) {  // outside the cache: nothing read or written, the output is NaN
         if (t < 128) out[(size_t)head * 128 + t] = __ushort_as_half((unsigned short)0x7e00);
@@ -300,6 +311,17 @@ __global__ __launch_bounds__(1024) void rope_attn_decode_kernel(
         }
     }
     __syncthreads();
+    // The V rows are requested only now: a wavefront reaches a barrier when its requests have been
+    // ACCEPTED, and one compute unit accepts about 32 KB per microsecond -- with the V rows in front
+    // of it the barrier opened when all 128 KB of a 256-position cache had been taken (3 to 4 us);
+    // they are not needed before the softmax is done and travel while the scores are formed.
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const u4_t r = __builtin_amdgcn_raw_buffer_load_b128(rvc, (row + 64 * u) * 256 + l16 * 16, 0, 0);
+        v_first[u] = make_uint4(r[0], r[1], r[2], r[3]);
+    }
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
     // q . k over the lane's 8 dimensions as four packed fp16 dot products (fp32 accumulation), the 16
     // lanes of a row then add up with DPP rotations
     const uint4 qv = *reinterpret_cast<const uint4 *>(&s_qh[8 * l16]);
