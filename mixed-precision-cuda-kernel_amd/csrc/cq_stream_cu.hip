@@ -101,9 +101,17 @@ constexpr int kCuSeparate = 0, kCuSiluPair = 1;  // epilogues: every layer's res
 // units; each layer's compaction is staged by S / MEM of the staging wavefronts (the layers keep
 // different cherry channels).  EPI: kCuSeparate stores every layer's result, kCuSiluPair (MEM 2)
 // fp16(fp16(silu(layer 0)) * layer 1) of the two rounded results instead.
-template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, int PRO, bool WALK, int MEM = 1, int EPI = kCuSeparate>
+// EXTRA (one layer per workgroup, S == W, no walking): a workgroup whose compute unit gets one tile
+// more than it has teams hands that tile to its staging wavefronts, which work on it as one more
+// team once the row is staged.  q / k / v of 4096 columns each are 3 x 256 tiles on 85 / 85 / 86
+// workgroups of three teams: 255 slots for 256 tiles, so one team of a member walked a second
+// tile and the launch carried the walking code (7.23 us against 6.17 us for 3 x 255 tiles).
+template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, int PRO, bool WALK, int MEM = 1, int EPI = kCuSeparate,
+          bool EXTRA = false>
 __device__ __forceinline__ void stream_cu_body(const CuJob &job) {
     constexpr int NC = W * TEAMS;  // computing wavefronts
+    constexpr int NCX = NC + (EXTRA ? S : 0);  // ... and the staging wavefronts when they take a tile of their own
+    static_assert(!EXTRA || (S == W && MEM == 1 && !WALK && EPI == kCuSeparate), "the staging wavefronts as one more team");
     constexpr int NT = 64 * (NC + S);
     constexpr int UB = BITS == 4 ? 1024 : 768;
     constexpr float kGrid = BITS == 4 ? -7.5f : -3.5f;
@@ -140,6 +148,140 @@ __device__ __forceinline__ void stream_cu_body(const CuJob &job) {
     float *s_xsum = reinterpret_cast<float *>(s_xs + MEM * Knp512);         // [MEM][4 nblk]
     float *s_red = s_xsum + MEM * 4 * nblk;
     const int tstride = G * TSLOTS;
+
+    // ---- a team's wavefront at work: wavefront `cls` of the team whose partial sums go to row `cwv` of
+    // s_red, on tile slot `slot` of layer `mem`.  AFTER: called behind the workgroup barrier (the staging
+    // wavefronts as one more team): no barrier inside, one tile.
+    auto team_work = [&](auto after_tag, const int cwv, const int slot, const int cls, const int mem) {
+        constexpr bool AFTER = decltype(after_tag)::value;
+        const uint8_t *__restrict__ stream = stream_of(mem);
+        const unsigned short *xs_m = s_xs + mem * Knp512;
+        const float *xsum_m = s_xsum + mem * 4 * nblk;
+        const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(stream + hdr_bytes), 0, (int)min((unsigned long long)ntiles * record_bytes, 0xffffffffull), kSFlags);
+        const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc((void *)stream, 0, (int)hdr_bytes, kSFlags);
+        uint32_t sc[L / 4];
+        su4 wbuf[D];
+        su4 cw[4];
+        su4 civ[4];
+        const bool cherry_wave = cls == W - 1;
+        constexpr bool WALKX = WALK && !AFTER;
+        int tcur = bid + G * slot;
+        bool vcur = tcur < ntiles;
+        uint32_t tb = (uint32_t)tcur * record_bytes;
+        auto load_cherry = [&](uint32_t base, bool valid) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int lg = 4 * j + kq;
+                if (32 * j < C)
+                    cw[j] = __builtin_amdgcn_raw_buffer_load_b128(
+                        rt, valid && 8 * lg < C ? off_cherry + (uint32_t)(lg * 16 + nn) * 16u : kSOob, base, 2);
+            }
+        };
+        // lane group kq keeps the scales of the units i with i % 4 == kq (every lane group ends up
+        // with the same MFMA results, so each finishes a quarter of the units)
+        const uint32_t sc_off = (uint32_t)((cls + kq * W) * 32 + nn * 2);
+        auto load_scale = [&](int i4, uint32_t base, bool valid) -> uint32_t {
+            return __builtin_amdgcn_raw_buffer_load_b16(rt, valid && cls + (4 * i4 + kq) * W < ng ? sc_off : kSOob,
+                                                        base + 4 * i4 * W * 32, 0);
+        };
+        // a unit past the last one of the column, or of a tile that does not exist, reads zeros:
+        // the vector offset alone lies outside the descriptor
+        const uint32_t w_off = off_units + (uint32_t)(cls * UB + lane * (BITS * 4));
+        auto load_unit = [&](int i, uint32_t base, bool valid) -> su4 {
+            const uint32_t off = valid && cls + i * W < ng ? w_off : kSOob;
+            if constexpr (BITS == 4) {
+                return __builtin_amdgcn_raw_buffer_load_b128(rt, off, base + i * W * UB, 2);
+            } else {
+                const su3 v = __builtin_amdgcn_raw_buffer_load_b96(rt, off, base + i * W * UB, 2);
+                return (su4){v[0], v[1], v[2], 0u};
+            }
+        };
+        // The barrier at which the staging wavefronts exchange their sums of squares (kCuNorm) opens
+        // when every wavefront's requests so far have been ACCEPTED by the compute unit.  With several
+        // layers per workgroup (two staging wavefronts per layer, four blocks each) the computing
+        // wavefronts pass it before they request anything: RMSNorm + gate/up + SiLU 10.25 -> 9.92 us;
+        // with one layer per workgroup the same order is slower (gate/up as a group 9.94 -> 10.43 us).
+        constexpr bool kNormFirst = PRO == kCuNorm && MEM > 1;
+        if constexpr (kNormFirst && !AFTER) __builtin_amdgcn_s_barrier();
+        if (cherry_wave) {
+            // the cherry columns of the lane's A operands (positions 32 q + 8 kq + 0..7 of the list) and the rows
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+                if (32 * q < C) civ[q] = __builtin_amdgcn_raw_buffer_load_b128(rh, (uint32_t)(Knp512 + 64 * q + 16 * kq), 0, 0);
+            load_cherry(tb, vcur);
+        }
+#pragma unroll
+        for (int i = 0; i < L / 4; i++) sc[i] = load_scale(i, tb, vcur);
+#pragma unroll
+        for (int i = 0; i < D0; i++) wbuf[i] = load_unit(i, tb, vcur);
+        if constexpr (!AFTER) {
+            if constexpr (PRO == kCuNorm && !kNormFirst) {
+                __builtin_amdgcn_s_barrier();  // (the staging wavefronts exchange their sums of squares)
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+            __builtin_amdgcn_s_barrier();
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+#pragma unroll
+        for (int i = D0; i < D; i++) wbuf[i] = load_unit(i, tb, vcur);
+        // cherry activations straight from the raw row in LDS; list entries past the last channel
+        // name column K, which holds a zero (out-of-range part of the last slice)
+        su4 ca[4];
+        if (cherry_wave) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                if (32 * q < C) {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const uint32_t c0 = min(civ[q][j] & 0xffffu, (uint32_t)K), c1 = min(civ[q][j] >> 16, (uint32_t)K);
+                        ca[q][j] = (uint32_t)s_raw[c0] | ((uint32_t)s_raw[c1] << 16);
+                    }
+                }
+            }
+        }
+        const int P = WALKX ? job.P : 1;
+#pragma unroll 1
+        for (int j = 0; j < P; j++) {
+            const int tnext = tcur + tstride;
+            const bool vnext = WALKX && tnext < ntiles;
+            const uint32_t tbn = (uint32_t)tnext * record_bytes;
+            float totc = 0.f;
+            if (cherry_wave) {
+                sf4_t dc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    if (32 * q < C) dc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(ca[q]), as_h8(cw[q]), dc, 0, 0, 0);
+                totc = dc[0];
+                if constexpr (WALKX) load_cherry(tbn, vnext);
+            }
+            float tt = 0.f;
+#pragma unroll
+            for (int i = 0; i < L; i++) {
+                // a unit past the column's last reads zero codes and a zero scale; its activations
+                // and unit sum are those of unit 0, which every layer has
+                const bool real = cls + i * W < ng;
+                const int up = real ? cls + i * W : 0;
+                const float sf = (i & 3) == kq ? __half2float(__ushort_as_half((unsigned short)sc[i >> 2])) : 0.f;
+                const su4 w = wbuf[i % D];
+                const float v = unit_dot<BITS>(w, xs_m + up * kStreamUnitK + 32 * kq);
+                if (i + D < L) wbuf[i % D] = load_unit(i + D, tb, vcur);
+                else if constexpr (WALKX) wbuf[i % D] = load_unit(i + D - L, tbn, vnext);
+                tt += (v + kGrid * xsum_m[up]) * sf;
+                if constexpr (WALKX) {
+                    if ((i & 3) == 3) sc[i >> 2] = load_scale(i >> 2, tbn, vnext);
+                }
+            }
+            // the four lane groups' quarters
+            tt = swap32_add(tt, tt);
+            tt = swap16_add(tt, tt) + totc;
+            if (kq == 0) s_red[(j * NCX + cwv) * 16 + nn] = tt;
+            tcur = tnext;
+            vcur = vnext;
+            tb = tbn;
+            if (!vcur) break;
+        }
+    };
 
     if (wave < S) {
         // ---- staging wavefront: its slice of the row, its blocks' gather table; gather; unit sums
@@ -284,135 +426,16 @@ __device__ __forceinline__ void stream_cu_body(const CuJob &job) {
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
         __builtin_amdgcn_s_barrier();
+        if constexpr (EXTRA) {
+            // one more tile for this compute unit than it has teams: the staging wavefronts take it
+            if (bid + G * TEAMS < ntiles) team_work(std::true_type{}, NC + wave, TEAMS, wave, 0);
+        }
     } else {
         // ---- computing wavefront
         const int cwv = wave - S;
         const int team = cwv / W, cls = cwv % W;
         const int mem = MEM > 1 ? team % MEM : 0, slot = MEM > 1 ? team / MEM : team;   // the team's layer, its tile slot
-        const uint8_t *__restrict__ stream = stream_of(mem);
-        const unsigned short *xs_m = s_xs + mem * Knp512;
-        const float *xsum_m = s_xsum + mem * 4 * nblk;
-        const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)(stream + hdr_bytes), 0, (int)min((unsigned long long)ntiles * record_bytes, 0xffffffffull), kSFlags);
-        const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc((void *)stream, 0, (int)hdr_bytes, kSFlags);
-        uint32_t sc[L / 4];
-        su4 wbuf[D];
-        su4 cw[4];
-        su4 civ[4];
-        const bool cherry_wave = cls == W - 1;
-        int tcur = bid + G * slot;
-        bool vcur = tcur < ntiles;
-        uint32_t tb = (uint32_t)tcur * record_bytes;
-        auto load_cherry = [&](uint32_t base, bool valid) {
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int lg = 4 * j + kq;
-                if (32 * j < C)
-                    cw[j] = __builtin_amdgcn_raw_buffer_load_b128(
-                        rt, valid && 8 * lg < C ? off_cherry + (uint32_t)(lg * 16 + nn) * 16u : kSOob, base, 2);
-            }
-        };
-        // lane group kq keeps the scales of the units i with i % 4 == kq (every lane group ends up
-        // with the same MFMA results, so each finishes a quarter of the units)
-        const uint32_t sc_off = (uint32_t)((cls + kq * W) * 32 + nn * 2);
-        auto load_scale = [&](int i4, uint32_t base, bool valid) -> uint32_t {
-            return __builtin_amdgcn_raw_buffer_load_b16(rt, valid && cls + (4 * i4 + kq) * W < ng ? sc_off : kSOob,
-                                                        base + 4 * i4 * W * 32, 0);
-        };
-        // a unit past the last one of the column, or of a tile that does not exist, reads zeros:
-        // the vector offset alone lies outside the descriptor
-        const uint32_t w_off = off_units + (uint32_t)(cls * UB + lane * (BITS * 4));
-        auto load_unit = [&](int i, uint32_t base, bool valid) -> su4 {
-            const uint32_t off = valid && cls + i * W < ng ? w_off : kSOob;
-            if constexpr (BITS == 4) {
-                return __builtin_amdgcn_raw_buffer_load_b128(rt, off, base + i * W * UB, 2);
-            } else {
-                const su3 v = __builtin_amdgcn_raw_buffer_load_b96(rt, off, base + i * W * UB, 2);
-                return (su4){v[0], v[1], v[2], 0u};
-            }
-        };
-        // The barrier at which the staging wavefronts exchange their sums of squares (kCuNorm) opens
-        // when every wavefront's requests so far have been ACCEPTED by the compute unit.  With several
-        // layers per workgroup (two staging wavefronts per layer, four blocks each) the computing
-        // wavefronts pass it before they request anything: RMSNorm + gate/up + SiLU 10.25 -> 9.92 us;
-        // with one layer per workgroup the same order is slower (gate/up as a group 9.94 -> 10.43 us).
-        constexpr bool kNormFirst = PRO == kCuNorm && MEM > 1;
-        if constexpr (kNormFirst) __builtin_amdgcn_s_barrier();
-        if (cherry_wave) {
-            // the cherry columns of the lane's A operands (positions 32 q + 8 kq + 0..7 of the list) and the rows
-#pragma unroll
-            for (int q = 0; q < 4; q++)
-                if (32 * q < C) civ[q] = __builtin_amdgcn_raw_buffer_load_b128(rh, (uint32_t)(Knp512 + 64 * q + 16 * kq), 0, 0);
-            load_cherry(tb, vcur);
-        }
-#pragma unroll
-        for (int i = 0; i < L / 4; i++) sc[i] = load_scale(i, tb, vcur);
-#pragma unroll
-        for (int i = 0; i < D0; i++) wbuf[i] = load_unit(i, tb, vcur);
-        if constexpr (PRO == kCuNorm && !kNormFirst) {
-            __builtin_amdgcn_s_barrier();  // (the staging wavefronts exchange their sums of squares)
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-#pragma unroll
-        for (int i = D0; i < D; i++) wbuf[i] = load_unit(i, tb, vcur);
-        // cherry activations straight from the raw row in LDS; list entries past the last channel
-        // name column K, which holds a zero (out-of-range part of the last slice)
-        su4 ca[4];
-        if (cherry_wave) {
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                if (32 * q < C) {
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const uint32_t c0 = min(civ[q][j] & 0xffffu, (uint32_t)K), c1 = min(civ[q][j] >> 16, (uint32_t)K);
-                        ca[q][j] = (uint32_t)s_raw[c0] | ((uint32_t)s_raw[c1] << 16);
-                    }
-                }
-            }
-        }
-        const int P = WALK ? job.P : 1;
-#pragma unroll 1
-        for (int j = 0; j < P; j++) {
-            const int tnext = tcur + tstride;
-            const bool vnext = WALK && tnext < ntiles;
-            const uint32_t tbn = (uint32_t)tnext * record_bytes;
-            float totc = 0.f;
-            if (cherry_wave) {
-                sf4_t dc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int q = 0; q < 4; q++)
-                    if (32 * q < C) dc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(ca[q]), as_h8(cw[q]), dc, 0, 0, 0);
-                totc = dc[0];
-                if constexpr (WALK) load_cherry(tbn, vnext);
-            }
-            float tt = 0.f;
-#pragma unroll
-            for (int i = 0; i < L; i++) {
-                // a unit past the column's last reads zero codes and a zero scale; its activations
-                // and unit sum are those of unit 0, which every layer has
-                const bool real = cls + i * W < ng;
-                const int up = real ? cls + i * W : 0;
-                const float sf = (i & 3) == kq ? __half2float(__ushort_as_half((unsigned short)sc[i >> 2])) : 0.f;
-                const su4 w = wbuf[i % D];
-                const float v = unit_dot<BITS>(w, xs_m + up * kStreamUnitK + 32 * kq);
-                if (i + D < L) wbuf[i % D] = load_unit(i + D, tb, vcur);
-                else if constexpr (WALK) wbuf[i % D] = load_unit(i + D - L, tbn, vnext);
-                tt += (v + kGrid * xsum_m[up]) * sf;
-                if constexpr (WALK) {
-                    if ((i & 3) == 3) sc[i >> 2] = load_scale(i >> 2, tbn, vnext);
-                }
-            }
-            // the four lane groups' quarters
-            tt = swap32_add(tt, tt);
-            tt = swap16_add(tt, tt) + totc;
-            if (kq == 0) s_red[(j * NC + cwv) * 16 + nn] = tt;
-            tcur = tnext;
-            vcur = vnext;
-            tb = tbn;
-            if (!vcur) break;
-        }
+        team_work(std::false_type{}, cwv, slot, cls, mem);
     }
 
     // ---- across a tile's wavefronts, then one store per output
@@ -420,7 +443,7 @@ __device__ __forceinline__ void stream_cu_body(const CuJob &job) {
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     const int P = WALK ? job.P : 1;
-    constexpr int OUTS = EPI == kCuSiluPair ? TSLOTS : TEAMS;   // 16-column pieces of output per walk step
+    constexpr int OUTS = EPI == kCuSiluPair ? TSLOTS : TEAMS + (EXTRA ? 1 : 0);   // 16-column pieces of output per walk step
     __half *mu0 = job.mul, *mu1 = MEM > 1 ? job.mul2 : job.mul, *mu2 = MEM > 2 ? job.mul3 : job.mul;
     if constexpr (MEM > 1) asm volatile("" : "+s"(mu0), "+s"(mu1), "+s"(mu2));
     for (int o = tid; o < 16 * P * OUTS; o += NT) {
@@ -428,7 +451,7 @@ __device__ __forceinline__ void stream_cu_body(const CuJob &job) {
         const int slot = EPI == kCuSiluPair ? t : t / MEM, mem = EPI == kCuSiluPair ? 0 : t - slot * MEM;
         const int tile = bid + G * (slot + TSLOTS * j), n = tile * 16 + col;
         if (tile < ntiles && n < N) {
-            const float *red = s_red + (j * NC + (slot * MEM + mem) * W) * 16 + col;
+            const float *red = s_red + (j * NCX + (slot * MEM + mem) * W) * 16 + col;
             if constexpr (EPI == kCuSiluPair) {
                 float g = 0.f, u = 0.f;
 #pragma unroll
@@ -476,7 +499,7 @@ struct CuGroupTail {
     __half *mul[kStreamMaxGroup];
     float eps;
 };
-template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, int PRO, bool WALK>
+template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, int PRO, bool WALK, bool EXTRA = false>
 __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_group_kernel(
     const __half *__restrict__ x, const __half *__restrict__ norm_w, const uint8_t *__restrict__ stream0,
     const uint8_t *__restrict__ stream1, const uint8_t *__restrict__ stream2, uint32_t kc, uint32_t n01, uint32_t n2p,
@@ -505,7 +528,7 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_group_kernel(
     job.P = (int)((n2p >> 16) & 0x7fffu);
     job.stream2 = job.stream3 = nullptr;
     job.mul2 = job.mul3 = nullptr;
-    stream_cu_body<BITS, W, L, TEAMS, S, NB, D0, D, PRO, WALK>(job);
+    stream_cu_body<BITS, W, L, TEAMS, S, NB, D0, D, PRO, WALK, 1, kCuSeparate, EXTRA>(job);
 }
 
 // MEM = 2 or 3 layers of the SAME shape that read the same row, every workgroup working on the same
@@ -663,11 +686,11 @@ static hipError_t cu_raise_lds(KERN kern, bool *raised) {
     return hipSuccess;
 }
 
-template <int BITS, int I, int PRO, bool GROUP, bool WALK>
+template <int BITS, int I, int PRO, bool GROUP, bool WALK, bool EXTRA = false>
 static hipError_t launch_cu_cfg(const __half *vec, const __half *norm_w, float eps, const StreamMember *members, int count,
                                 const StreamGeo &geo, const CuSplit &sp, int accumulate, hipStream_t s) {
     constexpr CuCfg c = kCuCfgs[I];
-    const size_t lds = cu_lds_bytes(geo, c, sp.walk);
+    const size_t lds = cu_lds_bytes(geo, c, sp.walk) + (EXTRA ? (size_t)c.S * 16 * 4 : 0);
     const dim3 grid(sp.total), block(64 * (c.W * c.TEAMS + c.S));
     static bool raised[kCuMaxDevices] = {};
     if constexpr (!GROUP) {
@@ -676,7 +699,7 @@ static hipError_t launch_cu_cfg(const __half *vec, const __half *norm_w, float e
         hipLaunchKernelGGL(kern, grid, block, lds, s, vec, members[0].stream, members[0].mul, geo.K, geo.C, members[0].N,
                            sp.wgs[0], accumulate, sp.walk);
     } else {
-        auto kern = stream_cu_group_kernel<BITS, c.W, c.L, c.TEAMS, c.S, c.NB, c.D0, c.D, PRO, WALK>;
+        auto kern = stream_cu_group_kernel<BITS, c.W, c.L, c.TEAMS, c.S, c.NB, c.D0, c.D, PRO, WALK, EXTRA>;
         if (hipError_t e = cu_raise_lds(kern, raised)) return e;
         CuGroupTail tail = {};
         const uint8_t *st[kStreamMaxGroup];
@@ -716,12 +739,28 @@ hipError_t launch_stream_cu(int bits, const __half *vec, const __half *norm_w, f
     const StreamGeo geo = stream_geo(bits, K, members[0].N, C);
     const int idx = cu_pick(geo.ng, ceil_div(all, kCuCus));
     if (idx < 0) return hipErrorInvalidValue;
-    const CuSplit sp = cu_split(tiles, count, kCuCfgs[idx].TEAMS);
+    CuSplit sp = cu_split(tiles, count, kCuCfgs[idx].TEAMS);
+    // one tile more than teams on some compute unit: the staging wavefronts take it instead of a team walking
+    bool extra = false;
+    if (sp.walk > 1 && (idx == 1 || idx == 2) && !gate && !attn_ml) {
+        const CuSplit sx = cu_split(tiles, count, kCuCfgs[idx].TEAMS + 1);
+        if (sx.walk == 1) {
+            sp = sx;
+            extra = true;
+        }
+    }
     if (sp.walk > kCuMaxWalk || sp.total > 1023) return hipErrorInvalidValue;
     const bool group = count > 1 || norm_w != nullptr || gate != nullptr, walk = sp.walk > 1;
     const __half *ml_slot = reinterpret_cast<const __half *>(attn_ml);
 #define CQ_CU_GO(BITS_, I_)                                                                                               \
     do {                                                                                                                  \
+        if (extra) {                                                                                                      \
+            if constexpr (I_ == 1 || I_ == 2)                                                                             \
+                return norm_w ? launch_cu_cfg<BITS_, I_, kCuNorm, true, false, true>(vec, norm_w, eps, members, count, geo, sp, accumulate, s)    \
+                              : launch_cu_cfg<BITS_, I_, kCuPlain, true, false, true>(vec, nullptr, 0.f, members, count, geo, sp, accumulate, s); \
+            else                                                                                                          \
+                return hipErrorInvalidValue;                                                                              \
+        }                                                                                                                 \
         if (attn_ml) {                                                                                                    \
             if constexpr (I_ <= kCuAttnMaxCfg)                                                                            \
                 return walk ? launch_cu_cfg<BITS_, I_, kCuAttn, true, true>(vec, ml_slot, 0.f, members, count, geo, sp, accumulate, s)   \
