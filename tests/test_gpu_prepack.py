@@ -63,7 +63,9 @@ SHAPES = [(4, 4096, 11008), (3, 4096, 11008), (4, 11008, 4096), (3, 11008, 4096)
           (4, 13824, 5120), (4, 16384, 264), (3, 13824, 264), (4, 28672, 264), (3, 28672, 264), (4, 20480, 4352),
           (3, 24576, 4104),
           # the geometries of the LLaMA-13B widths in the other bit width, and the 96-unit one (12 wavefronts on a tile)
-          (4, 5120, 5120), (4, 5120, 13824), (3, 12288, 4096), (4, 12288, 4104), (3, 13824, 8200)]
+          (4, 5120, 5120), (4, 5120, 13824), (3, 12288, 4096), (4, 12288, 4104), (3, 13824, 8200),
+          # 769 to 1024 tiles of up to 32 units: three teams per compute unit and the staging wavefronts as a fourth
+          (4, 4096, 16384), (3, 4096, 14008), (4, 1024, 12304)]
 
 
 @pytest.mark.parametrize("bits,k,n", SHAPES)
@@ -107,7 +109,7 @@ def test_prepacked_matvec_against_oracle(qc, bits, k, n):
 @pytest.mark.parametrize("bits,k,n", [(4, 4096, 4096), (3, 4096, 4096), (4, 11008, 512), (3, 11008, 512),
                                       (3, 5120, 520), (4, 8192, 264), (3, 13824, 264), (4, 28672, 264), (3, 28672, 264),
                                       (3, 11008, 4608), (4, 16384, 4112), (4, 5120, 8200), (3, 5120, 8200),
-                                      (3, 12288, 264), (4, 13824, 8200), (3, 13824, 8200)])
+                                      (3, 12288, 264), (4, 13824, 8200), (3, 13824, 8200), (3, 4096, 16384), (4, 2048, 14008)])
 def test_prepacked_one_hot_reads_back_dequantised_weights(qc, bits, k, n):
     """x = e_j returns column j of the dense weight: decode, gather around the cherry channels and
     the per-unit grid offset are exact.  Positions probe every code slot of a lane's 32 and both
