@@ -571,7 +571,10 @@ static constexpr CuCfg kCuCfgs[] = {
     {5, 8, 2, 6, 2, 3, 4},   // 7: up to 40 units (5120 input channels), two teams
     {4, 28, 2, 8, 4, 4, 7},  // 8: up to 112 units (13824 input channels), two tiles per compute unit
     {12, 8, 1, 4, 6, 3, 4},  // 9: up to 96 units, one team of 12 (12288 -> 4096: 6.5 / 6.1 us against 7.2 / 6.7 for entry 5)
+    {4, 12, 3, 4, 3, 3, 4},  // 10: up to 48 units, three teams and the staging wavefronts as a fourth (5120 -> 13824)
 };
+// entries whose staging wavefronts can work as one more team (as many of them as a team has wavefronts)
+constexpr bool cu_cfg_extra(int i) { return kCuCfgs[i].S == kCuCfgs[i].W; }
 // The LLaMA-13B widths (entries 7 and 8), us per launch, 4-bit / 3-bit, against the checkpoint layout's
 // 5.87 / 5.57 (5120 -> 5120), 10.15 / 8.80 (5120 -> 13824), 10.24 / 8.81 (13824 -> 5120):
 // 5120 -> 5120 (320 tiles): entry 7 4.52 / 4.65 (entry 3: 6.0 / 6.0; three teams of 4 x 12 units 5.4 / 5.9;
@@ -597,6 +600,7 @@ constexpr int kCuAttnMaxCfg = 3;  // the attention-combining prologue exists for
 
 static int cu_pick(int ng, int tiles_per_cu_ceil) {
     if (ng <= 32) return tiles_per_cu_ceil <= 1 ? 0 : tiles_per_cu_ceil == 2 ? 1 : 2;
+    if (ng <= 48 && tiles_per_cu_ceil >= 3 && tiles_per_cu_ceil <= 4) return 10;
     if (ng <= 40) return 7;
     if (ng <= 64) return 3;
     if (ng <= 88) return 4;
@@ -742,7 +746,7 @@ hipError_t launch_stream_cu(int bits, const __half *vec, const __half *norm_w, f
     CuSplit sp = cu_split(tiles, count, kCuCfgs[idx].TEAMS);
     // one tile more than teams on some compute unit: the staging wavefronts take it instead of a team walking
     bool extra = false;
-    if (sp.walk > 1 && (idx == 1 || idx == 2) && !gate && !attn_ml) {
+    if (sp.walk > 1 && cu_cfg_extra(idx) && !gate && !attn_ml) {
         const CuSplit sx = cu_split(tiles, count, kCuCfgs[idx].TEAMS + 1);
         if (sx.walk == 1) {
             sp = sx;
@@ -755,7 +759,7 @@ hipError_t launch_stream_cu(int bits, const __half *vec, const __half *norm_w, f
 #define CQ_CU_GO(BITS_, I_)                                                                                               \
     do {                                                                                                                  \
         if (extra) {                                                                                                      \
-            if constexpr (I_ == 1 || I_ == 2)                                                                             \
+            if constexpr (cu_cfg_extra(I_))                                                                               \
                 return norm_w ? launch_cu_cfg<BITS_, I_, kCuNorm, true, false, true>(vec, norm_w, eps, members, count, geo, sp, accumulate, s)    \
                               : launch_cu_cfg<BITS_, I_, kCuPlain, true, false, true>(vec, nullptr, 0.f, members, count, geo, sp, accumulate, s); \
             else                                                                                                          \
@@ -791,7 +795,8 @@ hipError_t launch_stream_cu(int bits, const __half *vec, const __half *norm_w, f
         case 6: CQ_CU_GO(BITS_, 6);  \
         case 7: CQ_CU_GO(BITS_, 7);  \
         case 8: CQ_CU_GO(BITS_, 8);  \
-        default: CQ_CU_GO(BITS_, 9); \
+        case 9: CQ_CU_GO(BITS_, 9);  \
+        default: CQ_CU_GO(BITS_, 10); \
     }
     if (bits == 4) CQ_CU_BITS(4)
     CQ_CU_BITS(3)
