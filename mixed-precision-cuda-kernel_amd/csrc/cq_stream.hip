@@ -1017,6 +1017,8 @@ __device__ inline sf4_t unit_dot_regs(const WB w, const su4 (&a)[4]) {
 
 // W wavefronts per team, 8 / W teams, L units per wavefront (W * L units per column at most), the
 // loads of R consecutive tiles of a team in flight (R * L per wavefront).
+constexpr int kRowsRegChunk = 4;  // tile steps whose partial outputs stream_rows_reg_kernel keeps in LDS between two barriers
+
 template <int BITS, int W, int L, int R>
 __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restrict__ xf, const float *__restrict__ xsum_g,
                                                               const su4 *__restrict__ xcf,
@@ -1026,9 +1028,13 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
     constexpr int TEAMS = 8 / W;
     constexpr int UB = BITS == 4 ? 1024 : 768;
     constexpr float kGrid = BITS == 4 ? -7.5f : -3.5f;
-    __shared__ float s_red[8][256];
+    // partial outputs of kRowsRegChunk consecutive tile steps: [step][wavefront][16 rows x 16 columns].  A
+    // wavefront reaches a barrier only when the compute unit has accepted all its requests so far, the
+    // next tiles' weights included: two barriers per tile cost more than the arithmetic between
+    // them, so the partial sums wait here and the workgroup meets once per chunk of steps.
     extern __shared__ __align__(16) unsigned char smem[];
-    float *s_xsum = reinterpret_cast<float *>(smem);  // [16][ng]
+    float *s_red = reinterpret_cast<float *>(smem);                  // [kRowsRegChunk][8][256]
+    float *s_xsum = s_red + kRowsRegChunk * 8 * 256;                 // [16][ng]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int team = wave / W, cls = wave % W;
@@ -1107,6 +1113,28 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
     const float *xsrow = s_xsum + (4 * kq) * ng;
     // the loop count is the same for every wavefront of the workgroup (barriers inside): as long as
     // the workgroup's first team, which has the lowest tile, has one in slot 0
+    int step = 0;   // tile steps of the workgroup so far (the same count in every wavefront)
+    auto flush = [&](int first_step, int count) {
+        // sums over a tile's wavefronts and the stores, for the `count` steps that started at `first_step`
+        __syncthreads();
+        for (int o = tid; o < count * TEAMS * 256; o += 512) {
+            const int j = o / (TEAMS * 256), rem = o - j * TEAMS * 256, tm = rem >> 8, t = rem & 255;
+            const int tl = blockIdx.x + tm * G + (first_step + j) * stride;
+            const int row = t >> 4, n = tl * kStreamTileCols + (t & 15);
+            if (tl < ntl && row < B && n < N) {
+                float v = 0.f;
+#pragma unroll
+                for (int c = 0; c < W; c++) v += s_red[(j * 8 + tm * W + c) * 256 + t];
+                __half *o16 = mul + (size_t)row * N + n;
+                if (accumulate) v += __half2float(*o16);
+                *o16 = __float2half_rn(v);
+            }
+        }
+        __syncthreads();
+    };
+    int chunk_first = 0;
+    // the loop count is the same for every wavefront of the workgroup (barriers inside): as long as
+    // the workgroup's first team, which has the lowest tile, has one in slot 0
     for (int t0 = blockIdx.x; t0 < ntl; t0 += R * stride) {
 #pragma unroll
         for (int s = 0; s < R; s++) {
@@ -1131,29 +1159,19 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
 #pragma unroll
                 for (int r = 0; r < 4; r++) acc[r] += (v[r] + kGrid * xsrow[r * ng + up]) * sf;
             }
-            float *red = &s_red[wave][0];
+            float *red = s_red + ((step - chunk_first) * 8 + wave) * 256;
 #pragma unroll
             for (int r = 0; r < 4; r++) red[(4 * kq + r) * 16 + nn] = acc[r];
-            __syncthreads();
-            {
-                const int t = tid - team * 64 * W;
-                if (t < 256 && valid[s]) {
-                    const int row = t >> 4, n = tile[s] * kStreamTileCols + (t & 15);
-                    if (row < B && n < N) {
-                        float v = 0.f;
-#pragma unroll
-                        for (int c = 0; c < W; c++) v += s_red[team * W + c][t];
-                        __half *o = mul + (size_t)row * N + n;
-                        if (accumulate) v += __half2float(*o);
-                        *o = __float2half_rn(v);
-                    }
-                }
-            }
-            __syncthreads();
             tile[s] = tnext;
             valid[s] = vnext;
+            step++;
+            if (step - chunk_first == kRowsRegChunk) {
+                flush(chunk_first, kRowsRegChunk);
+                chunk_first = step;
+            }
         }
     }
+    if (step > chunk_first) flush(chunk_first, step - chunk_first);
 }
 
 constexpr int kStreamWalk = 8;  // tiles one workgroup takes at most when a launch has more tiles than resident workgroups
@@ -1554,7 +1572,7 @@ hipError_t launch_stream_rows(int bits, const __half *vec, const uint8_t *stream
         if (e != hipSuccess) return e;
         const bool w4 = geo.ng <= 32;
         const int grid = geo.ntiles < kStreamCus ? geo.ntiles : kStreamCus;  // one team of 8 wavefronts per workgroup
-        const size_t lds = (size_t)16 * geo.ng * 4;
+        const size_t lds = (size_t)kRowsRegChunk * 8 * 256 * 4 + (size_t)16 * geo.ng * 4;
 #define CQ_REG_GO(BITS_, W_, L_, R_)                                                                                  \
     hipLaunchKernelGGL((stream_rows_reg_kernel<BITS_, W_, L_, R_>), dim3(grid), dim3(512), lds, s, xf, xsum, xcf, stream, mul,  \
                        B, accumulate, geo)
