@@ -1057,7 +1057,7 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
         const int u = cls + i * W;
 #pragma unroll
         for (int m = 0; m < 4; m++)
-            areg[i][m] = u < ng ? xf[((size_t)u * 4 + m) * 64 + lane] : (su4){0u, 0u, 0u, 0u};
+            areg[i][m] = u < ng && nn < B ? xf[((size_t)u * 4 + m) * 64 + lane] : (su4){0u, 0u, 0u, 0u};  // (rows from B on are zeros: not fetched)
     }
     __builtin_amdgcn_sched_barrier(0);
 
