@@ -55,9 +55,8 @@ MEASURED_TRAFFIC = {("llama7b_gate_up_w4", 1, "reference"): 25320960,
 # cycles / (kernel time x 2.4 GHz x 1024 SIMDs)); like the traffic figure it cannot be read while timing.
 MFMA_BUSY = {"llama70b_gate_up_w4": {"frac": 0.123, "kernel": "cq::stream_rows_reg_kernel<4, 8, 8, 1>",
                                      "profile": "profiles/rows16_w4_llama70b_gate_up_8192x28672_stream.md"},
-             "llama70b_down_w4": {"frac": 0.084, "kernel": "cq::batch_kernel<4>",
-                                  "profile": "profiles/batch_w4_llama70b_gate_up_8192x28672_b16_mfma_counters.md",
-                                  "note": "measured on the 8192 -> 28672 layer, same kernel and unit count per byte"}}
+             "llama70b_down_w4": {"frac": 0.135, "kernel": "cq::stream_rows_reg_kernel<4, 8, 8, 1, true>",
+                                  "profile": "profiles/rows16_w4_llama70b_down_28672x8192_stream.md"}}
 
 
 def algorithmic_bytes(bits, k, n, batch=1, group=128):
@@ -461,6 +460,8 @@ def main():
                 import quant_cuda
                 base_name = quant_cuda.prepacked_kernel_name(bits, k_in, n_out, -(-k_in // 256) // 8 * 8) if k_in and n_out else ""
                 return f"{base_name or 'cq::stream_cu_kernel'}<{bits}>"
+            if k_in > 64 * args.group + 128:  # deeper than 64 units: slices of units, partial outputs added by one more launch
+                return f"cq::stream_rows_frag_kernel + cq::stream_rows_reg_kernel<{bits}, slices> + cq::rows_reduce_kernel"
             if batch >= 8 or k_in > 32 * args.group:  # the rule of launch_stream_rows: activations in registers
                 return f"cq::stream_rows_frag_kernel + cq::stream_rows_reg_kernel<{bits}>"
             return f"cq::stream_rows_prep_kernel + cq::stream_rows_kernel<{bits}>"

@@ -255,7 +255,9 @@ int cherryq_matvec_prepacked_f16(int w_bits, const void *vec, const void *stream
  * are brought into matrix-core operand order once (a first small launch into an uninitialised
  * scratch buffer of cherryq_prepacked_scratch_bytes() bytes, 256-byte aligned; for up to 4 rows
  * inside the main launch) and then stay in LDS or in registers while a workgroup walks its
- * tiles; layers of up to 8192 + 128 input channels (64 units of 128 positions) are taken.  batch == 1 forwards to
+ * tiles.  Layers deeper than 8192 + 128 input channels (64 units of 128 positions), up to 256
+ * units, are taken in four slices of units with fp32 partial outputs in the scratch buffer and one
+ * more launch that adds them.  batch == 1 forwards to
  * cherryq_matvec_prepacked_f16 (scratch may then be NULL).  cherryq_prepack_supported(w_bits,
  * batch, ...) says whether a batch is taken.  vec must be 16-byte aligned (the rows are read as
  * 16-byte pieces; in_features is a multiple of 8, so every row then is).

@@ -1019,12 +1019,16 @@ __device__ inline sf4_t unit_dot_regs(const WB w, const su4 (&a)[4]) {
 // loads of R consecutive tiles of a team in flight (R * L per wavefront).
 constexpr int kRowsRegChunk = 4;  // tile steps whose partial outputs stream_rows_reg_kernel keeps in LDS between two barriers
 
-template <int BITS, int W, int L, int R>
+// KS > 1 (layers deeper than W * L units): the workgroups form KS slices, slice z takes units
+// [z * US, (z + 1) * US) of every tile it visits and writes its fp32 partial sums to
+// part[z][16][N]; rows_reduce_kernel adds the slices up.  The cherry channels belong to slice 0.
+template <int BITS, int W, int L, int R, bool KSPLIT = false>
 __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restrict__ xf, const float *__restrict__ xsum_g,
                                                               const su4 *__restrict__ xcf,
                                                               const uint8_t *__restrict__ stream,
                                                               __half *__restrict__ mul, int B, int accumulate,
-                                                              StreamGeo geo) {
+                                                              StreamGeo geo, float *__restrict__ part = nullptr,
+                                                              int KS = 1, int US = 0) {
     constexpr int TEAMS = 8 / W;
     constexpr int UB = BITS == 4 ? 1024 : 768;
     constexpr float kGrid = BITS == 4 ? -7.5f : -3.5f;
@@ -1040,29 +1044,34 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
     const int team = wave / W, cls = wave % W;
     const int kq = lane >> 4, nn = lane & 15;
     const int C = geo.C, ng = geo.ng, N = geo.N;
+    const int G = KSPLIT ? gridDim.x / KS : gridDim.x;          // workgroups that share the tiles
+    const int slice = KSPLIT ? blockIdx.x / G : 0, bx = KSPLIT ? blockIdx.x - slice * G : blockIdx.x;
+    const int u0 = KSPLIT ? slice * US : 0;                       // the slice's first unit
+    const int ucount = KSPLIT ? min(US, ng - u0) : ng;            // and how many it has
     // ---- requests, in the order their data is needed: the small shared operands (cherry
     // activations, unit sums: they go through LDS and gate the barrier), the wavefront's own A
     // operands, then the first R tiles' weights -- all queued BEFORE the barrier, so that the weight
     // stream is under way while the workgroup still waits for its activations
-    const bool cherry_wave = cls == W - 1;
+    const bool cherry_wave = cls == W - 1 && slice == 0;
     __shared__ su4 s_acr[4 * 64];  // the cherry operands (read once per tile by each team's last wavefront)
     su4 acr_v = {0u, 0u, 0u, 0u};
     if (tid < 4 * 64) acr_v = xcf[tid];
-    float xs_v[4];
+    constexpr int XJ = KSPLIT ? 8 : 4;  // 512 * XJ unit sums at most: 16 rows of 64 units, 256 when split
+    float xs_v[XJ];
 #pragma unroll
-    for (int j = 0; j < 4; j++) xs_v[j] = tid + 512 * j < 16 * ng ? xsum_g[tid + 512 * j] : 0.f;
+    for (int j = 0; j < XJ; j++) xs_v[j] = tid + 512 * j < 16 * ng ? xsum_g[tid + 512 * j] : 0.f;
     su4 areg[L][4];
 #pragma unroll
     for (int i = 0; i < L; i++) {
-        const int u = cls + i * W;
+        const int u = u0 + cls + i * W;
 #pragma unroll
         for (int m = 0; m < 4; m++)
-            areg[i][m] = u < ng && nn < B ? xf[((size_t)u * 4 + m) * 64 + lane] : (su4){0u, 0u, 0u, 0u};  // (rows from B on are zeros: not fetched)
+            areg[i][m] = cls + i * W < ucount && nn < B ? xf[((size_t)u * 4 + m) * 64 + lane] : (su4){0u, 0u, 0u, 0u};  // (rows from B on are zeros: not fetched)
     }
     __builtin_amdgcn_sched_barrier(0);
 
     const int ntl = (N + kStreamTileCols - 1) / kStreamTileCols;
-    const int G = gridDim.x, stride = G * TEAMS;
+    const int stride = G * TEAMS;
     const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(
         (void *)(stream + geo.hdr_bytes), 0, (int)min((unsigned long long)ntl * geo.record_bytes, 0xffffffffull), kSFlags);
     typedef typename std::conditional<BITS == 4, su4, su3>::type WB;  // a unit: 4 or 3 dwords per lane
@@ -1078,12 +1087,12 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
         }
     };
     auto load_scale = [&](int i, uint32_t base, bool valid) -> uint32_t {
-        return __builtin_amdgcn_raw_buffer_load_b16(rt, valid && cls + i * W < ng ? (uint32_t)(cls * 32 + nn * 2) : kSOob,
+        return __builtin_amdgcn_raw_buffer_load_b16(rt, valid && cls + i * W < ucount ? (uint32_t)((u0 + cls) * 32 + nn * 2) : kSOob,
                                                     base + i * W * 32, 0);
     };
-    const uint32_t w_off = geo.off_units + (uint32_t)(cls * UB + lane * (BITS * 4));
+    const uint32_t w_off = geo.off_units + (uint32_t)((u0 + cls) * UB + lane * (BITS * 4));
     auto load_unit = [&](int i, uint32_t base, bool valid) -> WB {
-        const uint32_t off = valid && cls + i * W < ng ? w_off : kSOob;
+        const uint32_t off = valid && cls + i * W < ucount ? w_off : kSOob;
         if constexpr (BITS == 4) {
             return __builtin_amdgcn_raw_buffer_load_b128(rt, off, base + i * W * UB, 2);
         } else {
@@ -1095,7 +1104,7 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
     bool valid[R];
 #pragma unroll
     for (int s = 0; s < R; s++) {
-        tile[s] = blockIdx.x + team * G + s * stride;
+        tile[s] = bx + team * G + s * stride;
         valid[s] = tile[s] < ntl;
         const uint32_t tb = (uint32_t)tile[s] * geo.record_bytes;
         if (cherry_wave) load_cherry(cw[s], tb, valid[s]);
@@ -1107,7 +1116,7 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
     __builtin_amdgcn_sched_barrier(0);
     if (tid < 4 * 64) s_acr[tid] = acr_v;
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int j = 0; j < XJ; j++)
         if (tid + 512 * j < 16 * ng) s_xsum[tid + 512 * j] = xs_v[j];
     __syncthreads();
     const float *xsrow = s_xsum + (4 * kq) * ng;
@@ -1119,15 +1128,19 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
         __syncthreads();
         for (int o = tid; o < count * TEAMS * 256; o += 512) {
             const int j = o / (TEAMS * 256), rem = o - j * TEAMS * 256, tm = rem >> 8, t = rem & 255;
-            const int tl = blockIdx.x + tm * G + (first_step + j) * stride;
+            const int tl = bx + tm * G + (first_step + j) * stride;
             const int row = t >> 4, n = tl * kStreamTileCols + (t & 15);
             if (tl < ntl && row < B && n < N) {
                 float v = 0.f;
 #pragma unroll
                 for (int c = 0; c < W; c++) v += s_red[(j * 8 + tm * W + c) * 256 + t];
-                __half *o16 = mul + (size_t)row * N + n;
-                if (accumulate) v += __half2float(*o16);
-                *o16 = __float2half_rn(v);
+                if constexpr (KSPLIT) {
+                    part[((size_t)slice * 16 + row) * N + n] = v;
+                } else {
+                    __half *o16 = mul + (size_t)row * N + n;
+                    if (accumulate) v += __half2float(*o16);
+                    *o16 = __float2half_rn(v);
+                }
             }
         }
         __syncthreads();
@@ -1135,7 +1148,7 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
     int chunk_first = 0;
     // the loop count is the same for every wavefront of the workgroup (barriers inside): as long as
     // the workgroup's first team, which has the lowest tile, has one in slot 0
-    for (int t0 = blockIdx.x; t0 < ntl; t0 += R * stride) {
+    for (int t0 = bx; t0 < ntl; t0 += R * stride) {
 #pragma unroll
         for (int s = 0; s < R; s++) {
             const int tnext = tile[s] + R * stride;
@@ -1151,7 +1164,7 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
             }
 #pragma unroll
             for (int i = 0; i < L; i++) {
-                const int up = cls + i * W < ng ? cls + i * W : 0;  // (a unit past the last: zero codes, zero scale, zero operands; unit 0's sum, which exists)
+                const int up = cls + i * W < ucount ? u0 + cls + i * W : 0;  // (a unit past the last: zero codes, zero scale, zero operands; unit 0's sum, which exists)
                 const float sf = __half2float(__ushort_as_half((unsigned short)sc[s][i]));
                 const sf4_t v = unit_dot_regs<BITS, WB>(wbuf[s][i], areg[i]);
                 wbuf[s][i] = load_unit(i, tbn, vnext);
@@ -1172,6 +1185,19 @@ __global__ __launch_bounds__(512) void stream_rows_reg_kernel(const su4 *__restr
         }
     }
     if (step > chunk_first) flush(chunk_first, step - chunk_first);
+}
+
+// Sum of the KS slices' partial outputs (part[z][16][N], fp32) of a split rows launch, rounded to
+// fp16 once: out[b][n] = (accumulate ? out[b][n] : 0) + sum_z part[z][b][n].
+__global__ __launch_bounds__(256) void rows_reduce_kernel(const float *__restrict__ part, __half *__restrict__ mul, int B, int N,
+                                                          int KS, int accumulate) {
+    const int n = blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
+    if (n >= N || row >= B) return;
+    float v = 0.f;
+    for (int z = 0; z < KS; z++) v += part[((size_t)z * 16 + row) * N + n];
+    __half *o16 = mul + (size_t)row * N + n;
+    if (accumulate) v += __half2float(*o16);
+    *o16 = __float2half_rn(v);
 }
 
 constexpr int kStreamWalk = 8;  // tiles one workgroup takes at most when a launch has more tiles than resident workgroups
@@ -1513,10 +1539,18 @@ static RowsFrag rows_frag(const StreamGeo &g) {
     r.total = r.xcf + 4 * 64 * 16;
     return r;
 }
+// layers deeper than 64 units: slices of at most 64 units, each with its own share of the workgroups
+constexpr int kRowsMaxSlices = 4;
+// Measured (us per call, 4-bit, 16 rows; 2 / 3 / 4 / 5 / 8 slices): 11008 -> 4096 15.4 / 14.9 / 14.4 / 16.3 / 18.6,
+// 28672 -> 8192 - / - / 32.6 / 37.9 / 34.0; 13824 -> 5120 3-bit 17.9 / 19.0 / 17.0 / 18.9 / 21.9.  Layers of up to
+// 64 units are slower in slices (4096 -> 11008: 12.3 whole, 15.5 in two, 21.4 in four).
+static int rows_slices(const StreamGeo &g) { return g.ng <= 64 ? 1 : kRowsMaxSlices; }
 
 size_t stream_rows_scratch_bytes(int bits, int B, int K, int N, int C) {
     if (B < 2) return 0;
     const StreamGeo geo = stream_geo(bits, K, N, C);
+    const int ks = rows_slices(geo);
+    if (ks > 1) return rows_frag(geo).total + (size_t)ks * 16 * N * 4;  // the operands, then the slices' fp32 partial outputs
     const size_t a = rows_scratch(B < kRowsMax ? B : kRowsMax, geo).total, b = rows_frag(geo).total;
     return a > b ? a : b;
 }
@@ -1525,7 +1559,8 @@ bool stream_rows_supported(int bits, int B, int K, int N, int C, int G) {
     if (B < 2 || B > kRowsMax) return false;
     if (!stream_supported(bits, 1, K, N, C, G)) return false;
     const StreamGeo geo = stream_geo(bits, K, N, C);
-    return geo.ng <= 64;  // at most 8 units per wavefront, 8 wavefronts per team
+    // at most 8 units per wavefront, 8 wavefronts per team: 64 units, or up to 4 slices of that
+    return ceil_div(geo.ng, rows_slices(geo)) <= 64;
 }
 
 template <int BITS, int W, int L, int TEAMS, bool STAGE>
@@ -1561,6 +1596,40 @@ hipError_t launch_stream_rows(int bits, const __half *vec, const uint8_t *stream
     // Two main kernels.  Measured (us, whole call, 4-bit; rows in LDS / rows in registers): 4096 -> 11008
     // 5 rows 12.0 / 12.4, 8 rows 12.4 / 12.5, 16 rows 14.1 / 12.6; 4096 -> 4096 8 rows 9.9 / 9.4, 16 rows
     // 12.4 / 9.6; 8192 -> 28672 8 rows 35.2 / 27.6, 16 rows - / 29.2; 8192 -> 8192 8 rows 16.7 / 14.8.
+    const int ks = rows_slices(geo);
+    if (ks > 1) {
+        // Deeper than 64 units: the tiles' units split over ks slices of workgroups (each keeps only
+        // its slice of the operands in registers), fp32 partial outputs per slice, one more launch
+        // that adds them up in slice order.  (The slice that finishes last adding them up inside the
+        // launch -- device-scope fences around an arrival counter -- measured 50 us slower per call.)
+        const RowsFrag f = rows_frag(geo);
+        su4 *xf = reinterpret_cast<su4 *>(reinterpret_cast<char *>(scratch) + f.xf);
+        float *xsum = reinterpret_cast<float *>(reinterpret_cast<char *>(scratch) + f.xsum);
+        su4 *xcf = reinterpret_cast<su4 *>(reinterpret_cast<char *>(scratch) + f.xcf);
+        float *part = reinterpret_cast<float *>(reinterpret_cast<char *>(scratch) + f.total);
+        const int us = ceil_div(geo.ng, ks);
+        if (us > 64) return hipErrorInvalidValue;
+        const int per = geo.ntiles < kStreamCus / ks ? geo.ntiles : kStreamCus / ks;  // workgroups of one slice
+        hipLaunchKernelGGL(stream_rows_frag_kernel, dim3(geo.ng + 1), dim3(256), 0, s, vec, stream, xf, xsum, xcf, B, geo);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        const size_t lds = (size_t)kRowsRegChunk * 8 * 256 * 4 + (size_t)16 * geo.ng * 4;
+#define CQ_SPLIT_GO(BITS_, L_, R_)                                                                                     \
+    hipLaunchKernelGGL((stream_rows_reg_kernel<BITS_, 8, L_, R_, true>), dim3(per * ks), dim3(512), lds, s, xf, xsum, xcf,  \
+                       stream, mul, B, accumulate, geo, part, ks, us)
+        if (bits == 4) {
+            if (us <= 32) CQ_SPLIT_GO(4, 4, 2);
+            else CQ_SPLIT_GO(4, 8, 1);
+        } else {
+            if (us <= 32) CQ_SPLIT_GO(3, 4, 2);
+            else CQ_SPLIT_GO(3, 8, 1);
+        }
+#undef CQ_SPLIT_GO
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(rows_reduce_kernel, dim3(ceil_div(N, 256), B), dim3(256), 0, s, part, mul, B, N, ks, accumulate);
+        return hipGetLastError();
+    }
     if (B >= 8 || geo.ng > 32 || rows_lds_bytes(B, geo, 8, false) > 160 * 1024) {
         // the rows as matrix-core operands in a buffer, then the kernel that keeps them in registers
         const RowsFrag f = rows_frag(geo);

@@ -392,7 +392,9 @@ def prepacked_rows_recommended(w_bits, rows, in_features, out_features, num_cher
     from 4 rows on layers of up to 32 units of 128 input channels, from 8 rows on deeper ones
     (measured on MI355X, checkpoint layout / stream in us: 4096 -> 11008 4-bit 2 rows 9.1 / 9.9, 4 rows
     11.2 / 10.6, 8 rows 16.8 / 12.4; 5120 -> 5120 3-bit 4 rows 7.9 / 11.9, 8 rows 13.7 / 11.9;
-    5120 -> 13824 3-bit 4 rows 14.5 / 16.0, 8 rows 19.6 / 16.1)."""
+    5120 -> 13824 3-bit 4 rows 14.5 / 16.0, 8 rows 19.6 / 16.1; 11008 -> 4096 4-bit 4 rows 10.6 / 13.9,
+    8 rows 17.0 / 13.9, 16 rows 21.4 / 14.4; 28672 -> 8192 4-bit 2 rows 27.4 / 30.2, 8 rows 36.1 / 30.4,
+    16 rows 41.3 / 32.6; 13824 -> 5120 3-bit 4 rows 13.6 / 16.3, 8 rows 19.8 / 16.4)."""
     if rows == 1:
         return prepack_recommended(w_bits, in_features, out_features, num_cherries, group_size)
     if rows < 1 or not prepack_supported(w_bits, rows, in_features, out_features, num_cherries, group_size):

@@ -218,11 +218,11 @@ def test_prepacked_c_abi_rejections(qc):
     assert lib.cherryq_prepack_supported(4, 2, 4096, 4096, 16, 128) == 1      # 2 to 16 rows: the rows kernel
     assert lib.cherryq_prepack_supported(4, 17, 4096, 4096, 16, 128) == 0
     assert lib.cherryq_prepack_supported(4, 16, 8192, 8192, 32, 128) == 1     # rows kept in registers
-    assert lib.cherryq_prepack_supported(3, 2, 13824, 5120, 48, 128) == 0     # more than 64 units per column
+    assert lib.cherryq_prepack_supported(3, 2, 13824, 5120, 48, 128) == 1     # more than 64 units per column: in slices
     assert lib.cherryq_prepack_supported(4, 1, 4096, 4096, 16, 64) == 0       # group size a multiple of 128
     assert lib.cherryq_prepack_supported(4, 1, 28672, 8192, 112, 128) == 1    # 224 units per column: the deepest taken
     assert lib.cherryq_prepack_supported(4, 1, 32768, 8192, 128, 128) == 0    # more than 224 units
-    assert lib.cherryq_prepack_supported(4, 16, 28672, 8192, 112, 128) == 0   # 2 to 16 rows: up to 64 units
+    assert lib.cherryq_prepack_supported(4, 16, 28672, 8192, 112, 128) == 1   # 2 to 16 rows: four slices of 56 units
     assert lib.cherryq_prepack_supported(3, 1, 13824, 5120, 48, 128) == 1
     nbytes = lib.cherryq_prepack_bytes(4, 4096, 1024, 16)
     buf = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
@@ -378,7 +378,10 @@ def test_prepacked_layers_with_more_tiles_than_resident_workgroups(bits, k, n):
 @pytest.mark.parametrize("bits,k,n,b", [(4, 4096, 11008, 16), (3, 4096, 11008, 16), (4, 4096, 4096, 8), (3, 4096, 4096, 2),
                                         (4, 8192, 1024, 8), (3, 1160, 264, 5), (4, 4096, 32008, 13), (4, 1024, 520, 16),
                                         (4, 8192, 4096, 16), (3, 8192, 1032, 9), (4, 4096, 4096, 3),
-                                        (3, 4096, 4112, 8), (4, 2048, 16, 16), (3, 1160, 264, 12), (4, 8192, 8200, 16)])
+                                        (3, 4096, 4112, 8), (4, 2048, 16, 16), (3, 1160, 264, 12), (4, 8192, 8200, 16),
+                                        # deeper than 64 units: slices of units with fp32 partial outputs and a summing launch
+                                        (4, 11008, 4096, 16), (3, 11008, 4096, 2), (3, 13824, 5120, 8), (4, 13824, 264, 11),
+                                        (4, 28672, 1032, 16), (3, 28672, 8192, 4), (4, 8320, 528, 5), (3, 16512, 4112, 16)])
 def test_prepacked_rows_against_the_c_oracle(bits, k, n, b):
     """2 to 16 activation rows over the repacked stream (compaction launch + matrix-core launch with
     real rows): against the C oracle, one-hot rows bit for bit (also with rows of very different
@@ -466,6 +469,29 @@ def test_quantlinear_routes_rows_to_the_stream_after_prepack():
     assert m.prepack()
     m.cpu()
     assert m._stream is None and not m.qweight.is_cuda
+
+
+def test_quantlinear_deep_layer_rows_after_prepack():
+    """A layer deeper than 64 units (11008 input channels) after prepack(): 8 to 16 rows leave the
+    checkpoint-layout batch kernel for the stream in slices, fewer stay; with the checkpoint buffers
+    released every batch size runs over the stream.  All agree with the module before prepack()."""
+    import cherryq_decoder as dec
+    print("[case] QuantLinear deep rows routing", flush=True)
+    cfg = dec.DecoderConfig(w_bits=3, group_size=128, cherry_fraction=1 / 256)
+    m = dec.random_packed_linear(cfg, 11008, 1032, torch.Generator(device="cuda").manual_seed(5), "cuda")
+    xs = {b: torch.randn(b, 11008, device="cuda", generator=torch.Generator(device="cuda").manual_seed(b)).half()
+          for b in (1, 2, 5, 8, 16, 19)}
+    before = {b: m(x) for b, x in xs.items()}
+    assert m.prepack()
+    for b, x in xs.items():
+        got = m(x)
+        assert orc.rel_l2(got.float().cpu().numpy(), before[b].float().cpu().numpy().astype(np.float64)) <= 5e-4, b
+        if b in (2, 5, 19):
+            assert torch.equal(got, before[b]), b   # same kernel as before
+        assert torch.equal(got, m(x)), b
+    m.prepack(release_reference=True)
+    for b, x in xs.items():
+        assert orc.rel_l2(m(x).float().cpu().numpy(), before[b].float().cpu().numpy().astype(np.float64)) <= 5e-4, b
 
 
 def _column_sample(p, cols):
