@@ -406,7 +406,7 @@ int cherryq_decode_attention_combine_f16(const void *partial, const float *max_s
  * accumulation, one rounding; act = norm_weight * fp16(hidden * rsqrt(mean(hidden^2) + eps)), the
  * final RMSNorm (:1064, :75-89) fused into the launch, or hidden itself when norm_weight is NULL.
  * A plain HBM stream over the matrix (the largest single read of a token step).  hidden_size a
- * multiple of 512, at most 8192 (cherryq_decode_head_supported); hidden, norm_weight, lm_head
+ * multiple of 8, at most 8192 (cherryq_decode_head_supported); hidden, norm_weight, lm_head
  * 16-byte aligned.
  */
 int cherryq_decode_head_supported(int vocab, int hidden_size);

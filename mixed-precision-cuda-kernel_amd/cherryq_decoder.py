@@ -343,6 +343,8 @@ class CherryLlamaDecoder(nn.Module):
         self.device_ = torch.device(device)
         if cfg.head_dim * cfg.num_attention_heads != cfg.hidden_size:
             raise ValueError("hidden_size must be num_attention_heads * head_dim")
+        if not _lib.cherryq_decode_head_supported(cfg.vocab_size, cfg.hidden_size):
+            raise ValueError("hidden_size must be a multiple of 8, at most 8192 (the head kernel's range)")
         gen = torch.Generator(device=self.device_).manual_seed(seed)
         h = cfg.hidden_size
         self.embed_tokens = (torch.randn(cfg.vocab_size, h, device=self.device_, generator=gen) * 0.02).half()
@@ -371,10 +373,9 @@ class CherryLlamaDecoder(nn.Module):
         self.attn_ml = torch.zeros(ATTN_SLICES, cfg.num_attention_heads, 2, dtype=torch.float32, device=self.device_)  # ... and (maximum, sum)
         self.logits16 = torch.zeros(1, cfg.vocab_size, **f16)
         self.history = torch.zeros(ml, dtype=torch.int64, device=self.device_)  # history[p]: token predicted at position p
-        self.lm_head_t = self.lm_head.t()
         self._graph = None
         self.fuse_norm = True
-        self.fuse_head = True  # final RMSNorm + fp16 head as one launch of the library's own kernel
+        self.fuse_head = True  # final RMSNorm inside the head launch (False: a launch of its own in front)
         # Attention dealt to ATTN_SLICES workgroups per head, combined by a repacked o_proj's staging: None =
         # for caches of 1024 positions and more.  (Measured per layer: 256-position cache 5.5 -> 5.0 us for
         # the attention but 4.3 -> 6.5 us for the projection; 1000 of 4096 positions 18.1 -> 11.3 us, 4000
@@ -527,23 +528,20 @@ class CherryLlamaDecoder(nn.Module):
                 matvec_group([down], self.up, [self.hid], vec_gate=self.gate, accumulate=True)
             if self.layer_trace is not None:  # validation only (eager runs): the hidden state after every layer
                 self.layer_trace.append(self.hid.clone())
-        if self.fuse_head and _lib.cherryq_decode_head_supported(cfg.vocab_size, cfg.hidden_size):
-            self._head(normed=False)
+        if self.fuse_head:
+            self._head(self.hid, self.norm)
         else:
             self._norm(self.norm)
-            self._head()
+            self._head(self.normed, None)
 
-    def _head(self, normed=True):
-        """Unquantised fp16 head, then the greedy tail on the device: next_token = argmax, recorded
-        in history[pos]; its embedding becomes the next step's hidden state; pos += 1.
-        normed=False: the final RMSNorm has not been applied yet and is fused into the head launch."""
+    def _head(self, row, norm_weight):
+        """Unquantised fp16 head over `row` (the final RMSNorm applied inside the launch when
+        norm_weight is given), then the greedy tail on the device: next_token = argmax, recorded
+        in history[pos]; its embedding becomes the next step's hidden state; pos += 1."""
         cfg = self.cfg
-        if normed:
-            torch.matmul(self.normed, self.lm_head_t, out=self.logits16)
-        else:
-            _ok(_lib.cherryq_decode_head_f16(self.hid.data_ptr(), self.norm.data_ptr(), cfg.rms_norm_eps,
-                                             self.lm_head.data_ptr(), self.logits16.data_ptr(), cfg.vocab_size,
-                                             cfg.hidden_size, _stream()), "head")
+        _ok(_lib.cherryq_decode_head_f16(row.data_ptr(), norm_weight.data_ptr() if norm_weight is not None else None,
+                                         cfg.rms_norm_eps, self.lm_head.data_ptr(), self.logits16.data_ptr(),
+                                         cfg.vocab_size, cfg.hidden_size, _stream()), "head")
         _ok(_lib.cherryq_decode_argmax_embed_f16(self.logits16.data_ptr(), cfg.vocab_size, self.embed_tokens.data_ptr(),
                                                  cfg.hidden_size, self.hid.data_ptr(), self.next_token.data_ptr(),
                                                  self.history.data_ptr(), self.history.numel(), self.pos.data_ptr(),
@@ -606,7 +604,7 @@ class CherryLlamaDecoder(nn.Module):
         _ok(_lib.cherryq_decode_add_rmsnorm_f16(self.hid.data_ptr(), delta, self.norm.data_ptr(),
                                                 self.normed.data_ptr(), cfg.hidden_size, cfg.rms_norm_eps, _stream()),
             "final norm")
-        self._head()
+        self._head(self.normed, None)
 
     def reset(self):
         self.pos.zero_()
@@ -676,7 +674,7 @@ class CherryLlamaDecoder(nn.Module):
             h = h + layer.down_proj(torch.nn.functional.silu(layer.gate_proj(x)) * layer.up_proj(x))
         self.normed.copy_(norm(h[T - 1:T], self.norm))
         self.pos.fill_(T - 1)
-        self._head()  # logits of the last prompt position; greedy tail: history[T-1], next embedding, pos = T
+        self._head(self.normed, None)  # logits of the last prompt position; greedy tail: history[T-1], next embedding, pos = T
         return self.logits
 
     @torch.inference_mode()

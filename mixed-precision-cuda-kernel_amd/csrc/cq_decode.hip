@@ -683,29 +683,33 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const __half *__restrict_
 // HBM stream: every wavefront keeps the whole activation row in registers (CH pieces of 16 bytes
 // per lane), normalises it itself (no LDS, no barrier) and then takes rows v = w, w + waves, ...,
 // one row = CH loads of 1 KB, the next row's loads in flight while the current one is multiplied.
+// RAGGED: the hidden size Hr is not a multiple of 512 (CH = ceil(Hr / 512)); lanes whose piece of the
+// last 1 KB lies past the row read nothing and multiply zeros.
 typedef uint32_t hu4 __attribute__((ext_vector_type(4)));
 
-template <int CH>
+template <int CH, bool RAGGED>
 __global__ __launch_bounds__(256) void head_kernel(const __half *__restrict__ h, const __half *__restrict__ norm_w,
                                                    float eps, const __half *__restrict__ W,
-                                                   __half *__restrict__ logits, int V) {
-    constexpr int H = 512 * CH;
+                                                   __half *__restrict__ logits, int V, int Hr) {
+    const int H = RAGGED ? Hr : 512 * CH;
     const int lane = threadIdx.x & 63;
     const int w = blockIdx.x * 4 + (threadIdx.x >> 6), nw = gridDim.x * 4;
+    const hu4 zero = {0u, 0u, 0u, 0u};
+    auto has = [&](int c) { return !RAGGED || c < CH - 1 || ((CH - 1) * 64 + lane) * 8 < H; };  // (H % 8 == 0)
     auto load_row = [&](hu4 (&dst)[CH], int v) {
         const hu4 *row = reinterpret_cast<const hu4 *>(W + (size_t)v * H);
 #pragma unroll
-        for (int c = 0; c < CH; c++) dst[c] = __builtin_nontemporal_load(row + c * 64 + lane);
+        for (int c = 0; c < CH; c++) dst[c] = has(c) ? __builtin_nontemporal_load(row + c * 64 + lane) : zero;
     };
     float x[CH][8];
     {
         hu4 xr[CH];
 #pragma unroll
-        for (int c = 0; c < CH; c++) xr[c] = reinterpret_cast<const hu4 *>(h)[c * 64 + lane];
+        for (int c = 0; c < CH; c++) xr[c] = has(c) ? reinterpret_cast<const hu4 *>(h)[c * 64 + lane] : zero;
         if (norm_w) {
             hu4 nr[CH];
 #pragma unroll
-            for (int c = 0; c < CH; c++) nr[c] = reinterpret_cast<const hu4 *>(norm_w)[c * 64 + lane];
+            for (int c = 0; c < CH; c++) nr[c] = has(c) ? reinterpret_cast<const hu4 *>(norm_w)[c * 64 + lane] : zero;
             float ss = 0.f;
 #pragma unroll
             for (int c = 0; c < CH; c++)
@@ -760,17 +764,21 @@ __global__ __launch_bounds__(256) void head_kernel(const __half *__restrict__ h,
     }
 }
 
-bool head_supported(int vocab, int hidden) { return vocab > 0 && hidden >= 512 && hidden <= 8192 && hidden % 512 == 0; }
+bool head_supported(int vocab, int hidden) { return vocab > 0 && hidden >= 8 && hidden <= 8192 && hidden % 8 == 0; }
 
 hipError_t launch_head(const __half *h, const __half *norm_w, float eps, const __half *W, __half *logits, int vocab,
                        int hidden, hipStream_t stream) {
     if (!head_supported(vocab, hidden)) return hipErrorInvalidValue;
     int grid = ceil_div(vocab, 4);
     if (grid > 1024) grid = 1024;  // four wavefronts per SIMD
-    switch (hidden / 512) {
-#define CQ_HEAD_CASE(CH_)                                                                                         \
-    case CH_:                                                                                                     \
-        hipLaunchKernelGGL(head_kernel<CH_>, dim3(grid), dim3(256), 0, stream, h, norm_w, eps, W, logits, vocab); \
+    const bool ragged = hidden % 512 != 0;
+    switch (ceil_div(hidden, 512)) {
+#define CQ_HEAD_CASE(CH_)                                                                                                       \
+    case CH_:                                                                                                                   \
+        if (ragged)                                                                                                             \
+            hipLaunchKernelGGL((head_kernel<CH_, true>), dim3(grid), dim3(256), 0, stream, h, norm_w, eps, W, logits, vocab, hidden);  \
+        else                                                                                                                    \
+            hipLaunchKernelGGL((head_kernel<CH_, false>), dim3(grid), dim3(256), 0, stream, h, norm_w, eps, W, logits, vocab, hidden); \
         break;
         CQ_HEAD_CASE(1) CQ_HEAD_CASE(2) CQ_HEAD_CASE(3) CQ_HEAD_CASE(4) CQ_HEAD_CASE(5) CQ_HEAD_CASE(6) CQ_HEAD_CASE(7)
         CQ_HEAD_CASE(8) CQ_HEAD_CASE(9) CQ_HEAD_CASE(10) CQ_HEAD_CASE(11) CQ_HEAD_CASE(12) CQ_HEAD_CASE(13)

@@ -136,7 +136,9 @@ def test_silu_mul_kernel(dec):
     assert rel(o, torch.nn.functional.silu(g) * u) < 1e-3
 
 
-@pytest.mark.parametrize("V,H", [(32000, 4096), (1000, 1024), (517, 512), (32003, 5120), (4099, 8192)])
+@pytest.mark.parametrize("V,H", [(32000, 4096), (1000, 1024), (517, 512), (32003, 5120), (4099, 8192),
+                                 # hidden sizes that are not whole kilobyte pieces per wavefront
+                                 (1000, 256), (4099, 384), (517, 8), (2003, 4104), (1000, 6656 + 128), (333, 8184)])
 def test_head_kernel_with_fused_final_norm(dec, V, H):
     """fp16 head (final RMSNorm fused or not) against float64 on the same fp16 operands: one
     rounding of the fp32-accumulated sum, rel-L2 below 1e-3; a one-hot row returns the matrix
@@ -176,11 +178,11 @@ def test_head_validation(dec):
     W = torch.zeros(8, 4096, dtype=torch.float16, device="cuda")
     out = torch.zeros(1, 8, dtype=torch.float16, device="cuda")
     assert lib.cherryq_decode_head_supported(32000, 4096) == 1
-    assert lib.cherryq_decode_head_supported(32000, 256) == 0 and lib.cherryq_decode_head_supported(32000, 8704) == 0
-    assert lib.cherryq_decode_head_supported(32000, 4100) == 0
+    assert lib.cherryq_decode_head_supported(32000, 256) == 1 and lib.cherryq_decode_head_supported(32000, 8704) == 0
+    assert lib.cherryq_decode_head_supported(32000, 4100) == 0 and lib.cherryq_decode_head_supported(32000, 0) == 0
     assert lib.cherryq_decode_head_f16(None, None, 0.0, W.data_ptr(), out.data_ptr(), 8, 4096, stream()) == -1
     assert lib.cherryq_decode_head_f16(h.data_ptr(), None, 0.0, W.data_ptr(), out.data_ptr(), 0, 4096, stream()) == -2
-    assert lib.cherryq_decode_head_f16(h.data_ptr(), None, 0.0, W.data_ptr(), out.data_ptr(), 8, 256, stream()) == -7
+    assert lib.cherryq_decode_head_f16(h.data_ptr(), None, 0.0, W.data_ptr(), out.data_ptr(), 8, 252, stream()) == -7
     assert lib.cherryq_decode_head_f16(h.data_ptr() + 2, None, 0.0, W.data_ptr(), out.data_ptr(), 8, 4096, stream()) == -6
 
 
