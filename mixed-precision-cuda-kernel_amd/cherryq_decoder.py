@@ -426,19 +426,21 @@ class CherryLlamaDecoder(nn.Module):
                 m._stream = None
         self._graph = None
 
-    def prepack(self, only_recommended=True):
+    def prepack(self, only_recommended=True, release_reference=False):
         """Repack, once, every linear whose shape the library recommends it for (on MI355X: all
         seven projections of the LLaMA-7B, -13B and -70B shapes) into the weight stream the batch-1
         kernel reads fastest; the token step then uses the stream kernels for them.  The
-        checkpoint-layout buffers stay (the batched prompt pass reads them).  Returns the number of
-        layers repacked."""
+        checkpoint-layout buffers stay (the batched prompt pass reads them) unless
+        `release_reference` frees them: one copy of the weights in memory, the prompt pass then goes
+        over the streams 16 rows at a time, and state_dict() needs unprepack() first.  Returns the
+        number of layers repacked."""
         n = 0
         for layer in self.layers:
             for m in layer.children():
                 if only_recommended and not quant_cuda.prepack_recommended(m.w_bits, m.in_features, m.out_features,
                                                                            m.num_cherries, m.group_size):
                     continue
-                n += bool(m.prepack())
+                n += bool(m.prepack(release_reference=release_reference))
         self._graph = None
         return n
 
@@ -453,10 +455,13 @@ class CherryLlamaDecoder(nn.Module):
         n = self.lm_head.numel() * 2
         for layer in self.layers:
             for m in layer.children():
-                n += sum(b.numel() * b.element_size() for b in (m.qweight, m.scales, m.cherry_weight, m.cherry_indices))
+                n += m.packed_bytes()
         return n
 
     def _linear(self, m: QuantLinear, x, out):
+        if getattr(m, "_released", False):  # only the weight stream is left
+            quant_cuda.matvec_prepacked_cherryq(m.w_bits, x, m._stream, out, m.in_features, m.num_cherries)
+            return
         quant_cuda.matmul_cherryq(m.w_bits, x, m.qweight, m.cherry_weight, m.cherry_indices, m.scales, out,
                                   m.group_size, accumulate=False)
 

@@ -207,6 +207,13 @@ class QuantLinear(nn.Module):
         return super().state_dict(*args, **kwargs)
 
     @torch.no_grad()
+    def packed_bytes(self) -> int:
+        """Bytes of the four checkpoint buffers (codes, scales, cherry rows, cherry indices), also
+        while prepack(release_reference=True) holds them only as a weight stream."""
+        kn = self.in_features - self.num_cherries
+        groups = -(-kn // self.group_size)
+        return (kn // 8 * self.w_bits + 2 * groups + 2 * self.num_cherries) * self.out_features + 2 * self.num_cherries
+
     def prepack(self, release_reference: bool = False):
         """Rearrange the packed buffers, once, into the weight stream the batch-1 kernel of this
         GPU reads fastest (quant_cuda.prepack_cherryq).  The state-dict buffers stay as they are

@@ -102,12 +102,13 @@ def save_quantized(model: nn.Module, save_dir: str) -> str:
 
 
 def from_quantized(model_name_or_path: str, model_type: str = "llama", torch_dtype=None, device_map=None,
-                   prepack: bool = True):
+                   prepack: bool = True, release_reference: bool = False):
     """Build this package's decoder from a directory written by `save_quantized` (here or by the
     reference, utils.py:125-149) and load the packed weights.  `device_map` may be None / "cuda" /
     a device; the whole model lives on that one device.  `prepack` (default) also repacks, once,
     the layers whose shape the library recommends it for into the weight streams the batch-1
-    kernels read fastest (CherryLlamaDecoder.prepack); the checkpoint-layout buffers stay."""
+    kernels read fastest (CherryLlamaDecoder.prepack); the checkpoint-layout buffers stay unless
+    `release_reference` frees them (one copy of the weights on the device: a decode deployment)."""
     if model_type != "llama":
         raise NotImplementedError(f"model_type {model_type!r}")
     if torch_dtype not in (None, torch.float16):
@@ -132,5 +133,5 @@ def from_quantized(model_name_or_path: str, model_type: str = "llama", torch_dty
     sd = torch.load(path, map_location="cpu", weights_only=True)
     model.load_reference_state_dict(sd)
     if prepack and model.device_.type == "cuda":
-        model.prepack()
+        model.prepack(release_reference=release_reference)
     return model

@@ -295,7 +295,24 @@ def test_small_decoder_matches_dense_reference(dec, bits):
         _ = model.reference_logits(ids[:4])
         graph2 = model.step_logits(ids, use_graph=True)
         assert torch.equal(graph, eager) and torch.equal(graph2, eager), ("prepacked", fuse_norm)
+    # only the weight streams kept (one copy of the weights): the same token step bit for bit, the
+    # literal launch sequence and the batched prompt pass go over the streams too
+    bytes_before = model.step_bytes()
+    kept = eager
+    assert model.prepack(only_recommended=False, release_reference=True) == 14
+    assert all(m.qweight.numel() == 0 for layer in model.layers for m in layer.children())
+    assert model.step_bytes() == bytes_before
+    model._graph = None
+    assert torch.equal(model.step_logits(ids, use_graph=False), kept)
+    assert torch.equal(model.step_logits(ids, use_graph=True), kept)
+    literal = model.step_logits(ids, use_graph=False, grouped=False)
+    for t in range(ids.numel()):
+        assert rel(literal[t], want[t]) < 2e-2, (t, "released, literal")
+    assert rel(model.prefill(ids)[0], want[-1]) < 2e-2
+    with pytest.raises(RuntimeError):
+        model.layers[0].q_proj.state_dict()
     model.unprepack()
+    assert all(m.qweight.numel() > 0 for layer in model.layers for m in layer.children())
     model._graph = None
     model.fuse_norm = True
     out, times, total = model.generate(ids[:4], 8, use_graph=True)
@@ -357,6 +374,11 @@ def test_saved_checkpoint_reloads_to_identical_logits(dec, tmp_path):
     got = repacked.step_logits(ids)
     for t in range(ids.numel()):
         assert rel(got[t], want[t]) < 5e-3, t
+    # a decode deployment: only the streams stay on the device; same logits as with both layouts
+    lean = cq_utils.from_quantized(str(tmp_path), release_reference=True)
+    assert all(m.qweight.numel() == 0 and m._stream is not None for m in lean.layers[1].children())
+    assert torch.equal(lean.step_logits(ids), got)
+    assert lean.step_bytes() == repacked.step_bytes()
 
 
 def test_argmax_embed_tail_kernel(dec):
