@@ -129,6 +129,9 @@ hipError_t launch_stream_group(int bits, const __half *vec, const __half *norm_w
                                const StreamMember *members, int count, int K, int C, int accumulate, hipStream_t s);
 bool stream_group_supported(int bits, int K, int C, int G, const int *Ns, int count);
 // 2 to 16 activation rows over the stream: a compaction launch into `scratch`, then the main launch
+bool stream_cu_rows_supported(int bits, int B, int K, int N, int C);
+hipError_t launch_stream_cu_rows(int bits, const __half *vec, const uint8_t *stream, __half *mul, int B, int K, int N, int C,
+                                 int accumulate, hipStream_t s);
 size_t stream_rows_scratch_bytes(int bits, int B, int K, int N, int C);
 bool stream_rows_supported(int bits, int B, int K, int N, int C, int G);
 hipError_t launch_stream_rows(int bits, const __half *vec, const uint8_t *stream, __half *mul, int B, int K, int N,

@@ -1593,6 +1593,9 @@ static hipError_t launch_rows_cfg(const unsigned short *xs, const float *xsum, c
 hipError_t launch_stream_rows(int bits, const __half *vec, const uint8_t *stream, __half *mul, int B, int K, int N,
                               int C, int accumulate, void *scratch, hipStream_t s) {
     const StreamGeo geo = stream_geo(bits, K, N, C);
+    static const bool cu_rows_off = getenv("CHERRYQ_CU_ROWS_OFF") != nullptr;
+    if (!cu_rows_off && stream_cu_rows_supported(bits, B, K, N, C))
+        return launch_stream_cu_rows(bits, vec, stream, mul, B, K, N, C, accumulate, s);
     // Two main kernels.  Measured (us, whole call, 4-bit; rows in LDS / rows in registers): 4096 -> 11008
     // 5 rows 12.0 / 12.4, 8 rows 12.4 / 12.5, 16 rows 14.1 / 12.6; 4096 -> 4096 8 rows 9.9 / 9.4, 16 rows
     // 12.4 / 9.6; 8192 -> 28672 8 rows 35.2 / 27.6, 16 rows - / 29.2; 8192 -> 8192 8 rows 16.7 / 14.8.

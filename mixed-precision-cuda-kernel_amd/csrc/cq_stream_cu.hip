@@ -805,6 +805,353 @@ hipError_t launch_stream_cu(int bits, const __half *vec, const __half *norm_w, f
 }
 
 
+// ---- two to four activation rows --------------------------------------------------------------------
+// The matrix-core tile that the one-row kernel fills with 16 copies of its row takes four different
+// rows at the same price: A row m holds activation row m % 4, so accumulator entry r of EVERY lane
+// group is row r's sum and the lane groups still share the units' scales a quarter each.  Same
+// launch shape as stream_cu_body (one workgroup per compute unit, staging wavefronts first, D0 units
+// requested before the barrier, a ring of D behind it); what changes is the staging: a row's slice
+// of NB blocks is a task, all wavefronts share the tasks of the B rows (the computing ones once
+// their first requests are out), each passes its tasks through a piece of LDS of its own, and the
+// rows' cherry activations are left in LDS for the teams' cherry wavefronts.
+template <int BITS>
+__device__ inline sf4_t unit_dot_rows(const su4 w, const unsigned short *xa) {
+    const sf4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (BITS == 4) {
+        const su4 y = {w[0] >> 8, w[1] >> 8, w[2] >> 8, w[3] >> 8};
+        const sh8_t a0 = *reinterpret_cast<const sh8_t *>(xa);
+        const sh8_t a1 = *reinterpret_cast<const sh8_t *>(xa + 8);
+        const sh8_t a2 = *reinterpret_cast<const sh8_t *>(xa + 16);
+        const sh8_t a3 = *reinterpret_cast<const sh8_t *>(xa + 24);
+        const su4 b0 = {w[0] & 0x000f000fu, y[0] & 0x000f000fu, w[1] & 0x000f000fu, y[1] & 0x000f000fu};
+        const su4 b1 = {w[2] & 0x000f000fu, y[2] & 0x000f000fu, w[3] & 0x000f000fu, y[3] & 0x000f000fu};
+        const su4 b2 = {w[0] & 0x00f000f0u, y[0] & 0x00f000f0u, w[1] & 0x00f000f0u, y[1] & 0x00f000f0u};
+        const su4 b3 = {w[2] & 0x00f000f0u, y[2] & 0x00f000f0u, w[3] & 0x00f000f0u, y[3] & 0x00f000f0u};
+        sf4_t dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, as_h8(b0), zero4, 0, 0, 0);
+        sf4_t dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, as_h8(b2), zero4, 0, 0, 0);
+        dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, as_h8(b1), dl, 0, 0, 0);
+        dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(a3, as_h8(b3), dh, 0, 0, 0);
+        return dl * 16777216.0f + dh * 1048576.0f;
+    } else {
+        const su3 y = {w[0] >> 9, w[1] >> 9, w[2] >> 9};
+        const sh8_t a0 = *reinterpret_cast<const sh8_t *>(xa);
+        const sh8_t a2 = *reinterpret_cast<const sh8_t *>(xa + 8);
+        const sh8_t a4 = *reinterpret_cast<const sh8_t *>(xa + 16);
+        const sh8_t a1 = *reinterpret_cast<const sh8_t *>(xa + 24);
+        const uint32_t z = (y[0] & 0x00400040u) | ((y[1] & 0x00400040u) << 1) | ((y[2] & 0x00400040u) << 2);
+        const su4 b0 = {w[0] & 0x00070007u, w[1] & 0x00070007u, w[2] & 0x00070007u, y[0] & 0x00070007u};
+        const su4 b2 = {w[0] & 0x00380038u, w[1] & 0x00380038u, w[2] & 0x00380038u, y[0] & 0x00380038u};
+        const su4 b4 = {w[0] & 0x01c001c0u, w[1] & 0x01c001c0u, w[2] & 0x01c001c0u, z};
+        const su4 b1 = {y[1] & 0x00070007u, y[2] & 0x00070007u, (y[1] >> 3) & 0x00070007u, (y[2] >> 3) & 0x00070007u};
+        sf4_t d0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, as_h8(b0), zero4, 0, 0, 0);
+        const sf4_t d3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, as_h8(b2), zero4, 0, 0, 0);
+        const sf4_t d6 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a4, as_h8(b4), zero4, 0, 0, 0);
+        d0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, as_h8(b1), d0, 0, 0, 0);
+        return d0 * 16777216.0f + d3 * 2097152.0f + d6 * 262144.0f;
+    }
+}
+
+constexpr int kCuRows = 4;     // activation rows of a stream_cu_rows_kernel launch (fewer: the rest are not staged)
+constexpr int kCuRowsNB = 2;   // blocks of 512 compacted positions per staging task
+constexpr int kCuRowsPad = 8;  // halves between the compacted rows in LDS: the four rows a load instruction reads lie in different banks
+
+template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D>
+__global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_rows_kernel(const __half *__restrict__ x,
+                                                                               const uint8_t *__restrict__ stream,
+                                                                               __half *__restrict__ mul, int K, int C, int N,
+                                                                               int G, int accumulate, int P, int B) {
+    constexpr int R = kCuRows;
+    constexpr int NC = W * TEAMS;
+    constexpr int NT = 64 * (NC + S);
+    constexpr int UB = BITS == 4 ? 1024 : 768;
+    constexpr float kGrid = BITS == 4 ? -7.5f : -3.5f;
+    constexpr int NBR = kCuRowsNB;
+    constexpr int XS = NBR + 1;
+    constexpr int NW = NC + S;                          // all wavefronts stage: the computing ones once their first requests are out
+    constexpr int TPW = (kCuRows * ((W * L + 4 * NBR - 1) / (4 * NBR)) + NW - 1) / NW;  // staging tasks (a row's slice of NBR blocks) per wavefront at most
+    constexpr int TB = XS <= 3 ? TPW : 1;               // ... requested at a time (what the registers hold)
+    constexpr int PIECE = XS * 512 + 8;                 // halves of a wavefront's piece of LDS
+    static_assert(D0 <= D && D <= L && L % D == 0 && L % 4 == 0, "ring slots are fixed per unit across tiles");
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kq = lane >> 4, nn = lane & 15;
+    const int bid = blockIdx.x;
+    const int ng = (K - C + kStreamUnitK - 1) / kStreamUnitK;
+    const int Knp512 = (ng * kStreamUnitK + 511) & ~511;
+    const int nblk = Knp512 >> 9;
+    const uint32_t off_cherry = ((uint32_t)ng * 32u + 255u) & ~255u;
+    const uint32_t off_units = off_cherry + (((uint32_t)C * 32u + 255u) & ~255u);
+    const uint32_t record_bytes = off_units + (uint32_t)ng * UB;
+    const uint32_t hdr_bytes = ((uint32_t)(Knp512 + 2 * ((C + 31) & ~31)) + 255u) & ~255u;
+    const int ntiles = (N + kStreamTileCols - 1) / kStreamTileCols;
+    // LDS: the wavefronts' pieces | compacted rows [R][Knp512 + pad] | unit sums [4 nblk][R] | cherry activations [R][128] | partial outputs [P][NC][R][16]
+    const int XROW = Knp512 + kCuRowsPad;
+    unsigned short *s_piece = reinterpret_cast<unsigned short *>(smem);
+    unsigned short *s_xs = s_piece + NW * PIECE;
+    float *s_xsum = reinterpret_cast<float *>(s_xs + R * XROW);
+    unsigned short *s_cx = reinterpret_cast<unsigned short *>(s_xsum + 4 * nblk * R);
+    float *s_red = reinterpret_cast<float *>(s_cx + R * 128);
+    const int tstride = G * TEAMS;
+
+    // ---- staging: task t = slice t % nslices (NBR blocks of 512 compacted positions) of row t / nslices;
+    // wavefront w takes the tasks w, w + NW, ...: raw slice -> its piece of LDS -> gather, unit sums,
+    // and the row's activations at the cherry channels whose columns start in the slice
+    const int nslices = (nblk + NBR - 1) / NBR, ntasks = B * nslices;
+    auto stage_tasks = [&]() {
+        const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc((void *)stream, 0, (int)hdr_bytes, kSFlags);
+        unsigned short *piece = s_piece + wave * PIECE;
+#pragma unroll
+        for (int t0 = 0; t0 < TPW; t0 += TB) {
+            su4 xr[TB][XS];
+            su2 tb[TB][NBR];
+            uint32_t cl[TB][2];
+#pragma unroll
+            for (int tt = 0; tt < TB; tt++) {
+                const int task = wave + (t0 + tt) * NW;
+                const bool on = task < ntasks;
+                const int r = task / nslices, sl = task - r * nslices, b0 = sl * NBR, b1 = min(nblk, b0 + NBR);
+                // (a descriptor per row: what lies behind the row's end reads as zeros)
+                const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)(x + (size_t)(on ? r : 0) * K), 0, K * 2, kSFlags);
+#pragma unroll
+                for (int i = 0; i < XS; i++)
+                    xr[tt][i] = __builtin_amdgcn_raw_buffer_load_b128(rx, on ? (uint32_t)(b0 * 512 + i * 512 + lane * 8) * 2u : kSOob, 0, 0);
+#pragma unroll
+                for (int i = 0; i < NBR; i++)
+                    tb[tt][i] = __builtin_amdgcn_raw_buffer_load_b64(rh, on && b0 + i < b1 ? (uint32_t)((b0 + i) * 512 + lane * 8) : kSOob, 0, 0);
+#pragma unroll
+                for (int h = 0; h < 2; h++)
+                    cl[tt][h] = __builtin_amdgcn_raw_buffer_load_b16(rh, on && lane + 64 * h < C ? (uint32_t)(Knp512 + 2 * (lane + 64 * h)) : kSOob, 0, 0);
+            }
+#pragma unroll
+            for (int tt = 0; tt < TB; tt++) {
+                const int task = wave + (t0 + tt) * NW;
+                if (task < ntasks) {
+                    const int r = task / nslices, sl = task - r * nslices, b0 = sl * NBR, b1 = min(nblk, b0 + NBR);
+                    unsigned short *xs_r = s_xs + r * XROW;
+#pragma unroll
+                    for (int i = 0; i < XS; i++) reinterpret_cast<su4 *>(piece + i * 512)[lane] = xr[tt][i];
+#pragma unroll
+                    for (int i = 0; i < NBR; i++) {
+                        const int blk = b0 + i;
+                        if (blk < b1) {
+                            const su2 t = tb[tt][i];
+                            unsigned short h[8];
+#pragma unroll
+                            for (int j = 0; j < 8; j++)
+                                h[j] = piece[i * 512 + 64 * j + lane + (int)((t[j >> 2] >> (8 * (j & 3))) & 0xffu)];
+                            float f[4];
+#pragma unroll
+                            for (int j = 0; j < 8; j++) xs_r[blk * 512 + 64 * j + lane] = h[j];
+#pragma unroll
+                            for (int u = 0; u < 4; u++)
+                                f[u] = __half2float(__ushort_as_half(h[2 * u])) + __half2float(__ushort_as_half(h[2 * u + 1]));
+                            const float s01 = swap32_add(f[0], f[1]);
+                            const float s23 = swap32_add(f[2], f[3]);
+                            const float rs = row_sum(swap16_add(s01, s23));
+                            if (nn == 0) s_xsum[(blk * 4 + ((kq >> 1) | ((kq & 1) << 1))) * R + r] = rs;
+                        }
+                    }
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        const int e = lane + 64 * h, col = (int)(cl[tt][h] & 0xffffu);
+                        const int owner = min(col / (NBR * 512), nslices - 1);
+                        if (e < C) {
+                            if (owner == sl) s_cx[r * 128 + e] = piece[col - b0 * 512];
+                        } else if (sl == 0) {
+                            s_cx[r * 128 + e] = 0;
+                        }
+                    }
+                }
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_wave_barrier();  // (the piece is rewritten for the next task)
+            }
+        }
+    };
+
+    if (wave < S) {
+        __builtin_amdgcn_s_setprio(3);
+        stage_tasks();
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+    } else {
+        // ---- computing wavefront `cls` of team `team`, on tiles bid + G (team + TEAMS j)
+        const int cwv = wave - S;
+        const int team = cwv / W, cls = cwv % W;
+        const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(stream + hdr_bytes), 0, (int)min((unsigned long long)ntiles * record_bytes, 0xffffffffull), kSFlags);
+        uint32_t sc[L / 4];
+        su4 wbuf[D];
+        su4 cw[4];
+        const bool cherry_wave = cls == W - 1;
+        int tcur = bid + G * team;
+        bool vcur = tcur < ntiles;
+        uint32_t tb = (uint32_t)tcur * record_bytes;
+        auto load_cherry = [&](uint32_t base, bool valid) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int lg = 4 * j + kq;
+                if (32 * j < C)
+                    cw[j] = __builtin_amdgcn_raw_buffer_load_b128(
+                        rt, valid && 8 * lg < C ? off_cherry + (uint32_t)(lg * 16 + nn) * 16u : kSOob, base, 2);
+            }
+        };
+        const uint32_t sc_off = (uint32_t)((cls + kq * W) * 32 + nn * 2);
+        auto load_scale = [&](int i4, uint32_t base, bool valid) -> uint32_t {
+            return __builtin_amdgcn_raw_buffer_load_b16(rt, valid && cls + (4 * i4 + kq) * W < ng ? sc_off : kSOob,
+                                                        base + 4 * i4 * W * 32, 0);
+        };
+        const uint32_t w_off = off_units + (uint32_t)(cls * UB + lane * (BITS * 4));
+        auto load_unit = [&](int i, uint32_t base, bool valid) -> su4 {
+            const uint32_t off = valid && cls + i * W < ng ? w_off : kSOob;
+            if constexpr (BITS == 4) {
+                return __builtin_amdgcn_raw_buffer_load_b128(rt, off, base + i * W * UB, 2);
+            } else {
+                const su3 v = __builtin_amdgcn_raw_buffer_load_b96(rt, off, base + i * W * UB, 2);
+                return (su4){v[0], v[1], v[2], 0u};
+            }
+        };
+        if (cherry_wave) load_cherry(tb, vcur);
+#pragma unroll
+        for (int i = 0; i < L / 4; i++) sc[i] = load_scale(i, tb, vcur);
+#pragma unroll
+        for (int i = 0; i < D0; i++) wbuf[i] = load_unit(i, tb, vcur);
+        __builtin_amdgcn_sched_barrier(0);
+        stage_tasks();
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+#pragma unroll
+        for (int i = D0; i < D; i++) wbuf[i] = load_unit(i, tb, vcur);
+        const unsigned short *xs_l = s_xs + (nn & (R - 1)) * XROW + 32 * kq;   // A row nn holds activation row nn % 4
+        su4 ca[4];
+        if (cherry_wave) {
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+                if (32 * q < C) ca[q] = *reinterpret_cast<const su4 *>(s_cx + (nn & (R - 1)) * 128 + 32 * q + 8 * kq);
+        }
+#pragma unroll 1
+        for (int j = 0; j < P; j++) {
+            const int tnext = tcur + tstride;
+            const bool vnext = tnext < ntiles;
+            const uint32_t tbn = (uint32_t)tnext * record_bytes;
+            sf4_t dc = {0.f, 0.f, 0.f, 0.f};
+            if (cherry_wave) {
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    if (32 * q < C) dc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(ca[q]), as_h8(cw[q]), dc, 0, 0, 0);
+                load_cherry(tbn, vnext);
+            }
+            sf4_t tt = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < L; i++) {
+                const bool real = cls + i * W < ng;
+                const int up = real ? cls + i * W : 0;
+                const float sf = (i & 3) == kq ? __half2float(__ushort_as_half((unsigned short)sc[i >> 2])) : 0.f;
+                const su4 w = wbuf[i % D];
+                const sf4_t v = unit_dot_rows<BITS>(w, xs_l + up * kStreamUnitK);
+                if (i + D < L) wbuf[i % D] = load_unit(i + D, tb, vcur);
+                else wbuf[i % D] = load_unit(i + D - L, tbn, vnext);
+                const sf4_t xsum = *reinterpret_cast<const sf4_t *>(s_xsum + up * R);
+                tt += (v + kGrid * xsum) * sf;
+                if ((i & 3) == 3) sc[i >> 2] = load_scale(i >> 2, tbn, vnext);
+            }
+            // the four lane groups' quarters; lane group kq then stores row kq
+            float out = 0.f;
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                float t = swap32_add(tt[r], tt[r]);
+                t = swap16_add(t, t) + dc[r];
+                out = kq == r ? t : out;
+            }
+            s_red[((j * NC + cwv) * R + kq) * 16 + nn] = out;
+            tcur = tnext;
+            vcur = vnext;
+            tb = tbn;
+            if (!vcur) break;
+        }
+    }
+
+    // ---- across a tile's wavefronts, then one store per output and row
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    for (int o = tid; o < 16 * R * P * TEAMS; o += NT) {
+        const int col = o & 15, r = (o >> 4) & (R - 1), jt = o >> 6, j = jt / TEAMS, t = jt - j * TEAMS;
+        const int tile = bid + G * (t + TEAMS * j), n = tile * 16 + col;
+        if (tile < ntiles && n < N && r < B) {
+            const float *red = s_red + ((j * NC + t * W) * R + r) * 16 + col;
+            float v = 0.f;
+#pragma unroll
+            for (int c = 0; c < W; c++) v += red[c * R * 16];
+            __half *o16 = mul + (size_t)r * N + n;
+            if (accumulate) v += __half2float(*o16);
+            *o16 = __float2half_rn(v);
+        }
+    }
+}
+
+static size_t cu_rows_lds_bytes(const StreamGeo &g, const CuCfg &c, int P) {
+    const int Knp512 = (g.ng * kStreamUnitK + 511) & ~511;
+    size_t need = (size_t)(c.W * c.TEAMS + c.S) * ((kCuRowsNB + 1) * 512 + 8) * 2 + (size_t)kCuRows * (Knp512 + kCuRowsPad) * 2 + (size_t)(Knp512 / 128) * kCuRows * 4 +
+                  (size_t)kCuRows * 128 * 2 + (size_t)P * c.W * c.TEAMS * kCuRows * 16 * 4;
+    const size_t alone = 80 * 1024 + 1024;  // more than half of a compute unit's LDS: one workgroup per compute unit
+    return need > alone ? need : alone;
+}
+
+// (entries 5, 6 and 8 -- more than 96 units per column, 16 wavefronts of 128 registers -- would spill with four rows' sums)
+constexpr bool cu_rows_cfg(int i) { return i != 5 && i != 6 && i != 8; }
+
+bool stream_cu_rows_supported(int bits, int B, int K, int N, int C) {
+    if (B < 2 || B > kCuRows || N % 8) return false;
+    const int Ns[1] = {N};
+    if (!stream_cu_supported(bits, K, C, Ns, 1)) return false;
+    const StreamGeo geo = stream_geo(bits, K, N, C);
+    const int idx = cu_pick(geo.ng, ceil_div(geo.ntiles, kCuCus));
+    if (!cu_rows_cfg(idx)) return false;
+    const int tiles[1] = {geo.ntiles};
+    const CuSplit sp = cu_split(tiles, 1, kCuCfgs[idx].TEAMS);
+    return cu_rows_lds_bytes(geo, kCuCfgs[idx], sp.walk) <= 160 * 1024;
+}
+
+template <int BITS, int I>
+static hipError_t launch_cu_rows_cfg(const __half *vec, const uint8_t *stream, __half *mul, int B, const StreamGeo &geo,
+                                     const CuSplit &sp, int accumulate, hipStream_t s) {
+    constexpr CuCfg c = kCuCfgs[I];
+    auto kern = stream_cu_rows_kernel<BITS, c.W, c.L, c.TEAMS, c.S, c.NB, c.D0, c.D>;
+    static bool raised[kCuMaxDevices] = {};
+    if (hipError_t e = cu_raise_lds(kern, raised)) return e;
+    const size_t lds = cu_rows_lds_bytes(geo, c, sp.walk);
+    hipLaunchKernelGGL(kern, dim3(sp.total), dim3(64 * (c.W * c.TEAMS + c.S)), lds, s, vec, stream, mul, geo.K, geo.C, geo.N,
+                       sp.wgs[0], accumulate, sp.walk, B);
+    return hipGetLastError();
+}
+
+// vec (B, K), mul (B, N), 2 <= B <= 4; the caller has asked stream_cu_rows_supported()
+hipError_t launch_stream_cu_rows(int bits, const __half *vec, const uint8_t *stream, __half *mul, int B, int K, int N, int C,
+                                 int accumulate, hipStream_t s) {
+    const StreamGeo geo = stream_geo(bits, K, N, C);
+    const int idx = cu_pick(geo.ng, ceil_div(geo.ntiles, kCuCus));
+    if (idx < 0 || !cu_rows_cfg(idx) || B < 2 || B > kCuRows) return hipErrorInvalidValue;
+    const int tiles[1] = {geo.ntiles};
+    const CuSplit sp = cu_split(tiles, 1, kCuCfgs[idx].TEAMS);
+    if (sp.walk > kCuMaxWalk) return hipErrorInvalidValue;
+#define CQ_ROWS_BITS(BITS_)                                                                               \
+    switch (idx) {                                                                                        \
+        case 0: return launch_cu_rows_cfg<BITS_, 0>(vec, stream, mul, B, geo, sp, accumulate, s);          \
+        case 1: return launch_cu_rows_cfg<BITS_, 1>(vec, stream, mul, B, geo, sp, accumulate, s);          \
+        case 2: return launch_cu_rows_cfg<BITS_, 2>(vec, stream, mul, B, geo, sp, accumulate, s);          \
+        case 3: return launch_cu_rows_cfg<BITS_, 3>(vec, stream, mul, B, geo, sp, accumulate, s);          \
+        case 4: return launch_cu_rows_cfg<BITS_, 4>(vec, stream, mul, B, geo, sp, accumulate, s);          \
+        case 7: return launch_cu_rows_cfg<BITS_, 7>(vec, stream, mul, B, geo, sp, accumulate, s);          \
+        case 9: return launch_cu_rows_cfg<BITS_, 9>(vec, stream, mul, B, geo, sp, accumulate, s);          \
+        default: return launch_cu_rows_cfg<BITS_, 10>(vec, stream, mul, B, geo, sp, accumulate, s);        \
+    }
+    if (bits == 4) CQ_ROWS_BITS(4)
+    CQ_ROWS_BITS(3)
+#undef CQ_ROWS_BITS
+}
+
 // ---- several layers of one shape in every workgroup -----------------------------------------------
 // gate_proj + up_proj -> fp16(fp16(silu(gate)) * up).  Up to 32 units per column: three pairs of
 // two-wavefront teams (16 units per wavefront) and 2 + 2 staging wavefronts of four blocks, i.e. the
