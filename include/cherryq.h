@@ -234,6 +234,14 @@ int cherryq_prepack_supported(int w_bits, int batch, int in_features, int out_fe
  * LLaMA-7B, -13B and -70B projection among them; within 3 % at worst on the shapes measured), 0
  * elsewhere or if unsupported: what a loader asks before spending the extra copy of the weights. */
 int cherryq_prepack_recommended(int w_bits, int in_features, int out_features, int num_cherries, int group_size);
+/* The same for `batch` activation rows, for a caller that holds both layouts: 1 where
+ * cherryq_matmul_prepacked_f16 measured faster on MI355X than cherryq_vecquant{3,4}matmul_f16 over
+ * the checkpoint layout -- one row as above; 2 to 4 rows wherever the four-row form of the
+ * one-workgroup-per-compute-unit kernel takes the layer (up to 96 units of 128 input channels);
+ * from 4 rows on layers of up to 32 units and from 8 rows on deeper ones otherwise; 0 beyond 16
+ * rows.  No counterpart in the reference (its kernel loops over the rows, quant_cuda_kernel.cu:797). */
+int cherryq_prepack_rows_recommended(int w_bits, int batch, int in_features, int out_features, int num_cherries,
+                                     int group_size);
 /* The kernel cherryq_matvec_prepacked_f16 launches for a layer, as it appears in a profiler's
  * kernel trace (without template arguments): "cq::stream_cu_kernel" (one workgroup per compute
  * unit) or "cq::stream_kernel"; "" for shapes the entry point does not take. */

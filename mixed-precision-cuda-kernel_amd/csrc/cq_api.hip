@@ -422,6 +422,15 @@ int cherryq_prepack_recommended(int w_bits, int in_features, int out_features, i
     return cq::stream_faster(w_bits, in_features, out_features, num_cherries) ? 1 : 0;
 }
 
+int cherryq_prepack_rows_recommended(int w_bits, int batch, int in_features, int out_features, int num_cherries,
+                                     int group_size) {
+    if (batch == 1) return cherryq_prepack_recommended(w_bits, in_features, out_features, num_cherries, group_size);
+    if (batch < 1 || !cherryq_prepack_supported(w_bits, batch, in_features, out_features, num_cherries, group_size)) return 0;
+    if (cq::stream_cu_rows_supported(w_bits, batch, in_features, out_features, num_cherries)) return 1;
+    const int units = (in_features - num_cherries + cq::kStreamUnitK - 1) / cq::kStreamUnitK;
+    return batch >= (units <= 32 ? 4 : 8) ? 1 : 0;
+}
+
 const char *cherryq_matvec_prepacked_kernel_name(int w_bits, int in_features, int out_features, int num_cherries) {
     if (!cq::stream_supported(w_bits, 1, in_features, out_features, num_cherries, cq::kStreamUnitK)) return "";
     return cq::stream_uses_cu(w_bits, in_features, out_features, num_cherries) ? "cq::stream_cu_kernel" : "cq::stream_kernel";

@@ -869,7 +869,6 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_rows_kernel(co
     constexpr int XS = NBR + 1;
     constexpr int NW = NC + S;                          // all wavefronts stage: the computing ones once their first requests are out
     constexpr int TPW = (kCuRows * ((W * L + 4 * NBR - 1) / (4 * NBR)) + NW - 1) / NW;  // staging tasks (a row's slice of NBR blocks) per wavefront at most
-    constexpr int TB = XS <= 3 ? TPW : 1;               // ... requested at a time (what the registers hold)
     constexpr int PIECE = XS * 512 + 8;                 // halves of a wavefront's piece of LDS
     static_assert(D0 <= D && D <= L && L % D == 0 && L % 4 == 0, "ring slots are fixed per unit across tiles");
     extern __shared__ __align__(16) unsigned char smem[];
@@ -898,80 +897,80 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_rows_kernel(co
     // wavefront w takes the tasks w, w + NW, ...: raw slice -> its piece of LDS -> gather, unit sums,
     // and the row's activations at the cherry channels whose columns start in the slice
     const int nslices = (nblk + NBR - 1) / NBR, ntasks = B * nslices;
-    auto stage_tasks = [&]() {
+    su4 xr[TPW][XS];
+    su2 tbl[TPW][NBR];
+    uint32_t cl[TPW][2];
+    auto stage_request = [&]() {
         const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc((void *)stream, 0, (int)hdr_bytes, kSFlags);
+#pragma unroll
+        for (int tt = 0; tt < TPW; tt++) {
+            const int task = wave + tt * NW;
+            const bool on = task < ntasks;
+            const int r = task / nslices, sl = task - r * nslices, b0 = sl * NBR, b1 = min(nblk, b0 + NBR);
+            // (a descriptor per row: what lies behind the row's end reads as zeros)
+            const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)(x + (size_t)(on ? r : 0) * K), 0, K * 2, kSFlags);
+#pragma unroll
+            for (int i = 0; i < XS; i++)
+                xr[tt][i] = __builtin_amdgcn_raw_buffer_load_b128(rx, on ? (uint32_t)(b0 * 512 + i * 512 + lane * 8) * 2u : kSOob, 0, 0);
+#pragma unroll
+            for (int i = 0; i < NBR; i++)
+                tbl[tt][i] = __builtin_amdgcn_raw_buffer_load_b64(rh, on && b0 + i < b1 ? (uint32_t)((b0 + i) * 512 + lane * 8) : kSOob, 0, 0);
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+                cl[tt][h] = __builtin_amdgcn_raw_buffer_load_b16(rh, on && lane + 64 * h < C ? (uint32_t)(Knp512 + 2 * (lane + 64 * h)) : kSOob, 0, 0);
+        }
+    };
+    auto stage_process = [&]() {
         unsigned short *piece = s_piece + wave * PIECE;
 #pragma unroll
-        for (int t0 = 0; t0 < TPW; t0 += TB) {
-            su4 xr[TB][XS];
-            su2 tb[TB][NBR];
-            uint32_t cl[TB][2];
-#pragma unroll
-            for (int tt = 0; tt < TB; tt++) {
-                const int task = wave + (t0 + tt) * NW;
-                const bool on = task < ntasks;
+        for (int tt = 0; tt < TPW; tt++) {
+            const int task = wave + tt * NW;
+            if (task < ntasks) {
                 const int r = task / nslices, sl = task - r * nslices, b0 = sl * NBR, b1 = min(nblk, b0 + NBR);
-                // (a descriptor per row: what lies behind the row's end reads as zeros)
-                const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)(x + (size_t)(on ? r : 0) * K), 0, K * 2, kSFlags);
+                unsigned short *xs_r = s_xs + r * XROW;
 #pragma unroll
-                for (int i = 0; i < XS; i++)
-                    xr[tt][i] = __builtin_amdgcn_raw_buffer_load_b128(rx, on ? (uint32_t)(b0 * 512 + i * 512 + lane * 8) * 2u : kSOob, 0, 0);
+                for (int i = 0; i < XS; i++) reinterpret_cast<su4 *>(piece + i * 512)[lane] = xr[tt][i];
 #pragma unroll
-                for (int i = 0; i < NBR; i++)
-                    tb[tt][i] = __builtin_amdgcn_raw_buffer_load_b64(rh, on && b0 + i < b1 ? (uint32_t)((b0 + i) * 512 + lane * 8) : kSOob, 0, 0);
+                for (int i = 0; i < NBR; i++) {
+                    const int blk = b0 + i;
+                    if (blk < b1) {
+                        const su2 t = tbl[tt][i];
+                        unsigned short h[8];
 #pragma unroll
-                for (int h = 0; h < 2; h++)
-                    cl[tt][h] = __builtin_amdgcn_raw_buffer_load_b16(rh, on && lane + 64 * h < C ? (uint32_t)(Knp512 + 2 * (lane + 64 * h)) : kSOob, 0, 0);
-            }
+                        for (int j = 0; j < 8; j++)
+                            h[j] = piece[i * 512 + 64 * j + lane + (int)((t[j >> 2] >> (8 * (j & 3))) & 0xffu)];
+                        float f[4];
 #pragma unroll
-            for (int tt = 0; tt < TB; tt++) {
-                const int task = wave + (t0 + tt) * NW;
-                if (task < ntasks) {
-                    const int r = task / nslices, sl = task - r * nslices, b0 = sl * NBR, b1 = min(nblk, b0 + NBR);
-                    unsigned short *xs_r = s_xs + r * XROW;
+                        for (int j = 0; j < 8; j++) xs_r[blk * 512 + 64 * j + lane] = h[j];
 #pragma unroll
-                    for (int i = 0; i < XS; i++) reinterpret_cast<su4 *>(piece + i * 512)[lane] = xr[tt][i];
-#pragma unroll
-                    for (int i = 0; i < NBR; i++) {
-                        const int blk = b0 + i;
-                        if (blk < b1) {
-                            const su2 t = tb[tt][i];
-                            unsigned short h[8];
-#pragma unroll
-                            for (int j = 0; j < 8; j++)
-                                h[j] = piece[i * 512 + 64 * j + lane + (int)((t[j >> 2] >> (8 * (j & 3))) & 0xffu)];
-                            float f[4];
-#pragma unroll
-                            for (int j = 0; j < 8; j++) xs_r[blk * 512 + 64 * j + lane] = h[j];
-#pragma unroll
-                            for (int u = 0; u < 4; u++)
-                                f[u] = __half2float(__ushort_as_half(h[2 * u])) + __half2float(__ushort_as_half(h[2 * u + 1]));
-                            const float s01 = swap32_add(f[0], f[1]);
-                            const float s23 = swap32_add(f[2], f[3]);
-                            const float rs = row_sum(swap16_add(s01, s23));
-                            if (nn == 0) s_xsum[(blk * 4 + ((kq >> 1) | ((kq & 1) << 1))) * R + r] = rs;
-                        }
-                    }
-#pragma unroll
-                    for (int h = 0; h < 2; h++) {
-                        const int e = lane + 64 * h, col = (int)(cl[tt][h] & 0xffffu);
-                        const int owner = min(col / (NBR * 512), nslices - 1);
-                        if (e < C) {
-                            if (owner == sl) s_cx[r * 128 + e] = piece[col - b0 * 512];
-                        } else if (sl == 0) {
-                            s_cx[r * 128 + e] = 0;
-                        }
+                        for (int u = 0; u < 4; u++)
+                            f[u] = __half2float(__ushort_as_half(h[2 * u])) + __half2float(__ushort_as_half(h[2 * u + 1]));
+                        const float s01 = swap32_add(f[0], f[1]);
+                        const float s23 = swap32_add(f[2], f[3]);
+                        const float rs = row_sum(swap16_add(s01, s23));
+                        if (nn == 0) s_xsum[(blk * 4 + ((kq >> 1) | ((kq & 1) << 1))) * R + r] = rs;
                     }
                 }
-                asm volatile("" ::: "memory");
-                __builtin_amdgcn_wave_barrier();  // (the piece is rewritten for the next task)
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const int e = lane + 64 * h, col = (int)(cl[tt][h] & 0xffffu);
+                    const int owner = min(col / (NBR * 512), nslices - 1);
+                    if (e < C) {
+                        if (owner == sl) s_cx[r * 128 + e] = piece[col - b0 * 512];
+                    } else if (sl == 0) {
+                        s_cx[r * 128 + e] = 0;
+                    }
+                }
             }
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_wave_barrier();  // (the piece is rewritten for the next task)
         }
     };
 
     if (wave < S) {
         __builtin_amdgcn_s_setprio(3);
-        stage_tasks();
+        stage_request();
+        stage_process();
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
         __builtin_amdgcn_s_barrier();
     } else {
@@ -1011,13 +1010,15 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_rows_kernel(co
                 return (su4){v[0], v[1], v[2], 0u};
             }
         };
+        stage_request();   // (activations first: the barrier waits for them, not for the weights)
+        __builtin_amdgcn_sched_barrier(0);
         if (cherry_wave) load_cherry(tb, vcur);
 #pragma unroll
         for (int i = 0; i < L / 4; i++) sc[i] = load_scale(i, tb, vcur);
 #pragma unroll
         for (int i = 0; i < D0; i++) wbuf[i] = load_unit(i, tb, vcur);
         __builtin_amdgcn_sched_barrier(0);
-        stage_tasks();
+        stage_process();
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");

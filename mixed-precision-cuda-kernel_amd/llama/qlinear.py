@@ -69,11 +69,6 @@ class QuantLinear(nn.Module):
     # instead of the fused dequantise + MFMA kernel (measured crossover on MI355X: the fused kernel
     # is 1.6x faster at 128 rows of a 4096 -> 11008 layer, level at 512, 1.3x slower at 2048).
     prefill_rows = 512
-    # from this many rows (up to 16) a prepack()ed layer runs the rows kernel over the weight stream;
-    # measured on 4096 -> 11008, 4-bit (us, stream / checkpoint layout): 2 rows 9.8 / 9.2, 4 rows
-    # 10.5 / 11.3, 8 rows 12.5 / 16.8, 16 rows 12.7 / 19.0
-    stream_rows_min = 4
-
     @classmethod
     @contextmanager
     def dmode(cls, layerwise_dequantize=True):
@@ -266,12 +261,12 @@ class QuantLinear(nn.Module):
             rows = x2.shape[0]
             # over the repacked stream: one row, and the small batches that measured faster there than on
             # the checkpoint layout's kernels (the matrix-core tile of the one-row kernel filled with real
-            # rows: from 4 rows, from 8 on layers of more than 32 units); with the checkpoint buffers
-            # released, everything the stream kernels take
+            # rows: quant_cuda.prepacked_rows_recommended); with the checkpoint buffers released,
+            # everything the stream kernels take
             shape = (self.w_bits, rows, self.in_features, self.out_features, self.num_cherries, self.group_size)
             if stream is not None and (rows == 1 or (2 <= rows <= 16 and (
                     quant_cuda.prepack_supported(*shape) if self._released else
-                    rows >= self.stream_rows_min and quant_cuda.prepacked_rows_recommended(*shape)))):
+                    quant_cuda.prepacked_rows_recommended(*shape)))):
                 out = torch.empty(rows, self.out_features, dtype=torch.float16, device=stream.device)
                 quant_cuda.matvec_prepacked_cherryq(self.w_bits, x2, stream, out, self.in_features, self.num_cherries)
             elif self._released:

@@ -66,6 +66,8 @@ _lib.cherryq_prepack_supported.argtypes = [_int, _int, _int, _int, _int, _int]
 _lib.cherryq_prepack_supported.restype = _int
 _lib.cherryq_prepack_recommended.argtypes = [_int, _int, _int, _int, _int]
 _lib.cherryq_prepack_recommended.restype = _int
+_lib.cherryq_prepack_rows_recommended.argtypes = [_int, _int, _int, _int, _int, _int]
+_lib.cherryq_prepack_rows_recommended.restype = _int
 _lib.cherryq_prepack_f16.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _sz, _int, _int, _int, _int, _vp]
 _lib.cherryq_prepack_f16.restype = _int
 _lib.cherryq_unprepack_f16.argtypes = [_int, _vp, _sz, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp]
@@ -388,19 +390,15 @@ def prepack_recommended(w_bits, in_features, out_features, num_cherries, group_s
 
 def prepacked_rows_recommended(w_bits, rows, in_features, out_features, num_cherries, group_size) -> bool:
     """Whether `rows` activation rows run faster over a layer's repacked stream than over its
-    checkpoint buffers (for a caller that holds both).  One row: prepack_recommended().  Several:
-    from 4 rows on layers of up to 32 units of 128 input channels, from 8 rows on deeper ones
-    (measured on MI355X, checkpoint layout / stream in us: 4096 -> 11008 4-bit 2 rows 9.1 / 9.9, 4 rows
-    11.2 / 10.6, 8 rows 16.8 / 12.4; 5120 -> 5120 3-bit 4 rows 7.9 / 11.9, 8 rows 13.7 / 11.9;
-    5120 -> 13824 3-bit 4 rows 14.5 / 16.0, 8 rows 19.6 / 16.1; 11008 -> 4096 4-bit 4 rows 10.6 / 13.9,
-    8 rows 17.0 / 13.9, 16 rows 21.4 / 14.4; 28672 -> 8192 4-bit 2 rows 27.4 / 30.2, 8 rows 36.1 / 30.4,
-    16 rows 41.3 / 32.6; 13824 -> 5120 3-bit 4 rows 13.6 / 16.3, 8 rows 19.8 / 16.4)."""
-    if rows == 1:
-        return prepack_recommended(w_bits, in_features, out_features, num_cherries, group_size)
-    if rows < 1 or not prepack_supported(w_bits, rows, in_features, out_features, num_cherries, group_size):
-        return False
-    units = -(-(int(in_features) - int(num_cherries)) // 128)
-    return rows >= (4 if units <= 32 else 8)
+    checkpoint buffers (for a caller that holds both): cherryq_prepack_rows_recommended.  Measured on
+    MI355X, checkpoint layout / stream in us: 4096 -> 11008 4-bit 2 rows 9.1 / 6.6, 4 rows 11.3 / 7.4,
+    8 rows 16.8 / 12.4; 4096 -> 4096 4 rows 8.1 / 5.6; 5120 -> 5120 3-bit 4 rows 7.9 / 7.5, 8 rows 13.7 / 11.9;
+    5120 -> 13824 3-bit 4 rows 14.0 / 9.9, 8 rows 19.6 / 16.1; 8192 -> 28672 4 rows 32.9 / 23.1; 11008 -> 4096
+    4-bit 2 rows 8.9 / 8.3, 4 rows 11.1 / 9.8, 8 rows 17.0 / 13.9, 16 rows 21.4 / 14.4; 28672 -> 8192 4-bit
+    2 rows 27.4 / 30.2, 8 rows 36.1 / 30.4, 16 rows 41.3 / 32.6; 13824 -> 5120 3-bit 4 rows 13.6 / 16.3,
+    8 rows 19.8 / 16.4."""
+    return bool(_lib.cherryq_prepack_rows_recommended(int(w_bits), int(rows), int(in_features), int(out_features),
+                                                      int(num_cherries), int(group_size)))
 
 
 def prepacked_kernel_name(w_bits, in_features, out_features, num_cherries) -> str:

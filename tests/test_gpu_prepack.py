@@ -381,7 +381,12 @@ def test_prepacked_layers_with_more_tiles_than_resident_workgroups(bits, k, n):
                                         (3, 4096, 4112, 8), (4, 2048, 16, 16), (3, 1160, 264, 12), (4, 8192, 8200, 16),
                                         # deeper than 64 units: slices of units with fp32 partial outputs and a summing launch
                                         (4, 11008, 4096, 16), (3, 11008, 4096, 2), (3, 13824, 5120, 8), (4, 13824, 264, 11),
-                                        (4, 28672, 1032, 16), (3, 28672, 8192, 4), (4, 8320, 528, 5), (3, 16512, 4112, 16)])
+                                        (4, 28672, 1032, 16), (3, 28672, 8192, 4), (4, 8320, 528, 5), (3, 16512, 4112, 16),
+                                        # two to four rows on every geometry of the one-workgroup-per-compute-unit kernel
+                                        (4, 4096, 11008, 4), (3, 4096, 11008, 3), (4, 4096, 8200, 2), (3, 4096, 32008, 4),
+                                        (4, 5120, 5120, 4), (3, 5120, 13824, 4), (4, 6144, 12304, 3), (3, 8192, 8192, 4),
+                                        (4, 8192, 12304, 2), (4, 11008, 4096, 4), (3, 11008, 4096, 3), (4, 12288, 4096, 4),
+                                        (3, 12288, 1032, 2), (4, 1160, 264, 4), (3, 2048, 16, 2), (4, 8192, 1024, 3)])
 def test_prepacked_rows_against_the_c_oracle(bits, k, n, b):
     """2 to 16 activation rows over the repacked stream (compaction launch + matrix-core launch with
     real rows): against the C oracle, one-hot rows bit for bit (also with rows of very different
@@ -429,12 +434,13 @@ def test_prepacked_rows_against_the_c_oracle(bits, k, n, b):
 
 
 def test_quantlinear_routes_rows_to_the_stream_after_prepack():
-    """QuantLinear.forward after prepack(): 1 row and 4..16 rows run over the weight stream (also with
-    the checkpoint-layout buffers released), 2 / 3 / 17 rows on the checkpoint layout; all agree with
-    the module before prepack()."""
+    """QuantLinear.forward after prepack(): 1 to 16 rows run over the weight stream (also with the
+    checkpoint-layout buffers released), 17 rows on the checkpoint layout; all agree with the
+    module before prepack()."""
     from llama.qlinear import QuantLinear
     from llama.quantizer import FullSymQuantizer
     import cherryq_decoder as dec
+    import quant_cuda
     print("[case] QuantLinear rows routing", flush=True)
     cfg = dec.DecoderConfig(w_bits=4, group_size=128, cherry_fraction=1 / 256)
     m = dec.random_packed_linear(cfg, 4096, 1024, torch.Generator(device="cuda").manual_seed(2), "cuda")
@@ -446,8 +452,10 @@ def test_quantlinear_routes_rows_to_the_stream_after_prepack():
         got = m(x)
         assert got.shape == (b, 1024)
         assert orc.rel_l2(got.float().cpu().numpy(), before[b].float().cpu().numpy().astype(np.float64)) <= 5e-4, b
-        if b in (2, 3, 17):
+        if b == 17:
             assert torch.equal(got, before[b]), b   # same kernel as before
+        else:
+            assert quant_cuda.prepacked_rows_recommended(4, b, 4096, 1024, m.num_cherries, 128), b
     m.prepack(release_reference=True)
     # only the stream is left: every batch size runs over it (2 and 3 rows on the rows kernel,
     # more than 16 in pieces of 16)
@@ -472,21 +480,22 @@ def test_quantlinear_routes_rows_to_the_stream_after_prepack():
 
 
 def test_quantlinear_deep_layer_rows_after_prepack():
-    """A layer deeper than 64 units (11008 input channels) after prepack(): 8 to 16 rows leave the
-    checkpoint-layout batch kernel for the stream in slices, fewer stay; with the checkpoint buffers
-    released every batch size runs over the stream.  All agree with the module before prepack()."""
+    """A layer deeper than 64 units (11008 input channels) after prepack(): 2 to 4 rows take the
+    four-row form of the one-row kernel, 8 to 16 rows leave the checkpoint-layout batch kernel for
+    the stream in slices, 5 and 19 stay; with the checkpoint buffers released every batch size runs
+    over the stream.  All agree with the module before prepack()."""
     import cherryq_decoder as dec
     print("[case] QuantLinear deep rows routing", flush=True)
     cfg = dec.DecoderConfig(w_bits=3, group_size=128, cherry_fraction=1 / 256)
     m = dec.random_packed_linear(cfg, 11008, 1032, torch.Generator(device="cuda").manual_seed(5), "cuda")
     xs = {b: torch.randn(b, 11008, device="cuda", generator=torch.Generator(device="cuda").manual_seed(b)).half()
-          for b in (1, 2, 5, 8, 16, 19)}
+          for b in (1, 2, 4, 5, 8, 16, 19)}
     before = {b: m(x) for b, x in xs.items()}
     assert m.prepack()
     for b, x in xs.items():
         got = m(x)
         assert orc.rel_l2(got.float().cpu().numpy(), before[b].float().cpu().numpy().astype(np.float64)) <= 5e-4, b
-        if b in (2, 5, 19):
+        if b in (5, 19):
             assert torch.equal(got, before[b]), b   # same kernel as before
         assert torch.equal(got, m(x)), b
     m.prepack(release_reference=True)
