@@ -851,16 +851,19 @@ __device__ inline sf4_t unit_dot_rows(const su4 w, const unsigned short *xa) {
     }
 }
 
-constexpr int kCuRows = 4;     // activation rows of a stream_cu_rows_kernel launch (fewer: the rest are not staged)
+constexpr int kCuRows = 8;     // activation rows of a stream_cu_rows_kernel launch at most (R = 4 or 8; rows from B on are not staged)
 constexpr int kCuRowsNB = 2;   // blocks of 512 compacted positions per staging task
 constexpr int kCuRowsPad = 8;  // halves between the compacted rows in LDS: the four rows a load instruction reads lie in different banks
 
-template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D>
+// R = 8: A row m holds activation row m % 8, lane groups kq and kq ^ 2 receive the same four rows
+// (4 (kq & 1) + r) and share the units' scales half each.
+template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, int R>
 __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_rows_kernel(const __half *__restrict__ x,
                                                                                const uint8_t *__restrict__ stream,
                                                                                __half *__restrict__ mul, int K, int C, int N,
                                                                                int G, int accumulate, int P, int B) {
-    constexpr int R = kCuRows;
+    static_assert(R == 4 || R == 8, "rows per matrix-core tile");
+    constexpr int NRED = 16 / R;   // lane groups that receive the same rows: they share the units' scales
     constexpr int NC = W * TEAMS;
     constexpr int NT = 64 * (NC + S);
     constexpr int UB = BITS == 4 ? 1024 : 768;
@@ -868,7 +871,7 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_rows_kernel(co
     constexpr int NBR = kCuRowsNB;
     constexpr int XS = NBR + 1;
     constexpr int NW = NC + S;                          // all wavefronts stage: the computing ones once their first requests are out
-    constexpr int TPW = (kCuRows * ((W * L + 4 * NBR - 1) / (4 * NBR)) + NW - 1) / NW;  // staging tasks (a row's slice of NBR blocks) per wavefront at most
+    constexpr int TPW = (R * ((W * L + 4 * NBR - 1) / (4 * NBR)) + NW - 1) / NW;  // staging tasks (a row's slice of NBR blocks) per wavefront at most
     constexpr int PIECE = XS * 512 + 8;                 // halves of a wavefront's piece of LDS
     static_assert(D0 <= D && D <= L && L % D == 0 && L % 4 == 0, "ring slots are fixed per unit across tiles");
     extern __shared__ __align__(16) unsigned char smem[];
@@ -979,7 +982,9 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_rows_kernel(co
         const int team = cwv / W, cls = cwv % W;
         const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(
             (void *)(stream + hdr_bytes), 0, (int)min((unsigned long long)ntiles * record_bytes, 0xffffffffull), kSFlags);
-        uint32_t sc[L / 4];
+        uint32_t sc[L / NRED];
+        const int red_id = kq / (R / 4);            // which share of the units' scales this lane group keeps
+        const int rowbase = 4 * (kq % (R / 4));     // accumulator entry r of this lane is row rowbase + r
         su4 wbuf[D];
         su4 cw[4];
         const bool cherry_wave = cls == W - 1;
@@ -995,10 +1000,10 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_rows_kernel(co
                         rt, valid && 8 * lg < C ? off_cherry + (uint32_t)(lg * 16 + nn) * 16u : kSOob, base, 2);
             }
         };
-        const uint32_t sc_off = (uint32_t)((cls + kq * W) * 32 + nn * 2);
-        auto load_scale = [&](int i4, uint32_t base, bool valid) -> uint32_t {
-            return __builtin_amdgcn_raw_buffer_load_b16(rt, valid && cls + (4 * i4 + kq) * W < ng ? sc_off : kSOob,
-                                                        base + 4 * i4 * W * 32, 0);
+        const uint32_t sc_off = (uint32_t)((cls + red_id * W) * 32 + nn * 2);
+        auto load_scale = [&](int sl, uint32_t base, bool valid) -> uint32_t {
+            return __builtin_amdgcn_raw_buffer_load_b16(rt, valid && cls + (NRED * sl + red_id) * W < ng ? sc_off : kSOob,
+                                                        base + NRED * sl * W * 32, 0);
         };
         const uint32_t w_off = off_units + (uint32_t)(cls * UB + lane * (BITS * 4));
         auto load_unit = [&](int i, uint32_t base, bool valid) -> su4 {
@@ -1014,7 +1019,7 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_rows_kernel(co
         __builtin_amdgcn_sched_barrier(0);
         if (cherry_wave) load_cherry(tb, vcur);
 #pragma unroll
-        for (int i = 0; i < L / 4; i++) sc[i] = load_scale(i, tb, vcur);
+        for (int i = 0; i < L / NRED; i++) sc[i] = load_scale(i, tb, vcur);
 #pragma unroll
         for (int i = 0; i < D0; i++) wbuf[i] = load_unit(i, tb, vcur);
         __builtin_amdgcn_sched_barrier(0);
@@ -1031,6 +1036,7 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_rows_kernel(co
             for (int q = 0; q < 4; q++)
                 if (32 * q < C) ca[q] = *reinterpret_cast<const su4 *>(s_cx + (nn & (R - 1)) * 128 + 32 * q + 8 * kq);
         }
+        const float *xsum_l = s_xsum + rowbase;
 #pragma unroll 1
         for (int j = 0; j < P; j++) {
             const int tnext = tcur + tstride;
@@ -1048,24 +1054,30 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_rows_kernel(co
             for (int i = 0; i < L; i++) {
                 const bool real = cls + i * W < ng;
                 const int up = real ? cls + i * W : 0;
-                const float sf = (i & 3) == kq ? __half2float(__ushort_as_half((unsigned short)sc[i >> 2])) : 0.f;
+                const float sf = (i % NRED) == red_id ? __half2float(__ushort_as_half((unsigned short)sc[i / NRED])) : 0.f;
                 const su4 w = wbuf[i % D];
                 const sf4_t v = unit_dot_rows<BITS>(w, xs_l + up * kStreamUnitK);
                 if (i + D < L) wbuf[i % D] = load_unit(i + D, tb, vcur);
                 else wbuf[i % D] = load_unit(i + D - L, tbn, vnext);
-                const sf4_t xsum = *reinterpret_cast<const sf4_t *>(s_xsum + up * R);
+                const sf4_t xsum = *reinterpret_cast<const sf4_t *>(xsum_l + up * R);
                 tt += (v + kGrid * xsum) * sf;
-                if ((i & 3) == 3) sc[i >> 2] = load_scale(i >> 2, tbn, vnext);
+                if ((i % NRED) == NRED - 1) sc[i / NRED] = load_scale(i / NRED, tbn, vnext);
             }
-            // the four lane groups' quarters; lane group kq then stores row kq
-            float out = 0.f;
+            // the shares of the lane groups that hold the same rows; every lane then stores R / 4 of its rows
+            float fin[4];
 #pragma unroll
-            for (int r = 0; r < R; r++) {
+            for (int r = 0; r < 4; r++) {
                 float t = swap32_add(tt[r], tt[r]);
-                t = swap16_add(t, t) + dc[r];
-                out = kq == r ? t : out;
+                if constexpr (NRED == 4) t = swap16_add(t, t);
+                fin[r] = t + dc[r];
             }
-            s_red[((j * NC + cwv) * R + kq) * 16 + nn] = out;
+            float *red = s_red + ((j * NC + cwv) * R + rowbase) * 16 + nn;
+            if constexpr (R == 4) {
+                red[kq * 16] = kq == 0 ? fin[0] : kq == 1 ? fin[1] : kq == 2 ? fin[2] : fin[3];
+            } else {
+                red[(2 * red_id) * 16] = red_id ? fin[2] : fin[0];
+                red[(2 * red_id + 1) * 16] = red_id ? fin[3] : fin[1];
+            }
             tcur = tnext;
             vcur = vnext;
             tb = tbn;
@@ -1078,7 +1090,7 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_rows_kernel(co
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     for (int o = tid; o < 16 * R * P * TEAMS; o += NT) {
-        const int col = o & 15, r = (o >> 4) & (R - 1), jt = o >> 6, j = jt / TEAMS, t = jt - j * TEAMS;
+        const int col = o & 15, r = (o >> 4) & (R - 1), jt = o / (16 * R), j = jt / TEAMS, t = jt - j * TEAMS;
         const int tile = bid + G * (t + TEAMS * j), n = tile * 16 + col;
         if (tile < ntiles && n < N && r < B) {
             const float *red = s_red + ((j * NC + t * W) * R + r) * 16 + col;
@@ -1092,16 +1104,18 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_rows_kernel(co
     }
 }
 
-static size_t cu_rows_lds_bytes(const StreamGeo &g, const CuCfg &c, int P) {
+static size_t cu_rows_lds_bytes(const StreamGeo &g, const CuCfg &c, int P, int R) {
     const int Knp512 = (g.ng * kStreamUnitK + 511) & ~511;
-    size_t need = (size_t)(c.W * c.TEAMS + c.S) * ((kCuRowsNB + 1) * 512 + 8) * 2 + (size_t)kCuRows * (Knp512 + kCuRowsPad) * 2 + (size_t)(Knp512 / 128) * kCuRows * 4 +
-                  (size_t)kCuRows * 128 * 2 + (size_t)P * c.W * c.TEAMS * kCuRows * 16 * 4;
+    size_t need = (size_t)(c.W * c.TEAMS + c.S) * ((kCuRowsNB + 1) * 512 + 8) * 2 + (size_t)R * (Knp512 + kCuRowsPad) * 2 + (size_t)(Knp512 / 128) * R * 4 +
+                  (size_t)R * 128 * 2 + (size_t)P * c.W * c.TEAMS * R * 16 * 4;
     const size_t alone = 80 * 1024 + 1024;  // more than half of a compute unit's LDS: one workgroup per compute unit
     return need > alone ? need : alone;
 }
 
-// (entries 5, 6 and 8 -- more than 96 units per column, 16 wavefronts of 128 registers -- would spill with four rows' sums)
-constexpr bool cu_rows_cfg(int i) { return i != 5 && i != 6 && i != 8; }
+// (entries 5, 6 and 8 -- more than 96 units per column, 16 wavefronts of 128 registers -- would spill with four rows' sums;
+// eight rows of more than 48 units do not fit the LDS beside the wavefronts' staging pieces)
+constexpr bool cu_rows_cfg(int i, int R) { return R == 4 ? i != 5 && i != 6 && i != 8 : i <= 2 || i == 7 || i == 10; }
+static int cu_rows_tile(int B) { return B <= 4 ? 4 : 8; }
 
 bool stream_cu_rows_supported(int bits, int B, int K, int N, int C) {
     if (B < 2 || B > kCuRows || N % 8) return false;
@@ -1109,44 +1123,48 @@ bool stream_cu_rows_supported(int bits, int B, int K, int N, int C) {
     if (!stream_cu_supported(bits, K, C, Ns, 1)) return false;
     const StreamGeo geo = stream_geo(bits, K, N, C);
     const int idx = cu_pick(geo.ng, ceil_div(geo.ntiles, kCuCus));
-    if (!cu_rows_cfg(idx)) return false;
+    if (!cu_rows_cfg(idx, cu_rows_tile(B))) return false;
     const int tiles[1] = {geo.ntiles};
     const CuSplit sp = cu_split(tiles, 1, kCuCfgs[idx].TEAMS);
-    return cu_rows_lds_bytes(geo, kCuCfgs[idx], sp.walk) <= 160 * 1024;
+    return cu_rows_lds_bytes(geo, kCuCfgs[idx], sp.walk, cu_rows_tile(B)) <= 160 * 1024;
 }
 
-template <int BITS, int I>
+template <int BITS, int I, int R>
 static hipError_t launch_cu_rows_cfg(const __half *vec, const uint8_t *stream, __half *mul, int B, const StreamGeo &geo,
                                      const CuSplit &sp, int accumulate, hipStream_t s) {
     constexpr CuCfg c = kCuCfgs[I];
-    auto kern = stream_cu_rows_kernel<BITS, c.W, c.L, c.TEAMS, c.S, c.NB, c.D0, c.D>;
-    static bool raised[kCuMaxDevices] = {};
-    if (hipError_t e = cu_raise_lds(kern, raised)) return e;
-    const size_t lds = cu_rows_lds_bytes(geo, c, sp.walk);
-    hipLaunchKernelGGL(kern, dim3(sp.total), dim3(64 * (c.W * c.TEAMS + c.S)), lds, s, vec, stream, mul, geo.K, geo.C, geo.N,
-                       sp.wgs[0], accumulate, sp.walk, B);
-    return hipGetLastError();
+    if constexpr (!cu_rows_cfg(I, R)) {
+        return hipErrorInvalidValue;
+    } else {
+        auto kern = stream_cu_rows_kernel<BITS, c.W, c.L, c.TEAMS, c.S, c.NB, c.D0, c.D, R>;
+        static bool raised[kCuMaxDevices] = {};
+        if (hipError_t e = cu_raise_lds(kern, raised)) return e;
+        const size_t lds = cu_rows_lds_bytes(geo, c, sp.walk, R);
+        hipLaunchKernelGGL(kern, dim3(sp.total), dim3(64 * (c.W * c.TEAMS + c.S)), lds, s, vec, stream, mul, geo.K, geo.C, geo.N,
+                           sp.wgs[0], accumulate, sp.walk, B);
+        return hipGetLastError();
+    }
 }
 
-// vec (B, K), mul (B, N), 2 <= B <= 4; the caller has asked stream_cu_rows_supported()
+// vec (B, K), mul (B, N), 2 <= B <= 8; the caller has asked stream_cu_rows_supported()
 hipError_t launch_stream_cu_rows(int bits, const __half *vec, const uint8_t *stream, __half *mul, int B, int K, int N, int C,
                                  int accumulate, hipStream_t s) {
     const StreamGeo geo = stream_geo(bits, K, N, C);
     const int idx = cu_pick(geo.ng, ceil_div(geo.ntiles, kCuCus));
-    if (idx < 0 || !cu_rows_cfg(idx) || B < 2 || B > kCuRows) return hipErrorInvalidValue;
+    if (idx < 0 || B < 2 || B > kCuRows || !cu_rows_cfg(idx, cu_rows_tile(B))) return hipErrorInvalidValue;
     const int tiles[1] = {geo.ntiles};
     const CuSplit sp = cu_split(tiles, 1, kCuCfgs[idx].TEAMS);
     if (sp.walk > kCuMaxWalk) return hipErrorInvalidValue;
 #define CQ_ROWS_BITS(BITS_)                                                                               \
     switch (idx) {                                                                                        \
-        case 0: return launch_cu_rows_cfg<BITS_, 0>(vec, stream, mul, B, geo, sp, accumulate, s);          \
-        case 1: return launch_cu_rows_cfg<BITS_, 1>(vec, stream, mul, B, geo, sp, accumulate, s);          \
-        case 2: return launch_cu_rows_cfg<BITS_, 2>(vec, stream, mul, B, geo, sp, accumulate, s);          \
-        case 3: return launch_cu_rows_cfg<BITS_, 3>(vec, stream, mul, B, geo, sp, accumulate, s);          \
-        case 4: return launch_cu_rows_cfg<BITS_, 4>(vec, stream, mul, B, geo, sp, accumulate, s);          \
-        case 7: return launch_cu_rows_cfg<BITS_, 7>(vec, stream, mul, B, geo, sp, accumulate, s);          \
-        case 9: return launch_cu_rows_cfg<BITS_, 9>(vec, stream, mul, B, geo, sp, accumulate, s);          \
-        default: return launch_cu_rows_cfg<BITS_, 10>(vec, stream, mul, B, geo, sp, accumulate, s);        \
+        case 0: return B <= 4 ? launch_cu_rows_cfg<BITS_, 0, 4>(vec, stream, mul, B, geo, sp, accumulate, s) : launch_cu_rows_cfg<BITS_, 0, 8>(vec, stream, mul, B, geo, sp, accumulate, s);          \
+        case 1: return B <= 4 ? launch_cu_rows_cfg<BITS_, 1, 4>(vec, stream, mul, B, geo, sp, accumulate, s) : launch_cu_rows_cfg<BITS_, 1, 8>(vec, stream, mul, B, geo, sp, accumulate, s);          \
+        case 2: return B <= 4 ? launch_cu_rows_cfg<BITS_, 2, 4>(vec, stream, mul, B, geo, sp, accumulate, s) : launch_cu_rows_cfg<BITS_, 2, 8>(vec, stream, mul, B, geo, sp, accumulate, s);          \
+        case 3: return B <= 4 ? launch_cu_rows_cfg<BITS_, 3, 4>(vec, stream, mul, B, geo, sp, accumulate, s) : launch_cu_rows_cfg<BITS_, 3, 8>(vec, stream, mul, B, geo, sp, accumulate, s);          \
+        case 4: return B <= 4 ? launch_cu_rows_cfg<BITS_, 4, 4>(vec, stream, mul, B, geo, sp, accumulate, s) : launch_cu_rows_cfg<BITS_, 4, 8>(vec, stream, mul, B, geo, sp, accumulate, s);          \
+        case 7: return B <= 4 ? launch_cu_rows_cfg<BITS_, 7, 4>(vec, stream, mul, B, geo, sp, accumulate, s) : launch_cu_rows_cfg<BITS_, 7, 8>(vec, stream, mul, B, geo, sp, accumulate, s);          \
+        case 9: return B <= 4 ? launch_cu_rows_cfg<BITS_, 9, 4>(vec, stream, mul, B, geo, sp, accumulate, s) : launch_cu_rows_cfg<BITS_, 9, 8>(vec, stream, mul, B, geo, sp, accumulate, s);          \
+        default: return B <= 4 ? launch_cu_rows_cfg<BITS_, 10, 4>(vec, stream, mul, B, geo, sp, accumulate, s) : launch_cu_rows_cfg<BITS_, 10, 8>(vec, stream, mul, B, geo, sp, accumulate, s);        \
     }
     if (bits == 4) CQ_ROWS_BITS(4)
     CQ_ROWS_BITS(3)

@@ -386,7 +386,11 @@ def test_prepacked_layers_with_more_tiles_than_resident_workgroups(bits, k, n):
                                         (4, 4096, 11008, 4), (3, 4096, 11008, 3), (4, 4096, 8200, 2), (3, 4096, 32008, 4),
                                         (4, 5120, 5120, 4), (3, 5120, 13824, 4), (4, 6144, 12304, 3), (3, 8192, 8192, 4),
                                         (4, 8192, 12304, 2), (4, 11008, 4096, 4), (3, 11008, 4096, 3), (4, 12288, 4096, 4),
-                                        (3, 12288, 1032, 2), (4, 1160, 264, 4), (3, 2048, 16, 2), (4, 8192, 1024, 3)])
+                                        (3, 12288, 1032, 2), (4, 1160, 264, 4), (3, 2048, 16, 2), (4, 8192, 1024, 3),
+                                        # five to eight rows in the same kernel (layers of up to 48 units)
+                                        (4, 4096, 11008, 8), (3, 4096, 11008, 5), (4, 4096, 4096, 7), (3, 4096, 8200, 6),
+                                        (4, 5120, 5120, 8), (3, 5120, 13824, 8), (3, 6144, 12304, 7), (4, 1160, 264, 6),
+                                        (4, 4096, 32008, 8)])
 def test_prepacked_rows_against_the_c_oracle(bits, k, n, b):
     """2 to 16 activation rows over the repacked stream (compaction launch + matrix-core launch with
     real rows): against the C oracle, one-hot rows bit for bit (also with rows of very different
