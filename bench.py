@@ -460,11 +460,8 @@ def main():
                 import quant_cuda
                 base_name = quant_cuda.prepacked_kernel_name(bits, k_in, n_out, -(-k_in // 256) // 8 * 8) if k_in and n_out else ""
                 return f"{base_name or 'cq::stream_cu_kernel'}<{bits}>"
-            if k_in > 64 * args.group + 128:  # deeper than 64 units: slices of units, partial outputs added by one more launch
-                return f"cq::stream_rows_frag_kernel + cq::stream_rows_reg_kernel<{bits}, slices> + cq::rows_reduce_kernel"
-            if batch >= 8 or k_in > 32 * args.group:  # the rule of launch_stream_rows: activations in registers
-                return f"cq::stream_rows_frag_kernel + cq::stream_rows_reg_kernel<{bits}>"
-            return f"cq::stream_rows_prep_kernel + cq::stream_rows_kernel<{bits}>"
+            import quant_cuda
+            return f"{quant_cuda.prepacked_kernel_name(bits, k_in, n_out, -(-k_in // 256) // 8 * 8, rows=batch)} <{bits}-bit>"
         if batch == 1:
             return f"cq::matvec_kernel<{bits}>"
         if batch <= 4:

@@ -246,6 +246,8 @@ int cherryq_prepack_rows_recommended(int w_bits, int batch, int in_features, int
  * kernel trace (without template arguments): "cq::stream_cu_kernel" (one workgroup per compute
  * unit) or "cq::stream_kernel"; "" for shapes the entry point does not take. */
 const char *cherryq_matvec_prepacked_kernel_name(int w_bits, int in_features, int out_features, int num_cherries);
+/* The same for cherryq_matmul_prepacked_f16 with `batch` rows (2 to 16): its kernels in launch order, joined by " + ". */
+const char *cherryq_matmul_prepacked_kernel_name(int w_bits, int batch, int in_features, int out_features, int num_cherries);
 int cherryq_prepack_f16(int w_bits, const uint8_t *qweight, const void *cherry_weight, const int16_t *cherry_indices,
                         const void *scales, void *stream, size_t stream_bytes, int in_features, int out_features,
                         int num_cherries, int group_size, void *hip_stream);
@@ -259,7 +261,10 @@ int cherryq_matvec_prepacked_f16(int w_bits, const void *vec, const void *stream
 /*
  * The same over 2 to 16 activation rows (vec (batch, in_features), mul (batch, out_features)): the
  * matrix-core tile that the one-row kernel fills with copies of one row takes 16 different rows
- * at the same price, still without split-K or workspace.  The compacted activations of all rows
+ * at the same price, still without split-K or workspace.  Two to four rows (layers of up to 96
+ * units of 128 input channels) and five to eight rows (up to 48 units) run in the one-row kernel's
+ * own launch shape, tile row m holding activation row m mod 4 or 8: one launch, the scratch buffer
+ * is not touched.  Otherwise the compacted activations of all rows
  * are brought into matrix-core operand order once (a first small launch into an uninitialised
  * scratch buffer of cherryq_prepacked_scratch_bytes() bytes, 256-byte aligned; for up to 4 rows
  * inside the main launch) and then stay in LDS or in registers while a workgroup walks its

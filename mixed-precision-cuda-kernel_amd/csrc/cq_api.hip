@@ -436,6 +436,12 @@ const char *cherryq_matvec_prepacked_kernel_name(int w_bits, int in_features, in
     return cq::stream_uses_cu(w_bits, in_features, out_features, num_cherries) ? "cq::stream_cu_kernel" : "cq::stream_kernel";
 }
 
+const char *cherryq_matmul_prepacked_kernel_name(int w_bits, int batch, int in_features, int out_features, int num_cherries) {
+    if (batch == 1) return cherryq_matvec_prepacked_kernel_name(w_bits, in_features, out_features, num_cherries);
+    if (!cq::stream_rows_supported(w_bits, batch, in_features, out_features, num_cherries, cq::kStreamUnitK)) return "";
+    return cq::stream_rows_kernel_name(w_bits, batch, in_features, out_features, num_cherries);
+}
+
 static int prepack_check(int w_bits, int K, int N, int C, int G, size_t stream_bytes_given) {
     if (w_bits != 3 && w_bits != 4) return CHERRYQ_E_BITS;
     if (K <= 0 || N <= 0 || C < 0 || C >= K || K % 8 || N % 8 || C % 8) return CHERRYQ_E_SHAPE;

@@ -132,6 +132,7 @@ bool stream_group_supported(int bits, int K, int C, int G, const int *Ns, int co
 bool stream_cu_rows_supported(int bits, int B, int K, int N, int C);
 hipError_t launch_stream_cu_rows(int bits, const __half *vec, const uint8_t *stream, __half *mul, int B, int K, int N, int C,
                                  int accumulate, hipStream_t s);
+const char *stream_rows_kernel_name(int bits, int B, int K, int N, int C);
 size_t stream_rows_scratch_bytes(int bits, int B, int K, int N, int C);
 bool stream_rows_supported(int bits, int B, int K, int N, int C, int G);
 hipError_t launch_stream_rows(int bits, const __half *vec, const uint8_t *stream, __half *mul, int B, int K, int N,

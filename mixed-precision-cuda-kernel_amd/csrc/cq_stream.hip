@@ -1589,12 +1589,23 @@ static hipError_t launch_rows_cfg(const unsigned short *xs, const float *xsum, c
     return hipGetLastError();
 }
 
+// the kernels launch_stream_rows runs for a shape, as a profiler's kernel trace names them
+const char *stream_rows_kernel_name(int bits, int B, int K, int N, int C) {
+    const StreamGeo geo = stream_geo(bits, K, N, C);
+    if (stream_cu_rows_supported(bits, B, K, N, C)) return "cq::stream_cu_rows_kernel";
+    if (rows_slices(geo) > 1) return "cq::stream_rows_frag_kernel + cq::stream_rows_reg_kernel (slices of units) + cq::rows_reduce_kernel";
+    if (B >= 8 || geo.ng > 32 || rows_lds_bytes(B, geo, 8, false) > 160 * 1024)
+        return "cq::stream_rows_frag_kernel + cq::stream_rows_reg_kernel";
+    return B <= 4 ? "cq::stream_rows_kernel (rows staged in the launch)" : "cq::stream_rows_prep_kernel + cq::stream_rows_kernel";
+}
+
 // vec (B, K), mul (B, N), 2 <= B <= 16; scratch: stream_rows_scratch_bytes(), 256-byte aligned
 hipError_t launch_stream_rows(int bits, const __half *vec, const uint8_t *stream, __half *mul, int B, int K, int N,
                               int C, int accumulate, void *scratch, hipStream_t s) {
     const StreamGeo geo = stream_geo(bits, K, N, C);
-    static const bool cu_rows_off = getenv("CHERRYQ_CU_ROWS_OFF") != nullptr;
-    if (!cu_rows_off && stream_cu_rows_supported(bits, B, K, N, C))
+    // two to eight rows in the one-workgroup-per-compute-unit shape where it takes the layer: no launch in
+    // front, no scratch (4096 -> 11008, us: 2 rows 9.9 -> 6.6, 4 rows 10.5 -> 7.4, 8 rows 11.7 -> 8.6)
+    if (stream_cu_rows_supported(bits, B, K, N, C))
         return launch_stream_cu_rows(bits, vec, stream, mul, B, K, N, C, accumulate, s);
     // Two main kernels.  Measured (us, whole call, 4-bit; rows in LDS / rows in registers): 4096 -> 11008
     // 5 rows 12.0 / 12.4, 8 rows 12.4 / 12.5, 16 rows 14.1 / 12.6; 4096 -> 4096 8 rows 9.9 / 9.4, 16 rows

@@ -401,10 +401,10 @@ def prepacked_rows_recommended(w_bits, rows, in_features, out_features, num_cher
                                                       int(num_cherries), int(group_size)))
 
 
-def prepacked_kernel_name(w_bits, in_features, out_features, num_cherries) -> str:
-    """The kernel matvec_prepacked_cherryq launches for a one-row call on this layer, as a profiler names it."""
-    _lib.cherryq_matvec_prepacked_kernel_name.restype = ctypes.c_char_p
-    return _lib.cherryq_matvec_prepacked_kernel_name(int(w_bits), int(in_features), int(out_features),
+def prepacked_kernel_name(w_bits, in_features, out_features, num_cherries, rows=1) -> str:
+    """The kernels matvec_prepacked_cherryq launches for a call of `rows` rows on this layer, as a profiler names them."""
+    _lib.cherryq_matmul_prepacked_kernel_name.restype = ctypes.c_char_p
+    return _lib.cherryq_matmul_prepacked_kernel_name(int(w_bits), int(rows), int(in_features), int(out_features),
                                                      int(num_cherries)).decode()
 
 
