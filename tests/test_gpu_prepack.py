@@ -390,7 +390,9 @@ def test_prepacked_layers_with_more_tiles_than_resident_workgroups(bits, k, n):
                                         # five to eight rows in the same kernel (layers of up to 48 units)
                                         (4, 4096, 11008, 8), (3, 4096, 11008, 5), (4, 4096, 4096, 7), (3, 4096, 8200, 6),
                                         (4, 5120, 5120, 8), (3, 5120, 13824, 8), (3, 6144, 12304, 7), (4, 1160, 264, 6),
-                                        (4, 4096, 32008, 8)])
+                                        (4, 4096, 32008, 8),
+                                        # fewer units per column than a team has wavefronts
+                                        (4, 392, 24, 3), (3, 136, 8, 8), (4, 520, 40, 16)])
 def test_prepacked_rows_against_the_c_oracle(bits, k, n, b):
     """2 to 16 activation rows over the repacked stream (compaction launch + matrix-core launch with
     real rows): against the C oracle, one-hot rows bit for bit (also with rows of very different
