@@ -80,6 +80,38 @@ def test_weight_stream_shapes_taken_and_refused(lib):
     assert f(4, 1, 4096, n_ok + 16, 16, 128) == 0
 
 
+def test_small_batch_routing_over_the_weight_stream(lib):
+    """cherryq_prepack_rows_recommended / cherryq_matmul_prepacked_kernel_name are host arithmetic:
+    which row counts a caller with both layouts sends to the stream, and the kernels that serve
+    them (the LLaMA-7B / 13B / 70B layer shapes with their 1/256 cherry channels)."""
+    rec = lib.cherryq_prepack_rows_recommended
+    name = lib.cherryq_matmul_prepacked_kernel_name
+    name.restype = ctypes.c_char_p
+    name.argtypes = [ctypes.c_int] * 5
+    cherries = lambda k: -(-k // 256) // 8 * 8
+    for bits in (3, 4):
+        # up to 48 units of 128 channels: 2 to 8 rows in the one-row kernel's launch shape
+        for k, n in ((4096, 4096), (4096, 11008), (5120, 5120), (5120, 13824)):
+            for b in range(1, 17):
+                assert rec(bits, b, k, n, cherries(k), 128) == 1, (bits, b, k, n)
+            for b in (2, 4, 5, 8):
+                assert name(bits, b, k, n, cherries(k)) == b"cq::stream_cu_rows_kernel", (bits, b, k, n)
+            assert b"stream_rows_reg_kernel" in name(bits, 9, k, n, cherries(k))
+        # 64 to 96 units: 2 to 4 rows there, 5 to 7 stay on the checkpoint layout, 8 to 16 on the older stream kernels
+        for k, n in ((8192, 8192), (8192, 28672), (11008, 4096)):
+            got = [rec(bits, b, k, n, cherries(k), 128) for b in range(1, 18)]
+            assert got == [1, 1, 1, 1, 0, 0, 0] + [1] * 9 + [0], (bits, k, n, got)
+            assert name(bits, 3, k, n, cherries(k)) == b"cq::stream_cu_rows_kernel"
+        assert b"rows_reduce_kernel" in name(bits, 16, 11008, 4096, cherries(11008))
+        # deeper: only 8 to 16 rows, in slices of units
+        for k, n in ((13824, 5120), (28672, 8192)):
+            got = [rec(bits, b, k, n, cherries(k), 128) for b in range(1, 18)]
+            assert got == [1, 0, 0, 0, 0, 0, 0] + [1] * 9 + [0], (bits, k, n, got)
+            assert b"rows_reduce_kernel" in name(bits, 8, k, n, cherries(k))
+    assert rec(4, 4, 4096, 4096, 16, 64) == 0 and rec(5, 4, 4096, 4096, 16, 128) == 0
+    assert name(4, 17, 4096, 4096, 16) == b"" and name(4, 1, 4096, 4096, 16) == b"cq::stream_cu_kernel"
+
+
 def _call(fn, *, vec=0x1000, qw=0x1000, cw=0x1000, idx=0x1000, sc=0x1000, mul=0x1000, b=1, k=4096, n=4096,
           c=16, g=128, acc=1, ws=0x1000, wsb=1 << 30, scr=None, scrb=0, stream=None):
     fn.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 6 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
