@@ -263,8 +263,8 @@ int cherryq_matvec_prepacked_f16(int w_bits, const void *vec, const void *stream
  * matrix-core tile that the one-row kernel fills with copies of one row takes 16 different rows
  * at the same price, still without split-K or workspace.  Two to four rows (layers of up to 96
  * units of 128 input channels) and five to eight rows (up to 48 units) run in the one-row kernel's
- * own launch shape, tile row m holding activation row m mod 4 or 8: one launch, the scratch buffer
- * is not touched.  Otherwise the compacted activations of all rows
+ * own launch shape, tile row m holding activation row m mod 4 or 8: one launch, no scratch buffer
+ * (cherryq_prepacked_scratch_bytes() is 0 and scratch may be NULL).  Otherwise the compacted activations of all rows
  * are brought into matrix-core operand order once (a first small launch into an uninitialised
  * scratch buffer of cherryq_prepacked_scratch_bytes() bytes, 256-byte aligned; for up to 4 rows
  * inside the main launch) and then stay in LDS or in registers while a workgroup walks its

@@ -507,9 +507,8 @@ int cherryq_matmul_prepacked_f16(int w_bits, const void *vec, const void *stream
         return CHERRYQ_E_UNSUPPORTED;
     if (!vec || !stream || !mul) return CHERRYQ_E_NULL;
     if (!cq::aligned(stream, 256) || !cq::aligned(vec, 16) || !cq::aligned(mul, 2)) return CHERRYQ_E_ALIGN;
-    if (!scratch || !cq::aligned(scratch, 256) ||
-        scratch_bytes < cq::stream_rows_scratch_bytes(w_bits, batch, in_features, out_features, num_cherries))
-        return CHERRYQ_E_WORKSPACE;
+    const size_t need = cq::stream_rows_scratch_bytes(w_bits, batch, in_features, out_features, num_cherries);
+    if (need && (!scratch || !cq::aligned(scratch, 256) || scratch_bytes < need)) return CHERRYQ_E_WORKSPACE;
     return (int)cq::launch_stream_rows(w_bits, reinterpret_cast<const __half *>(vec), reinterpret_cast<const uint8_t *>(stream),
                                        reinterpret_cast<__half *>(mul), batch, in_features, out_features, num_cherries,
                                        accumulate, scratch, reinterpret_cast<hipStream_t>(hip_stream));

@@ -1547,7 +1547,7 @@ constexpr int kRowsMaxSlices = 4;
 static int rows_slices(const StreamGeo &g) { return g.ng <= 64 ? 1 : kRowsMaxSlices; }
 
 size_t stream_rows_scratch_bytes(int bits, int B, int K, int N, int C) {
-    if (B < 2) return 0;
+    if (B < 2 || stream_cu_rows_supported(bits, B, K, N, C)) return 0;  // (one row, or the rows staged inside the one launch)
     const StreamGeo geo = stream_geo(bits, K, N, C);
     const int ks = rows_slices(geo);
     if (ks > 1) return rows_frag(geo).total + (size_t)ks * 16 * N * 4;  // the operands, then the slices' fp32 partial outputs

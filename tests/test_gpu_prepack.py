@@ -239,16 +239,21 @@ def test_prepacked_c_abi_rejections(qc):
     # the entry point for 2 to 16 rows: needs its scratch buffer
     lib.cherryq_prepacked_scratch_bytes.restype = ctypes.c_size_t
     g = lib.cherryq_matmul_prepacked_f16
-    x4 = torch.zeros(4, 4096, dtype=torch.float16, device="cuda")
-    y4 = torch.zeros(4, 1024, dtype=torch.float16, device="cuda")
-    need = lib.cherryq_prepacked_scratch_bytes(4, 4, 4096, 1024, 16)
-    assert need >= 4 * 4096 * 2 and lib.cherryq_prepacked_scratch_bytes(4, 1, 4096, 1024, 16) == 0
+    x4 = torch.zeros(12, 4096, dtype=torch.float16, device="cuda")
+    y4 = torch.zeros(12, 1024, dtype=torch.float16, device="cuda")
+    need = lib.cherryq_prepacked_scratch_bytes(4, 12, 4096, 1024, 16)
+    assert need >= 12 * 4096 * 2 and lib.cherryq_prepacked_scratch_bytes(4, 1, 4096, 1024, 16) == 0
     sc = torch.empty(need, dtype=torch.uint8, device="cuda")
-    assert g(4, x4.data_ptr(), buf.data_ptr(), nbytes, y4.data_ptr(), 4, 4096, 1024, 16, 0, None, 0, None) == -4
-    assert g(4, x4.data_ptr(), buf.data_ptr(), nbytes, y4.data_ptr(), 4, 4096, 1024, 16, 0, sc.data_ptr(), need - 1, None) == -4
+    assert g(4, x4.data_ptr(), buf.data_ptr(), nbytes, y4.data_ptr(), 12, 4096, 1024, 16, 0, None, 0, None) == -4
+    assert g(4, x4.data_ptr(), buf.data_ptr(), nbytes, y4.data_ptr(), 12, 4096, 1024, 16, 0, sc.data_ptr(), need - 1, None) == -4
     assert g(4, x4.data_ptr(), buf.data_ptr(), nbytes, y4.data_ptr(), 17, 4096, 1024, 16, 0, sc.data_ptr(), need, None) == -7
-    assert g(4, x4.data_ptr(), buf.data_ptr(), nbytes, y4.data_ptr(), 4, 4096, 1024, 16, 0, sc.data_ptr(), need, None) == 0
-    assert g(4, x4.data_ptr() + 2, buf.data_ptr(), nbytes, y4.data_ptr(), 3, 4096, 1024, 16, 0, sc.data_ptr(), need, None) == -6
+    assert g(4, x4.data_ptr(), buf.data_ptr(), nbytes, y4.data_ptr(), 12, 4096, 1024, 16, 0, sc.data_ptr(), need, None) == 0
+    assert g(4, x4.data_ptr() + 2, buf.data_ptr(), nbytes, y4.data_ptr(), 11, 4096, 1024, 16, 0, sc.data_ptr(), need, None) == -6
+    # two to eight rows on this layer run in one launch: no scratch buffer
+    for rows in (2, 4, 8):
+        assert lib.cherryq_prepacked_scratch_bytes(4, rows, 4096, 1024, 16) == 0
+        assert g(4, x4.data_ptr(), buf.data_ptr(), nbytes, y4.data_ptr(), rows, 4096, 1024, 16, 0, None, 0, None) == 0
+    assert g(4, x4.data_ptr() + 2, buf.data_ptr(), nbytes, y4.data_ptr(), 3, 4096, 1024, 16, 0, None, 0, None) == -6
     assert g(4, x.data_ptr(), buf.data_ptr(), nbytes, y.data_ptr(), 1, 4096, 1024, 16, 0, None, 0, None) == 0
     torch.cuda.synchronize()
 
