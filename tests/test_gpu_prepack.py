@@ -444,6 +444,49 @@ def test_prepacked_rows_against_the_c_oracle(bits, k, n, b):
         np.testing.assert_array_equal(run(e), c_oracle.fused(e, p, bits, 128).astype(np.float16))
 
 
+def test_prepacked_rows_on_random_small_layers(qc):
+    """1 to 16 rows over randomly drawn small layers -- input widths that are no multiple of 512,
+    0 to 128 cherry channels at random places (neighbours, the first and the last columns), widths
+    that end inside a tile -- against the C oracle, and one-hot rows bit for bit."""
+    rng = np.random.default_rng(2024)
+    done = 0
+    for case in range(60):
+        bits = int(rng.choice([3, 4]))
+        c = int(rng.choice([0, 8, 16, 24, 40, 64, 96, 128]))
+        k = int(rng.integers(17 + c // 8, 420)) * 8
+        n = int(rng.integers(1, 90)) * 8
+        b = int(rng.integers(1, 17))
+        if k - c < 8:
+            continue
+        frac = (c + 0.5) / k if c else 1e-9
+        p = orc.synthetic_packed_fast(k, n, bits, 128, seed=1000 + case, cherry_fraction=frac)
+        if p["cherry_indices"].shape[0] != c or not qc.prepack_supported(bits, b, k, n, c, 128):
+            continue
+        if c and case % 3 == 0:   # neighbours at both ends of the row
+            idx = np.sort(np.unique(np.concatenate([np.arange(min(4, c)), k - 1 - np.arange(min(3, c)),
+                                                    p["cherry_indices"].astype(np.int64)]))[:c]).astype(np.int16)
+            if idx.shape[0] == c:
+                p["cherry_indices"] = idx
+        announce("random small layer", bits, k, n, c, b)
+        stream = prepack(qc, bits, p, k)
+        x = rng.standard_normal((b, k)).astype(np.float16)
+        out = torch.full((b, n), float("nan"), dtype=torch.float16, device="cuda")
+        qc.matvec_prepacked_cherryq(bits, torch.from_numpy(x).cuda(), stream, out, k, c)
+        torch.cuda.synchronize()
+        got, want = out.cpu().numpy(), c_oracle.fused(x, p, bits, 128)
+        for r in range(b):
+            assert orc.rel_l2(got[r], want[r]) <= TOL, (case, bits, k, n, c, b, r)
+        e = np.zeros((b, k), dtype=np.float16)
+        for r in range(b):
+            e[r, int(rng.integers(0, k))] = np.float16(2.0 ** int(rng.integers(-4, 4)))
+        qc.matvec_prepacked_cherryq(bits, torch.from_numpy(e).cuda(), stream, out, k, c)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(out.cpu().numpy(), c_oracle.fused(e, p, bits, 128).astype(np.float16),
+                                      err_msg=str((case, bits, k, n, c, b)))
+        done += 1
+    assert done >= 30, done
+
+
 def test_quantlinear_routes_rows_to_the_stream_after_prepack():
     """QuantLinear.forward after prepack(): 1 to 16 rows run over the weight stream (also with the
     checkpoint-layout buffers released), 17 rows on the checkpoint layout; all agree with the
