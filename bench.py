@@ -51,9 +51,13 @@ MEASURED_TRAFFIC = {("llama7b_gate_up_w4", 1, "reference"): 25320960,
                     ("llama7b_gate_up_w4", 1, "prepacked"): 23834070}
 
 
-# Matrix-core busy share of the 16-row kernels from rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES runs (busy
+# Matrix-core busy share of the 8- and 16-row kernels from rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES runs (busy
 # cycles / (kernel time x 2.4 GHz x 1024 SIMDs)); like the traffic figure it cannot be read while timing.
-MFMA_BUSY = {"llama70b_gate_up_w4": {"frac": 0.123, "kernel": "cq::stream_rows_reg_kernel<4, 8, 8, 1>",
+MFMA_BUSY = {("llama13b_gate_up_w3", 8): {"frac": 0.092, "kernel": "cq::stream_cu_rows_kernel<3, 4, 12, 3, 4, 3, 3, 4, 8>",
+                                          "profile": "profiles/stream_cu_rows_w3_w4_llama13b_llama7b_gate_up_rows4_rows8.md"},
+             ("llama13b_attn_w3", 8): {"frac": 0.057, "kernel": "cq::stream_cu_rows_kernel<3, 5, 8, 2, 6, 2, 3, 4, 8>",
+                                       "profile": "profiles/stream_cu_rows_w3_w4_llama13b_llama7b_gate_up_rows4_rows8.md"},
+             "llama70b_gate_up_w4": {"frac": 0.123, "kernel": "cq::stream_rows_reg_kernel<4, 8, 8, 1>",
                                      "profile": "profiles/rows16_w4_llama70b_gate_up_8192x28672_stream.md"},
              "llama70b_down_w4": {"frac": 0.135, "kernel": "cq::stream_rows_reg_kernel<4, 8, 8, 1, true>",
                                   "profile": "profiles/rows16_w4_llama70b_down_28672x8192_stream.md"}}
@@ -569,7 +573,7 @@ def main():
             # 3 bits at batch 1 / 4 / 8 (config 3), the LLaMA-70B shapes in 4 bits at batch 1 / 16 (config 4)
             result["config1_down"] = [side_record("llama7b_down_w4"), side_record("llama7b_down_w3")]
             result["config3"] = {"batch1": [side_record(w) for w in ("llama13b_attn_w3", "llama13b_gate_up_w3", "llama13b_down_w3")],
-                                 "batched": [batch_record(w, b) for w in ("llama13b_attn_w3", "llama13b_gate_up_w3") for b in (4, 8)]}
+                                 "batched": [batch_record(w, b, MFMA_BUSY.get((w, b))) for w in ("llama13b_attn_w3", "llama13b_gate_up_w3") for b in (4, 8)]}
             result["config4"] = {"batch1": [side_record(w) for w in ("llama70b_attn_w4", "llama70b_kv_w4", "llama70b_gate_up_w4",
                                                                      "llama70b_down_w4")],
                                  "batch16": [batch_record("llama70b_gate_up_w4", 16, MFMA_BUSY.get("llama70b_gate_up_w4")),
