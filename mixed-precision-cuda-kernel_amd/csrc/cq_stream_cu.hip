@@ -857,11 +857,13 @@ constexpr int kCuRowsPad = 8;  // halves between the compacted rows in LDS: the 
 
 // R = 8: A row m holds activation row m % 8, lane groups kq and kq ^ 2 receive the same four rows
 // (4 (kq & 1) + r) and share the units' scales half each.
-template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, int R>
+// WALK: some team takes more than one tile (the requests of the next tile then join the ring).
+template <int BITS, int W, int L, int TEAMS, int S, int NB, int D0, int D, int R, bool WALK>
 __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_rows_kernel(const __half *__restrict__ x,
                                                                                const uint8_t *__restrict__ stream,
                                                                                __half *__restrict__ mul, int K, int C, int N,
-                                                                               int G, int accumulate, int P, int B) {
+                                                                               int G, int accumulate, int Pw, int B) {
+    const int P = WALK ? Pw : 1;
     static_assert(R == 4 || R == 8, "rows per matrix-core tile");
     constexpr int NRED = 16 / R;   // lane groups that receive the same rows: they share the units' scales
     constexpr int NC = W * TEAMS;
@@ -1040,14 +1042,14 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_rows_kernel(co
 #pragma unroll 1
         for (int j = 0; j < P; j++) {
             const int tnext = tcur + tstride;
-            const bool vnext = tnext < ntiles;
+            const bool vnext = WALK && tnext < ntiles;
             const uint32_t tbn = (uint32_t)tnext * record_bytes;
             sf4_t dc = {0.f, 0.f, 0.f, 0.f};
             if (cherry_wave) {
 #pragma unroll
                 for (int q = 0; q < 4; q++)
                     if (32 * q < C) dc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(ca[q]), as_h8(cw[q]), dc, 0, 0, 0);
-                load_cherry(tbn, vnext);
+                if constexpr (WALK) load_cherry(tbn, vnext);
             }
             sf4_t tt = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -1058,10 +1060,12 @@ __global__ __launch_bounds__(64 * (W * TEAMS + S)) void stream_cu_rows_kernel(co
                 const su4 w = wbuf[i % D];
                 const sf4_t v = unit_dot_rows<BITS>(w, xs_l + up * kStreamUnitK);
                 if (i + D < L) wbuf[i % D] = load_unit(i + D, tb, vcur);
-                else wbuf[i % D] = load_unit(i + D - L, tbn, vnext);
+                else if constexpr (WALK) wbuf[i % D] = load_unit(i + D - L, tbn, vnext);
                 const sf4_t xsum = *reinterpret_cast<const sf4_t *>(xsum_l + up * R);
                 tt += (v + kGrid * xsum) * sf;
-                if ((i % NRED) == NRED - 1) sc[i / NRED] = load_scale(i / NRED, tbn, vnext);
+                if constexpr (WALK) {
+                    if ((i % NRED) == NRED - 1) sc[i / NRED] = load_scale(i / NRED, tbn, vnext);
+                }
             }
             // the shares of the lane groups that hold the same rows; every lane then stores R / 4 of its rows
             float fin[4];
@@ -1136,12 +1140,19 @@ static hipError_t launch_cu_rows_cfg(const __half *vec, const uint8_t *stream, _
     if constexpr (!cu_rows_cfg(I, R)) {
         return hipErrorInvalidValue;
     } else {
-        auto kern = stream_cu_rows_kernel<BITS, c.W, c.L, c.TEAMS, c.S, c.NB, c.D0, c.D, R>;
-        static bool raised[kCuMaxDevices] = {};
-        if (hipError_t e = cu_raise_lds(kern, raised)) return e;
         const size_t lds = cu_rows_lds_bytes(geo, c, sp.walk, R);
-        hipLaunchKernelGGL(kern, dim3(sp.total), dim3(64 * (c.W * c.TEAMS + c.S)), lds, s, vec, stream, mul, geo.K, geo.C, geo.N,
-                           sp.wgs[0], accumulate, sp.walk, B);
+        const dim3 grid(sp.total), block(64 * (c.W * c.TEAMS + c.S));
+        if (sp.walk > 1) {
+            auto kern = stream_cu_rows_kernel<BITS, c.W, c.L, c.TEAMS, c.S, c.NB, c.D0, c.D, R, true>;
+            static bool raised[kCuMaxDevices] = {};
+            if (hipError_t e = cu_raise_lds(kern, raised)) return e;
+            hipLaunchKernelGGL(kern, grid, block, lds, s, vec, stream, mul, geo.K, geo.C, geo.N, sp.wgs[0], accumulate, sp.walk, B);
+        } else {
+            auto kern = stream_cu_rows_kernel<BITS, c.W, c.L, c.TEAMS, c.S, c.NB, c.D0, c.D, R, false>;
+            static bool raised[kCuMaxDevices] = {};
+            if (hipError_t e = cu_raise_lds(kern, raised)) return e;
+            hipLaunchKernelGGL(kern, grid, block, lds, s, vec, stream, mul, geo.K, geo.C, geo.N, sp.wgs[0], accumulate, sp.walk, B);
+        }
         return hipGetLastError();
     }
 }
